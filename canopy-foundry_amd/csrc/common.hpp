@@ -1,0 +1,151 @@
+// Shared device helpers for the gfx950 FP8 kernels: bf16 <-> f32, OCP fp8
+// encode/decode, wavefront (64-lane) reductions, launch bookkeeping.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "cf_fp8.h"
+
+#ifndef __gfx950__
+#if defined(__HIP_DEVICE_COMPILE__)
+#error "this library is written for gfx950 (MI355X) only"
+#endif
+#endif
+
+namespace cf {
+
+constexpr int kWave = 64;
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ float bf16_to_f32(uint16_t b) { return __uint_as_float(static_cast<uint32_t>(b) << 16); }
+__device__ __forceinline__ float bf16_lo(uint32_t pair) { return __uint_as_float(pair << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t pair) { return __uint_as_float(pair & 0xffff0000u); }
+
+// Round-to-nearest-even, NaN kept quiet.
+__device__ __forceinline__ uint16_t f32_to_bf16(float v) {
+    const uint32_t bits = __float_as_uint(v);
+    if ((bits & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((bits >> 16) | 0x0040u);
+    return static_cast<uint16_t>((bits + 0x7fffu + ((bits >> 16) & 1u)) >> 16);
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    return static_cast<uint32_t>(f32_to_bf16(lo)) | (static_cast<uint32_t>(f32_to_bf16(hi)) << 16);
+}
+
+// ---- OCP fp8 encode -------------------------------------------------------
+// gfx950's v_cvt_pk_{fp8,bf8}_f32 round to nearest even onto OCP e4m3fn / e5m2.
+// Saturation to the largest finite value is applied here by clamping first
+// (v_med3_f32); NaN is restored afterwards as sign|0x7f.
+template <bool E5M2>
+__device__ __forceinline__ float fp8_clamp(float v) {
+    constexpr float m = E5M2 ? 57344.0f : 448.0f;
+    return __builtin_amdgcn_fmed3f(v, -m, m);
+}
+__device__ __forceinline__ uint32_t nan_fix(uint32_t packed, float v, int byte) {
+    if (v != v) {
+        const uint32_t code = ((__float_as_uint(v) >> 24) & 0x80u) | 0x7fu;
+        packed = (packed & ~(0xffu << (8 * byte))) | (code << (8 * byte));
+    }
+    return packed;
+}
+// four floats -> four fp8 bytes, byte i holds v_i
+template <bool E5M2>
+__device__ __forceinline__ uint32_t cvt4_fp8(float a, float b, float c, float d) {
+    int r = 0;
+    if constexpr (E5M2) {
+        r = __builtin_amdgcn_cvt_pk_bf8_f32(fp8_clamp<true>(a), fp8_clamp<true>(b), r, false);
+        r = __builtin_amdgcn_cvt_pk_bf8_f32(fp8_clamp<true>(c), fp8_clamp<true>(d), r, true);
+    } else {
+        r = __builtin_amdgcn_cvt_pk_fp8_f32(fp8_clamp<false>(a), fp8_clamp<false>(b), r, false);
+        r = __builtin_amdgcn_cvt_pk_fp8_f32(fp8_clamp<false>(c), fp8_clamp<false>(d), r, true);
+    }
+    uint32_t u = static_cast<uint32_t>(r);
+    u = nan_fix(u, a, 0); u = nan_fix(u, b, 1); u = nan_fix(u, c, 2); u = nan_fix(u, d, 3);
+    return u;
+}
+template <bool E5M2>
+__device__ __forceinline__ uint8_t cvt1_fp8(float a) {
+    return static_cast<uint8_t>(cvt4_fp8<E5M2>(a, 0.0f, 0.0f, 0.0f) & 0xffu);
+}
+
+// ---- fp8 decode (exact) -----------------------------------------------------
+__device__ __forceinline__ float e4m3_to_f32(uint8_t b) {
+    const uint32_t sign = (static_cast<uint32_t>(b) & 0x80u) << 24;
+    const uint32_t e = (b >> 3) & 0xfu, m = b & 7u;
+    float mag;
+    if (e == 0) mag = static_cast<float>(m) * 0.001953125f;           // m * 2^-9
+    else if (e == 15 && m == 7) mag = __uint_as_float(0x7fc00000u);
+    else mag = __uint_as_float(((e + 120u) << 23) | (m << 20));
+    return __uint_as_float(__float_as_uint(mag) | sign);
+}
+__device__ __forceinline__ float e5m2_to_f32(uint8_t b) {
+    const uint32_t sign = (static_cast<uint32_t>(b) & 0x80u) << 24;
+    const uint32_t e = (b >> 2) & 0x1fu, m = b & 3u;
+    float mag;
+    if (e == 0) mag = static_cast<float>(m) * 1.52587890625e-05f;     // m * 2^-16
+    else if (e == 31) mag = __uint_as_float(m == 0 ? 0x7f800000u : 0x7fc00000u);
+    else mag = __uint_as_float(((e + 112u) << 23) | (m << 21));
+    return __uint_as_float(__float_as_uint(mag) | sign);
+}
+
+// ---- 64-lane wavefront reductions ------------------------------------------
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+__device__ __forceinline__ int wave_sum_i(int v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+// |x| >= 0 orders like its bit pattern, so an integer max is a float max.
+__device__ __forceinline__ void atomic_max_nonneg(float* addr, float v) {
+    atomicMax(reinterpret_cast<int*>(addr), __float_as_int(v));
+}
+
+// ---- deterministic expf ------------------------------------------------------
+// Cody-Waite reduction + degree-6 polynomial with explicit FMAs and exact
+// power-of-two scaling.  Uses only IEEE-exact operations so that a host
+// restatement of the same steps yields the same bits.
+__device__ __forceinline__ float det_expf(float x) {
+    if (x != x) return x;
+    if (x > 88.72284f) return __uint_as_float(0x7f800000u);
+    if (x < -103.97208f) return 0.0f;
+    const float k = __builtin_rintf(x * 1.44269504f);
+    float r = __builtin_fmaf(k, -0.693359375f, x);
+    r = __builtin_fmaf(k, 2.12194440e-4f, r);
+    float p = 1.9875691500e-4f;
+    p = __builtin_fmaf(p, r, 1.3981999507e-3f);
+    p = __builtin_fmaf(p, r, 8.3334519073e-3f);
+    p = __builtin_fmaf(p, r, 4.1665795894e-2f);
+    p = __builtin_fmaf(p, r, 1.6666665459e-1f);
+    p = __builtin_fmaf(p, r, 5.0000001201e-1f);
+    p = __builtin_fmaf(p, r * r, r);
+    p = p + 1.0f;
+    const int ki = static_cast<int>(k);
+    if (ki < -126) return (p * __uint_as_float(static_cast<uint32_t>(ki + 227) << 23)) * 7.8886090522101181e-31f;
+    if (ki > 127) return (p * __uint_as_float(static_cast<uint32_t>(ki + 126) << 23)) * 2.0f;
+    return p * __uint_as_float(static_cast<uint32_t>(ki + 127) << 23);
+}
+__device__ __forceinline__ float stable_sigmoid(float x) {
+    if (x >= 0.0f) return 1.0f / (1.0f + det_expf(-x));
+    const float e = det_expf(x);
+    return e / (1.0f + e);
+}
+
+// ---- host-side launch helpers ----------------------------------------------
+inline hipStream_t as_stream(cf_stream_t s) { return static_cast<hipStream_t>(s); }
+inline int launch_status() {
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CF_OK : static_cast<int>(e);
+}
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline unsigned ceil_div(size_t a, size_t b) { return static_cast<unsigned>((a + b - 1) / b); }
+
+}  // namespace cf

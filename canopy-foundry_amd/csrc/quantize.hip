@@ -1,0 +1,629 @@
+// FP8 quantize family for gfx950: amax reduction, scale derivation, E4M3/E5M2
+// quantize (plain, recording, per-row, per-1x128, per-128x128, fp32 input),
+// delayed-scale history, clip probes, raw-byte E4M3 pack/unpack.
+//
+// All bulk kernels are HBM-bound: a lane moves 16 elements per step through
+// two 128-bit loads and one 128-bit store, a wavefront reduces with xor
+// shuffles, and a workgroup issues one atomic.
+#include "common.hpp"
+
+namespace cf {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kVec = 16;            // elements per lane per step
+constexpr unsigned kMaxBlocks = 4096;
+
+__device__ __forceinline__ float block_max(float v, float* sh) {
+    v = wave_max(v);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0) sh[wave] = v;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float m = sh[0];
+        for (int w = 1; w < (int)(blockDim.x >> 6); ++w) m = fmaxf(m, sh[w]);
+        sh[0] = m;
+    }
+    __syncthreads();
+    return sh[0];
+}
+
+struct Vec16 { uint4 lo, hi; };   // 16 bf16
+
+__device__ __forceinline__ Vec16 load16(const uint16_t* p) {
+    Vec16 v;
+    v.lo = *reinterpret_cast<const uint4*>(p);
+    v.hi = *reinterpret_cast<const uint4*>(p + 8);
+    return v;
+}
+__device__ __forceinline__ float amax16(const Vec16& v) {
+    const uint32_t w[8] = {v.lo.x, v.lo.y, v.lo.z, v.lo.w, v.hi.x, v.hi.y, v.hi.z, v.hi.w};
+    float m = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        m = fmaxf(m, fabsf(bf16_lo(w[i])));
+        m = fmaxf(m, fabsf(bf16_hi(w[i])));
+    }
+    return m;
+}
+template <bool E5M2>
+__device__ __forceinline__ uint4 quant16(const Vec16& v, float s) {
+    const uint32_t w[8] = {v.lo.x, v.lo.y, v.lo.z, v.lo.w, v.hi.x, v.hi.y, v.hi.z, v.hi.w};
+    uint4 o;
+    o.x = cvt4_fp8<E5M2>(bf16_lo(w[0]) * s, bf16_hi(w[0]) * s, bf16_lo(w[1]) * s, bf16_hi(w[1]) * s);
+    o.y = cvt4_fp8<E5M2>(bf16_lo(w[2]) * s, bf16_hi(w[2]) * s, bf16_lo(w[3]) * s, bf16_hi(w[3]) * s);
+    o.z = cvt4_fp8<E5M2>(bf16_lo(w[4]) * s, bf16_hi(w[4]) * s, bf16_lo(w[5]) * s, bf16_hi(w[5]) * s);
+    o.w = cvt4_fp8<E5M2>(bf16_lo(w[6]) * s, bf16_hi(w[6]) * s, bf16_lo(w[7]) * s, bf16_hi(w[7]) * s);
+    return o;
+}
+
+// ---- amax ------------------------------------------------------------------
+// VEC: x is 16-byte aligned and the body is read as 16-element vectors; the
+// n % 16 tail and the unaligned case go through the scalar loop.
+template <bool VEC>
+__global__ __launch_bounds__(kThreads) void k_amax_bf16(const uint16_t* __restrict__ x, size_t n,
+                                                        float* __restrict__ amax) {
+    __shared__ float sh[kThreads / 64];
+    float local = 0.0f;
+    const size_t tid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+    size_t done = 0;
+    if constexpr (VEC) {
+        const size_t nvec = n / kVec;
+        for (size_t i = tid; i < nvec; i += stride) local = fmaxf(local, amax16(load16(x + i * kVec)));
+        done = nvec * kVec;
+    }
+    for (size_t i = done + tid; i < n; i += stride) local = fmaxf(local, fabsf(bf16_to_f32(x[i])));
+    const float m = block_max(local, sh);
+    if (threadIdx.x == 0) atomic_max_nonneg(amax, m);
+}
+
+__global__ __launch_bounds__(kThreads) void k_amax_f32(const float* __restrict__ x, size_t n,
+                                                       float* __restrict__ amax, int vec) {
+    __shared__ float sh[kThreads / 64];
+    float local = 0.0f;
+    const size_t tid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+    size_t done = 0;
+    if (vec) {
+        const size_t nvec = n / 4;
+        for (size_t i = tid; i < nvec; i += stride) {
+            const float4 v = reinterpret_cast<const float4*>(x)[i];
+            local = fmaxf(fmaxf(local, fabsf(v.x)), fmaxf(fmaxf(fabsf(v.y), fabsf(v.z)), fabsf(v.w)));
+        }
+        done = nvec * 4;
+    }
+    for (size_t i = done + tid; i < n; i += stride) local = fmaxf(local, fabsf(x[i]));
+    const float m = block_max(local, sh);
+    if (threadIdx.x == 0) atomic_max_nonneg(amax, m);
+}
+
+__global__ void k_zero_f32(float* p) { *p = 0.0f; }
+
+// ---- scalar-state kernels --------------------------------------------------
+__global__ void k_scale_from_amax(const float* __restrict__ amax, float fp8_max,
+                                  float* __restrict__ scale, float* __restrict__ descale) {
+    const float a = fmaxf(*amax, 1e-12f);
+    *scale = fp8_max / a;
+    *descale = a / fp8_max;
+}
+
+__global__ void k_update_delayed_scale(const float* __restrict__ amax, float fp8_max,
+                                       float* __restrict__ scale, float* __restrict__ descale,
+                                       float* __restrict__ history, int history_len,
+                                       int* __restrict__ history_cursor, int* __restrict__ history_count) {
+    const float a = fmaxf(*amax, 1e-12f);
+    if (history_len <= 0) {
+        *scale = fp8_max / a;
+        *descale = a / fp8_max;
+        return;
+    }
+    int cursor = *history_cursor;
+    int count = *history_count;
+    if (cursor < 0 || cursor >= history_len) cursor = 0;
+    history[cursor] = a;
+    cursor = (cursor + 1) % history_len;
+    if (count < history_len) ++count;
+    float hist_max = history[0];
+    for (int i = 1; i < count; ++i) hist_max = fmaxf(hist_max, history[i]);
+    hist_max = fmaxf(hist_max, 1e-12f);
+    *history_cursor = cursor;
+    *history_count = count;
+    *scale = fp8_max / hist_max;
+    *descale = hist_max / fp8_max;
+}
+
+__global__ void k_clip_probe(const float* __restrict__ amax, const float* __restrict__ scale,
+                             float fp8_max, float* __restrict__ stats) {
+    const float a = *amax, s = *scale;
+    stats[2] += 1.0f;
+    if (fp8_max > 0.0f && s > 0.0f) {
+        const float ratio = a * s / fp8_max;
+        if (ratio > 1.0f) {
+            stats[0] += 1.0f;
+            if (ratio > stats[1]) stats[1] = ratio;
+        }
+    }
+}
+
+__global__ void k_calib_minmax(const float* __restrict__ amax, float* __restrict__ cmin,
+                               float* __restrict__ cmax) {
+    const float a = fmaxf(*amax, 1e-12f);
+    *cmin = fminf(*cmin, a);
+    *cmax = fmaxf(*cmax, a);
+}
+
+// ---- per-tensor quantize ---------------------------------------------------
+template <bool E5M2, bool RECORD, bool VEC>
+__global__ __launch_bounds__(kThreads) void k_quant(const uint16_t* __restrict__ x,
+                                                    uint8_t* __restrict__ out,
+                                                    const float* __restrict__ scale,
+                                                    float* __restrict__ amax, size_t n) {
+    __shared__ float sh[kThreads / 64];
+    const float s = *scale;
+    float local = 0.0f;
+    const size_t tid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+    size_t done = 0;
+    if constexpr (VEC) {
+        const size_t nvec = n / kVec;
+        for (size_t i = tid; i < nvec; i += stride) {
+            const Vec16 v = load16(x + i * kVec);
+            if constexpr (RECORD) local = fmaxf(local, amax16(v));
+            *reinterpret_cast<uint4*>(out + i * kVec) = quant16<E5M2>(v, s);
+        }
+        done = nvec * kVec;
+    }
+    for (size_t i = done + tid; i < n; i += stride) {
+        const float v = bf16_to_f32(x[i]);
+        if constexpr (RECORD) local = fmaxf(local, fabsf(v));
+        out[i] = cvt1_fp8<E5M2>(v * s);
+    }
+    if constexpr (RECORD) {
+        const float m = block_max(local, sh);
+        if (threadIdx.x == 0) atomic_max_nonneg(amax, m);
+    }
+}
+
+template <bool E5M2>
+__global__ __launch_bounds__(kThreads) void k_quant_f32(const float* __restrict__ x,
+                                                        uint8_t* __restrict__ out,
+                                                        const float* __restrict__ scale, size_t n,
+                                                        int vec) {
+    const float s = *scale;
+    const size_t tid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+    size_t done = 0;
+    if (vec) {
+        const size_t nvec = n / 4;
+        for (size_t i = tid; i < nvec; i += stride) {
+            const float4 v = reinterpret_cast<const float4*>(x)[i];
+            reinterpret_cast<uint32_t*>(out)[i] = cvt4_fp8<E5M2>(v.x * s, v.y * s, v.z * s, v.w * s);
+        }
+        done = nvec * 4;
+    }
+    for (size_t i = done + tid; i < n; i += stride) out[i] = cvt1_fp8<E5M2>(x[i] * s);
+}
+
+__global__ __launch_bounds__(kThreads) void k_elem_clip_count(const uint16_t* __restrict__ x,
+                                                              const float* __restrict__ scale,
+                                                              float fp8_max, size_t n,
+                                                              float* __restrict__ out) {
+    const float s = *scale;
+    int clipped = 0;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+         i += static_cast<size_t>(gridDim.x) * blockDim.x)
+        if (fabsf(bf16_to_f32(x[i])) * s > fp8_max) ++clipped;
+    clipped = wave_sum_i(clipped);
+    if ((threadIdx.x & 63) == 0 && clipped) atomicAdd(&out[0], static_cast<float>(clipped));
+    if (blockIdx.x == 0 && threadIdx.x == 0) atomicAdd(&out[1], static_cast<float>(n));
+}
+
+// ---- per-row quantize ---------------------------------------------------------
+// One wavefront per row.  The row stays in registers between the amax pass and
+// the convert pass, so HBM sees 2 B read + 1 B written per element.
+// MAXS = register-resident steps of 64 lanes x 16 elements.
+template <bool E5M2, int MAXS>
+__global__ __launch_bounds__(kThreads) void k_quant_rows(const uint16_t* __restrict__ x, int rows, int K,
+                                                         uint8_t* __restrict__ out,
+                                                         float* __restrict__ scale,
+                                                         float* __restrict__ descale) {
+    const int row = blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int lane = threadIdx.x & 63;
+    const uint16_t* xr = x + static_cast<size_t>(row) * K;
+    uint8_t* outr = out + static_cast<size_t>(row) * K;
+    Vec16 v[MAXS];
+    float local = 0.0f;
+#pragma unroll
+    for (int s = 0; s < MAXS; ++s) {
+        const int k = (s * 64 + lane) * kVec;
+        if (k < K) {
+            v[s] = load16(xr + k);
+            local = fmaxf(local, amax16(v[s]));
+        }
+    }
+    constexpr float fmax_ = E5M2 ? 57344.0f : 448.0f;
+    const float a = fmaxf(wave_max(local), 1e-12f);
+    const float sc = fmax_ / a;
+    if (lane == 0) { scale[row] = sc; descale[row] = a / fmax_; }
+#pragma unroll
+    for (int s = 0; s < MAXS; ++s) {
+        const int k = (s * 64 + lane) * kVec;
+        if (k < K) *reinterpret_cast<uint4*>(outr + k) = quant16<E5M2>(v[s], sc);
+    }
+}
+
+// Any K, any alignment: one workgroup per row, two passes over the row.
+template <bool E5M2>
+__global__ __launch_bounds__(kThreads) void k_quant_rows_generic(const uint16_t* __restrict__ x, int K,
+                                                                 uint8_t* __restrict__ out,
+                                                                 float* __restrict__ scale,
+                                                                 float* __restrict__ descale) {
+    __shared__ float sh[kThreads / 64];
+    const int row = blockIdx.x;
+    const uint16_t* xr = x + static_cast<size_t>(row) * K;
+    uint8_t* outr = out + static_cast<size_t>(row) * K;
+    float local = 0.0f;
+    for (int k = threadIdx.x; k < K; k += blockDim.x) local = fmaxf(local, fabsf(bf16_to_f32(xr[k])));
+    constexpr float fmax_ = E5M2 ? 57344.0f : 448.0f;
+    const float a = fmaxf(block_max(local, sh), 1e-12f);
+    const float sc = fmax_ / a;
+    if (threadIdx.x == 0) { scale[row] = sc; descale[row] = a / fmax_; }
+    for (int k = threadIdx.x; k < K; k += blockDim.x) outr[k] = cvt1_fp8<E5M2>(bf16_to_f32(xr[k]) * sc);
+}
+
+// ---- 1x128 groups ------------------------------------------------------------
+// K % 128 == 0, 16-byte aligned rows: a group is 8 neighbouring lanes.
+__global__ __launch_bounds__(kThreads) void k_quant_1x128(const uint16_t* __restrict__ x, size_t ngroups,
+                                                          uint8_t* __restrict__ out,
+                                                          float* __restrict__ scale,
+                                                          float* __restrict__ descale) {
+    const size_t tid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+    const size_t nvec = ngroups * 8;
+    // every lane of a wave runs the same number of iterations (nvec % 8 == 0, stride % 64 == 0)
+    for (size_t i = tid; i < ((nvec + 63) / 64) * 64; i += stride) {
+        const bool live = i < nvec;
+        Vec16 v = {};
+        if (live) v = load16(x + i * kVec);
+        float m = amax16(v);
+        m = fmaxf(m, __shfl_xor(m, 1, kWave));
+        m = fmaxf(m, __shfl_xor(m, 2, kWave));
+        m = fmaxf(m, __shfl_xor(m, 4, kWave));
+        const float a = fmaxf(m, 1e-12f);
+        const float sc = 448.0f / a;
+        if (live) {
+            if ((i & 7) == 0) { scale[i >> 3] = sc; descale[i >> 3] = a / 448.0f; }
+            *reinterpret_cast<uint4*>(out + i * kVec) = quant16<false>(v, sc);
+        }
+    }
+}
+
+// ragged K or unaligned rows: one wavefront per group
+__global__ __launch_bounds__(kThreads) void k_quant_1x128_generic(const uint16_t* __restrict__ x, int rows,
+                                                                  int K, uint8_t* __restrict__ out,
+                                                                  float* __restrict__ scale,
+                                                                  float* __restrict__ descale) {
+    const int kb = (K + 127) / 128;
+    const size_t g = static_cast<size_t>(blockIdx.x) * (kThreads / 64) + (threadIdx.x >> 6);
+    if (g >= static_cast<size_t>(rows) * kb) return;
+    const int lane = threadIdx.x & 63;
+    const int r = static_cast<int>(g / kb), b = static_cast<int>(g % kb);
+    const size_t base = static_cast<size_t>(r) * K + static_cast<size_t>(b) * 128;
+    const int len = min(128, K - b * 128);
+    float v0 = lane < len ? bf16_to_f32(x[base + lane]) : 0.0f;
+    float v1 = lane + 64 < len ? bf16_to_f32(x[base + lane + 64]) : 0.0f;
+    const float a = fmaxf(wave_max(fmaxf(fabsf(v0), fabsf(v1))), 1e-12f);
+    const float sc = 448.0f / a;
+    if (lane == 0) { scale[g] = sc; descale[g] = a / 448.0f; }
+    if (lane < len) out[base + lane] = cvt1_fp8<false>(v0 * sc);
+    if (lane + 64 < len) out[base + lane + 64] = cvt1_fp8<false>(v1 * sc);
+}
+
+// ---- 128x128 blocks ------------------------------------------------------------
+// One workgroup per block; a thread holds a 4 x 16 slice in registers.
+__global__ __launch_bounds__(kThreads) void k_quant_128x128(const uint16_t* __restrict__ x, int rows, int K,
+                                                            uint8_t* __restrict__ out,
+                                                            float* __restrict__ scale,
+                                                            float* __restrict__ descale, int vec) {
+    __shared__ float sh[kThreads / 64];
+    const int kb = (K + 127) / 128;
+    const int br = blockIdx.x / kb, bk = blockIdx.x % kb;
+    const int r0 = br * 128, k0 = bk * 128;
+    const int tr = threadIdx.x >> 3, tc = (threadIdx.x & 7) * kVec;    // 32 rows x 8 lanes per pass
+    float local = 0.0f;
+    if (vec) {
+        Vec16 v[4];
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const int r = r0 + p * 32 + tr;
+            v[p] = Vec16{};
+            if (r < rows) v[p] = load16(x + static_cast<size_t>(r) * K + k0 + tc);
+            local = fmaxf(local, amax16(v[p]));
+        }
+        const float a = fmaxf(block_max(local, sh), 1e-12f);
+        const float sc = 448.0f / a;
+        if (threadIdx.x == 0) { scale[blockIdx.x] = sc; descale[blockIdx.x] = a / 448.0f; }
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const int r = r0 + p * 32 + tr;
+            if (r < rows) *reinterpret_cast<uint4*>(out + static_cast<size_t>(r) * K + k0 + tc) = quant16<false>(v[p], sc);
+        }
+    } else {
+        const int klen = min(128, K - k0), rlen = min(128, rows - r0);
+        for (int i = threadIdx.x; i < rlen * 128; i += blockDim.x) {
+            const int r = i >> 7, k = i & 127;
+            if (k < klen) local = fmaxf(local, fabsf(bf16_to_f32(x[static_cast<size_t>(r0 + r) * K + k0 + k])));
+        }
+        const float a = fmaxf(block_max(local, sh), 1e-12f);
+        const float sc = 448.0f / a;
+        if (threadIdx.x == 0) { scale[blockIdx.x] = sc; descale[blockIdx.x] = a / 448.0f; }
+        for (int i = threadIdx.x; i < rlen * 128; i += blockDim.x) {
+            const int r = i >> 7, k = i & 127;
+            if (k < klen) {
+                const size_t idx = static_cast<size_t>(r0 + r) * K + k0 + k;
+                out[idx] = cvt1_fp8<false>(bf16_to_f32(x[idx]) * sc);
+            }
+        }
+    }
+}
+
+// ---- raw-byte E4M3 storage path --------------------------------------------------
+// The byte contract pack(): like the saturating convert for finite input,
+// nonfinite input -> sign|0x7f and flagged.
+__device__ __forceinline__ uint8_t pack_raw(float v, bool& finite) {
+    const uint32_t bits = __float_as_uint(v);
+    finite = (bits & 0x7f800000u) != 0x7f800000u;
+    if (!finite) return static_cast<uint8_t>(((bits >> 24) & 0x80u) | 0x7fu);
+    return cvt1_fp8<false>(v);
+}
+
+__global__ __launch_bounds__(kThreads) void k_raw_stats(const uint16_t* __restrict__ x, size_t n,
+                                                        float* __restrict__ amax, int* __restrict__ bad) {
+    __shared__ float sh[kThreads / 64];
+    float local = 0.0f;
+    int nbad = 0;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+         i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+        const float v = bf16_to_f32(x[i]);
+        if ((__float_as_uint(v) & 0x7f800000u) == 0x7f800000u) ++nbad;
+        else local = fmaxf(local, fabsf(v));
+    }
+    nbad = wave_sum_i(nbad);
+    if ((threadIdx.x & 63) == 0 && nbad) atomicAdd(bad, nbad);
+    const float m = block_max(local, sh);
+    if (threadIdx.x == 0) atomic_max_nonneg(amax, m);
+}
+
+template <bool DEQUANT>
+__global__ __launch_bounds__(kThreads) void k_raw_pack(const uint16_t* __restrict__ x,
+                                                       uint8_t* __restrict__ out,
+                                                       uint16_t* __restrict__ dequant,
+                                                       const float* __restrict__ scale,
+                                                       const float* __restrict__ descale,
+                                                       int* __restrict__ bad, size_t n) {
+    const float s = *scale;
+    const float d = DEQUANT ? *descale : 0.0f;
+    int nbad = 0;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+         i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+        bool fin;
+        const uint8_t code = pack_raw(bf16_to_f32(x[i]) * s, fin);
+        out[i] = code;
+        if constexpr (DEQUANT) dequant[i] = f32_to_bf16(e4m3_to_f32(code) * d);
+        if (!fin) ++nbad;
+    }
+    nbad = wave_sum_i(nbad);
+    if ((threadIdx.x & 63) == 0 && nbad) atomicAdd(bad, nbad);
+}
+
+__global__ __launch_bounds__(kThreads) void k_raw_unpack(const uint8_t* __restrict__ in,
+                                                         const float* __restrict__ descale,
+                                                         uint16_t* __restrict__ out, size_t n) {
+    const float d = *descale;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+         i += static_cast<size_t>(gridDim.x) * blockDim.x)
+        out[i] = f32_to_bf16(e4m3_to_f32(in[i]) * d);
+}
+
+__global__ void k_zero_raw(float* amax, int* bad) { *amax = 0.0f; *bad = 0; }
+
+unsigned blocks_for(size_t items) {
+    const size_t b = (items + kThreads - 1) / kThreads;
+    return static_cast<unsigned>(b < 1 ? 1 : (b > kMaxBlocks ? kMaxBlocks : b));
+}
+
+template <bool E5M2, bool RECORD>
+int launch_quant(const uint16_t* x, void* out, const float* scale, float* amax, size_t n, cf_stream_t st) {
+    if (n == 0) return CF_OK;
+    if (!x || !out || !scale || (RECORD && !amax)) return CF_ERR_INVALID_ARG;
+    auto* o = static_cast<uint8_t*>(out);
+    if (aligned16(x) && aligned16(out))
+        k_quant<E5M2, RECORD, true><<<blocks_for((n + kVec - 1) / kVec), kThreads, 0, as_stream(st)>>>(x, o, scale, amax, n);
+    else
+        k_quant<E5M2, RECORD, false><<<blocks_for(n), kThreads, 0, as_stream(st)>>>(x, o, scale, amax, n);
+    return launch_status();
+}
+
+}  // namespace
+}  // namespace cf
+
+using namespace cf;
+
+extern "C" {
+
+int cf_fp8_amax_bf16(const uint16_t* d_x, size_t n, float* d_amax, cf_stream_t stream) {
+    if (!d_amax || (n > 0 && !d_x)) return CF_ERR_INVALID_ARG;
+    // a one-thread fill, not a memset node, so the call can sit inside a captured graph
+    k_zero_f32<<<1, 1, 0, as_stream(stream)>>>(d_amax);
+    if (n == 0) return launch_status();
+    if (aligned16(d_x))
+        k_amax_bf16<true><<<blocks_for((n + kVec - 1) / kVec), kThreads, 0, as_stream(stream)>>>(d_x, n, d_amax);
+    else
+        k_amax_bf16<false><<<blocks_for(n), kThreads, 0, as_stream(stream)>>>(d_x, n, d_amax);
+    return launch_status();
+}
+
+int cf_fp8_amax_f32(const float* d_x, size_t n, float* d_amax, cf_stream_t stream) {
+    if (!d_amax || (n > 0 && !d_x)) return CF_ERR_INVALID_ARG;
+    k_zero_f32<<<1, 1, 0, as_stream(stream)>>>(d_amax);
+    if (n == 0) return launch_status();
+    const int vec = aligned16(d_x);
+    k_amax_f32<<<blocks_for(vec ? (n + 3) / 4 : n), kThreads, 0, as_stream(stream)>>>(d_x, n, d_amax, vec);
+    return launch_status();
+}
+
+int cf_fp8_scale_from_amax(const float* d_amax, float fp8_max, float* d_scale, float* d_descale,
+                           cf_stream_t stream) {
+    if (!d_amax || !d_scale || !d_descale) return CF_ERR_INVALID_ARG;
+    k_scale_from_amax<<<1, 1, 0, as_stream(stream)>>>(d_amax, fp8_max, d_scale, d_descale);
+    return launch_status();
+}
+
+int cf_fp8_quantize_e4m3(const uint16_t* d_x, void* d_out, const float* d_scale, size_t n, cf_stream_t stream) {
+    return launch_quant<false, false>(d_x, d_out, d_scale, nullptr, n, stream);
+}
+int cf_fp8_quantize_e5m2(const uint16_t* d_x, void* d_out, const float* d_scale, size_t n, cf_stream_t stream) {
+    return launch_quant<true, false>(d_x, d_out, d_scale, nullptr, n, stream);
+}
+int cf_fp8_quantize_e4m3_record(const uint16_t* d_x, void* d_out, const float* d_scale, float* d_amax,
+                                size_t n, cf_stream_t stream) {
+    return launch_quant<false, true>(d_x, d_out, d_scale, d_amax, n, stream);
+}
+int cf_fp8_quantize_e5m2_record(const uint16_t* d_x, void* d_out, const float* d_scale, float* d_amax,
+                                size_t n, cf_stream_t stream) {
+    return launch_quant<true, true>(d_x, d_out, d_scale, d_amax, n, stream);
+}
+
+int cf_fp8_quantize_f32_e4m3(const float* d_x, void* d_out, const float* d_scale, size_t n, cf_stream_t stream) {
+    if (n == 0) return CF_OK;
+    if (!d_x || !d_out || !d_scale) return CF_ERR_INVALID_ARG;
+    const int vec = aligned16(d_x) && (reinterpret_cast<uintptr_t>(d_out) & 3u) == 0;
+    k_quant_f32<false><<<blocks_for(vec ? (n + 3) / 4 : n), kThreads, 0, as_stream(stream)>>>(
+        d_x, static_cast<uint8_t*>(d_out), d_scale, n, vec);
+    return launch_status();
+}
+int cf_fp8_quantize_f32_e5m2(const float* d_x, void* d_out, const float* d_scale, size_t n, cf_stream_t stream) {
+    if (n == 0) return CF_OK;
+    if (!d_x || !d_out || !d_scale) return CF_ERR_INVALID_ARG;
+    const int vec = aligned16(d_x) && (reinterpret_cast<uintptr_t>(d_out) & 3u) == 0;
+    k_quant_f32<true><<<blocks_for(vec ? (n + 3) / 4 : n), kThreads, 0, as_stream(stream)>>>(
+        d_x, static_cast<uint8_t*>(d_out), d_scale, n, vec);
+    return launch_status();
+}
+
+int cf_fp8_update_delayed_scale(const float* d_amax, float fp8_max, float* d_scale, float* d_descale,
+                                float* d_history, int history_len, int* d_history_cursor,
+                                int* d_history_count, cf_stream_t stream) {
+    if (!d_amax || !d_scale || !d_descale) return CF_ERR_INVALID_ARG;
+    if (history_len > 0 && (!d_history || !d_history_cursor || !d_history_count)) return CF_ERR_INVALID_ARG;
+    k_update_delayed_scale<<<1, 1, 0, as_stream(stream)>>>(d_amax, fp8_max, d_scale, d_descale, d_history,
+                                                           history_len, d_history_cursor, d_history_count);
+    return launch_status();
+}
+
+int cf_fp8_clip_probe(const float* d_amax, const float* d_scale, float fp8_max, float* d_stats,
+                      cf_stream_t stream) {
+    if (!d_amax || !d_scale || !d_stats) return CF_ERR_INVALID_ARG;
+    k_clip_probe<<<1, 1, 0, as_stream(stream)>>>(d_amax, d_scale, fp8_max, d_stats);
+    return launch_status();
+}
+
+int cf_fp8_elem_clip_count(const uint16_t* d_x, const float* d_scale, float fp8_max, size_t n, float* d_out,
+                           cf_stream_t stream) {
+    if (!d_scale || !d_out || (n > 0 && !d_x)) return CF_ERR_INVALID_ARG;
+    k_elem_clip_count<<<blocks_for(n), kThreads, 0, as_stream(stream)>>>(d_x, d_scale, fp8_max, n, d_out);
+    return launch_status();
+}
+
+int cf_fp8_calib_minmax_update(const float* d_amax, float* d_cmin, float* d_cmax, cf_stream_t stream) {
+    if (!d_amax || !d_cmin || !d_cmax) return CF_ERR_INVALID_ARG;
+    k_calib_minmax<<<1, 1, 0, as_stream(stream)>>>(d_amax, d_cmin, d_cmax);
+    return launch_status();
+}
+
+int cf_fp8_quantize_rows(const uint16_t* d_x, int rows, int K, int is_e5m2, void* d_out, float* d_scale,
+                         float* d_descale, cf_stream_t stream) {
+    if (rows < 0 || K < 0) return CF_ERR_INVALID_ARG;
+    if (rows == 0) return CF_OK;
+    if (!d_scale || !d_descale || (K > 0 && (!d_x || !d_out))) return CF_ERR_INVALID_ARG;
+    auto* o = static_cast<uint8_t*>(d_out);
+    hipStream_t st = as_stream(stream);
+    const bool vec = aligned16(d_x) && aligned16(d_out) && K % kVec == 0 && K > 0;
+    const unsigned grid = ceil_div(rows, kThreads / 64);
+    if (vec && K <= 4 * 1024) {
+        if (is_e5m2) k_quant_rows<true, 4><<<grid, kThreads, 0, st>>>(d_x, rows, K, o, d_scale, d_descale);
+        else         k_quant_rows<false, 4><<<grid, kThreads, 0, st>>>(d_x, rows, K, o, d_scale, d_descale);
+    } else if (vec && K <= 16 * 1024) {
+        if (is_e5m2) k_quant_rows<true, 16><<<grid, kThreads, 0, st>>>(d_x, rows, K, o, d_scale, d_descale);
+        else         k_quant_rows<false, 16><<<grid, kThreads, 0, st>>>(d_x, rows, K, o, d_scale, d_descale);
+    } else {
+        if (is_e5m2) k_quant_rows_generic<true><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);
+        else         k_quant_rows_generic<false><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);
+    }
+    return launch_status();
+}
+
+int cf_fp8_quantize_block_1x128(const uint16_t* d_x, int rows, int K, void* d_out, float* d_scale,
+                                float* d_descale, cf_stream_t stream) {
+    if (rows < 0 || K < 0) return CF_ERR_INVALID_ARG;
+    if (rows == 0 || K == 0) return CF_OK;
+    if (!d_x || !d_out || !d_scale || !d_descale) return CF_ERR_INVALID_ARG;
+    auto* o = static_cast<uint8_t*>(d_out);
+    if (K % 128 == 0 && aligned16(d_x) && aligned16(d_out)) {
+        const size_t ngroups = static_cast<size_t>(rows) * (K / 128);
+        k_quant_1x128<<<blocks_for(ngroups * 8), kThreads, 0, as_stream(stream)>>>(d_x, ngroups, o, d_scale, d_descale);
+    } else {
+        const size_t ngroups = static_cast<size_t>(rows) * ((K + 127) / 128);
+        k_quant_1x128_generic<<<ceil_div(ngroups, kThreads / 64), kThreads, 0, as_stream(stream)>>>(
+            d_x, rows, K, o, d_scale, d_descale);
+    }
+    return launch_status();
+}
+
+int cf_fp8_quantize_block_128x128(const uint16_t* d_x, int rows, int K, void* d_out, float* d_scale,
+                                  float* d_descale, cf_stream_t stream) {
+    if (rows < 0 || K < 0) return CF_ERR_INVALID_ARG;
+    if (rows == 0 || K == 0) return CF_OK;
+    if (!d_x || !d_out || !d_scale || !d_descale) return CF_ERR_INVALID_ARG;
+    const int vec = K % 128 == 0 && aligned16(d_x) && aligned16(d_out);
+    const unsigned grid = static_cast<unsigned>(((rows + 127) / 128) * ((K + 127) / 128));
+    k_quant_128x128<<<grid, kThreads, 0, as_stream(stream)>>>(d_x, rows, K, static_cast<uint8_t*>(d_out),
+                                                              d_scale, d_descale, vec);
+    return launch_status();
+}
+
+int cf_fp8_pack_bf16_e4m3_raw(const uint16_t* d_x, uint8_t* d_out, float* d_amax, float* d_scale,
+                              float* d_descale, int* d_bad_count, size_t n, cf_stream_t stream) {
+    if (!d_amax || !d_scale || !d_descale || !d_bad_count || (n > 0 && (!d_x || !d_out))) return CF_ERR_INVALID_ARG;
+    hipStream_t st = as_stream(stream);
+    k_zero_raw<<<1, 1, 0, st>>>(d_amax, d_bad_count);
+    if (n) k_raw_stats<<<blocks_for(n), kThreads, 0, st>>>(d_x, n, d_amax, d_bad_count);
+    k_scale_from_amax<<<1, 1, 0, st>>>(d_amax, 448.0f, d_scale, d_descale);
+    if (n) k_raw_pack<false><<<blocks_for(n), kThreads, 0, st>>>(d_x, d_out, nullptr, d_scale, d_descale, d_bad_count, n);
+    return launch_status();
+}
+
+int cf_fp8_pack_bf16_e4m3_raw_and_dequant(const uint16_t* d_x, uint8_t* d_out, uint16_t* d_dequant,
+                                          float* d_amax, float* d_scale, float* d_descale,
+                                          int* d_bad_count, size_t n, cf_stream_t stream) {
+    if (!d_amax || !d_scale || !d_descale || !d_bad_count || (n > 0 && (!d_x || !d_out || !d_dequant)))
+        return CF_ERR_INVALID_ARG;
+    hipStream_t st = as_stream(stream);
+    k_zero_raw<<<1, 1, 0, st>>>(d_amax, d_bad_count);
+    if (n) k_raw_stats<<<blocks_for(n), kThreads, 0, st>>>(d_x, n, d_amax, d_bad_count);
+    k_scale_from_amax<<<1, 1, 0, st>>>(d_amax, 448.0f, d_scale, d_descale);
+    if (n) k_raw_pack<true><<<blocks_for(n), kThreads, 0, st>>>(d_x, d_out, d_dequant, d_scale, d_descale, d_bad_count, n);
+    return launch_status();
+}
+
+int cf_fp8_unpack_e4m3_raw_bf16(const uint8_t* d_in, const float* d_descale, uint16_t* d_out, size_t n,
+                                cf_stream_t stream) {
+    if (n == 0) return CF_OK;
+    if (!d_in || !d_descale || !d_out) return CF_ERR_INVALID_ARG;
+    k_raw_unpack<<<blocks_for(n), kThreads, 0, as_stream(stream)>>>(d_in, d_descale, d_out, n);
+    return launch_status();
+}
+
+}  // extern "C"

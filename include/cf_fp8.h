@@ -1,0 +1,142 @@
+/*
+ * cf_fp8.h -- C ABI of the MI355X (gfx950) FP8 hot-path library.
+ *
+ * Every entry point replaces one function of the reference's kernel library
+ * (C++ free functions in namespace ida_native, declared in
+ * include/ida_native/kernels.hpp of the reference tree) or one of the static
+ * cuBLASLt wrappers in src/trainer.cu; the citation after each declaration
+ * names it.  Conventions, all taken from the reference call sites:
+ *   - every pointer is device memory owned by the caller, scalars included
+ *     (amax / scale / descale / history / cursor / count are device scalars);
+ *   - work is enqueued on `stream` (a hipStream_t passed as void*) and nothing
+ *     synchronises;
+ *   - bf16 tensors are passed as uint16_t*, fp8 tensors as void* / uint8_t*;
+ *   - the library allocates nothing and keeps no mutable global state.
+ * The reference functions return void and throw; the C ABI returns 0 on
+ * success, a positive hipError_t when the runtime reports one, or a negative
+ * CF_ERR_* code for an argument the kernels cannot honour.
+ */
+#ifndef CF_FP8_H
+#define CF_FP8_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* cf_stream_t; /* hipStream_t */
+
+#define CF_OK                 0
+#define CF_ERR_INVALID_ARG   (-1)  /* null pointer with n > 0, negative size       */
+#define CF_ERR_UNSUPPORTED   (-2)  /* shape / alignment outside what a kernel takes */
+
+#define CF_E4M3_MAX 448.0f
+#define CF_E5M2_MAX 57344.0f
+
+/* library identification: returns a static string naming arch and build */
+const char* cf_version(void);
+
+/* ---- per-tensor quantize family: kernels/fp8.cu --------------------------- */
+
+/* fp8_amax_bf16, kernels.hpp:983, kernels/fp8.cu:250-253.  Zeroes *d_amax then
+ * max-reduces |x| into it. */
+int cf_fp8_amax_bf16(const uint16_t* d_x, size_t n, float* d_amax, cf_stream_t stream);
+
+/* fp8_scale_from_amax, kernels.hpp:1002, kernels/fp8.cu:255-259. */
+int cf_fp8_scale_from_amax(const float* d_amax, float fp8_max, float* d_scale,
+                           float* d_descale, cf_stream_t stream);
+
+/* fp8_quantize_e4m3 / fp8_quantize_e5m2, kernels.hpp:1004-1007,
+ * kernels/fp8.cu:261-279.  out[i] = cvt_rne_satfinite(f32(x[i]) * *d_scale). */
+int cf_fp8_quantize_e4m3(const uint16_t* d_x, void* d_out, const float* d_scale,
+                         size_t n, cf_stream_t stream);
+int cf_fp8_quantize_e5m2(const uint16_t* d_x, void* d_out, const float* d_scale,
+                         size_t n, cf_stream_t stream);
+
+/* fp8_quantize_e4m3_record / _e5m2_record, kernels.hpp:1021-1026,
+ * kernels/fp8.cu:310-330.  Quantizes with *d_scale and max-combines the amax
+ * of the unscaled input into *d_amax (caller zeroes it). */
+int cf_fp8_quantize_e4m3_record(const uint16_t* d_x, void* d_out, const float* d_scale,
+                                float* d_amax, size_t n, cf_stream_t stream);
+int cf_fp8_quantize_e5m2_record(const uint16_t* d_x, void* d_out, const float* d_scale,
+                                float* d_amax, size_t n, cf_stream_t stream);
+
+/* fp8_update_delayed_scale, kernels.hpp:1042-1052, kernels/fp8.cu:396-417. */
+int cf_fp8_update_delayed_scale(const float* d_amax, float fp8_max, float* d_scale,
+                                float* d_descale, float* d_history, int history_len,
+                                int* d_history_cursor, int* d_history_count,
+                                cf_stream_t stream);
+
+/* fp8_quantize_transpose_e4m3, kernels.hpp:1009-1010, kernels/fp8.cu:281-290.
+ * w[K,N] bf16 -> out[N,K] E4M3. */
+int cf_fp8_quantize_transpose_e4m3(const uint16_t* d_w, void* d_out, const float* d_scale,
+                                   int K, int N, cf_stream_t stream);
+
+/* fp8_quant_and_transpose_e4m3, kernels.hpp:1015-1017, kernels/fp8.cu:292-308.
+ * in[K,N] bf16 -> act8[K,N] and snap[N,K], one read. */
+int cf_fp8_quant_and_transpose_e4m3(const uint16_t* d_in, void* d_act8_out, void* d_snap_out,
+                                    const float* d_scale, int K, int N, cf_stream_t stream);
+
+/* transpose_u8, static at src/trainer.cu:1441-1448.  in[rows,cols] -> out[cols,rows]. */
+int cf_transpose_u8(const void* d_in, void* d_out, int rows, int cols, cf_stream_t stream);
+
+/* fp8_clip_probe / fp8_elem_clip_count, kernels.hpp:1033-1041,
+ * kernels/fp8.cu:358-394. */
+int cf_fp8_clip_probe(const float* d_amax, const float* d_scale, float fp8_max,
+                      float* d_stats, cf_stream_t stream);
+int cf_fp8_elem_clip_count(const uint16_t* d_x, const float* d_scale, float fp8_max,
+                           size_t n, float* d_out, cf_stream_t stream);
+
+/* fp8_pack_bf16_e4m3_raw / _raw_and_dequant / fp8_unpack_e4m3_raw_bf16,
+ * kernels.hpp:988-1001, kernels/fp8.cu:491-528.  Byte contract of
+ * include/ida_native/fp8_e4m3.hpp (nonfinite -> sign|0x7f and counted).
+ * *d_bad_count is nonzero iff an input or a packed product was nonfinite. */
+int cf_fp8_pack_bf16_e4m3_raw(const uint16_t* d_x, uint8_t* d_out, float* d_amax,
+                              float* d_scale, float* d_descale, int* d_bad_count,
+                              size_t n, cf_stream_t stream);
+int cf_fp8_pack_bf16_e4m3_raw_and_dequant(const uint16_t* d_x, uint8_t* d_out,
+                                          uint16_t* d_dequant, float* d_amax, float* d_scale,
+                                          float* d_descale, int* d_bad_count, size_t n,
+                                          cf_stream_t stream);
+int cf_fp8_unpack_e4m3_raw_bf16(const uint8_t* d_in, const float* d_descale, uint16_t* d_out,
+                                size_t n, cf_stream_t stream);
+
+/* k_calib_minmax_update, static at src/trainer.cu:3789-3795. */
+int cf_fp8_calib_minmax_update(const float* d_amax, float* d_cmin, float* d_cmax,
+                               cf_stream_t stream);
+
+/* ---- scale groups finer than per-tensor ------------------------------------
+ * The reference scales per tensor only (kernels/fp8.cu:13-16); these apply the
+ * same formula (kernels/fp8.cu:37-39,49) per row, per 1x128 group and per
+ * 128x128 block, and to fp32 input, for the benchmark configurations that ask
+ * for them.  Scale tensors are fp32: [rows], [rows, ceil(K/128)],
+ * [ceil(rows/128), ceil(K/128)]. */
+int cf_fp8_amax_f32(const float* d_x, size_t n, float* d_amax, cf_stream_t stream);
+int cf_fp8_quantize_f32_e4m3(const float* d_x, void* d_out, const float* d_scale, size_t n,
+                             cf_stream_t stream);
+int cf_fp8_quantize_f32_e5m2(const float* d_x, void* d_out, const float* d_scale, size_t n,
+                             cf_stream_t stream);
+int cf_fp8_quantize_rows(const uint16_t* d_x, int rows, int K, int is_e5m2, void* d_out,
+                         float* d_scale, float* d_descale, cf_stream_t stream);
+int cf_fp8_quantize_block_1x128(const uint16_t* d_x, int rows, int K, void* d_out,
+                                float* d_scale, float* d_descale, cf_stream_t stream);
+int cf_fp8_quantize_block_128x128(const uint16_t* d_x, int rows, int K, void* d_out,
+                                  float* d_scale, float* d_descale, cf_stream_t stream);
+
+/* ---- elementwise epilogue ops (also fused into the GEMM epilogue) ---------- */
+
+/* swiglu_forward, kernels.hpp:159-165, kernels/activations.cu:76-87.
+ * n < 0 or a null pointer with n > 0 is CF_ERR_INVALID_ARG (the reference
+ * throws std::invalid_argument, kernels/activations.cu:61-72). */
+int cf_swiglu_forward(const uint16_t* d_gate, const uint16_t* d_up, uint16_t* d_out, int n,
+                      cf_stream_t stream);
+/* bias_add_strided_bf16, kernels.hpp:243-247, kernels/moe.cu:349-356. */
+int cf_bias_add_strided_bf16(uint16_t* d_inout, const uint16_t* d_bias, int rows, int cols,
+                             int row_stride, int base, cf_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CF_FP8_H */

@@ -1,0 +1,41 @@
+"""The C-ABI library loads on a machine without a GPU and exports every symbol the header declares."""
+import ctypes
+import re
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+def test_library_exports_every_declared_symbol(cf):
+    assert len(cf.decls) >= 25
+    dll = ctypes.CDLL(str(ROOT / "canopy-foundry_amd" / "libcf_fp8.so"))
+    for name in cf.decls:
+        assert getattr(dll, name) is not None
+    assert b"gfx950" in cf.cf_version()
+
+
+def test_every_declaration_cites_the_reference():
+    text = (ROOT / "include" / "cf_fp8.h").read_text()
+    # each exported function is preceded (within its comment block) by a reference file:line or an explicit note
+    for m in re.finditer(r"\n(?:int|const char\*) (cf_\w+)\(", text):
+        head = text[: m.start()]
+        block = head[head.rfind("/*"):]
+        assert re.search(r"\w+\.(cu|hpp|cpp):\d+", block) or "no counterpart" in block or "identification" in block, m.group(1)
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    import __graft_entry__ as entry
+    import pytest
+    pkg = entry.load_package()
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        pkg.Lib(tmp_path / "libcf_fp8.so")
+
+
+def test_argument_errors_do_not_need_a_gpu(cf):
+    # argument validation happens before any launch
+    assert cf.raw_cf_swiglu_forward(None, None, None, -1, None) == -1
+    assert cf.raw_cf_swiglu_forward(None, None, None, 4, None) == -1
+    assert cf.raw_cf_swiglu_forward(None, None, None, 0, None) == 0
+    assert cf.raw_cf_fp8_quantize_e4m3(None, None, None, 0, None) == 0
+    assert cf.raw_cf_fp8_quantize_e4m3(None, None, None, 8, None) == -1
+    assert cf.raw_cf_fp8_quantize_rows(None, -1, 4, 0, None, None, None, None) == -1

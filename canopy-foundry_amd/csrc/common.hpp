@@ -78,7 +78,7 @@ __device__ __forceinline__ float e4m3_to_f32(uint8_t b) {
     const uint32_t e = (b >> 3) & 0xfu, m = b & 7u;
     float mag;
     if (e == 0) mag = static_cast<float>(m) * 0.001953125f;           // m * 2^-9
-    else if (e == 15 && m == 7) mag = __uint_as_float(0x7fc00000u);
+    else if (e == 15 && m == 7) return __uint_as_float(0x7fc00000u);   // one NaN for both signs, as unpack() does
     else mag = __uint_as_float(((e + 120u) << 23) | (m << 20));
     return __uint_as_float(__float_as_uint(mag) | sign);
 }
@@ -87,7 +87,8 @@ __device__ __forceinline__ float e5m2_to_f32(uint8_t b) {
     const uint32_t e = (b >> 2) & 0x1fu, m = b & 3u;
     float mag;
     if (e == 0) mag = static_cast<float>(m) * 1.52587890625e-05f;     // m * 2^-16
-    else if (e == 31) mag = __uint_as_float(m == 0 ? 0x7f800000u : 0x7fc00000u);
+    else if (e == 31 && m != 0) return __uint_as_float(0x7fc00000u);
+    else if (e == 31) mag = __uint_as_float(0x7f800000u);
     else mag = __uint_as_float(((e + 112u) << 23) | (m << 21));
     return __uint_as_float(__float_as_uint(mag) | sign);
 }

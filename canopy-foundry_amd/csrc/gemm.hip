@@ -1,0 +1,424 @@
+// Scaled FP8 GEMM for gfx950:  C[M,N] = epilogue( (A[M,K] * sa) . (B[N,K] * sb)^T ).
+//
+// Workgroup tile 256 x 256 x 128, four wavefronts in a 2 x 2 arrangement, each
+// owning a 128 x 128 sub-tile = 4 x 4 tiles of v_mfma_f32_32x32x64_f8f6f4 with
+// fp32 accumulators (256 accumulator registers per lane, one wave per SIMD).
+// A and B tiles are staged through LDS, double buffered: while the matrix cores
+// work on stage s the next K-tile is fetched from HBM/L2 with 128-bit loads
+// into registers and written to stage s^1; one barrier per K-tile.
+//
+// LDS tile layout: [256 rows][128 bytes], the eight 16-byte chunks of a row are
+// xor-swizzled with f(row) = (row ^ (row >> 3)) & 7 (low five row bits only) so
+// both the 128-bit staging writes and the 128-bit operand reads are spread over
+// all banks.
+//
+// The weight operand goes to the MFMA "A" side and the activation to the "B"
+// side, so a lane ends up holding four consecutive OUTPUT COLUMNS of one output
+// row per accumulator quad: the epilogue scales, applies bias / SiLU-gate, rounds
+// to bf16 and stores 8 bytes per lane without a transpose.
+//
+// Workgroup -> tile mapping is XCD aware: consecutive workgroup ids go round-robin
+// to the 8 XCDs, so each XCD is given a contiguous range of tiles, walked in
+// 8 (M) x 4 (N) patches whose operands fit its own L2.
+#include "common.hpp"
+
+#include <mutex>
+
+namespace cf {
+namespace {
+
+constexpr int BM = 256, BN = 256, BK = 128;
+constexpr int kThreads = 256;
+constexpr int kTileBytes = BM * BK;               // 32 KiB per operand tile
+constexpr int kStageBytes = 2 * kTileBytes;       // X tile + W tile
+constexpr int kLdsBytes = 2 * kStageBytes;        // double buffered: 128 KiB
+constexpr int kXcds = 8;
+
+enum { EPI_NONE = 0, EPI_BIAS = 1, EPI_SILU_GATE = 2, EPI_ACCUM_F32 = 3, EPI_ACCUM_BF16 = 4 };
+enum { SCALE_TENSOR = 0, SCALE_ROWCOL = 1 };
+
+struct GemmArgs {
+    int M, N, K;                 // N = output columns
+    const uint8_t* A; int lda;   // activations [M,K]
+    const uint8_t* B; int ldb;   // weights [N,K] (gate weights for EPI_SILU_GATE)
+    const uint8_t* B2;           // up weights [N,K] for EPI_SILU_GATE
+    const float* sa;             // descale of A: [1] or [M]
+    const float* sb;             // descale of B: [1] or [N]
+    const float* sb2;            // descale of B2
+    const uint16_t* bias;        // bf16 [N] for EPI_BIAS
+    uint16_t* C; int ldc;        // bf16 [M,N]
+    float* Cf;                   // fp32 [M,N] for EPI_ACCUM_F32 (C += product)
+    int tiles_m, tiles_n;
+};
+
+__device__ __forceinline__ int swz(int row) { return (row ^ ((row >> 3) & 3)) & 7; }
+
+// tile index -> (tile_m, tile_n): contiguous range per XCD, 8 x 4 patches inside it
+__device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, int& tm, int& tn) {
+    const int total = tiles_m * tiles_n;
+    const int per_xcd = (total + kXcds - 1) / kXcds;
+    int t = (bid % kXcds) * per_xcd + bid / kXcds;
+    if (total % kXcds != 0) t = bid;                       // ragged tile counts keep the plain order
+    constexpr int GM = 8;
+    const int group = t / (GM * tiles_n);
+    const int first_m = group * GM;
+    const int gm = min(GM, tiles_m - first_m);
+    const int in_group = t - group * GM * tiles_n;
+    tm = first_m + in_group % gm;
+    tn = in_group / gm;
+}
+
+// FMT bit 0: A (activation side) is E5M2; bit 1: B (weight side) is E5M2
+template <int FMT, int EPI, int SCALE>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void k_gemm_nt(const GemmArgs p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+    int tile_m, tile_n;
+    tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+    constexpr int OUT_BN = EPI == EPI_SILU_GATE ? BN / 2 : BN;     // output columns per workgroup
+    const int m0 = tile_m * BM, n0 = tile_n * OUT_BN;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+
+    // ---- global -> register staging: thread owns chunk c of rows r0 + 32 i ----
+    const int r0 = tid >> 3, c = tid & 7;
+    const int lds_w = r0 * BK + ((c ^ swz(r0)) << 4);
+    const uint8_t* xsrc[8];
+    const uint8_t* wsrc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int row = r0 + 32 * i;
+        xsrc[i] = p.A + static_cast<size_t>(min(m0 + row, p.M - 1)) * p.lda + c * 16;
+        if constexpr (EPI == EPI_SILU_GATE) {
+            // LDS weight rows of a wave: [gate 32 | up 32 | gate 32 | up 32] over the same 64 output columns
+            const int t = (row >> 5) & 3, w = row >> 7;
+            const int n = n0 + w * 64 + (t >> 1) * 32 + (row & 31);
+            wsrc[i] = ((t & 1) ? p.B2 : p.B) + static_cast<size_t>(min(n, p.N - 1)) * p.ldb + c * 16;
+        } else {
+            wsrc[i] = p.B + static_cast<size_t>(min(n0 + row, p.N - 1)) * p.ldb + c * 16;
+        }
+    }
+    const bool kfull = (p.K % BK) == 0;
+    uint4 xr[8], wr[8];
+    auto fetch = [&](int k0) {
+        const bool live = kfull || (k0 + c * 16 < p.K);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            xr[i] = live ? *reinterpret_cast<const uint4*>(xsrc[i] + k0) : make_uint4(0, 0, 0, 0);
+            wr[i] = live ? *reinterpret_cast<const uint4*>(wsrc[i] + k0) : make_uint4(0, 0, 0, 0);
+        }
+    };
+    auto stash = [&](int stage) {
+        uint8_t* xs = smem + stage * kStageBytes + lds_w;
+        uint8_t* ws = xs + kTileBytes;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            *reinterpret_cast<uint4*>(xs + i * 32 * BK) = xr[i];
+            *reinterpret_cast<uint4*>(ws + i * 32 * BK) = wr[i];
+        }
+    };
+
+    // ---- LDS -> MFMA operand addressing ----
+    const int frow = lane & 31, khalf = lane >> 5, fs = swz(frow);
+    int rd[2][2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) rd[s][j] = frow * BK + (((s * 4 + khalf * 2 + j) ^ fs) << 4);
+    const int x_base = wm * 128 * BK, w_base = kTileBytes + wn * 128 * BK;
+
+    v16f acc[4][4];   // [weight tile][activation tile]
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
+
+    const int ktiles = (p.K + BK - 1) / BK;
+    fetch(0);
+    stash(0);
+    __syncthreads();
+
+    for (int kt = 0; kt < ktiles; ++kt) {
+        const int stage = kt & 1;
+        const bool more = kt + 1 < ktiles;
+        if (more) fetch((kt + 1) * BK);
+        const uint8_t* st = smem + stage * kStageBytes;
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            v8i wf[4], xf[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const uint4 w0 = *reinterpret_cast<const uint4*>(st + w_base + t * 32 * BK + rd[s][0]);
+                const uint4 w1 = *reinterpret_cast<const uint4*>(st + w_base + t * 32 * BK + rd[s][1]);
+                wf[t] = v8i{(int)w0.x, (int)w0.y, (int)w0.z, (int)w0.w, (int)w1.x, (int)w1.y, (int)w1.z, (int)w1.w};
+                const uint4 x0 = *reinterpret_cast<const uint4*>(st + x_base + t * 32 * BK + rd[s][0]);
+                const uint4 x1 = *reinterpret_cast<const uint4*>(st + x_base + t * 32 * BK + rd[s][1]);
+                xf[t] = v8i{(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w, (int)x1.x, (int)x1.y, (int)x1.z, (int)x1.w};
+            }
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+#pragma unroll
+                for (int b = 0; b < 4; ++b)
+                    acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                        wf[a], xf[b], acc[a][b], (FMT >> 1) & 1 /* weight side */, FMT & 1 /* activation side */, 0, 0, 0, 0);
+        }
+        if (more) stash(stage ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue ----
+    // acc[a][b][r]: output row m = m0 + wm*128 + b*32 + (lane & 31),
+    // weight row (within the wave's 128) = a*32 + 8*(r/4) + 4*(lane>>5) + r%4
+    const bool vec_ok = EPI == EPI_ACCUM_F32 ? (p.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.Cf) & 15u) == 0)
+                                             : (p.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.C) & 7u) == 0);
+    const float sa_t = SCALE == SCALE_TENSOR ? p.sa[0] : 0.0f;
+    const float sb_t = SCALE == SCALE_TENSOR ? p.sb[0] : 0.0f;
+    const float sb2_t = (SCALE == SCALE_TENSOR && EPI == EPI_SILU_GATE) ? p.sb2[0] : 0.0f;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        const int m = m0 + wm * 128 + b * 32 + (lane & 31);
+        if (m >= p.M) continue;
+        const float sa = SCALE == SCALE_TENSOR ? sa_t : p.sa[m];
+        uint16_t* crow = EPI == EPI_ACCUM_F32 ? nullptr : p.C + static_cast<size_t>(m) * p.ldc;
+        if constexpr (EPI == EPI_SILU_GATE) {
+#pragma unroll
+            for (int pair = 0; pair < 2; ++pair) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int n = n0 + wn * 64 + pair * 32 + g * 8 + khalf * 4;
+                    uint16_t o[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int nn = min(n + q, p.N - 1);
+                        const float sg = SCALE == SCALE_TENSOR ? sb_t : p.sb[nn];
+                        const float su = SCALE == SCALE_TENSOR ? sb2_t : p.sb2[nn];
+                        // the reference rounds gate and up to bf16 before the SiLU product
+                        const float gate = bf16_to_f32(f32_to_bf16(acc[2 * pair][b][g * 4 + q] * (sa * sg)));
+                        const float up = bf16_to_f32(f32_to_bf16(acc[2 * pair + 1][b][g * 4 + q] * (sa * su)));
+                        o[q] = f32_to_bf16((gate * stable_sigmoid(gate)) * up);
+                    }
+                    if (vec_ok && n + 3 < p.N) {
+                        *reinterpret_cast<uint2*>(crow + n) = make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
+                    } else {
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) if (n + q < p.N) crow[n + q] = o[q];
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int n = n0 + wn * 128 + a * 32 + g * 8 + khalf * 4;
+                    if constexpr (EPI == EPI_ACCUM_F32) {
+                        // beta = 1: the product is added to what the caller's fp32 buffer holds
+                        float* frow = p.Cf + static_cast<size_t>(m) * p.ldc + n;
+                        if (vec_ok && n + 3 < p.N) {
+                            float4 c4 = *reinterpret_cast<const float4*>(frow);
+                            c4.x += acc[a][b][g * 4 + 0] * (sa * sb_t);
+                            c4.y += acc[a][b][g * 4 + 1] * (sa * sb_t);
+                            c4.z += acc[a][b][g * 4 + 2] * (sa * sb_t);
+                            c4.w += acc[a][b][g * 4 + 3] * (sa * sb_t);
+                            *reinterpret_cast<float4*>(frow) = c4;
+                        } else {
+#pragma unroll
+                            for (int q = 0; q < 4; ++q) if (n + q < p.N) frow[q] += acc[a][b][g * 4 + q] * (sa * sb_t);
+                        }
+                        continue;
+                    }
+                    uint16_t o[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int nn = min(n + q, p.N - 1);
+                        const float sb = SCALE == SCALE_TENSOR ? sb_t : p.sb[nn];
+                        float v = acc[a][b][g * 4 + q] * (sa * sb);
+                        if constexpr (EPI == EPI_ACCUM_BF16) {
+                            if (n + q < p.N) v += bf16_to_f32(crow[n + q]);
+                        }
+                        if constexpr (EPI == EPI_BIAS)
+                            v = bf16_to_f32(f32_to_bf16(v)) + bf16_to_f32(p.bias[nn]);   // bias is added to the bf16 result
+                        o[q] = f32_to_bf16(v);
+                    }
+                    if (vec_ok && n + 3 < p.N) {
+                        *reinterpret_cast<uint2*>(crow + n) = make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
+                    } else {
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) if (n + q < p.N) crow[n + q] = o[q];
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ---- naive kernel: any shape, any alignment; also the on-device cross-check ----
+// one lane per output element, fp32 accumulate in k order
+__global__ __launch_bounds__(256) void k_gemm_nt_naive(const GemmArgs p, int fmt, int epi, int scale_mode) {
+    const long long idx = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= static_cast<long long>(p.M) * p.N) return;
+    const int m = static_cast<int>(idx / p.N), n = static_cast<int>(idx % p.N);
+    const uint8_t* a = p.A + static_cast<size_t>(m) * p.lda;
+    const uint8_t* b = p.B + static_cast<size_t>(n) * p.ldb;
+    const uint8_t* b2 = epi == EPI_SILU_GATE ? p.B2 + static_cast<size_t>(n) * p.ldb : nullptr;
+    float acc = 0.0f, acc2 = 0.0f;
+    for (int k = 0; k < p.K; ++k) {
+        const float av = (fmt & 1) ? e5m2_to_f32(a[k]) : e4m3_to_f32(a[k]);
+        acc = __builtin_fmaf(av, (fmt & 2) ? e5m2_to_f32(b[k]) : e4m3_to_f32(b[k]), acc);
+        if (b2) acc2 = __builtin_fmaf(av, e4m3_to_f32(b2[k]), acc2);
+    }
+    const float sa = scale_mode == SCALE_TENSOR ? p.sa[0] : p.sa[m];
+    const float sb = scale_mode == SCALE_TENSOR ? p.sb[0] : p.sb[n];
+    float v = acc * (sa * sb);
+    if (epi == EPI_ACCUM_F32) { p.Cf[static_cast<size_t>(m) * p.ldc + n] += v; return; }
+    if (epi == EPI_ACCUM_BF16) v += bf16_to_f32(p.C[static_cast<size_t>(m) * p.ldc + n]);
+    if (epi == EPI_BIAS) v = bf16_to_f32(f32_to_bf16(v)) + bf16_to_f32(p.bias[n]);
+    if (epi == EPI_SILU_GATE) {
+        const float su = scale_mode == SCALE_TENSOR ? p.sb2[0] : p.sb2[n];
+        const float gate = bf16_to_f32(f32_to_bf16(v));
+        const float up = bf16_to_f32(f32_to_bf16(acc2 * (sa * su)));
+        v = (gate * stable_sigmoid(gate)) * up;
+    }
+    p.C[static_cast<size_t>(m) * p.ldc + n] = f32_to_bf16(v);
+}
+
+template <int FMT, int EPI, int SCALE>
+int launch_tiled(const GemmArgs& p, hipStream_t st) {
+    static std::once_flag once;
+    static hipError_t attr_err = hipSuccess;
+    std::call_once(once, [] {
+        attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_nt<FMT, EPI, SCALE>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    });
+    if (attr_err != hipSuccess) return static_cast<int>(attr_err);
+    k_gemm_nt<FMT, EPI, SCALE><<<p.tiles_m * p.tiles_n, kThreads, kLdsBytes, st>>>(p);
+    return launch_status();
+}
+
+template <int FMT, int EPI>
+int dispatch_scale(const GemmArgs& p, int scale_mode, hipStream_t st) {
+    return scale_mode == SCALE_TENSOR ? launch_tiled<FMT, EPI, SCALE_TENSOR>(p, st)
+                                      : launch_tiled<FMT, EPI, SCALE_ROWCOL>(p, st);
+}
+// forward family: activations E4M3 or E5M2, weights E4M3
+template <int FMT>
+int dispatch_epi(const GemmArgs& p, int epi, int scale_mode, hipStream_t st) {
+    switch (epi) {
+        case EPI_NONE: return dispatch_scale<FMT, EPI_NONE>(p, scale_mode, st);
+        case EPI_BIAS: return dispatch_scale<FMT, EPI_BIAS>(p, scale_mode, st);
+        default:       return dispatch_scale<FMT, EPI_SILU_GATE>(p, scale_mode, st);
+    }
+}
+
+int gemm_nt(GemmArgs p, int fmt, int epi, int scale_mode, int force_naive, cf_stream_t stream) {
+    if (p.M < 0 || p.N < 0 || p.K < 0) return CF_ERR_INVALID_ARG;
+    if (p.M == 0 || p.N == 0) return CF_OK;
+    if (!p.A || !p.B || !(epi == EPI_ACCUM_F32 ? (void*)p.Cf : (void*)p.C) || !p.sa || !p.sb) return CF_ERR_INVALID_ARG;
+    if (epi < EPI_NONE || epi > EPI_ACCUM_BF16 || scale_mode < SCALE_TENSOR || scale_mode > SCALE_ROWCOL)
+        return CF_ERR_INVALID_ARG;
+    if (epi == EPI_BIAS && !p.bias) return CF_ERR_INVALID_ARG;
+    if (epi == EPI_SILU_GATE && (!p.B2 || !p.sb2)) return CF_ERR_INVALID_ARG;
+    if (p.lda < p.K || p.ldb < p.K || p.ldc < p.N) return CF_ERR_INVALID_ARG;
+    hipStream_t st = as_stream(stream);
+    const bool tiled_ok = p.K > 0 && p.K % 16 == 0 && p.lda % 16 == 0 && p.ldb % 16 == 0 && aligned16(p.A) &&
+                          aligned16(p.B) && (epi != EPI_SILU_GATE || aligned16(p.B2));
+    if (force_naive || !tiled_ok) {
+        const long long total = static_cast<long long>(p.M) * p.N;
+        k_gemm_nt_naive<<<static_cast<unsigned>((total + 255) / 256), 256, 0, st>>>(p, fmt, epi, scale_mode);
+        return launch_status();
+    }
+    const int out_bn = epi == EPI_SILU_GATE ? BN / 2 : BN;
+    p.tiles_m = (p.M + BM - 1) / BM;
+    p.tiles_n = (p.N + out_bn - 1) / out_bn;
+    if (epi == EPI_ACCUM_F32 || epi == EPI_ACCUM_BF16) {
+        // weight-gradient family: per-tensor scales only, any operand format pair
+        if (scale_mode != SCALE_TENSOR) return CF_ERR_UNSUPPORTED;
+        const bool f32 = epi == EPI_ACCUM_F32;
+        switch (fmt & 3) {
+            case 0: return f32 ? launch_tiled<0, EPI_ACCUM_F32, SCALE_TENSOR>(p, st) : launch_tiled<0, EPI_ACCUM_BF16, SCALE_TENSOR>(p, st);
+            case 1: return f32 ? launch_tiled<1, EPI_ACCUM_F32, SCALE_TENSOR>(p, st) : launch_tiled<1, EPI_ACCUM_BF16, SCALE_TENSOR>(p, st);
+            case 2: return f32 ? launch_tiled<2, EPI_ACCUM_F32, SCALE_TENSOR>(p, st) : launch_tiled<2, EPI_ACCUM_BF16, SCALE_TENSOR>(p, st);
+            default: return f32 ? launch_tiled<3, EPI_ACCUM_F32, SCALE_TENSOR>(p, st) : launch_tiled<3, EPI_ACCUM_BF16, SCALE_TENSOR>(p, st);
+        }
+    }
+    if (fmt & 2) return CF_ERR_UNSUPPORTED;     // forward weights are always E4M3
+    return (fmt & 1) ? dispatch_epi<1>(p, epi, scale_mode, st) : dispatch_epi<0>(p, epi, scale_mode, st);
+}
+
+}  // namespace
+}  // namespace cf
+
+using namespace cf;
+
+extern "C" {
+
+int cf_fp8_gemm_nt_bf16(int M, int N, int K, const void* A, int lda, int a_is_e5m2, const float* a_descale,
+                        const void* B, const float* b_descale, uint16_t* C, int ldc, cf_stream_t stream) {
+    GemmArgs p{};
+    p.M = M; p.N = N; p.K = K;
+    p.A = static_cast<const uint8_t*>(A); p.lda = lda;
+    p.B = static_cast<const uint8_t*>(B); p.ldb = K;
+    p.sa = a_descale; p.sb = b_descale;
+    p.C = C; p.ldc = ldc;
+    return gemm_nt(p, a_is_e5m2 ? 1 : 0, EPI_NONE, SCALE_TENSOR, 0, stream);
+}
+
+int cf_fp8_gemm_nt_bf16_ex(int M, int N, int K, const void* A, int lda, int a_is_e5m2, const float* a_descale,
+                           const void* B, int ldb, const float* b_descale, int scale_mode, int epilogue,
+                           const uint16_t* bias, const void* B_up, const float* b_up_descale, uint16_t* C,
+                           int ldc, int flags, cf_stream_t stream) {
+    GemmArgs p{};
+    p.M = M; p.N = N; p.K = K;
+    p.A = static_cast<const uint8_t*>(A); p.lda = lda;
+    p.B = static_cast<const uint8_t*>(B); p.ldb = ldb;
+    p.B2 = static_cast<const uint8_t*>(B_up);
+    p.sa = a_descale; p.sb = b_descale; p.sb2 = b_up_descale;
+    p.bias = bias;
+    p.C = C; p.ldc = ldc;
+    if (epilogue > EPI_SILU_GATE) return CF_ERR_INVALID_ARG;
+    return gemm_nt(p, a_is_e5m2 ? 1 : 0, epilogue, scale_mode, flags & CF_GEMM_FLAG_NAIVE, stream);
+}
+
+// dW[M,N] += X^T . dY with both operands pre-transposed to K-contiguous rows:
+// "A" = X^T [M,K] E4M3, "B" = dY^T [N,K] E5M2.
+int cf_fp8_gemm_tn_accum_f32(int M, int N, int K, const void* Xt_e4m3, const float* ds_x, const void* dYt_e5m2,
+                             const float* ds_dy, float* dW, int ldc_dw, cf_stream_t stream) {
+    GemmArgs p{};
+    p.M = M; p.N = N; p.K = K;
+    p.A = static_cast<const uint8_t*>(Xt_e4m3); p.lda = K;
+    p.B = static_cast<const uint8_t*>(dYt_e5m2); p.ldb = K;
+    p.sa = ds_x; p.sb = ds_dy;
+    p.Cf = dW; p.ldc = ldc_dw;
+    return gemm_nt(p, 2, EPI_ACCUM_F32, SCALE_TENSOR, 0, stream);
+}
+
+int cf_fp8_gemm_tn_accum_bf16(int M, int N, int K, const void* Xt_e4m3, const float* ds_x, const void* dYt_e5m2,
+                              const float* ds_dy, uint16_t* dW, int ldc_dw, cf_stream_t stream) {
+    GemmArgs p{};
+    p.M = M; p.N = N; p.K = K;
+    p.A = static_cast<const uint8_t*>(Xt_e4m3); p.lda = K;
+    p.B = static_cast<const uint8_t*>(dYt_e5m2); p.ldb = K;
+    p.sa = ds_x; p.sb = ds_dy;
+    p.C = dW; p.ldc = ldc_dw;
+    return gemm_nt(p, 2, EPI_ACCUM_BF16, SCALE_TENSOR, 0, stream);
+}
+
+// Cross-check form of the accumulate GEMMs: any format pair, optional naive kernel.
+int cf_fp8_gemm_nt_accum_f32_ex(int M, int N, int K, const void* A, int lda, int a_is_e5m2, const float* a_descale,
+                                const void* B, int ldb, int b_is_e5m2, const float* b_descale, float* C, int ldc,
+                                int flags, cf_stream_t stream) {
+    GemmArgs p{};
+    p.M = M; p.N = N; p.K = K;
+    p.A = static_cast<const uint8_t*>(A); p.lda = lda;
+    p.B = static_cast<const uint8_t*>(B); p.ldb = ldb;
+    p.sa = a_descale; p.sb = b_descale;
+    p.Cf = C; p.ldc = ldc;
+    return gemm_nt(p, (a_is_e5m2 ? 1 : 0) | (b_is_e5m2 ? 2 : 0), EPI_ACCUM_F32, SCALE_TENSOR,
+                   flags & CF_GEMM_FLAG_NAIVE, stream);
+}
+
+}  // extern "C"

@@ -136,6 +136,61 @@ int cf_swiglu_forward(const uint16_t* d_gate, const uint16_t* d_up, uint16_t* d_
 int cf_bias_add_strided_bf16(uint16_t* d_inout, const uint16_t* d_bias, int rows, int cols,
                              int row_stride, int base, cf_stream_t stream);
 
+/* ---- scaled FP8 GEMM -------------------------------------------------------
+ * Replaces the reference's cuBLASLt wrappers, which are static functions of
+ * src/trainer.cu bound to its Fp8Ctx (handle, workspace, plan cache); the
+ * entry points take the same operands without the context.  fp32 accumulate. */
+
+#define CF_SCALE_PER_TENSOR 0  /* a_descale[1], b_descale[1] (device scalars)   */
+#define CF_SCALE_ROW_COL    1  /* a_descale[M] per token, b_descale[N] per channel */
+#define CF_SCALE_BLOCK_128  2  /* a_descale[M, ceil(K/128)], b_descale[ceil(N/128), ceil(K/128)] */
+
+#define CF_EPI_NONE      0     /* C = bf16(acc * sa * sb)                          */
+#define CF_EPI_BIAS      1     /* C = bf16(bf16(acc * sa * sb) + bias[n]), i.e. the GEMM followed by
+                                  bias_add_strided_bf16 (kernels/moe.cu:325-334)   */
+#define CF_EPI_SILU_GATE 2     /* C = swiglu(bf16(gate), bf16(up)): two weight matrices, the GEMMs at
+                                  src/trainer.cu:6310-6312 followed by swiglu_forward (:6322) */
+
+#define CF_GEMM_FLAG_NAIVE 1   /* run the one-lane-per-output cross-check kernel  */
+
+/* lt_gemm_fp8_nt, static at src/trainer.cu:4498-4534 (plan lookup :4402-4496).
+ * C[M,N] bf16 (row stride ldc) = (A[M,K] fp8, row stride lda, E4M3 or E5M2) .
+ * (B[N,K] E4M3, contiguous)^T, per-tensor device descales, alpha 1, beta 0. */
+int cf_fp8_gemm_nt_bf16(int M, int N, int K, const void* d_A, int lda, int a_is_e5m2,
+                        const float* d_a_descale, const void* d_B, const float* d_b_descale,
+                        uint16_t* d_C, int ldc, cf_stream_t stream);
+
+/* Extended form of the same GEMM for the scale groups and fused epilogues of
+ * the benchmark configurations (the reference runs src/trainer.cu:4498 and
+ * then kernels/activations.cu:76-87 or kernels/moe.cu:349-356 as separate
+ * launches).  d_bias is bf16 [N] for CF_EPI_BIAS; d_B_up / d_b_up_descale are
+ * the second ("up") weight matrix [N,K] and its descale for CF_EPI_SILU_GATE;
+ * unused pointers may be null. */
+int cf_fp8_gemm_nt_bf16_ex(int M, int N, int K, const void* d_A, int lda, int a_is_e5m2,
+                           const float* d_a_descale, const void* d_B, int ldb,
+                           const float* d_b_descale, int scale_mode, int epilogue,
+                           const uint16_t* d_bias, const void* d_B_up,
+                           const float* d_b_up_descale, uint16_t* d_C, int ldc, int flags,
+                           cf_stream_t stream);
+
+/* lt_gemm_fp8_tn_accum_f32, fp32 overload, static at src/trainer.cu:4596-4627 (plan :4539-4594).
+ * dW[M,N] fp32 (row stride ldc_dw) += (X^T[M,K] E4M3 * ds_x) . (dY^T[N,K] E5M2 * ds_dy)^T,
+ * both operands contiguous with K innermost (pre-transposed), alpha 1, beta 1. */
+int cf_fp8_gemm_tn_accum_f32(int M, int N, int K, const void* d_Xt_e4m3, const float* d_ds_x,
+                             const void* d_dYt_e5m2, const float* d_ds_dy, float* d_dW,
+                             int ldc_dw, cf_stream_t stream);
+/* lt_gemm_fp8_tn_accum_f32, bf16 overload, static at src/trainer.cu:4670-4691. */
+int cf_fp8_gemm_tn_accum_bf16(int M, int N, int K, const void* d_Xt_e4m3, const float* d_ds_x,
+                              const void* d_dYt_e5m2, const float* d_ds_dy, uint16_t* d_dW,
+                              int ldc_dw, cf_stream_t stream);
+/* The accumulate GEMM of src/trainer.cu:4596-4627 with free operand formats and row strides, and
+ * CF_GEMM_FLAG_NAIVE for the cross-check kernel; used by the tests and for fp32 inspection of
+ * the accumulators. */
+int cf_fp8_gemm_nt_accum_f32_ex(int M, int N, int K, const void* d_A, int lda, int a_is_e5m2,
+                                const float* d_a_descale, const void* d_B, int ldb, int b_is_e5m2,
+                                const float* d_b_descale, float* d_C, int ldc, int flags,
+                                cf_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,186 @@
+"""GPU parity: the scaled FP8 GEMM against the CPU oracle (matmul of the dequantised operands,
+carried in double).  Bar: relative L2 error <= 1e-3 and max error <= 2 bf16 ulps of |ref|
+(see oracle_lib.assert_gemm_close for the accumulation-order term near cancellation)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle_lib as orc
+from gpu_util import bf16_bits, case, dev_arr, dev_bf16, host, scalar, stream
+
+pytestmark = pytest.mark.gpu
+
+PER_TENSOR, ROW_COL = 0, 1
+EPI_NONE, EPI_BIAS, EPI_SILU = 0, 1, 2
+NAIVE = 1
+
+
+def rand_fp8(rng, shape, e5m2=False, sigma=1.0):
+    """Quantised operand bytes drawn like a real tensor: N(0, sigma) scaled to the format's range."""
+    x = (rng.standard_normal(shape) * sigma).astype(np.float32)
+    fmax = 57344.0 if e5m2 else 448.0
+    s = np.float32(fmax) / np.abs(x).max()
+    q = orc.e5m2_satfinite(x * s) if e5m2 else orc.e4m3_satfinite(x * s)
+    return q, np.float32(1.0) / s
+
+
+def silu_ref(gate_ref, up_ref):
+    """The reference epilogue on exact inputs: bf16(gate), bf16(up) -> bf16(silu*up) (kernels/activations.cu:28-40)."""
+    g = orc.bf16_to_f32(orc.bf16_from_f32(gate_ref.astype(np.float32))).astype(np.float64)
+    u = orc.bf16_to_f32(orc.bf16_from_f32(up_ref.astype(np.float32))).astype(np.float64)
+    return g / (1.0 + np.exp(-g)) * u
+
+
+def run_gemm(cf, dev, A, B, sa, sb, *, lda=None, a_e5m2=False, mode=PER_TENSOR, epi=EPI_NONE, bias=None,
+             B2=None, sb2=None, flags=0, ldc=None):
+    M, K = A.shape[0], B.shape[1]
+    N = B.shape[0]
+    lda = A.shape[1] if lda is None else lda
+    ldc = N if ldc is None else ldc
+    Ad, Bd = dev_arr(A, dev), dev_arr(B, dev)
+    C = torch.full((M, ldc), float("nan"), dtype=torch.bfloat16, device=dev)
+    cf.cf_fp8_gemm_nt_bf16_ex(M, N, K, Ad, lda, int(a_e5m2), dev_arr(np.atleast_1d(sa).astype(np.float32), dev),
+                              Bd, K, dev_arr(np.atleast_1d(sb).astype(np.float32), dev), mode, epi,
+                              None if bias is None else dev_bf16(bias, dev),
+                              None if B2 is None else dev_arr(B2, dev),
+                              None if sb2 is None else dev_arr(np.atleast_1d(sb2).astype(np.float32), dev),
+                              C, ldc, flags, stream())
+    torch.cuda.synchronize()
+    return orc.bf16_to_f32(bf16_bits(C)).astype(np.float64)
+
+
+SHAPES = [(256, 256, 128), (512, 768, 1024), (300, 200, 144), (1, 1, 16), (33, 500, 208), (257, 129, 4096), (64, 1408, 2048)]
+
+
+@pytest.mark.parametrize("M,N,K", SHAPES)
+@pytest.mark.parametrize("flags", [0, NAIVE])
+def test_gemm_per_tensor(cf, dev, M, N, K, flags):
+    case(f"gemm per-tensor {M}x{N}x{K} flags={flags}")
+    rng = np.random.default_rng(M + N + K)
+    A, sa = rand_fp8(rng, (M, K))
+    B, sb = rand_fp8(rng, (N, K), sigma=0.02)
+    got = run_gemm(cf, dev, A, B, sa, sb, flags=flags)
+    ref, absdot = orc.gemm_nt_ref(A, B, [sa], [sb])
+    orc.assert_gemm_close(got, ref, absdot, what=f"{M}x{N}x{K}", acc=orc.ACC_FP32 if flags else orc.ACC_MFMA)
+    # without any allowance: only cancellation points (|ref| << sum|a b|) may exceed 2 bf16 ulps
+    off = np.abs(got - ref) > 2 * orc.bf16_ulp(ref)
+    assert off.mean() <= 0.03 and np.all(np.abs(ref[off]) <= 2.0 ** -9 * absdot[off])
+
+
+def test_gemm_exact_small_integers_equals_numpy_matmul(cf, dev):
+    """All scales 1 and operands small integers: every product and partial sum is exact in fp32,
+    so the GEMM must equal numpy's matmul to the last bit of the bf16 rounding."""
+    case("gemm exact integers")
+    rng = np.random.default_rng(0)
+    M, N, K = 256, 512, 256
+    ai = rng.integers(-3, 4, (M, K)).astype(np.float32)
+    bi = rng.integers(-2, 3, (N, K)).astype(np.float32)
+    A, B = orc.e4m3_satfinite(ai), orc.e4m3_satfinite(bi)
+    got = run_gemm(cf, dev, A, B, 1.0, 1.0)
+    want = orc.bf16_to_f32(orc.bf16_from_f32((ai @ bi.T).astype(np.float32)))
+    assert np.array_equal(got, want)
+    # a transposed or misindexed operand cannot pass this: the matrix is far from symmetric
+    assert not np.array_equal(got[:256, :256], got[:256, :256].T)
+
+
+@pytest.mark.parametrize("flags", [0, NAIVE])
+def test_gemm_e5m2_activations_and_row_stride(cf, dev, flags):
+    case(f"gemm e5m2 A + lda flags={flags}")
+    rng = np.random.default_rng(5)
+    M, N, K, lda = 200, 300, 512, 512 + 64
+    A, sa = rand_fp8(rng, (M, lda), e5m2=True, sigma=1e-3)
+    B, sb = rand_fp8(rng, (N, K), sigma=0.02)
+    got = run_gemm(cf, dev, A, B, sa, sb, lda=lda, a_e5m2=True, flags=flags, ldc=N + 8)[:, :N]
+    ref, absdot = orc.gemm_nt_ref(A, B, [sa], [sb], a_e5m2=True, lda=lda)
+    orc.assert_gemm_close(got, ref, absdot)
+
+
+@pytest.mark.parametrize("flags", [0, NAIVE])
+def test_gemm_row_col_scales_and_bias(cf, dev, flags):
+    case(f"gemm row/col scales + bias flags={flags}")
+    rng = np.random.default_rng(6)
+    M, N, K = 300, 260, 384
+    A, _ = rand_fp8(rng, (M, K))
+    B, _ = rand_fp8(rng, (N, K), sigma=0.02)
+    sa = rng.uniform(0.001, 0.02, M).astype(np.float32)
+    sb = rng.uniform(1e-5, 1e-4, N).astype(np.float32)
+    got = run_gemm(cf, dev, A, B, sa, sb, mode=ROW_COL, flags=flags)
+    ref, absdot = orc.gemm_nt_ref(A, B, sa, sb, scale_mode=1)
+    orc.assert_gemm_close(got, ref, absdot)
+    bias = orc.bf16_from_f32((rng.standard_normal(N) * np.abs(ref).mean()).astype(np.float32))
+    gotb = run_gemm(cf, dev, A, B, sa, sb, mode=ROW_COL, epi=EPI_BIAS, bias=bias, flags=flags)
+    # bias is added to the bf16-rounded product (GEMM then bias_add_strided_bf16): exact given the plain result
+    want = orc.bf16_to_f32(orc.bf16_from_f32((got + orc.bf16_to_f32(bias)[None, :].astype(np.float64)).astype(np.float32)))
+    assert np.array_equal(gotb, want)
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 128, 256), (300, 200, 512), (512, 1408, 2048)])
+@pytest.mark.parametrize("mode", [PER_TENSOR, ROW_COL])
+def test_gemm_fused_silu_gate(cf, dev, M, N, K, mode):
+    case(f"gemm silu-gate {M}x{N}x{K} mode={mode}")
+    rng = np.random.default_rng(M + N + mode)
+    A, sa = rand_fp8(rng, (M, K))
+    Bg, sg = rand_fp8(rng, (N, K), sigma=0.02)
+    Bu, su = rand_fp8(rng, (N, K), sigma=0.02)
+    if mode == ROW_COL:
+        sa = (sa * rng.uniform(0.5, 2, M)).astype(np.float32)
+        sg = (sg * rng.uniform(0.5, 2, N)).astype(np.float32)
+        su = (su * rng.uniform(0.5, 2, N)).astype(np.float32)
+    fused = run_gemm(cf, dev, A, Bg, sa, sg, mode=mode, epi=EPI_SILU, B2=Bu, sb2=su)
+    # (1) identical to running the two plain GEMMs and the stand-alone swiglu kernel
+    gate = run_gemm(cf, dev, A, Bg, sa, sg, mode=mode)
+    up = run_gemm(cf, dev, A, Bu, sa, su, mode=mode)
+    want = orc.bf16_to_f32(orc.swiglu_forward(orc.bf16_from_f32(gate.astype(np.float32)), orc.bf16_from_f32(up.astype(np.float32))))
+    assert np.array_equal(fused, want)
+    naive = run_gemm(cf, dev, A, Bg, sa, sg, mode=mode, epi=EPI_SILU, B2=Bu, sb2=su, flags=NAIVE)
+    # (2) close to the exact-input reference epilogue; gate/up each carry <= 1 bf16 ulp of input rounding
+    gref, _ = orc.gemm_nt_ref(A, Bg, np.atleast_1d(sa), np.atleast_1d(sg), scale_mode=mode, want_abs=False)
+    uref, _ = orc.gemm_nt_ref(A, Bu, np.atleast_1d(sa), np.atleast_1d(su), scale_mode=mode, want_abs=False)
+    exact = silu_ref(gref, uref)
+    for got in (fused, naive):
+        rel = np.sqrt(((got - exact) ** 2).sum() / (exact ** 2).sum())
+        assert rel <= 4e-3, rel      # three bf16 roundings (gate, up, product): ~2^-9 * sqrt(3) relative
+
+
+def test_gemm_config2_shape_sampled_rows_and_naive_crosscheck(cf, dev):
+    """M=8192, K=4096, N=14336 (the benchmark shape): per-token / per-channel scales, outliers at +-40."""
+    case("gemm config 2 full size")
+    M, N, K = 8192, 14336, 4096
+    g = torch.Generator(device=dev).manual_seed(22)
+    x = torch.randn((M, K), generator=g, device=dev)
+    u = torch.rand((M, K), generator=g, device=dev)
+    x = torch.where(u < 0.0005, torch.full_like(x, 40.0), x)
+    x = torch.where(u > 0.9995, torch.full_like(x, -40.0), x).to(torch.bfloat16)
+    w = (torch.randn((N, K), generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    xq = torch.empty((M, K), dtype=torch.uint8, device=dev); xs = torch.empty(M, device=dev); xd = torch.empty(M, device=dev)
+    wq = torch.empty((N, K), dtype=torch.uint8, device=dev); ws = torch.empty(N, device=dev); wd = torch.empty(N, device=dev)
+    cf.cf_fp8_quantize_rows(x, M, K, 0, xq, xs, xd, stream())
+    cf.cf_fp8_quantize_rows(w, N, K, 0, wq, ws, wd, stream())
+    C = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+    Cn = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+    cf.cf_fp8_gemm_nt_bf16_ex(M, N, K, xq, K, 0, xd, wq, K, wd, ROW_COL, EPI_NONE, None, None, None, C, N, 0, stream())
+    cf.cf_fp8_gemm_nt_bf16_ex(M, N, K, xq, K, 0, xd, wq, K, wd, ROW_COL, EPI_NONE, None, None, None, Cn, N, NAIVE, stream())
+    torch.cuda.synchronize()
+    # tiled vs naive over the whole output: both are fp32 accumulations of the same products
+    diff = (C.float() - Cn.float()).abs()
+    ulp = torch.maximum(Cn.float().abs(), torch.tensor(1e-30, device=dev)).log2().floor().sub(7).exp2()
+    frac_off = (diff > 2 * ulp).float().mean().item()
+    assert frac_off < 5e-3, frac_off      # cancellation points only: the MFMA keeps fewer bits than an fp32 FMA chain
+    rel = (diff.double().pow(2).sum() / Cn.double().pow(2).sum()).sqrt().item()
+    assert rel < 1e-3
+    # sampled rows against the CPU oracle
+    rows = np.sort(np.random.default_rng(1).choice(M, 48, replace=False))
+    ridx = torch.from_numpy(rows).to(dev)
+    ref, absdot = orc.gemm_nt_ref(host(xq[ridx]), host(wq), host(xd[ridx]), host(wd), scale_mode=1)
+    got = orc.bf16_to_f32(bf16_bits(C[ridx])).astype(np.float64)
+    orc.assert_gemm_close(got, ref, absdot, what="config 2 sampled rows")
+
+
+def test_gemm_argument_errors(cf, dev):
+    a = torch.zeros(16, dtype=torch.uint8, device=dev)
+    c = torch.zeros(16, dtype=torch.bfloat16, device=dev)
+    s = scalar(1.0, dev)
+    assert cf.raw_cf_fp8_gemm_nt_bf16(-1, 1, 16, a.data_ptr(), 16, 0, s.data_ptr(), a.data_ptr(), s.data_ptr(), c.data_ptr(), 1, None) == -1
+    assert cf.raw_cf_fp8_gemm_nt_bf16(1, 1, 16, None, 16, 0, s.data_ptr(), a.data_ptr(), s.data_ptr(), c.data_ptr(), 1, None) == -1
+    assert cf.raw_cf_fp8_gemm_nt_bf16(1, 1, 16, a.data_ptr(), 8, 0, s.data_ptr(), a.data_ptr(), s.data_ptr(), c.data_ptr(), 1, None) == -1
+    assert cf.raw_cf_fp8_gemm_nt_bf16(0, 1, 16, a.data_ptr(), 16, 0, s.data_ptr(), a.data_ptr(), s.data_ptr(), c.data_ptr(), 1, None) == 0

@@ -10,7 +10,7 @@ from pathlib import Path
 PKG = Path(__file__).resolve().parent
 CSRC = PKG / "csrc"
 INCLUDE = PKG.parent / "include"
-LIB = PKG / "libcf_fp8.so"
+LIB = Path(os.environ.get("CF_LIB_OUT", PKG / "libcf_fp8.so"))
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -38,8 +38,8 @@ def _compile(src: Path, obj: Path, extra: list[str]) -> None:
 def build(force: bool = True, extra: list[str] | None = None, jobs: int = 8) -> Path:
     """Compiles every .hip under csrc/ and links libcf_fp8.so next to this file."""
     extra = list(extra or [])
-    objdir = CSRC / "build"
-    objdir.mkdir(exist_ok=True)
+    objdir = Path(os.environ.get("CF_OBJ_DIR", CSRC / "build"))
+    objdir.mkdir(exist_ok=True, parents=True)
     srcs = sources()
     hdrs = list(CSRC.glob("*.hpp")) + list(INCLUDE.glob("*.h"))
     newest_hdr = max((h.stat().st_mtime for h in hdrs), default=0.0)

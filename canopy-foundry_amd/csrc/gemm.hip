@@ -23,6 +23,7 @@
 #include "common.hpp"
 
 #include <mutex>
+#include <type_traits>
 
 namespace cf {
 namespace {
@@ -49,6 +50,7 @@ struct GemmArgs {
     uint16_t* C; int ldc;        // bf16 [M,N]
     float* Cf;                   // fp32 [M,N] for EPI_ACCUM_F32 (C += product)
     int tiles_m, tiles_n;
+    int force_staged;            // take the register-staged kernel even when the ring kernel applies
 };
 
 __device__ __forceinline__ int swz(int row) { return (row ^ ((row >> 3) & 3)) & 7; }
@@ -66,6 +68,96 @@ __device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, i
     const int in_group = t - group * GM * tiles_n;
     tm = first_m + in_group % gm;
     tn = in_group / gm;
+}
+
+// ---- epilogue shared by the tiled kernels ----------------------------------------
+// acc[a][b][r]: output row m = m0 + wm*128 + b*32 + (lane & 31); weight row within the
+// wave's 128 = a*32 + 8*(r/4) + 4*(lane>>5) + r%4, i.e. four consecutive output columns per quad.
+template <int EPI, int SCALE>
+__device__ __forceinline__ void epilogue(v16f (&acc)[4][4], const GemmArgs& p, int m0, int n0, int wm, int wn,
+                                         int lane) {
+    const int khalf = lane >> 5;
+    const bool vec_ok = EPI == EPI_ACCUM_F32 ? (p.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.Cf) & 15u) == 0)
+                                             : (p.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.C) & 7u) == 0);
+    const float sa_t = SCALE == SCALE_TENSOR ? p.sa[0] : 0.0f;
+    const float sb_t = SCALE == SCALE_TENSOR ? p.sb[0] : 0.0f;
+    const float sb2_t = (SCALE == SCALE_TENSOR && EPI == EPI_SILU_GATE) ? p.sb2[0] : 0.0f;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        const int m = m0 + wm * 128 + b * 32 + (lane & 31);
+        if (m >= p.M) continue;
+        const float sa = SCALE == SCALE_TENSOR ? sa_t : p.sa[m];
+        uint16_t* crow = EPI == EPI_ACCUM_F32 ? nullptr : p.C + static_cast<size_t>(m) * p.ldc;
+        if constexpr (EPI == EPI_SILU_GATE) {
+#pragma unroll
+            for (int pair = 0; pair < 2; ++pair) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int n = n0 + wn * 64 + pair * 32 + g * 8 + khalf * 4;
+                    uint16_t o[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int nn = min(n + q, p.N - 1);
+                        const float sg = SCALE == SCALE_TENSOR ? sb_t : p.sb[nn];
+                        const float su = SCALE == SCALE_TENSOR ? sb2_t : p.sb2[nn];
+                        // the reference rounds gate and up to bf16 before the SiLU product
+                        const float gate = bf16_to_f32(f32_to_bf16(acc[2 * pair][b][g * 4 + q] * (sa * sg)));
+                        const float up = bf16_to_f32(f32_to_bf16(acc[2 * pair + 1][b][g * 4 + q] * (sa * su)));
+                        o[q] = f32_to_bf16((gate * stable_sigmoid(gate)) * up);
+                    }
+                    if (vec_ok && n + 3 < p.N) {
+                        *reinterpret_cast<uint2*>(crow + n) = make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
+                    } else {
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) if (n + q < p.N) crow[n + q] = o[q];
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int n = n0 + wn * 128 + a * 32 + g * 8 + khalf * 4;
+                    if constexpr (EPI == EPI_ACCUM_F32) {
+                        // beta = 1: the product is added to what the caller's fp32 buffer holds
+                        float* frow = p.Cf + static_cast<size_t>(m) * p.ldc + n;
+                        if (vec_ok && n + 3 < p.N) {
+                            float4 c4 = *reinterpret_cast<const float4*>(frow);
+                            c4.x += acc[a][b][g * 4 + 0] * (sa * sb_t);
+                            c4.y += acc[a][b][g * 4 + 1] * (sa * sb_t);
+                            c4.z += acc[a][b][g * 4 + 2] * (sa * sb_t);
+                            c4.w += acc[a][b][g * 4 + 3] * (sa * sb_t);
+                            *reinterpret_cast<float4*>(frow) = c4;
+                        } else {
+#pragma unroll
+                            for (int q = 0; q < 4; ++q) if (n + q < p.N) frow[q] += acc[a][b][g * 4 + q] * (sa * sb_t);
+                        }
+                        continue;
+                    }
+                    uint16_t o[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int nn = min(n + q, p.N - 1);
+                        const float sb = SCALE == SCALE_TENSOR ? sb_t : p.sb[nn];
+                        float v = acc[a][b][g * 4 + q] * (sa * sb);
+                        if constexpr (EPI == EPI_ACCUM_BF16) {
+                            if (n + q < p.N) v += bf16_to_f32(crow[n + q]);
+                        }
+                        if constexpr (EPI == EPI_BIAS)
+                            v = bf16_to_f32(f32_to_bf16(v)) + bf16_to_f32(p.bias[nn]);   // bias is added to the bf16 result
+                        o[q] = f32_to_bf16(v);
+                    }
+                    if (vec_ok && n + 3 < p.N) {
+                        *reinterpret_cast<uint2*>(crow + n) = make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
+                    } else {
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) if (n + q < p.N) crow[n + q] = o[q];
+                    }
+                }
+            }
+        }
+    }
 }
 
 // FMT bit 0: A (activation side) is E5M2; bit 1: B (weight side) is E5M2
@@ -170,90 +262,173 @@ void k_gemm_nt(const GemmArgs p) {
         __syncthreads();
     }
 
-    // ---- epilogue ----
-    // acc[a][b][r]: output row m = m0 + wm*128 + b*32 + (lane & 31),
-    // weight row (within the wave's 128) = a*32 + 8*(r/4) + 4*(lane>>5) + r%4
-    const bool vec_ok = EPI == EPI_ACCUM_F32 ? (p.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.Cf) & 15u) == 0)
-                                             : (p.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.C) & 7u) == 0);
-    const float sa_t = SCALE == SCALE_TENSOR ? p.sa[0] : 0.0f;
-    const float sb_t = SCALE == SCALE_TENSOR ? p.sb[0] : 0.0f;
-    const float sb2_t = (SCALE == SCALE_TENSOR && EPI == EPI_SILU_GATE) ? p.sb2[0] : 0.0f;
+    epilogue<EPI, SCALE>(acc, p, m0, n0, wm, wn, lane);
+}
+
+
+// ---- ring kernel: direct-to-LDS copies into five 32 KiB slots --------------------------------
+// Needs K % 128 == 0 and K >= 256.  global_load_lds_dwordx4 copies 16 bytes per lane from global
+// memory straight into LDS (lane l lands at base + 16*l): no staging registers, and eight lanes
+// fetch one full 128-byte line of a row (half-line requests reach only ~60% of the L2 rate).
+// A slot holds one operand tile [256 rows][128 bytes], chunks xor-swizzled as in the staged kernel.
+// Operand tile i (X of K-tile i/2 for even i, W for odd i) lives in slot i % 5, so while K-tile kt is
+// being multiplied, K-tile kt+1 is resident or landing and the X half of kt+2 is already on its way.
+//
+// A K-tile is two MFMA steps (k-halves of 64).  Step (kt,0): 16 MFMAs, the operand reads of (kt,1),
+// the 8 copies of X(kt+2).  Step (kt,1): 2 MFMAs, wait for K-tile kt+1, barrier, 14 MFMAs woven
+// with the operand reads of (kt+1,0) and the 8 copies of W(kt+2).  One barrier per 2048 MFMA cycles;
+// a copy has two to three steps (2000-3000 cycles) to land.
+constexpr int kSlotBytes = BM * BK;               // 32 KiB
+constexpr int kSlots = 5;
+constexpr int kRingLds = kSlots * kSlotBytes;     // 160 KiB: all of a CU's LDS
+
+// s_waitcnt immediates: vmcnt in bits [3:0] and [15:14], expcnt [6:4] and lgkmcnt [11:8] left at no-wait
+constexpr int kWaitVm0 = 0x0f70, kWaitVm8 = 0x0f78, kWaitVm16 = 0x4f70;
+
+template <int FMT, int EPI, int SCALE>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void k_gemm_nt_ring(const GemmArgs p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+    int tile_m, tile_n;
+    tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+    constexpr int OUT_BN = EPI == EPI_SILU_GATE ? BN / 2 : BN;
+    const int m0 = tile_m * BM, n0 = tile_n * OUT_BN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+
+    // ---- global -> LDS: wave w copies rows [64w, 64w+64) of an operand tile, 8 rows per instruction ----
+    const int lrow = lane >> 3, lslot = lane & 7;
+    const uint8_t* xsrc[8];
+    const uint8_t* wsrc[8];
 #pragma unroll
-    for (int b = 0; b < 4; ++b) {
-        const int m = m0 + wm * 128 + b * 32 + (lane & 31);
-        if (m >= p.M) continue;
-        const float sa = SCALE == SCALE_TENSOR ? sa_t : p.sa[m];
-        uint16_t* crow = EPI == EPI_ACCUM_F32 ? nullptr : p.C + static_cast<size_t>(m) * p.ldc;
+    for (int j = 0; j < 8; ++j) {
+        const int row = wave * 64 + j * 8 + lrow;
+        const int gchunk = (lslot ^ swz(row)) * 16;
+        xsrc[j] = p.A + static_cast<size_t>(min(m0 + row, p.M - 1)) * p.lda + gchunk;
         if constexpr (EPI == EPI_SILU_GATE) {
-#pragma unroll
-            for (int pair = 0; pair < 2; ++pair) {
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int n = n0 + wn * 64 + pair * 32 + g * 8 + khalf * 4;
-                    uint16_t o[4];
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const int nn = min(n + q, p.N - 1);
-                        const float sg = SCALE == SCALE_TENSOR ? sb_t : p.sb[nn];
-                        const float su = SCALE == SCALE_TENSOR ? sb2_t : p.sb2[nn];
-                        // the reference rounds gate and up to bf16 before the SiLU product
-                        const float gate = bf16_to_f32(f32_to_bf16(acc[2 * pair][b][g * 4 + q] * (sa * sg)));
-                        const float up = bf16_to_f32(f32_to_bf16(acc[2 * pair + 1][b][g * 4 + q] * (sa * su)));
-                        o[q] = f32_to_bf16((gate * stable_sigmoid(gate)) * up);
-                    }
-                    if (vec_ok && n + 3 < p.N) {
-                        *reinterpret_cast<uint2*>(crow + n) = make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
-                    } else {
-#pragma unroll
-                        for (int q = 0; q < 4; ++q) if (n + q < p.N) crow[n + q] = o[q];
-                    }
-                }
-            }
+            const int t = (row >> 5) & 3, w = row >> 7;
+            const int n = n0 + w * 64 + (t >> 1) * 32 + (row & 31);
+            wsrc[j] = ((t & 1) ? p.B2 : p.B) + static_cast<size_t>(min(n, p.N - 1)) * p.ldb + gchunk;
         } else {
-#pragma unroll
-            for (int a = 0; a < 4; ++a) {
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int n = n0 + wn * 128 + a * 32 + g * 8 + khalf * 4;
-                    if constexpr (EPI == EPI_ACCUM_F32) {
-                        // beta = 1: the product is added to what the caller's fp32 buffer holds
-                        float* frow = p.Cf + static_cast<size_t>(m) * p.ldc + n;
-                        if (vec_ok && n + 3 < p.N) {
-                            float4 c4 = *reinterpret_cast<const float4*>(frow);
-                            c4.x += acc[a][b][g * 4 + 0] * (sa * sb_t);
-                            c4.y += acc[a][b][g * 4 + 1] * (sa * sb_t);
-                            c4.z += acc[a][b][g * 4 + 2] * (sa * sb_t);
-                            c4.w += acc[a][b][g * 4 + 3] * (sa * sb_t);
-                            *reinterpret_cast<float4*>(frow) = c4;
-                        } else {
-#pragma unroll
-                            for (int q = 0; q < 4; ++q) if (n + q < p.N) frow[q] += acc[a][b][g * 4 + q] * (sa * sb_t);
-                        }
-                        continue;
-                    }
-                    uint16_t o[4];
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const int nn = min(n + q, p.N - 1);
-                        const float sb = SCALE == SCALE_TENSOR ? sb_t : p.sb[nn];
-                        float v = acc[a][b][g * 4 + q] * (sa * sb);
-                        if constexpr (EPI == EPI_ACCUM_BF16) {
-                            if (n + q < p.N) v += bf16_to_f32(crow[n + q]);
-                        }
-                        if constexpr (EPI == EPI_BIAS)
-                            v = bf16_to_f32(f32_to_bf16(v)) + bf16_to_f32(p.bias[nn]);   // bias is added to the bf16 result
-                        o[q] = f32_to_bf16(v);
-                    }
-                    if (vec_ok && n + 3 < p.N) {
-                        *reinterpret_cast<uint2*>(crow + n) = make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
-                    } else {
-#pragma unroll
-                        for (int q = 0; q < 4; ++q) if (n + q < p.N) crow[n + q] = o[q];
-                    }
-                }
-            }
+            wsrc[j] = p.B + static_cast<size_t>(min(n0 + row, p.N - 1)) * p.ldb + gchunk;
         }
     }
+    // The copies are issued through inline assembly: the compiler cannot tell that an LDS-DMA write
+    // and a later LDS read touch different slots, and would wait for every outstanding copy before
+    // each operand read.  Their completion is tracked by hand with s_waitcnt vmcnt before the barriers.
+    const uint32_t lds_wave = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(smem)) +
+                              __builtin_amdgcn_readfirstlane(wave) * (64 * BK);
+    // copy instruction j (0..7) of operand tile `op` (2*kt for X, 2*kt+1 for W)
+    auto dma_one = [&](int op, int j) {
+        const uint32_t dst = lds_wave + (op % kSlots) * kSlotBytes + j * 8 * BK;
+        const int k0 = (op >> 1) * BK;
+        const uint8_t* src = (op & 1) ? wsrc[j] + k0 : xsrc[j] + k0;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(src) : "memory");
+    };
+
+    // ---- LDS -> MFMA operands ----
+    const int frow = lane & 31, khalf = lane >> 5, fs = swz(frow);
+    int rd[2][2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) rd[h][j] = frow * BK + (((h * 4 + khalf * 2 + j) ^ fs) << 4);
+    const uint8_t* xrd = smem + wm * 128 * BK;
+    const uint8_t* wrd = smem + wn * 128 * BK;
+
+    v16f acc[4][4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
+
+    // operand registers, two sets: k-half h of any K-tile lives in set h
+    v8i wq[2][4], xq[2][4];
+    auto put = [](v8i& dst, int half, const uint4 v) {
+        dst[4 * half + 0] = (int)v.x; dst[4 * half + 1] = (int)v.y; dst[4 * half + 2] = (int)v.z; dst[4 * half + 3] = (int)v.w;
+    };
+    // the 16 reads of (kt, h) in the order its MFMAs need them: w0 x0 x1 x2 x3 w1 w2 w3, two reads each
+    auto read_one = [&](int kt, int h, int i) {
+        const int xoff = ((2 * kt) % kSlots) * kSlotBytes, woff = ((2 * kt + 1) % kSlots) * kSlotBytes;
+        const int t = i >> 1, half = i & 1;
+        const int r = rd[h][half];
+        if (t == 0)      put(wq[h][0], half, *reinterpret_cast<const uint4*>(wrd + woff + r));
+        else if (t <= 4) put(xq[h][t - 1], half, *reinterpret_cast<const uint4*>(xrd + xoff + (t - 1) * 32 * BK + r));
+        else             put(wq[h][t - 4], half, *reinterpret_cast<const uint4*>(wrd + woff + (t - 4) * 32 * BK + r));
+    };
+    auto mfma_one = [&](int h, int i) {
+        const int a = i >> 2, b = i & 3;
+        acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wq[h][a], xq[h][b], acc[a][b],
+                                                                     (FMT >> 1) & 1, FMT & 1, 0, 0, 0, 0);
+    };
+
+    const int ktiles = p.K / BK;      // >= 2, checked by the launcher
+    // prologue: K-tiles 0 and 1 in flight, tile 0 landed and visible, operands (0,0) in set 0
+#pragma unroll
+    for (int op = 0; op < 4; ++op)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) dma_one(op, j);
+    __builtin_amdgcn_s_waitcnt(kWaitVm16);
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 16; ++i) read_one(0, 0, i);
+
+    // step (kt,0): no synchronisation; COPY: start X(kt+2)
+    auto step0 = [&](int kt, auto copy_c) {
+        constexpr bool COPY = decltype(copy_c)::value != 0;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            mfma_one(0, i);
+            read_one(kt, 1, i);
+            if constexpr (COPY) {
+                if (i >= 2 && i < 10) dma_one(2 * kt + 4, i - 2);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    // step (kt,1).  MODE 0: steady (X(kt+2) stays in flight, start W(kt+2)); MODE 1: K-tile kt+1 is the
+    // last one (nothing else in flight, no copies); MODE 2: kt is the last K-tile (MFMAs only).
+    auto step1 = [&](int kt, auto mode_c) {
+        constexpr int MODE = decltype(mode_c)::value;
+        mfma_one(1, 0);
+        mfma_one(1, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (MODE != 2) {
+            __builtin_amdgcn_s_waitcnt(MODE == 0 ? kWaitVm8 : kWaitVm0);
+            __syncthreads();
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int i = 2; i < 16; ++i) {
+            mfma_one(1, i);
+            if constexpr (MODE != 2) {
+                read_one(kt + 1, 0, i - 2);
+                if (i >= 14) read_one(kt + 1, 0, i);              // reads 14 and 15 ride with the last two MFMAs
+            }
+            if constexpr (MODE == 0) {
+                if (i >= 4 && i < 12) dma_one(2 * kt + 5, i - 4);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    using C0 = std::integral_constant<int, 0>;
+    using C1 = std::integral_constant<int, 1>;
+    using C2 = std::integral_constant<int, 2>;
+
+    int kt = 0;
+    for (; kt + 2 < ktiles; ++kt) {
+        step0(kt, C1{});
+        step1(kt, C0{});
+    }
+    step0(kt, C0{});          // kt == ktiles - 2
+    step1(kt, C1{});
+    step0(kt + 1, C0{});      // last K-tile
+    step1(kt + 1, C2{});
+
+    epilogue<EPI, SCALE>(acc, p, m0, n0, wm, wn, lane);
 }
 
 // ---- naive kernel: any shape, any alignment; also the on-device cross-check ----
@@ -295,6 +470,17 @@ int launch_tiled(const GemmArgs& p, hipStream_t st) {
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
     });
     if (attr_err != hipSuccess) return static_cast<int>(attr_err);
+    if (p.K % BK == 0 && p.K >= 2 * BK && !p.force_staged) {
+        static std::once_flag once_ring;
+        static hipError_t ring_err = hipSuccess;
+        std::call_once(once_ring, [] {
+            ring_err = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_nt_ring<FMT, EPI, SCALE>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, kRingLds);
+        });
+        if (ring_err != hipSuccess) return static_cast<int>(ring_err);
+        k_gemm_nt_ring<FMT, EPI, SCALE><<<p.tiles_m * p.tiles_n, kThreads, kRingLds, st>>>(p);
+        return launch_status();
+    }
     k_gemm_nt<FMT, EPI, SCALE><<<p.tiles_m * p.tiles_n, kThreads, kLdsBytes, st>>>(p);
     return launch_status();
 }
@@ -380,6 +566,7 @@ int cf_fp8_gemm_nt_bf16_ex(int M, int N, int K, const void* A, int lda, int a_is
     p.bias = bias;
     p.C = C; p.ldc = ldc;
     if (epilogue > EPI_SILU_GATE) return CF_ERR_INVALID_ARG;
+    p.force_staged = (flags & CF_GEMM_FLAG_STAGED) != 0;
     return gemm_nt(p, a_is_e5m2 ? 1 : 0, epilogue, scale_mode, flags & CF_GEMM_FLAG_NAIVE, stream);
 }
 
@@ -417,6 +604,7 @@ int cf_fp8_gemm_nt_accum_f32_ex(int M, int N, int K, const void* A, int lda, int
     p.B = static_cast<const uint8_t*>(B); p.ldb = ldb;
     p.sa = a_descale; p.sb = b_descale;
     p.Cf = C; p.ldc = ldc;
+    p.force_staged = (flags & CF_GEMM_FLAG_STAGED) != 0;
     return gemm_nt(p, (a_is_e5m2 ? 1 : 0) | (b_is_e5m2 ? 2 : 0), EPI_ACCUM_F32, SCALE_TENSOR,
                    flags & CF_GEMM_FLAG_NAIVE, stream);
 }

@@ -26,6 +26,7 @@ def lib_path() -> Path:
     return PKG / "libcf_fp8.so"
 
 
+
 _CTYPES = {
     "int": ctypes.c_int, "float": ctypes.c_float, "size_t": ctypes.c_size_t,
     "cf_stream_t": ctypes.c_void_p, "long long": ctypes.c_longlong, "int64_t": ctypes.c_int64,

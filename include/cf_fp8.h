@@ -152,6 +152,7 @@ int cf_bias_add_strided_bf16(uint16_t* d_inout, const uint16_t* d_bias, int rows
                                   src/trainer.cu:6310-6312 followed by swiglu_forward (:6322) */
 
 #define CF_GEMM_FLAG_NAIVE 1   /* run the one-lane-per-output cross-check kernel  */
+#define CF_GEMM_FLAG_STAGED 2  /* take the register-staged tile kernel (the K % 64 != 0 path) */
 
 /* lt_gemm_fp8_nt, static at src/trainer.cu:4498-4534 (plan lookup :4402-4496).
  * C[M,N] bf16 (row stride ldc) = (A[M,K] fp8, row stride lda, E4M3 or E5M2) .

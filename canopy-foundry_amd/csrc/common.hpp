@@ -36,6 +36,15 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
     return static_cast<uint32_t>(f32_to_bf16(lo)) | (static_cast<uint32_t>(f32_to_bf16(hi)) << 16);
 }
 
+// Two floats -> packed bf16 pair on gfx950's v_cvt_pk_bf16_f32 (round to nearest even).
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2_hw(float lo, float hi) {
+    const f32x2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+__device__ __forceinline__ float round_bf16_hw(float v) { return __uint_as_float(pack_bf16x2_hw(v, 0.0f) << 16); }
+
 // ---- OCP fp8 encode -------------------------------------------------------
 // gfx950's v_cvt_pk_{fp8,bf8}_f32 round to nearest even onto OCP e4m3fn / e5m2.
 // Saturation to the largest finite value is applied here by clamping first

@@ -55,12 +55,14 @@ struct GemmArgs {
 
 __device__ __forceinline__ int swz(int row) { return (row ^ ((row >> 3) & 3)) & 7; }
 
-// tile index -> (tile_m, tile_n): contiguous range per XCD, 8 x 4 patches inside it
-__device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, int& tm, int& tn) {
+// Position `pos` in launch order -> (tile_m, tile_n).  Workgroups are handed to the 8 XCDs round-robin,
+// so positions with the same pos % 8 share an XCD (and its L2): each XCD gets a contiguous range of
+// tiles, walked in patches of 8 (M) x tiles_n... x 4 (N) whose operands its L2 can hold.
+__device__ __forceinline__ void tile_coords(int pos, int tiles_m, int tiles_n, int& tm, int& tn) {
     const int total = tiles_m * tiles_n;
-    const int per_xcd = (total + kXcds - 1) / kXcds;
-    int t = (bid % kXcds) * per_xcd + bid / kXcds;
-    if (total % kXcds != 0) t = bid;                       // ragged tile counts keep the plain order
+    const int per_xcd = total / kXcds;
+    int t = pos;
+    if (total % kXcds == 0) t = (pos % kXcds) * per_xcd + pos / kXcds;   // ragged counts keep the plain order
     constexpr int GM = 8;
     const int group = t / (GM * tiles_n);
     const int first_m = group * GM;
@@ -73,89 +75,120 @@ __device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, i
 // ---- epilogue shared by the tiled kernels ----------------------------------------
 // acc[a][b][r]: output row m = m0 + wm*128 + b*32 + (lane & 31); weight row within the
 // wave's 128 = a*32 + 8*(r/4) + 4*(lane>>5) + r%4, i.e. four consecutive output columns per quad.
+// Column scales are fetched once per quad as a float4 and reused for the four row tiles.
+
+// SiLU gate for the fused epilogue: x * 1/(1 + 2^(-x*log2 e)) on the hardware exp2 and reciprocal
+// (1 ulp each).  The stand-alone swiglu kernel keeps the correctly-rounded divide and the
+// reproducible expf; the two differ by at most one bf16 ulp of the product.
+__device__ __forceinline__ float fast_silu(float x) {
+    const float e = __builtin_amdgcn_exp2f(-1.44269504f * x);
+    return x * __builtin_amdgcn_rcpf(1.0f + e);
+}
+
+__device__ __forceinline__ float4 load_scale4(const float* s, int n, int N, bool fast) {
+    if (fast) return *reinterpret_cast<const float4*>(s + n);
+    return make_float4(s[min(n, N - 1)], s[min(n + 1, N - 1)], s[min(n + 2, N - 1)], s[min(n + 3, N - 1)]);
+}
+
 template <int EPI, int SCALE>
 __device__ __forceinline__ void epilogue(v16f (&acc)[4][4], const GemmArgs& p, int m0, int n0, int wm, int wn,
                                          int lane) {
     const int khalf = lane >> 5;
+    constexpr bool GATE = EPI == EPI_SILU_GATE;
+    constexpr int NT = GATE ? 2 : 4;                       // 32-wide output column tiles per wave
+    const int nbase = n0 + wn * (NT * 32) + khalf * 4;     // + t*32 + g*8
     const bool vec_ok = EPI == EPI_ACCUM_F32 ? (p.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.Cf) & 15u) == 0)
                                              : (p.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.C) & 7u) == 0);
-    const float sa_t = SCALE == SCALE_TENSOR ? p.sa[0] : 0.0f;
-    const float sb_t = SCALE == SCALE_TENSOR ? p.sb[0] : 0.0f;
-    const float sb2_t = (SCALE == SCALE_TENSOR && EPI == EPI_SILU_GATE) ? p.sb2[0] : 0.0f;
+    const bool full_n = n0 + (GATE ? BN / 2 : BN) <= p.N;
+
+    float s1 = 0.0f, s2 = 0.0f;
+    if constexpr (SCALE == SCALE_TENSOR) {
+        s1 = p.sa[0] * p.sb[0];
+        if constexpr (GATE) s2 = p.sa[0] * p.sb2[0];
+    }
+    const bool fast = SCALE != SCALE_TENSOR && full_n && ((reinterpret_cast<uintptr_t>(p.sb) & 15u) == 0) &&
+                      (!GATE || (reinterpret_cast<uintptr_t>(p.sb2) & 15u) == 0);
+    // row factors and row validity of this lane's four output rows
+    float sa[4];
+    int mrow[4];
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
-        const int m = m0 + wm * 128 + b * 32 + (lane & 31);
-        if (m >= p.M) continue;
-        const float sa = SCALE == SCALE_TENSOR ? sa_t : p.sa[m];
-        uint16_t* crow = EPI == EPI_ACCUM_F32 ? nullptr : p.C + static_cast<size_t>(m) * p.ldc;
-        if constexpr (EPI == EPI_SILU_GATE) {
+        mrow[b] = m0 + wm * 128 + b * 32 + (lane & 31);
+        sa[b] = SCALE == SCALE_TENSOR ? 1.0f : p.sa[min(mrow[b], p.M - 1)];
+    }
+
 #pragma unroll
-            for (int pair = 0; pair < 2; ++pair) {
+    for (int t = 0; t < NT; ++t) {
+        // per-quad column factors of this 32-column tile: [g] -> 4 columns
+        float4 cs[4], cs2[4];
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int n = n0 + wn * 64 + pair * 32 + g * 8 + khalf * 4;
-                    uint16_t o[4];
+        for (int g = 0; g < 4; ++g) {
+            if constexpr (SCALE == SCALE_TENSOR) {
+                cs[g] = make_float4(s1, s1, s1, s1);
+                cs2[g] = make_float4(s2, s2, s2, s2);
+            } else {
+                cs[g] = load_scale4(p.sb, nbase + t * 32 + g * 8, p.N, fast);
+                if constexpr (GATE) cs2[g] = load_scale4(p.sb2, nbase + t * 32 + g * 8, p.N, fast);
+            }
+        }
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const int nn = min(n + q, p.N - 1);
-                        const float sg = SCALE == SCALE_TENSOR ? sb_t : p.sb[nn];
-                        const float su = SCALE == SCALE_TENSOR ? sb2_t : p.sb2[nn];
-                        // the reference rounds gate and up to bf16 before the SiLU product
-                        const float gate = bf16_to_f32(f32_to_bf16(acc[2 * pair][b][g * 4 + q] * (sa * sg)));
-                        const float up = bf16_to_f32(f32_to_bf16(acc[2 * pair + 1][b][g * 4 + q] * (sa * su)));
-                        o[q] = f32_to_bf16((gate * stable_sigmoid(gate)) * up);
-                    }
+        for (int b = 0; b < 4; ++b) {
+            const int m = mrow[b];
+            if (m >= p.M) continue;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int n = nbase + t * 32 + g * 8;
+                const float c4[4] = {cs[g].x, cs[g].y, cs[g].z, cs[g].w};
+                if constexpr (EPI == EPI_ACCUM_F32) {
+                    // beta = 1: the product is added to what the caller's fp32 buffer holds
+                    float* frow = p.Cf + static_cast<size_t>(m) * p.ldc + n;
                     if (vec_ok && n + 3 < p.N) {
-                        *reinterpret_cast<uint2*>(crow + n) = make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
+                        float4 v = *reinterpret_cast<const float4*>(frow);
+                        v.x += acc[t][b][g * 4 + 0] * c4[0];
+                        v.y += acc[t][b][g * 4 + 1] * c4[1];
+                        v.z += acc[t][b][g * 4 + 2] * c4[2];
+                        v.w += acc[t][b][g * 4 + 3] * c4[3];
+                        *reinterpret_cast<float4*>(frow) = v;
                     } else {
 #pragma unroll
-                        for (int q = 0; q < 4; ++q) if (n + q < p.N) crow[n + q] = o[q];
+                        for (int q = 0; q < 4; ++q) if (n + q < p.N) frow[q] += acc[t][b][g * 4 + q] * c4[q];
                     }
-                }
-            }
-        } else {
+                } else {
+                    uint16_t* crow = p.C + static_cast<size_t>(m) * p.ldc + n;
+                    float v[4];
 #pragma unroll
-            for (int a = 0; a < 4; ++a) {
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int n = n0 + wn * 128 + a * 32 + g * 8 + khalf * 4;
-                    if constexpr (EPI == EPI_ACCUM_F32) {
-                        // beta = 1: the product is added to what the caller's fp32 buffer holds
-                        float* frow = p.Cf + static_cast<size_t>(m) * p.ldc + n;
-                        if (vec_ok && n + 3 < p.N) {
-                            float4 c4 = *reinterpret_cast<const float4*>(frow);
-                            c4.x += acc[a][b][g * 4 + 0] * (sa * sb_t);
-                            c4.y += acc[a][b][g * 4 + 1] * (sa * sb_t);
-                            c4.z += acc[a][b][g * 4 + 2] * (sa * sb_t);
-                            c4.w += acc[a][b][g * 4 + 3] * (sa * sb_t);
-                            *reinterpret_cast<float4*>(frow) = c4;
+                    for (int q = 0; q < 4; ++q) {
+                        if constexpr (GATE) {
+                            const float u4[4] = {cs2[g].x, cs2[g].y, cs2[g].z, cs2[g].w};
+                            // the reference rounds gate and up to bf16 before the SiLU product
+                            const float gate = round_bf16_hw(acc[2 * t][b][g * 4 + q] * (sa[b] * c4[q]));
+                            const float up = round_bf16_hw(acc[2 * t + 1][b][g * 4 + q] * (sa[b] * u4[q]));
+                            v[q] = fast_silu(gate) * up;
                         } else {
-#pragma unroll
-                            for (int q = 0; q < 4; ++q) if (n + q < p.N) frow[q] += acc[a][b][g * 4 + q] * (sa * sb_t);
+                            v[q] = acc[t][b][g * 4 + q] * (sa[b] * c4[q]);
+                            if constexpr (EPI == EPI_ACCUM_BF16) {
+                                if (n + q < p.N) v[q] += bf16_to_f32(crow[q]);
+                            }
+                            if constexpr (EPI == EPI_BIAS)   // bias is added to the bf16 result, as the separate kernel does
+                                v[q] = round_bf16_hw(v[q]) + bf16_to_f32(p.bias[min(n + q, p.N - 1)]);
                         }
-                        continue;
                     }
-                    uint16_t o[4];
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const int nn = min(n + q, p.N - 1);
-                        const float sb = SCALE == SCALE_TENSOR ? sb_t : p.sb[nn];
-                        float v = acc[a][b][g * 4 + q] * (sa * sb);
-                        if constexpr (EPI == EPI_ACCUM_BF16) {
-                            if (n + q < p.N) v += bf16_to_f32(crow[n + q]);
-                        }
-                        if constexpr (EPI == EPI_BIAS)
-                            v = bf16_to_f32(f32_to_bf16(v)) + bf16_to_f32(p.bias[nn]);   // bias is added to the bf16 result
-                        o[q] = f32_to_bf16(v);
-                    }
+                    const uint32_t o01 = pack_bf16x2_hw(v[0], v[1]), o23 = pack_bf16x2_hw(v[2], v[3]);
+#ifdef CF_ABLATE_STORE
+                    if (p.ldc < 0)
+#endif
                     if (vec_ok && n + 3 < p.N) {
-                        *reinterpret_cast<uint2*>(crow + n) = make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
+                        *reinterpret_cast<uint2*>(crow) = make_uint2(o01, o23);
                     } else {
+                        const uint16_t o[4] = {(uint16_t)(o01 & 0xffffu), (uint16_t)(o01 >> 16), (uint16_t)(o23 & 0xffffu), (uint16_t)(o23 >> 16)};
 #pragma unroll
-                        for (int q = 0; q < 4; ++q) if (n + q < p.N) crow[n + q] = o[q];
+                        for (int q = 0; q < 4; ++q) if (n + q < p.N) crow[q] = o[q];
                     }
                 }
             }
+            // keep the scheduler from pulling every accumulator into VGPRs at once: in the persistent
+            // kernel the next tile's operands are live across the epilogue
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 }
@@ -285,44 +318,54 @@ constexpr int kRingLds = kSlots * kSlotBytes;     // 160 KiB: all of a CU's LDS
 // s_waitcnt immediates: vmcnt in bits [3:0] and [15:14], expcnt [6:4] and lgkmcnt [11:8] left at no-wait
 constexpr int kWaitVm0 = 0x0f70, kWaitVm8 = 0x0f78, kWaitVm16 = 0x4f70;
 
+// The kernel is persistent: workgroup w walks tiles w, w + grid, w + 2*grid, ... of the XCD-aware
+// order, and the copy stream simply runs on into the next tile, so only a workgroup's very first
+// K-tiles pay memory latency; the epilogue of one tile runs while the next tile's first two K-tiles land.
 template <int FMT, int EPI, int SCALE>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void k_gemm_nt_ring(const GemmArgs p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
-    int tile_m, tile_n;
-    tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
     constexpr int OUT_BN = EPI == EPI_SILU_GATE ? BN / 2 : BN;
-    const int m0 = tile_m * BM, n0 = tile_n * OUT_BN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
+    const int total_tiles = p.tiles_m * p.tiles_n;
+    const int my_tiles = (total_tiles - static_cast<int>(blockIdx.x) + static_cast<int>(gridDim.x) - 1) / static_cast<int>(gridDim.x);
+    const int ktiles = p.K / BK;      // >= 2, checked by the launcher
+    const int total_g = my_tiles * ktiles;          // K-tiles this workgroup multiplies, over all its tiles
 
     // ---- global -> LDS: wave w copies rows [64w, 64w+64) of an operand tile, 8 rows per instruction ----
     const int lrow = lane >> 3, lslot = lane & 7;
     const uint8_t* xsrc[8];
     const uint8_t* wsrc[8];
+    auto aim = [&](int seq) {                        // point the copy stream at this workgroup's seq-th tile
+        int tile_m, tile_n;
+        tile_coords(blockIdx.x + seq * gridDim.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+        const int m0 = tile_m * BM, n0 = tile_n * OUT_BN;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const int row = wave * 64 + j * 8 + lrow;
-        const int gchunk = (lslot ^ swz(row)) * 16;
-        xsrc[j] = p.A + static_cast<size_t>(min(m0 + row, p.M - 1)) * p.lda + gchunk;
-        if constexpr (EPI == EPI_SILU_GATE) {
-            const int t = (row >> 5) & 3, w = row >> 7;
-            const int n = n0 + w * 64 + (t >> 1) * 32 + (row & 31);
-            wsrc[j] = ((t & 1) ? p.B2 : p.B) + static_cast<size_t>(min(n, p.N - 1)) * p.ldb + gchunk;
-        } else {
-            wsrc[j] = p.B + static_cast<size_t>(min(n0 + row, p.N - 1)) * p.ldb + gchunk;
+        for (int j = 0; j < 8; ++j) {
+            const int row = wave * 64 + j * 8 + lrow;
+            const int gchunk = (lslot ^ swz(row)) * 16;
+            xsrc[j] = p.A + static_cast<size_t>(min(m0 + row, p.M - 1)) * p.lda + gchunk;
+            if constexpr (EPI == EPI_SILU_GATE) {
+                // LDS weight rows of a wave: [gate 32 | up 32 | gate 32 | up 32] over the same 64 output columns
+                const int t = (row >> 5) & 3, w = row >> 7;
+                const int n = n0 + w * 64 + (t >> 1) * 32 + (row & 31);
+                wsrc[j] = ((t & 1) ? p.B2 : p.B) + static_cast<size_t>(min(n, p.N - 1)) * p.ldb + gchunk;
+            } else {
+                wsrc[j] = p.B + static_cast<size_t>(min(n0 + row, p.N - 1)) * p.ldb + gchunk;
+            }
         }
-    }
+    };
     // The copies are issued through inline assembly: the compiler cannot tell that an LDS-DMA write
     // and a later LDS read touch different slots, and would wait for every outstanding copy before
     // each operand read.  Their completion is tracked by hand with s_waitcnt vmcnt before the barriers.
     const uint32_t lds_wave = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(smem)) +
                               __builtin_amdgcn_readfirstlane(wave) * (64 * BK);
-    // copy instruction j (0..7) of operand tile `op` (2*kt for X, 2*kt+1 for W)
-    auto dma_one = [&](int op, int j) {
+    // copy instruction j (0..7) of operand tile `op` (2*g for X, 2*g+1 for W of K-tile g of the stream),
+    // reading K offset k0 of the tile the stream is aimed at
+    auto dma_one = [&](int op, int k0, int j) {
         const uint32_t dst = lds_wave + (op % kSlots) * kSlotBytes + j * 8 * BK;
-        const int k0 = (op >> 1) * BK;
         const uint8_t* src = (op & 1) ? wsrc[j] + k0 : xsrc[j] + k0;
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(src) : "memory");
     };
@@ -338,21 +381,24 @@ void k_gemm_nt_ring(const GemmArgs p) {
     const uint8_t* wrd = smem + wn * 128 * BK;
 
     v16f acc[4][4];
+    auto zero_acc = [&]() {
 #pragma unroll
-    for (int a = 0; a < 4; ++a)
+        for (int a = 0; a < 4; ++a)
 #pragma unroll
-        for (int b = 0; b < 4; ++b)
+            for (int b = 0; b < 4; ++b)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
+                for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
+    };
+    zero_acc();
 
     // operand registers, two sets: k-half h of any K-tile lives in set h
     v8i wq[2][4], xq[2][4];
     auto put = [](v8i& dst, int half, const uint4 v) {
         dst[4 * half + 0] = (int)v.x; dst[4 * half + 1] = (int)v.y; dst[4 * half + 2] = (int)v.z; dst[4 * half + 3] = (int)v.w;
     };
-    // the 16 reads of (kt, h) in the order its MFMAs need them: w0 x0 x1 x2 x3 w1 w2 w3, two reads each
-    auto read_one = [&](int kt, int h, int i) {
-        const int xoff = ((2 * kt) % kSlots) * kSlotBytes, woff = ((2 * kt + 1) % kSlots) * kSlotBytes;
+    // the 16 reads of (g, h) in the order its MFMAs need them: w0 x0 x1 x2 x3 w1 w2 w3, two reads each
+    auto read_one = [&](int g, int h, int i) {
+        const int xoff = ((2 * g) % kSlots) * kSlotBytes, woff = ((2 * g + 1) % kSlots) * kSlotBytes;
         const int t = i >> 1, half = i & 1;
         const int r = rd[h][half];
         if (t == 0)      put(wq[h][0], half, *reinterpret_cast<const uint4*>(wrd + woff + r));
@@ -365,33 +411,33 @@ void k_gemm_nt_ring(const GemmArgs p) {
                                                                      (FMT >> 1) & 1, FMT & 1, 0, 0, 0, 0);
     };
 
-    const int ktiles = p.K / BK;      // >= 2, checked by the launcher
-    // prologue: K-tiles 0 and 1 in flight, tile 0 landed and visible, operands (0,0) in set 0
+    // prologue: K-tiles 0 and 1 of the stream in flight, tile 0 landed and visible, operands (0,0) in set 0
+    aim(0);
 #pragma unroll
     for (int op = 0; op < 4; ++op)
 #pragma unroll
-        for (int j = 0; j < 8; ++j) dma_one(op, j);
+        for (int j = 0; j < 8; ++j) dma_one(op, (op >> 1) * BK, j);
     __builtin_amdgcn_s_waitcnt(kWaitVm16);
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < 16; ++i) read_one(0, 0, i);
 
-    // step (kt,0): no synchronisation; COPY: start X(kt+2)
-    auto step0 = [&](int kt, auto copy_c) {
+    // step (g,0): no synchronisation; COPY: start X of stream K-tile g+2 (tile-local K offset dk0)
+    auto step0 = [&](int g, int dk0, auto copy_c) {
         constexpr bool COPY = decltype(copy_c)::value != 0;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             mfma_one(0, i);
-            read_one(kt, 1, i);
+            read_one(g, 1, i);
             if constexpr (COPY) {
-                if (i >= 2 && i < 10) dma_one(2 * kt + 4, i - 2);
+                if (i >= 2 && i < 10) dma_one(2 * g + 4, dk0, i - 2);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
     };
-    // step (kt,1).  MODE 0: steady (X(kt+2) stays in flight, start W(kt+2)); MODE 1: K-tile kt+1 is the
-    // last one (nothing else in flight, no copies); MODE 2: kt is the last K-tile (MFMAs only).
-    auto step1 = [&](int kt, auto mode_c) {
+    // step (g,1).  MODE 0: steady (X(g+2) stays in flight, start W(g+2)); MODE 1: K-tile g+1 is the
+    // last of the stream (nothing else in flight, no copies); MODE 2: g is the last K-tile (MFMAs only).
+    auto step1 = [&](int g, int dk0, auto mode_c) {
         constexpr int MODE = decltype(mode_c)::value;
         mfma_one(1, 0);
         mfma_one(1, 1);
@@ -405,11 +451,11 @@ void k_gemm_nt_ring(const GemmArgs p) {
         for (int i = 2; i < 16; ++i) {
             mfma_one(1, i);
             if constexpr (MODE != 2) {
-                read_one(kt + 1, 0, i - 2);
-                if (i >= 14) read_one(kt + 1, 0, i);              // reads 14 and 15 ride with the last two MFMAs
+                read_one(g + 1, 0, i - 2);
+                if (i >= 14) read_one(g + 1, 0, i);               // reads 14 and 15 ride with the last two MFMAs
             }
             if constexpr (MODE == 0) {
-                if (i >= 4 && i < 12) dma_one(2 * kt + 5, i - 4);
+                if (i >= 4 && i < 12) dma_one(2 * g + 5, dk0, i - 4);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -418,17 +464,32 @@ void k_gemm_nt_ring(const GemmArgs p) {
     using C1 = std::integral_constant<int, 1>;
     using C2 = std::integral_constant<int, 2>;
 
-    int kt = 0;
-    for (; kt + 2 < ktiles; ++kt) {
-        step0(kt, C1{});
-        step1(kt, C0{});
+    // copy position: two K-tiles ahead of the compute position (ktiles >= 2, so at most one tile ahead)
+    int dkt = 2 % ktiles, dseq = 2 / ktiles;
+    if (dseq == 1 && my_tiles > 1) aim(1);
+    int g = 0;                                     // K-tile index in this workgroup's stream
+    for (int seq = 0; seq < my_tiles; ++seq) {
+        const bool last_tile = seq + 1 == my_tiles;
+        const int steady = last_tile ? ktiles - 2 : ktiles;
+        for (int kt = 0; kt < steady; ++kt, ++g) {
+            step0(g, dkt * BK, C1{});
+            step1(g, dkt * BK, C0{});
+            if (++dkt == ktiles) {               // the stream moves on to the next tile
+                dkt = 0;
+                if (++dseq < my_tiles) aim(dseq);
+            }
+        }
+        if (last_tile) {
+            step0(g, 0, C0{});
+            step1(g, 0, C1{});
+            step0(g + 1, 0, C0{});
+            step1(g + 1, 0, C2{});
+        }
+        int tile_m, tile_n;
+        tile_coords(blockIdx.x + seq * gridDim.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+        epilogue<EPI, SCALE>(acc, p, tile_m * BM, tile_n * OUT_BN, wm, wn, lane);
+        zero_acc();
     }
-    step0(kt, C0{});          // kt == ktiles - 2
-    step1(kt, C1{});
-    step0(kt + 1, C0{});      // last K-tile
-    step1(kt + 1, C2{});
-
-    epilogue<EPI, SCALE>(acc, p, m0, n0, wm, wn, lane);
 }
 
 // ---- naive kernel: any shape, any alignment; also the on-device cross-check ----
@@ -461,6 +522,16 @@ __global__ __launch_bounds__(256) void k_gemm_nt_naive(const GemmArgs p, int fmt
     p.C[static_cast<size_t>(m) * p.ldc + n] = f32_to_bf16(v);
 }
 
+inline int num_cus() {
+    static int n = [] {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) != hipSuccess) return 256;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) return 256;
+        return v;
+    }();
+    return n;
+}
+
 template <int FMT, int EPI, int SCALE>
 int launch_tiled(const GemmArgs& p, hipStream_t st) {
     static std::once_flag once;
@@ -478,7 +549,12 @@ int launch_tiled(const GemmArgs& p, hipStream_t st) {
                                            hipFuncAttributeMaxDynamicSharedMemorySize, kRingLds);
         });
         if (ring_err != hipSuccess) return static_cast<int>(ring_err);
-        k_gemm_nt_ring<FMT, EPI, SCALE><<<p.tiles_m * p.tiles_n, kThreads, kRingLds, st>>>(p);
+        // persistent: one workgroup per CU (the kernel uses a CU's whole LDS and register file);
+        // a grid that is a multiple of 8 keeps "position % 8 = XCD" true for every tile a workgroup walks
+        const int total = p.tiles_m * p.tiles_n;
+        int grid = total < num_cus() ? total : num_cus();
+        if (grid >= kXcds) grid -= grid % kXcds;
+        k_gemm_nt_ring<FMT, EPI, SCALE><<<grid, kThreads, kRingLds, st>>>(p);
         return launch_status();
     }
     k_gemm_nt<FMT, EPI, SCALE><<<p.tiles_m * p.tiles_n, kThreads, kLdsBytes, st>>>(p);

@@ -1,0 +1,366 @@
+// MoE routing and dispatch for gfx950: row softmax, top-k select + renormalise,
+// deterministic per-expert row lists, offsets, row gather (token permute) and the
+// weighted scatter-accumulate (unpermute).
+//
+// Routing is bit-reproducible: the softmax uses the library's deterministic expf and
+// a fixed reduction tree (32-lane xor butterflies, then the group sums), top-k picks
+// by (value descending, index ascending), and row lists are filled in ascending row
+// order by a scan instead of atomics.
+#include "common.hpp"
+
+namespace cf {
+namespace {
+
+constexpr int kThreads = 256;
+
+// xor butterfly over the 32-lane group a lane belongs to (offsets 16..1)
+__device__ __forceinline__ float group32_sum(float v) {
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+__device__ __forceinline__ float group32_max(float v) {
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+
+// ---- softmax, cols <= 64: one wavefront per row, lane = column ----------------
+// Matches a launch of T = cols threads: one element per thread, 32-lane butterflies,
+// then the (at most two) group sums added.
+__device__ __forceinline__ float row_softmax_wave(float x, bool live, float& out_max) {
+    const float m32 = group32_max(live ? x : -3.402823466e+38f);
+    const float mx = fmaxf(m32, __shfl_xor(m32, 32, kWave));
+    const float e = live ? det_expf(x - mx) : 0.0f;
+    const float s32 = group32_sum(e);
+    // second level: the butterfly over {s_lo, s_hi, 0, ...} reduces to s_lo + s_hi
+    const float lo = __shfl(s32, 0, kWave), hi = __shfl(s32, 32, kWave);
+    const float sum = lo + hi;
+    const float inv = 1.0f / sum;
+    out_max = mx;
+    return e * inv;
+}
+
+__global__ __launch_bounds__(kThreads) void k_softmax_wave(float* __restrict__ x, int rows, int cols) {
+    const int row = blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int lane = threadIdx.x & 63;
+    const bool live = lane < cols;
+    float* r = x + static_cast<size_t>(row) * cols;
+    float mx;
+    const float p = row_softmax_wave(live ? r[lane] : 0.0f, live, mx);
+    if (live) r[lane] = p;
+}
+
+// ---- softmax, any cols: one workgroup per row, T = min(cols,256) virtual threads ----
+__global__ __launch_bounds__(kThreads) void k_softmax_block(float* __restrict__ x, int cols) {
+    __shared__ float sh[8];
+    __shared__ float bc;
+    float* r = x + static_cast<size_t>(blockIdx.x) * cols;
+    const int T = min(cols, 256), t = threadIdx.x;
+    float lm = -3.402823466e+38f;
+    if (t < T) for (int c = t; c < cols; c += T) lm = fmaxf(lm, r[c]);
+    lm = group32_max(lm);
+    if ((t & 31) == 0) sh[t >> 5] = lm;
+    __syncthreads();
+    if (t == 0) { float m = sh[0]; for (int w = 1; w < 8; ++w) m = fmaxf(m, sh[w]); bc = m; }
+    __syncthreads();
+    const float mx = bc;
+    float ls = 0.0f;
+    if (t < T) for (int c = t; c < cols; c += T) ls += det_expf(r[c] - mx);
+    ls = group32_sum(ls);
+    __syncthreads();
+    if ((t & 31) == 0) sh[t >> 5] = ls;          // groups past T hold 0
+    __syncthreads();
+    if (t == 0) {
+        // butterfly over the 32-entry array of group sums (only the first 8 can be non-zero):
+        // offsets 16 and 8 add zeros, then (w0+w4),(w1+w5),(w2+w6),(w3+w7); (.. + ..) pairs 2 apart; then 1 apart
+        const float a0 = sh[0] + sh[4], a1 = sh[1] + sh[5], a2 = sh[2] + sh[6], a3 = sh[3] + sh[7];
+        bc = (a0 + a2) + (a1 + a3);
+    }
+    __syncthreads();
+    const float inv = 1.0f / bc;
+    if (t < T) for (int c = t; c < cols; c += T) r[c] = det_expf(r[c] - mx) * inv;
+}
+
+// ---- top-k, E <= 64: one wavefront per row, lane = expert ----------------------
+// Optionally fused with the softmax (SOFTMAX) so the logits are read once.
+template <bool SOFTMAX>
+__global__ __launch_bounds__(kThreads) void k_topk_wave(float* __restrict__ scores, float* __restrict__ row_sum_save,
+                                                        float* __restrict__ scores_save, int rows, int E, int top_k,
+                                                        int normalize) {
+    const int row = blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int lane = threadIdx.x & 63;
+    const bool live = lane < E;
+    float* s = scores + static_cast<size_t>(row) * E;
+    float v = live ? s[lane] : 0.0f;
+    if constexpr (SOFTMAX) {
+        float mx;
+        v = row_softmax_wave(v, live, mx);
+        if (scores_save && live) scores_save[static_cast<size_t>(row) * E + lane] = v;
+    }
+    const int k = min(top_k, E);
+    bool kept = false;
+    for (int pick = 0; pick < k; ++pick) {
+        // candidates must beat -1 strictly (NaN never does); largest value, lowest lane among equals
+        const bool cand = live && !kept && v > -1.0f;
+        float best = cand ? v : -2.0f;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) best = fmaxf(best, __shfl_xor(best, off, kWave));
+        const unsigned long long hit = __ballot(cand && v == best);
+        if (hit == 0ull) break;
+        if (lane == __builtin_ctzll(hit)) kept = true;
+    }
+    // kept sum in ascending expert order, one fp32 add per kept expert
+    unsigned long long mask = __ballot(kept);
+    float sum = 0.0f;
+    while (mask) {
+        const int e = __builtin_ctzll(mask);
+        mask &= mask - 1;
+        sum += __shfl(v, e, kWave);
+    }
+    if (row_sum_save && lane == 0) row_sum_save[row] = sum;
+    const float inv_sum = (normalize && sum > 0.0f) ? (1.0f / sum) : 1.0f;
+    if (live) s[lane] = kept ? v * inv_sum : 0.0f;
+}
+
+// ---- top-k, any E up to 2048: one lane per row ----------------------------------
+constexpr int kMaxExpertsGeneric = 2048;
+__global__ __launch_bounds__(128) void k_topk_generic(float* __restrict__ scores, float* __restrict__ row_sum_save,
+                                                      int rows, int E, int top_k, int normalize) {
+    const int row = blockIdx.x * blockDim.x + threadIdx.x;
+    if (row >= rows) return;
+    float* s = scores + static_cast<size_t>(row) * E;
+    uint32_t kept[kMaxExpertsGeneric / 32];
+    for (int w = 0; w < (E + 31) / 32; ++w) kept[w] = 0u;
+    const int k = min(top_k, E);
+    for (int pick = 0; pick < k; ++pick) {
+        int best = -1;
+        float best_v = -1.0f;
+        for (int e = 0; e < E; ++e)
+            if (!((kept[e >> 5] >> (e & 31)) & 1u) && s[e] > best_v) { best_v = s[e]; best = e; }
+        if (best < 0) break;
+        kept[best >> 5] |= 1u << (best & 31);
+    }
+    float sum = 0.0f;
+    for (int e = 0; e < E; ++e) if ((kept[e >> 5] >> (e & 31)) & 1u) sum += s[e];
+    if (row_sum_save) row_sum_save[row] = sum;
+    const float inv_sum = (normalize && sum > 0.0f) ? (1.0f / sum) : 1.0f;
+    for (int e = 0; e < E; ++e) s[e] = ((kept[e >> 5] >> (e & 31)) & 1u) ? s[e] * inv_sum : 0.0f;
+}
+
+// ---- per-expert row lists ----------------------------------------------------------
+// One workgroup per expert scans the rows 1024 at a time: ballot + popcount inside a
+// wavefront, wavefront totals through LDS, so slots come out in ascending row order.
+__global__ __launch_bounds__(1024) void k_build_row_lists(const float* __restrict__ route_weights,
+                                                          int* __restrict__ counts, int* __restrict__ row_indices,
+                                                          int rows, int E) {
+    __shared__ int wave_tot[16];
+    __shared__ int base_sh;
+    const int e = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    int* out = row_indices + static_cast<size_t>(e) * rows;
+    if (t == 0) base_sh = 0;
+    __syncthreads();
+    for (int r0 = 0; r0 < rows; r0 += 1024) {
+        const int row = r0 + t;
+        const bool sel = row < rows && route_weights[static_cast<size_t>(row) * E + e] > 0.0f;
+        const unsigned long long m = __ballot(sel);
+        const int rank = __builtin_popcountll(m & ((1ull << lane) - 1ull));
+        if (lane == 0) wave_tot[wave] = __builtin_popcountll(m);
+        __syncthreads();
+        int before = base_sh;
+        for (int w = 0; w < wave; ++w) before += wave_tot[w];
+        if (sel) out[before + rank] = row;
+        __syncthreads();
+        if (t == 0) { int s = 0; for (int w = 0; w < 16; ++w) s += wave_tot[w]; base_sh += s; }
+        __syncthreads();
+    }
+    if (t == 0) counts[e] = base_sh;
+}
+
+__global__ void k_offsets(const int* __restrict__ counts, int* __restrict__ offsets, int E) {
+    int sum = 0;
+    for (int e = 0; e < E; ++e) { offsets[e] = sum; sum += counts[e]; }
+}
+
+// ---- row gather (token permute) -----------------------------------------------------
+// dst[i, :] = src[row_indices[i], :], rows of `width` bytes; 16 bytes per lane when aligned.
+__global__ __launch_bounds__(kThreads) void k_gather_rows16(const uint4* __restrict__ src, uint4* __restrict__ dst,
+                                                            const int* __restrict__ row_indices, int n_rows,
+                                                            int vec_per_row) {
+    const size_t total = static_cast<size_t>(n_rows) * vec_per_row;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total;
+         i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+        const int r = static_cast<int>(i / vec_per_row), c = static_cast<int>(i % vec_per_row);
+        dst[i] = src[static_cast<size_t>(row_indices[r]) * vec_per_row + c];
+    }
+}
+template <typename T>
+__global__ __launch_bounds__(kThreads) void k_gather_rows_scalar(const T* __restrict__ src, T* __restrict__ dst,
+                                                                 const int* __restrict__ row_indices, int n_rows,
+                                                                 int width) {
+    const size_t total = static_cast<size_t>(n_rows) * width;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total;
+         i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+        const int r = static_cast<int>(i / width), c = static_cast<int>(i % width);
+        dst[i] = src[static_cast<size_t>(row_indices[r]) * width + c];
+    }
+}
+
+// ---- weighted scatter-accumulate (unpermute) -------------------------------------------
+// mixed[row,h] = bf16(fma(w, compact[i,h], mixed[row,h])): one fused multiply-add (what the
+// CUDA compiler makes of `m + w * c` by default) and one bf16 rounding.
+__device__ __forceinline__ uint32_t fma2_bf16(uint32_t m, uint32_t c, float w) {
+    const float lo = __builtin_fmaf(w, bf16_lo(c), bf16_lo(m));
+    const float hi = __builtin_fmaf(w, bf16_hi(c), bf16_hi(m));
+    return pack_bf16x2(lo, hi);
+}
+// rows of `compact` map to rows of `mixed` through row_indices (or identically when it is null)
+__global__ __launch_bounds__(kThreads) void k_scatter_accumulate(uint16_t* __restrict__ mixed,
+                                                                 const uint16_t* __restrict__ compact,
+                                                                 const float* __restrict__ route_weights,
+                                                                 const int* __restrict__ row_indices, int n_rows,
+                                                                 int expert_idx, int E, int H, int vec) {
+    if (vec) {
+        const int vpr = H / 8;
+        const size_t total = static_cast<size_t>(n_rows) * vpr;
+        for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total;
+             i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+            const int r = static_cast<int>(i / vpr), c = static_cast<int>(i % vpr);
+            const int row = row_indices ? row_indices[r] : r;
+            const float w = route_weights[static_cast<size_t>(row) * E + expert_idx];
+            uint4* dst = reinterpret_cast<uint4*>(mixed + static_cast<size_t>(row) * H) + c;
+            const uint4 cv = reinterpret_cast<const uint4*>(compact + static_cast<size_t>(r) * H)[c];
+            uint4 mv = *dst;
+            mv.x = fma2_bf16(mv.x, cv.x, w); mv.y = fma2_bf16(mv.y, cv.y, w);
+            mv.z = fma2_bf16(mv.z, cv.z, w); mv.w = fma2_bf16(mv.w, cv.w, w);
+            *dst = mv;
+        }
+    } else {
+        const size_t total = static_cast<size_t>(n_rows) * H;
+        for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total;
+             i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+            const int r = static_cast<int>(i / H), h = static_cast<int>(i % H);
+            const int row = row_indices ? row_indices[r] : r;
+            const float w = route_weights[static_cast<size_t>(row) * E + expert_idx];
+            uint16_t* dst = mixed + static_cast<size_t>(row) * H + h;
+            *dst = f32_to_bf16(__builtin_fmaf(w, bf16_to_f32(compact[i]), bf16_to_f32(*dst)));
+        }
+    }
+}
+
+unsigned grid_for(size_t items) {
+    const size_t b = (items + kThreads - 1) / kThreads;
+    return static_cast<unsigned>(b < 1 ? 1 : (b > 8192 ? 8192 : b));
+}
+
+}  // namespace
+}  // namespace cf
+
+using namespace cf;
+
+extern "C" {
+
+int cf_softmax_inplace_f32(float* d_x, int rows, int cols, cf_stream_t stream) {
+    if (rows < 0 || cols < 0) return CF_ERR_INVALID_ARG;
+    if (rows == 0 || cols == 0) return CF_OK;
+    if (!d_x) return CF_ERR_INVALID_ARG;
+    if (cols <= 64) k_softmax_wave<<<ceil_div(rows, kThreads / 64), kThreads, 0, as_stream(stream)>>>(d_x, rows, cols);
+    else k_softmax_block<<<rows, kThreads, 0, as_stream(stream)>>>(d_x, cols);
+    return launch_status();
+}
+
+int cf_moe_topk_route_f32(float* d_scores, int rows, int num_experts, int top_k, cf_stream_t stream,
+                          float* d_row_sum_save, float* d_scores_save, int normalize_topk) {
+    if (rows < 0 || num_experts < 0) return CF_ERR_INVALID_ARG;
+    if (rows == 0 || num_experts == 0) return CF_OK;
+    if (!d_scores) return CF_ERR_INVALID_ARG;
+    if (num_experts > kMaxExpertsGeneric) return CF_ERR_UNSUPPORTED;
+    hipStream_t st = as_stream(stream);
+    if (num_experts <= 64) {
+        k_topk_wave<true><<<ceil_div(rows, kThreads / 64), kThreads, 0, st>>>(d_scores, d_row_sum_save, d_scores_save,
+                                                                               rows, num_experts, top_k, normalize_topk);
+        return launch_status();
+    }
+    k_softmax_block<<<rows, kThreads, 0, st>>>(d_scores, num_experts);
+    if (d_scores_save) {
+        const hipError_t e = hipMemcpyAsync(d_scores_save, d_scores, static_cast<size_t>(rows) * num_experts * sizeof(float),
+                                            hipMemcpyDeviceToDevice, st);
+        if (e != hipSuccess) return static_cast<int>(e);
+    }
+    k_topk_generic<<<ceil_div(rows, 128), 128, 0, st>>>(d_scores, d_row_sum_save, rows, num_experts, top_k, normalize_topk);
+    return launch_status();
+}
+
+int cf_moe_build_expert_row_lists(const float* d_route_weights, int* d_counts, int* d_row_indices, int rows,
+                                  int num_experts, cf_stream_t stream) {
+    if (rows < 0 || num_experts < 0) return CF_ERR_INVALID_ARG;
+    if (num_experts == 0) return CF_OK;
+    if (!d_counts || (rows > 0 && (!d_route_weights || !d_row_indices))) return CF_ERR_INVALID_ARG;
+    k_build_row_lists<<<num_experts, 1024, 0, as_stream(stream)>>>(d_route_weights, d_counts, d_row_indices, rows, num_experts);
+    return launch_status();
+}
+
+int cf_moe_expert_offsets_from_counts(const int* d_counts, int* d_offsets, int num_experts, cf_stream_t stream) {
+    if (num_experts < 0) return CF_ERR_INVALID_ARG;
+    if (num_experts == 0) return CF_OK;
+    if (!d_counts || !d_offsets) return CF_ERR_INVALID_ARG;
+    k_offsets<<<1, 1, 0, as_stream(stream)>>>(d_counts, d_offsets, num_experts);
+    return launch_status();
+}
+
+int cf_moe_gather_rows_u8(const uint8_t* d_src, uint8_t* d_dst, const int* d_row_indices, int n_rows, int width,
+                          cf_stream_t stream) {
+    if (n_rows < 0 || width < 0) return CF_ERR_INVALID_ARG;
+    if (n_rows == 0 || width == 0) return CF_OK;
+    if (!d_src || !d_dst || !d_row_indices) return CF_ERR_INVALID_ARG;
+    const size_t total = static_cast<size_t>(n_rows) * width;
+    if (width % 16 == 0 && aligned16(d_src) && aligned16(d_dst))
+        k_gather_rows16<<<grid_for(total / 16), kThreads, 0, as_stream(stream)>>>(
+            reinterpret_cast<const uint4*>(d_src), reinterpret_cast<uint4*>(d_dst), d_row_indices, n_rows, width / 16);
+    else
+        k_gather_rows_scalar<uint8_t><<<grid_for(total), kThreads, 0, as_stream(stream)>>>(d_src, d_dst, d_row_indices, n_rows, width);
+    return launch_status();
+}
+
+int cf_moe_gather_rows_bf16(const uint16_t* d_src, uint16_t* d_dst, const int* d_row_indices, int n_rows, int width,
+                            cf_stream_t stream) {
+    if (n_rows < 0 || width < 0) return CF_ERR_INVALID_ARG;
+    if (n_rows == 0 || width == 0) return CF_OK;
+    if (!d_src || !d_dst || !d_row_indices) return CF_ERR_INVALID_ARG;
+    const size_t total = static_cast<size_t>(n_rows) * width;
+    if (width % 8 == 0 && aligned16(d_src) && aligned16(d_dst))
+        k_gather_rows16<<<grid_for(total / 8), kThreads, 0, as_stream(stream)>>>(
+            reinterpret_cast<const uint4*>(d_src), reinterpret_cast<uint4*>(d_dst), d_row_indices, n_rows, width / 8);
+    else
+        k_gather_rows_scalar<uint16_t><<<grid_for(total), kThreads, 0, as_stream(stream)>>>(d_src, d_dst, d_row_indices, n_rows, width);
+    return launch_status();
+}
+
+int cf_moe_scatter_accumulate_rows_bf16(uint16_t* d_mixed, const uint16_t* d_compact, const float* d_route_weights,
+                                        const int* d_row_indices, int n_rows, int expert_idx, int num_experts, int H,
+                                        cf_stream_t stream) {
+    if (n_rows < 0 || H < 0 || expert_idx < 0 || expert_idx >= num_experts) return CF_ERR_INVALID_ARG;
+    if (n_rows == 0 || H == 0) return CF_OK;
+    if (!d_mixed || !d_compact || !d_route_weights || !d_row_indices) return CF_ERR_INVALID_ARG;
+    const int vec = H % 8 == 0 && aligned16(d_mixed) && aligned16(d_compact);
+    const size_t items = static_cast<size_t>(n_rows) * (vec ? H / 8 : H);
+    k_scatter_accumulate<<<grid_for(items), kThreads, 0, as_stream(stream)>>>(d_mixed, d_compact, d_route_weights, d_row_indices,
+                                                                              n_rows, expert_idx, num_experts, H, vec);
+    return launch_status();
+}
+
+int cf_moe_scale_accumulate_bf16(uint16_t* d_mixed, const uint16_t* d_term, const float* d_route_weights, int rows,
+                                 int expert_idx, int num_experts, int H, cf_stream_t stream) {
+    if (rows < 0 || H < 0 || expert_idx < 0 || expert_idx >= num_experts) return CF_ERR_INVALID_ARG;
+    if (rows == 0 || H == 0) return CF_OK;
+    if (!d_mixed || !d_term || !d_route_weights) return CF_ERR_INVALID_ARG;
+    const int vec = H % 8 == 0 && aligned16(d_mixed) && aligned16(d_term);
+    const size_t items = static_cast<size_t>(rows) * (vec ? H / 8 : H);
+    k_scatter_accumulate<<<grid_for(items), kThreads, 0, as_stream(stream)>>>(d_mixed, d_term, d_route_weights, nullptr, rows,
+                                                                              expert_idx, num_experts, H, vec);
+    return launch_status();
+}
+
+}  // extern "C"

@@ -192,6 +192,52 @@ int cf_fp8_gemm_nt_accum_f32_ex(int M, int N, int K, const void* d_A, int lda, i
                                 const float* d_b_descale, float* d_C, int ldc, int flags,
                                 cf_stream_t stream);
 
+/* ---- MoE routing and dispatch: kernels/moe.cu, kernels/cross_entropy.cu --------
+ * Routing results are reproducible bit for bit: fixed reduction order, a
+ * deterministic expf, ties broken towards the lowest expert index, row lists in
+ * ascending row order (the reference fills them in atomicAdd arrival order,
+ * kernels/moe.cu:576-577, so its lists equal these as sets). */
+
+/* softmax_inplace_f32, kernels.hpp:193, kernels/cross_entropy.cu:193-197. */
+int cf_softmax_inplace_f32(float* d_x, int rows, int cols, cf_stream_t stream);
+
+/* moe_topk_route_f32, kernels.hpp:313-317, kernels/moe.cu:409-422: softmax, keep the
+ * top_k probabilities per row (strict >, lowest index wins ties), zero the rest,
+ * optionally renormalise the kept ones to sum 1.  The save pointers may be null.
+ * The reference's kept[32] flag array (kernels/moe.cu:383) limits it to 32 experts;
+ * this entry point takes up to 2048. */
+int cf_moe_topk_route_f32(float* d_scores, int rows, int num_experts, int top_k,
+                          cf_stream_t stream, float* d_row_sum_save, float* d_scores_save,
+                          int normalize_topk);
+
+/* moe_build_expert_row_lists, kernels.hpp:361-364, kernels/moe.cu:702-710.
+ * counts[E]; row_indices[E, rows] expert-major, first counts[e] entries valid. */
+int cf_moe_build_expert_row_lists(const float* d_route_weights, int* d_counts,
+                                  int* d_row_indices, int rows, int num_experts,
+                                  cf_stream_t stream);
+
+/* moe_expert_offsets_from_counts, kernels.hpp:397-399, kernels/moe.cu:859-863. */
+int cf_moe_expert_offsets_from_counts(const int* d_counts, int* d_offsets, int num_experts,
+                                      cf_stream_t stream);
+
+/* moe_gather_rows_u8 / moe_gather_rows_bf16, kernels.hpp:365-372, kernels/moe.cu:712-728.
+ * width is in elements. */
+int cf_moe_gather_rows_u8(const uint8_t* d_src, uint8_t* d_dst, const int* d_row_indices,
+                          int n_rows, int width, cf_stream_t stream);
+int cf_moe_gather_rows_bf16(const uint16_t* d_src, uint16_t* d_dst, const int* d_row_indices,
+                            int n_rows, int width, cf_stream_t stream);
+
+/* moe_scatter_accumulate_rows_bf16, kernels.hpp:373-377, kernels/moe.cu:730-738:
+ * mixed[row_indices[i], h] = bf16(mixed + w[row, expert_idx] * compact[i, h]). */
+int cf_moe_scatter_accumulate_rows_bf16(uint16_t* d_mixed, const uint16_t* d_compact,
+                                        const float* d_route_weights, const int* d_row_indices,
+                                        int n_rows, int expert_idx, int num_experts, int H,
+                                        cf_stream_t stream);
+/* moe_scale_accumulate_bf16, kernels.hpp:340-343, kernels/moe.cu:677-683 (dense form). */
+int cf_moe_scale_accumulate_bf16(uint16_t* d_mixed, const uint16_t* d_term,
+                                 const float* d_route_weights, int rows, int expert_idx,
+                                 int num_experts, int H, cf_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -149,7 +149,9 @@ void orc_moe_gather_rows_bf16(const uint16_t* src, uint16_t* dst, const int* row
         memcpy(dst + (size_t)i * width, src + (size_t)row_indices[i] * width, (size_t)width * 2);
 }
 
-/* kernels/moe.cu:607-622: one fp32 multiply, one fp32 add, one bf16 rounding */
+/* kernels/moe.cu:607-622: `mixed + w * compact` in fp32, then one bf16 rounding.  The reference builds
+ * its device code with the CUDA compiler's defaults (no -fmad=false in CMakeLists.txt), which contract
+ * a multiply feeding an add into one fused multiply-add, so the restatement is fmaf. */
 void orc_moe_scatter_accumulate_rows_bf16(uint16_t* mixed, const uint16_t* compact,
                                           const float* route_weights, const int* row_indices,
                                           int n_rows, int expert_idx, int num_experts, int H) {
@@ -158,13 +160,12 @@ void orc_moe_scatter_accumulate_rows_bf16(uint16_t* mixed, const uint16_t* compa
         const float w = route_weights[(size_t)row * num_experts + expert_idx];
         for (int h = 0; h < H; ++h) {
             uint16_t* dst = mixed + (size_t)row * H + h;
-            const float prod = w * orc_bf16_to_f32(compact[(size_t)i * H + h]);
-            *dst = orc_bf16_from_f32(orc_bf16_to_f32(*dst) + prod);
+            *dst = orc_bf16_from_f32(fmaf(w, orc_bf16_to_f32(compact[(size_t)i * H + h]), orc_bf16_to_f32(*dst)));
         }
     }
 }
 
-/* kernels/moe.cu:529-542 */
+/* kernels/moe.cu:529-542 (same contraction as above) */
 void orc_moe_scale_accumulate_bf16(uint16_t* mixed, const uint16_t* term,
                                    const float* route_weights, int rows, int expert_idx,
                                    int num_experts, int H) {
@@ -172,8 +173,7 @@ void orc_moe_scale_accumulate_bf16(uint16_t* mixed, const uint16_t* term,
         const float w = route_weights[(size_t)row * num_experts + expert_idx];
         for (int h = 0; h < H; ++h) {
             uint16_t* dst = mixed + (size_t)row * H + h;
-            const float prod = w * orc_bf16_to_f32(term[(size_t)row * H + h]);
-            *dst = orc_bf16_from_f32(orc_bf16_to_f32(*dst) + prod);
+            *dst = orc_bf16_from_f32(fmaf(w, orc_bf16_to_f32(term[(size_t)row * H + h]), orc_bf16_to_f32(*dst)));
         }
     }
 }

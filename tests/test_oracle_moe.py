@@ -98,6 +98,20 @@ def test_topk_brute_force_all_tie_patterns_tiny():
             assert np.array_equal(got, py_topk(orc.softmax(logits), k))
 
 
+def fma32(a, b, c):
+    """Correctly rounded fp32 fused multiply-add, by exact rational arithmetic."""
+    from fractions import Fraction
+    a, b, c = np.broadcast_arrays(np.asarray(a, np.float32), np.asarray(b, np.float32), np.asarray(c, np.float32))
+    out = np.empty(a.shape, np.float32)
+    for i in np.ndindex(a.shape):
+        exact = Fraction(float(a[i])) * Fraction(float(b[i])) + Fraction(float(c[i]))
+        guess = np.float32(float(exact))                       # may be double-rounded: repair against the neighbours
+        cands = [guess, np.nextafter(guess, np.float32(np.inf)), np.nextafter(guess, np.float32(-np.inf))]
+        best = min(cands, key=lambda v: (abs(Fraction(float(v)) - exact), int(np.float32(v).view(np.uint32)) & 1))
+        out[i] = best
+    return out
+
+
 def test_row_lists_offsets_gather_scatter():
     rng = np.random.default_rng(2)
     rows, E, k, H = 301, 16, 3, 24
@@ -114,18 +128,16 @@ def test_row_lists_offsets_gather_scatter():
     assert np.array_equal(orc.moe_gather_rows_u8(src8, idx[3, : counts[3]]), src8[idx[3, : counts[3]]])
     src16 = rng.integers(0, 65536, (rows, H)).astype(np.uint16)
     assert np.array_equal(orc.moe_gather_rows_bf16(src16, idx[5, : counts[5]]), src16[idx[5, : counts[5]]])
-    # weighted unpermute: one fp32 multiply-add and one bf16 rounding per element, only selected rows change
+    # weighted unpermute: one FUSED multiply-add and one bf16 rounding per element, only selected rows change
     mixed = orc.bf16_from_f32(rng.standard_normal((rows, H)).astype(np.float32))
     compact = orc.bf16_from_f32(rng.standard_normal((counts[3], H)).astype(np.float32))
     out = orc.moe_scatter_accumulate(mixed, compact, rw, idx[3, : counts[3]], 3)
     sel = idx[3, : counts[3]]
-    prod = (rw[sel, 3][:, None] * orc.bf16_to_f32(compact)).astype(np.float32)
     want = mixed.copy()
-    want[sel] = orc.bf16_from_f32(orc.bf16_to_f32(mixed[sel]) + prod)
+    want[sel] = orc.bf16_from_f32(fma32(rw[sel, 3][:, None], orc.bf16_to_f32(compact), orc.bf16_to_f32(mixed[sel])))
     assert np.array_equal(out, want)
     dense = orc.moe_scale_accumulate(mixed, mixed, rw, 3)
-    prod = (rw[:, 3][:, None] * orc.bf16_to_f32(mixed)).astype(np.float32)
-    assert np.array_equal(dense, orc.bf16_from_f32(orc.bf16_to_f32(mixed) + prod))
+    assert np.array_equal(dense, orc.bf16_from_f32(fma32(rw[:, 3][:, None], orc.bf16_to_f32(mixed), orc.bf16_to_f32(mixed))))
 
 
 @pytest.mark.parametrize("mode", [0, 1, 2])

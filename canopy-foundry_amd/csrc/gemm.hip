@@ -51,7 +51,15 @@ struct GemmArgs {
     float* Cf;                   // fp32 [M,N] for EPI_ACCUM_F32 (C += product)
     int tiles_m, tiles_n;
     int force_staged;            // take the register-staged kernel even when the ring kernel applies
+    // grouped (per-expert) form, ring kernel only; all null / 0 for a dense GEMM
+    const int* tile_map;         // [0] = number of row tiles, then (expert, first row, end row) per row tile
+    const int* a_row_index;      // compact row r reads A row (and its descale) a_row_index[r]; null = r
+    long long b_expert_stride;   // bytes between the weight matrices of consecutive experts
+    int sb_expert_stride;        // elements between the channel descales of consecutive experts
 };
+
+// where a workgroup's tile lives: rows [m0, m_end) of the output, columns from n0, weights of `expert`
+struct TilePos { int m0, m_end, n0, expert; };
 
 __device__ __forceinline__ int swz(int row) { return (row ^ ((row >> 3) & 3)) & 7; }
 
@@ -114,7 +122,12 @@ __device__ __forceinline__ void epilogue(v16f (&acc)[4][4], const GemmArgs& p, i
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
         mrow[b] = m0 + wm * 128 + b * 32 + (lane & 31);
-        sa[b] = SCALE == SCALE_TENSOR ? 1.0f : p.sa[min(mrow[b], p.M - 1)];
+        if constexpr (SCALE == SCALE_TENSOR) {
+            sa[b] = 1.0f;
+        } else {
+            const int r = min(mrow[b], p.M - 1);
+            sa[b] = p.sa[p.a_row_index ? p.a_row_index[r] : r];
+        }
     }
 
 #pragma unroll
@@ -318,6 +331,30 @@ constexpr int kRingLds = kSlots * kSlotBytes;     // 160 KiB: all of a CU's LDS
 // s_waitcnt immediates: vmcnt in bits [3:0] and [15:14], expcnt [6:4] and lgkmcnt [11:8] left at no-wait
 constexpr int kWaitVm0 = 0x0f70, kWaitVm8 = 0x0f78, kWaitVm16 = 0x4f70;
 
+template <int OUT_BN>
+__device__ __forceinline__ TilePos locate_tile(const GemmArgs& p, int pos) {
+    TilePos t;
+    if (p.tile_map) {
+        // grouped: row tiles come from the table, column tiles vary fastest so neighbours share an A tile
+        const int total = p.tile_map[0] * p.tiles_n;
+        int lin = pos;
+        if (total % kXcds == 0) lin = (pos % kXcds) * (total / kXcds) + pos / kXcds;
+        const int mt = lin / p.tiles_n, nt = lin - mt * p.tiles_n;
+        t.expert = p.tile_map[1 + 3 * mt];
+        t.m0 = p.tile_map[2 + 3 * mt];
+        t.m_end = p.tile_map[3 + 3 * mt];
+        t.n0 = nt * OUT_BN;
+    } else {
+        int tile_m, tile_n;
+        tile_coords(pos, p.tiles_m, p.tiles_n, tile_m, tile_n);
+        t.expert = 0;
+        t.m0 = tile_m * BM;
+        t.m_end = p.M;
+        t.n0 = tile_n * OUT_BN;
+    }
+    return t;
+}
+
 // The kernel is persistent: workgroup w walks tiles w, w + grid, w + 2*grid, ... of the XCD-aware
 // order, and the copy stream simply runs on into the next tile, so only a workgroup's very first
 // K-tiles pay memory latency; the epilogue of one tile runs while the next tile's first two K-tiles land.
@@ -329,8 +366,9 @@ void k_gemm_nt_ring(const GemmArgs p) {
     constexpr int OUT_BN = EPI == EPI_SILU_GATE ? BN / 2 : BN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int total_tiles = p.tiles_m * p.tiles_n;
+    const int total_tiles = (p.tile_map ? p.tile_map[0] : p.tiles_m) * p.tiles_n;
     const int my_tiles = (total_tiles - static_cast<int>(blockIdx.x) + static_cast<int>(gridDim.x) - 1) / static_cast<int>(gridDim.x);
+    if (my_tiles <= 0) return;        // grouped launches size the grid by an upper bound of the tile count
     const int ktiles = p.K / BK;      // >= 2, checked by the launcher
     const int total_g = my_tiles * ktiles;          // K-tiles this workgroup multiplies, over all its tiles
 
@@ -339,21 +377,23 @@ void k_gemm_nt_ring(const GemmArgs p) {
     const uint8_t* xsrc[8];
     const uint8_t* wsrc[8];
     auto aim = [&](int seq) {                        // point the copy stream at this workgroup's seq-th tile
-        int tile_m, tile_n;
-        tile_coords(blockIdx.x + seq * gridDim.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
-        const int m0 = tile_m * BM, n0 = tile_n * OUT_BN;
+        const TilePos t = locate_tile<OUT_BN>(p, blockIdx.x + seq * gridDim.x);
+        const uint8_t* wbase = p.B + t.expert * p.b_expert_stride;
+        const uint8_t* wbase2 = EPI == EPI_SILU_GATE ? p.B2 + t.expert * p.b_expert_stride : nullptr;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int row = wave * 64 + j * 8 + lrow;
             const int gchunk = (lslot ^ swz(row)) * 16;
-            xsrc[j] = p.A + static_cast<size_t>(min(m0 + row, p.M - 1)) * p.lda + gchunk;
+            int arow = min(t.m0 + row, t.m_end - 1);
+            if (p.a_row_index) arow = p.a_row_index[arow];
+            xsrc[j] = p.A + static_cast<size_t>(arow) * p.lda + gchunk;
             if constexpr (EPI == EPI_SILU_GATE) {
                 // LDS weight rows of a wave: [gate 32 | up 32 | gate 32 | up 32] over the same 64 output columns
-                const int t = (row >> 5) & 3, w = row >> 7;
-                const int n = n0 + w * 64 + (t >> 1) * 32 + (row & 31);
-                wsrc[j] = ((t & 1) ? p.B2 : p.B) + static_cast<size_t>(min(n, p.N - 1)) * p.ldb + gchunk;
+                const int tt = (row >> 5) & 3, w = row >> 7;
+                const int n = t.n0 + w * 64 + (tt >> 1) * 32 + (row & 31);
+                wsrc[j] = ((tt & 1) ? wbase2 : wbase) + static_cast<size_t>(min(n, p.N - 1)) * p.ldb + gchunk;
             } else {
-                wsrc[j] = p.B + static_cast<size_t>(min(n0 + row, p.N - 1)) * p.ldb + gchunk;
+                wsrc[j] = wbase + static_cast<size_t>(min(t.n0 + row, p.N - 1)) * p.ldb + gchunk;
             }
         }
     };
@@ -485,9 +525,14 @@ void k_gemm_nt_ring(const GemmArgs p) {
             step0(g + 1, 0, C0{});
             step1(g + 1, 0, C2{});
         }
-        int tile_m, tile_n;
-        tile_coords(blockIdx.x + seq * gridDim.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
-        epilogue<EPI, SCALE>(acc, p, tile_m * BM, tile_n * OUT_BN, wm, wn, lane);
+        const TilePos t = locate_tile<OUT_BN>(p, blockIdx.x + seq * gridDim.x);
+        GemmArgs q = p;                        // the epilogue sees this tile's row bound and this expert's channel scales
+        q.M = t.m_end;
+        if (SCALE == SCALE_ROWCOL) {
+            q.sb += static_cast<size_t>(t.expert) * p.sb_expert_stride;
+            if (EPI == EPI_SILU_GATE) q.sb2 += static_cast<size_t>(t.expert) * p.sb_expert_stride;
+        }
+        epilogue<EPI, SCALE>(acc, q, t.m0, t.n0, wm, wn, lane);
         zero_acc();
     }
 }
@@ -551,7 +596,7 @@ int launch_tiled(const GemmArgs& p, hipStream_t st) {
         if (ring_err != hipSuccess) return static_cast<int>(ring_err);
         // persistent: one workgroup per CU (the kernel uses a CU's whole LDS and register file);
         // a grid that is a multiple of 8 keeps "position % 8 = XCD" true for every tile a workgroup walks
-        const int total = p.tiles_m * p.tiles_n;
+        const int total = p.tiles_m * p.tiles_n;     // grouped: tiles_m is the host-side upper bound of row tiles
         int grid = total < num_cus() ? total : num_cus();
         if (grid >= kXcds) grid -= grid % kXcds;
         k_gemm_nt_ring<FMT, EPI, SCALE><<<grid, kThreads, kRingLds, st>>>(p);
@@ -574,6 +619,22 @@ int dispatch_epi(const GemmArgs& p, int epi, int scale_mode, hipStream_t st) {
         case EPI_BIAS: return dispatch_scale<FMT, EPI_BIAS>(p, scale_mode, st);
         default:       return dispatch_scale<FMT, EPI_SILU_GATE>(p, scale_mode, st);
     }
+}
+
+// one thread: row tiles of every expert in expert order
+__global__ void k_build_tile_map(const int* __restrict__ counts, const int* __restrict__ offsets, int num_experts,
+                                 int max_row_tiles, int* __restrict__ tile_map) {
+    int n = 0;
+    for (int e = 0; e < num_experts; ++e) {
+        const int first = offsets[e], end = first + counts[e];
+        for (int r = first; r < end && n < max_row_tiles; r += BM) {
+            tile_map[1 + 3 * n] = e;
+            tile_map[2 + 3 * n] = r;
+            tile_map[3 + 3 * n] = min(r + BM, end);
+            ++n;
+        }
+    }
+    tile_map[0] = n;
 }
 
 int gemm_nt(GemmArgs p, int fmt, int epi, int scale_mode, int force_naive, cf_stream_t stream) {
@@ -668,6 +729,57 @@ int cf_fp8_gemm_tn_accum_bf16(int M, int N, int K, const void* Xt_e4m3, const fl
     p.sa = ds_x; p.sb = ds_dy;
     p.C = dW; p.ldc = ldc_dw;
     return gemm_nt(p, 2, EPI_ACCUM_BF16, SCALE_TENSOR, 0, stream);
+}
+
+int cf_fp8_grouped_gemm_workspace_bytes(int total_rows, int num_experts, size_t* bytes) {
+    if (total_rows < 0 || num_experts < 0 || !bytes) return CF_ERR_INVALID_ARG;
+    const size_t max_row_tiles = static_cast<size_t>(total_rows) / BM + static_cast<size_t>(num_experts);
+    *bytes = (1 + 3 * max_row_tiles) * sizeof(int);
+    return CF_OK;
+}
+
+int cf_fp8_grouped_gemm_nt_bf16_ex(int total_rows, int N, int K, int num_experts, const int* d_counts,
+                                   const int* d_offsets, const void* A, int lda, const int* d_a_row_index,
+                                   const float* a_descale, const void* B, const float* b_descale, int scale_mode,
+                                   int epilogue, const void* B_up, const float* b_up_descale, uint16_t* C, int ldc,
+                                   void* d_workspace, size_t workspace_bytes, cf_stream_t stream) {
+    if (total_rows < 0 || N < 0 || K < 0 || num_experts < 0) return CF_ERR_INVALID_ARG;
+    if (total_rows == 0 || N == 0 || num_experts == 0) return CF_OK;
+    if (!d_counts || !d_offsets || !A || !B || !C || !a_descale || !b_descale || !d_workspace) return CF_ERR_INVALID_ARG;
+    if (epilogue != EPI_NONE && epilogue != EPI_SILU_GATE) return CF_ERR_INVALID_ARG;
+    if (epilogue == EPI_SILU_GATE && (!B_up || !b_up_descale)) return CF_ERR_INVALID_ARG;
+    if (scale_mode != SCALE_TENSOR && scale_mode != SCALE_ROWCOL) return CF_ERR_INVALID_ARG;
+    size_t need = 0;
+    cf_fp8_grouped_gemm_workspace_bytes(total_rows, num_experts, &need);
+    if (workspace_bytes < need || (reinterpret_cast<uintptr_t>(d_workspace) & 3u)) return CF_ERR_INVALID_ARG;
+    // the grouped form runs on the ring kernel only
+    if (K % BK != 0 || K < 2 * BK || lda % 16 != 0 || !aligned16(A) || !aligned16(B) ||
+        (epilogue == EPI_SILU_GATE && !aligned16(B_up)) || lda < K || ldc < N)
+        return CF_ERR_UNSUPPORTED;
+    hipStream_t st = as_stream(stream);
+    const int max_row_tiles = total_rows / BM + num_experts;
+    int* tile_map = static_cast<int*>(d_workspace);
+    k_build_tile_map<<<1, 1, 0, st>>>(d_counts, d_offsets, num_experts, max_row_tiles, tile_map);
+    GemmArgs p{};
+    p.M = total_rows; p.N = N; p.K = K;
+    p.A = static_cast<const uint8_t*>(A); p.lda = lda;
+    p.B = static_cast<const uint8_t*>(B); p.ldb = K;
+    p.B2 = static_cast<const uint8_t*>(B_up);
+    p.sa = a_descale; p.sb = b_descale; p.sb2 = b_up_descale;
+    p.C = C; p.ldc = ldc;
+    p.tile_map = tile_map;
+    p.a_row_index = d_a_row_index;
+    p.b_expert_stride = static_cast<long long>(N) * K;
+    p.sb_expert_stride = scale_mode == SCALE_ROWCOL ? N : 0;
+    const int out_bn = epilogue == EPI_SILU_GATE ? BN / 2 : BN;
+    p.tiles_m = max_row_tiles;
+    p.tiles_n = (N + out_bn - 1) / out_bn;
+    if (scale_mode == SCALE_TENSOR) {
+        // per-tensor descales: one device scalar per expert for the weights
+        return CF_ERR_UNSUPPORTED;
+    }
+    return epilogue == EPI_SILU_GATE ? launch_tiled<0, EPI_SILU_GATE, SCALE_ROWCOL>(p, st)
+                                     : launch_tiled<0, EPI_NONE, SCALE_ROWCOL>(p, st);
 }
 
 // Cross-check form of the accumulate GEMMs: any format pair, optional naive kernel.

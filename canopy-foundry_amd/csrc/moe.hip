@@ -250,6 +250,82 @@ __global__ __launch_bounds__(kThreads) void k_scatter_accumulate(uint16_t* __res
     }
 }
 
+// ---- compact row index: the row lists of all experts back to back --------------------
+__global__ __launch_bounds__(kThreads) void k_compact_index(const int* __restrict__ counts, const int* __restrict__ offsets,
+                                                            const int* __restrict__ row_indices, int rows,
+                                                            int* __restrict__ compact) {
+    const int e = blockIdx.y;
+    const int n = counts[e], base = offsets[e];
+    for (int s = blockIdx.x * blockDim.x + threadIdx.x; s < n; s += gridDim.x * blockDim.x)
+        compact[base + s] = row_indices[static_cast<size_t>(e) * rows + s];
+}
+
+// ---- fused weighted unpermute ------------------------------------------------------------
+// One workgroup per token row.  For every expert with a positive route weight, in ascending expert
+// order: mixed[row] = bf16(fma(w, y[slot], mixed[row])), slot = offsets[e] + rank of the row in the
+// expert's (ascending) row list, found by binary search.  Same arithmetic and order as one
+// scatter-accumulate launch per expert.
+__global__ __launch_bounds__(kThreads) void k_unpermute(uint16_t* __restrict__ mixed, const uint16_t* __restrict__ y,
+                                                        const float* __restrict__ route_weights,
+                                                        const int* __restrict__ counts, const int* __restrict__ offsets,
+                                                        const int* __restrict__ row_indices, int rows, int E, int H) {
+    __shared__ int sl_slot[64];
+    __shared__ float sl_w[64];
+    __shared__ int sl_n;
+    const int row = blockIdx.x, t = threadIdx.x;
+    uint16_t* mrow = mixed + static_cast<size_t>(row) * H;
+    for (int e0 = 0; e0 < E; e0 += 64) {
+        if (t < 64) {
+            const int e = e0 + t;
+            const float w = e < E ? route_weights[static_cast<size_t>(row) * E + e] : 0.0f;
+            const bool sel = w > 0.0f;
+            int slot = -1;
+            if (sel) {
+                const int* list = row_indices + static_cast<size_t>(e) * rows;
+                int lo = 0, hi = counts[e] - 1;
+                while (lo <= hi) {
+                    const int mid = (lo + hi) >> 1;
+                    const int v = list[mid];
+                    if (v == row) { slot = offsets[e] + mid; break; }
+                    if (v < row) lo = mid + 1; else hi = mid - 1;
+                }
+            }
+            const bool ok = sel && slot >= 0;
+            const unsigned long long m = __ballot(ok);
+            if (ok) {
+                const int pos = __builtin_popcountll(m & ((1ull << t) - 1ull));
+                sl_slot[pos] = slot;
+                sl_w[pos] = w;
+            }
+            if (t == 0) sl_n = __builtin_popcountll(m);
+        }
+        __syncthreads();
+        const int n = sl_n;
+        if (n > 0) {
+            if ((H & 7) == 0) {
+                for (int c = t; c < H / 8; c += blockDim.x) {
+                    uint4 mv = reinterpret_cast<uint4*>(mrow)[c];
+                    for (int i = 0; i < n; ++i) {
+                        const uint4 yv = reinterpret_cast<const uint4*>(y + static_cast<size_t>(sl_slot[i]) * H)[c];
+                        const float w = sl_w[i];
+                        mv.x = fma2_bf16(mv.x, yv.x, w); mv.y = fma2_bf16(mv.y, yv.y, w);
+                        mv.z = fma2_bf16(mv.z, yv.z, w); mv.w = fma2_bf16(mv.w, yv.w, w);
+                    }
+                    reinterpret_cast<uint4*>(mrow)[c] = mv;
+                }
+            } else {
+                for (int h = t; h < H; h += blockDim.x) {
+                    float m = bf16_to_f32(mrow[h]);
+                    for (int i = 0; i < n; ++i)
+                        m = bf16_to_f32(f32_to_bf16(__builtin_fmaf(sl_w[i], bf16_to_f32(y[static_cast<size_t>(sl_slot[i]) * H + h]), m)));
+                    mrow[h] = f32_to_bf16(m);
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
 unsigned grid_for(size_t items) {
     const size_t b = (items + kThreads - 1) / kThreads;
     return static_cast<unsigned>(b < 1 ? 1 : (b > 8192 ? 8192 : b));
@@ -361,6 +437,96 @@ int cf_moe_scale_accumulate_bf16(uint16_t* d_mixed, const uint16_t* d_term, cons
     k_scatter_accumulate<<<grid_for(items), kThreads, 0, as_stream(stream)>>>(d_mixed, d_term, d_route_weights, nullptr, rows,
                                                                               expert_idx, num_experts, H, vec);
     return launch_status();
+}
+
+int cf_moe_compact_row_index(const int* d_counts, const int* d_offsets, const int* d_row_indices, int rows,
+                             int num_experts, int* d_compact_index, cf_stream_t stream) {
+    if (rows < 0 || num_experts < 0) return CF_ERR_INVALID_ARG;
+    if (rows == 0 || num_experts == 0) return CF_OK;
+    if (!d_counts || !d_offsets || !d_row_indices || !d_compact_index) return CF_ERR_INVALID_ARG;
+    dim3 grid(ceil_div(rows, kThreads) < 16 ? ceil_div(rows, kThreads) : 16, num_experts);
+    k_compact_index<<<grid, kThreads, 0, as_stream(stream)>>>(d_counts, d_offsets, d_row_indices, rows, d_compact_index);
+    return launch_status();
+}
+
+int cf_moe_unpermute_weighted_bf16(uint16_t* d_mixed, const uint16_t* d_compact_out, const float* d_route_weights,
+                                   const int* d_counts, const int* d_offsets, const int* d_row_indices, int rows,
+                                   int num_experts, int H, cf_stream_t stream) {
+    if (rows < 0 || num_experts < 0 || H < 0) return CF_ERR_INVALID_ARG;
+    if (rows == 0 || num_experts == 0 || H == 0) return CF_OK;
+    if (!d_mixed || !d_compact_out || !d_route_weights || !d_counts || !d_offsets || !d_row_indices) return CF_ERR_INVALID_ARG;
+    if ((H & 7) == 0 && !(aligned16(d_mixed) && aligned16(d_compact_out))) return CF_ERR_UNSUPPORTED;
+    k_unpermute<<<rows, kThreads, 0, as_stream(stream)>>>(d_mixed, d_compact_out, d_route_weights, d_counts, d_offsets,
+                                                          d_row_indices, rows, num_experts, H);
+    return launch_status();
+}
+
+// ---- grouped SwiGLU expert bank -----------------------------------------------------------------
+namespace {
+struct SwigluWs { size_t tile_map, index, act, actq, act_scale, act_descale, y, total; };
+SwigluWs swiglu_layout(int total_rows, int num_experts, int H, int Ie) {
+    auto up = [](size_t v) { return (v + 255) & ~static_cast<size_t>(255); };
+    SwigluWs w{};
+    size_t map_bytes = 0;
+    cf_fp8_grouped_gemm_workspace_bytes(total_rows, num_experts, &map_bytes);
+    size_t off = 0;
+    w.tile_map = off; off = up(off + map_bytes);
+    w.index = off; off = up(off + sizeof(int) * static_cast<size_t>(total_rows));
+    w.act = off; off = up(off + 2 * static_cast<size_t>(total_rows) * Ie);
+    w.actq = off; off = up(off + static_cast<size_t>(total_rows) * Ie);
+    w.act_scale = off; off = up(off + sizeof(float) * static_cast<size_t>(total_rows));
+    w.act_descale = off; off = up(off + sizeof(float) * static_cast<size_t>(total_rows));
+    w.y = off; off = up(off + 2 * static_cast<size_t>(total_rows) * H);
+    w.total = off;
+    return w;
+}
+}  // namespace
+
+int cf_moe_grouped_swiglu_workspace_bytes(int total_selected_rows, int num_experts, int H, int Ie, size_t* bytes) {
+    if (total_selected_rows < 0 || num_experts < 0 || H < 0 || Ie < 0 || !bytes) return CF_ERR_INVALID_ARG;
+    *bytes = swiglu_layout(total_selected_rows, num_experts, H, Ie).total;
+    return CF_OK;
+}
+
+int cf_moe_grouped_swiglu_forward_fp8(const void* d_hidden_e4m3, const float* d_hidden_descale,
+                                      const float* d_route_weights, const int* d_counts, const int* d_offsets,
+                                      const int* d_row_indices, const void* d_w_gate, const float* d_w_gate_descale,
+                                      const void* d_w_up, const float* d_w_up_descale, const void* d_w_down,
+                                      const float* d_w_down_descale, uint16_t* d_mixed, int rows, int H, int Ie,
+                                      int num_experts, int total_selected_rows, void* d_workspace,
+                                      size_t workspace_bytes, cf_stream_t stream) {
+    if (rows < 0 || H < 0 || Ie < 0 || num_experts < 0 || total_selected_rows < 0) return CF_ERR_INVALID_ARG;
+    if (rows == 0 || num_experts == 0 || total_selected_rows == 0) return CF_OK;
+    if (!d_hidden_e4m3 || !d_hidden_descale || !d_route_weights || !d_counts || !d_offsets || !d_row_indices ||
+        !d_w_gate || !d_w_gate_descale || !d_w_up || !d_w_up_descale || !d_w_down || !d_w_down_descale || !d_mixed ||
+        !d_workspace)
+        return CF_ERR_INVALID_ARG;
+    const SwigluWs w = swiglu_layout(total_selected_rows, num_experts, H, Ie);
+    if (workspace_bytes < w.total || (reinterpret_cast<uintptr_t>(d_workspace) & 255u)) return CF_ERR_INVALID_ARG;
+    auto* base = static_cast<uint8_t*>(d_workspace);
+    int* index = reinterpret_cast<int*>(base + w.index);
+    auto* act = reinterpret_cast<uint16_t*>(base + w.act);
+    auto* actq = base + w.actq;
+    auto* act_scale = reinterpret_cast<float*>(base + w.act_scale);
+    auto* act_descale = reinterpret_cast<float*>(base + w.act_descale);
+    auto* y = reinterpret_cast<uint16_t*>(base + w.y);
+    size_t map_bytes = 0;
+    cf_fp8_grouped_gemm_workspace_bytes(total_selected_rows, num_experts, &map_bytes);
+    int rc = cf_moe_compact_row_index(d_counts, d_offsets, d_row_indices, rows, num_experts, index, stream);
+    if (rc) return rc;
+    // gate/up: rows gathered through the compact index (the token permute is fused into the operand fetch)
+    rc = cf_fp8_grouped_gemm_nt_bf16_ex(total_selected_rows, Ie, H, num_experts, d_counts, d_offsets, d_hidden_e4m3, H, index,
+                                        d_hidden_descale, d_w_gate, d_w_gate_descale, CF_SCALE_ROW_COL, CF_EPI_SILU_GATE,
+                                        d_w_up, d_w_up_descale, act, Ie, base + w.tile_map, map_bytes, stream);
+    if (rc) return rc;
+    rc = cf_fp8_quantize_rows(act, total_selected_rows, Ie, 0, actq, act_scale, act_descale, stream);
+    if (rc) return rc;
+    rc = cf_fp8_grouped_gemm_nt_bf16_ex(total_selected_rows, H, Ie, num_experts, d_counts, d_offsets, actq, Ie, nullptr,
+                                        act_descale, d_w_down, d_w_down_descale, CF_SCALE_ROW_COL, CF_EPI_NONE, nullptr,
+                                        nullptr, y, H, base + w.tile_map, map_bytes, stream);
+    if (rc) return rc;
+    return cf_moe_unpermute_weighted_bf16(d_mixed, y, d_route_weights, d_counts, d_offsets, d_row_indices, rows,
+                                          num_experts, H, stream);
 }
 
 }  // extern "C"

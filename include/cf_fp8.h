@@ -238,6 +238,64 @@ int cf_moe_scale_accumulate_bf16(uint16_t* d_mixed, const uint16_t* d_term,
                                  const float* d_route_weights, int rows, int expert_idx,
                                  int num_experts, int H, cf_stream_t stream);
 
+/* ---- grouped (per-expert) FP8 GEMM and the SwiGLU expert bank --------------------
+ * The reference runs its selected-row expert path as a host loop of variable-M
+ * cuBLASLt GEMMs after copying the counts to the host (src/trainer.cu:6876-6934), or as
+ * one scalar-FMA kernel per (expert, row tile) (kernels/moe.cu:950-1127).  These entry
+ * points keep the counts on the device and run every expert's tiles in one MFMA launch. */
+
+/* Bytes of the tile table cf_fp8_grouped_gemm_nt_bf16_ex needs in d_workspace.  The reference's GEMM
+ * workspace is the 32 MiB block owned by Fp8Ctx (src/trainer.cu:3300-3301); here the caller owns it. */
+int cf_fp8_grouped_gemm_workspace_bytes(int total_rows, int num_experts, size_t* bytes);
+
+/* For each expert e: C[offsets[e] .. +counts[e], :] = A_rows . B[e]^T with the per-token x
+ * per-channel scales and epilogues of cf_fp8_gemm_nt_bf16_ex (replaces the per-expert
+ * lt_gemm_fp8_nt calls at src/trainer.cu:6893-6931).  A row r of the compact output reads A row
+ * d_a_row_index[r] (and its descale) when the index is given, so the token permute
+ * (moe_gather_rows_u8, kernels/moe.cu:720-728) is fused into the operand fetch; null = row r.
+ * B is [num_experts, N, K] E4M3, b_descale [num_experts, N].  total_rows is the host-side upper
+ * bound rows * top_k; counts / offsets stay on the device.  Needs K % 128 == 0, K >= 256. */
+int cf_fp8_grouped_gemm_nt_bf16_ex(int total_rows, int N, int K, int num_experts,
+                                   const int* d_counts, const int* d_offsets, const void* d_A,
+                                   int lda, const int* d_a_row_index, const float* d_a_descale,
+                                   const void* d_B, const float* d_b_descale, int scale_mode,
+                                   int epilogue, const void* d_B_up, const float* d_b_up_descale,
+                                   uint16_t* d_C, int ldc, void* d_workspace,
+                                   size_t workspace_bytes, cf_stream_t stream);
+
+/* Row lists of all experts back to back: compact[offsets[e] + s] = row_indices[e, s]
+ * (the gather order of moe_gather_rows_u8 over all experts, kernels/moe.cu:594-606). */
+int cf_moe_compact_row_index(const int* d_counts, const int* d_offsets, const int* d_row_indices,
+                             int rows, int num_experts, int* d_compact_index, cf_stream_t stream);
+
+/* All per-expert moe_scatter_accumulate_rows_bf16 launches (kernels/moe.cu:730-738,
+ * src/trainer.cu:6932-6934) in one: experts in ascending order per token row, one bf16
+ * rounding per expert.  compact_out is [sum counts, H] in compact-row order; the row lists
+ * must be ascending (as cf_moe_build_expert_row_lists builds them). */
+int cf_moe_unpermute_weighted_bf16(uint16_t* d_mixed, const uint16_t* d_compact_out,
+                                   const float* d_route_weights, const int* d_counts,
+                                   const int* d_offsets, const int* d_row_indices, int rows,
+                                   int num_experts, int H, cf_stream_t stream);
+
+/* The grouped SwiGLU expert bank of benchmark config 5 (the FP8 form of the expert loop in
+ * moe_expert_bank_forward, src/trainer.cu:6876-6934, with the SwiGLU experts of
+ * moe_generic_forward, src/trainer.cu:6510-6529): permute -> gate/up GEMM with fused SiLU gate
+ * -> per-token E4M3 quantize -> down GEMM -> weighted unpermute added into d_mixed.
+ * hidden [rows,H] E4M3 with per-token descales; w_gate / w_up [E,Ie,H], w_down [E,H,Ie] E4M3 with
+ * per-channel descales [E,Ie] / [E,H].  d_workspace: 256-byte aligned,
+ * cf_moe_grouped_swiglu_workspace_bytes() bytes. */
+int cf_moe_grouped_swiglu_workspace_bytes(int total_selected_rows, int num_experts, int H,
+                                          int Ie, size_t* bytes);
+int cf_moe_grouped_swiglu_forward_fp8(const void* d_hidden_e4m3, const float* d_hidden_descale,
+                                      const float* d_route_weights, const int* d_counts,
+                                      const int* d_offsets, const int* d_row_indices,
+                                      const void* d_w_gate, const float* d_w_gate_descale,
+                                      const void* d_w_up, const float* d_w_up_descale,
+                                      const void* d_w_down, const float* d_w_down_descale,
+                                      uint16_t* d_mixed, int rows, int H, int Ie, int num_experts,
+                                      int total_selected_rows, void* d_workspace,
+                                      size_t workspace_bytes, cf_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

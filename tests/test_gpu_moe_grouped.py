@@ -1,0 +1,144 @@
+"""GPU parity: grouped (per-expert) FP8 GEMM and the SwiGLU expert bank of benchmark config 5.
+
+Integer / byte stages (compact index, per-token quantize of the activations, weighted unpermute) are bit-exact
+against the oracle given their inputs; the GEMM stages meet the GEMM bar against the oracle's double reference."""
+import numpy as np
+import pytest
+import torch
+
+import oracle_lib as orc
+from gpu_util import bf16_bits, case, dev_arr, dev_bf16, host, stream
+from test_gpu_gemm import silu_ref
+
+pytestmark = pytest.mark.gpu
+ROW_COL, EPI_NONE, EPI_SILU = 1, 0, 2
+
+
+def quant_rows_np(x):
+    """float32 [r,c] -> (E4M3 bytes, descale[r]) with the library's per-row scale formula."""
+    q, s, d = orc.quantize_rows(orc.bf16_from_f32(x))
+    return q, d
+
+
+class Bank:
+    """Synthetic expert bank + routing, everything the stages need on host and device."""
+
+    def __init__(self, dev, rows, E, k, H, Ie, seed, zero_expert=None):
+        rng = np.random.default_rng(seed)
+        self.rows, self.E, self.k, self.H, self.Ie = rows, E, k, H, Ie
+        logits = rng.standard_normal((rows, E)).astype(np.float32)
+        if zero_expert is not None:
+            logits[:, zero_expert] = -50.0                   # an expert nobody selects
+        self.rw = orc.moe_topk_route(logits, k)
+        self.counts, self.idx = orc.moe_build_expert_row_lists(self.rw)
+        self.offsets = orc.moe_expert_offsets(self.counts)
+        self.total = rows * k
+        self.hq, self.hd = quant_rows_np(rng.standard_normal((rows, H)).astype(np.float32))
+        self.wg, self.wgd = quant_rows_np((0.02 * rng.standard_normal((E * Ie, H))).astype(np.float32))
+        self.wu, self.wud = quant_rows_np((0.02 * rng.standard_normal((E * Ie, H))).astype(np.float32))
+        self.wd, self.wdd = quant_rows_np((0.02 * rng.standard_normal((E * H, Ie))).astype(np.float32))
+        self.mixed0 = orc.bf16_from_f32(rng.standard_normal((rows, H)).astype(np.float32))
+        d = lambda a: dev_arr(a, dev)
+        self.d = {n: d(getattr(self, n)) for n in ("rw", "counts", "offsets", "idx", "hq", "hd", "wg", "wgd", "wu", "wud", "wd", "wdd")}
+        self.dev = dev
+
+    def compact_index(self):
+        return np.concatenate([self.idx[e, : self.counts[e]] for e in range(self.E)])
+
+
+def run_stages(cf, b: Bank):
+    """The bank through the individual entry points; returns every intermediate."""
+    dev, E, H, Ie, total = b.dev, b.E, b.H, b.Ie, b.total
+    nbytes = np.zeros(1, np.uint64)
+    import ctypes
+    sz = ctypes.c_size_t(0)
+    assert cf.raw_cf_fp8_grouped_gemm_workspace_bytes(total, E, ctypes.byref(sz)) == 0
+    ws = torch.empty(sz.value, dtype=torch.uint8, device=dev)
+    cidx = torch.full((total,), -1, dtype=torch.int32, device=dev)
+    cf.cf_moe_compact_row_index(b.d["counts"], b.d["offsets"], b.d["idx"], b.rows, E, cidx, stream())
+    act = torch.zeros((total, Ie), dtype=torch.bfloat16, device=dev)
+    cf.cf_fp8_grouped_gemm_nt_bf16_ex(total, Ie, H, E, b.d["counts"], b.d["offsets"], b.d["hq"], H, cidx, b.d["hd"],
+                                      b.d["wg"], b.d["wgd"], ROW_COL, EPI_SILU, b.d["wu"], b.d["wud"], act, Ie, ws, sz.value, stream())
+    actq = torch.empty((total, Ie), dtype=torch.uint8, device=dev)
+    a_s = torch.empty(total, device=dev); a_d = torch.empty(total, device=dev)
+    cf.cf_fp8_quantize_rows(act, total, Ie, 0, actq, a_s, a_d, stream())
+    y = torch.zeros((total, H), dtype=torch.bfloat16, device=dev)
+    cf.cf_fp8_grouped_gemm_nt_bf16_ex(total, H, Ie, E, b.d["counts"], b.d["offsets"], actq, Ie, None, a_d,
+                                      b.d["wd"], b.d["wdd"], ROW_COL, EPI_NONE, None, None, y, H, ws, sz.value, stream())
+    mixed = dev_bf16(b.mixed0, dev)
+    cf.cf_moe_unpermute_weighted_bf16(mixed, y, b.d["rw"], b.d["counts"], b.d["offsets"], b.d["idx"], b.rows, E, H, stream())
+    torch.cuda.synchronize()
+    return dict(cidx=host(cidx), act=bf16_bits(act), actq=host(actq), a_s=host(a_s), a_d=host(a_d), y=bf16_bits(y), mixed=bf16_bits(mixed))
+
+
+def run_fused(cf, b: Bank):
+    import ctypes
+    sz = ctypes.c_size_t(0)
+    assert cf.raw_cf_moe_grouped_swiglu_workspace_bytes(b.total, b.E, b.H, b.Ie, ctypes.byref(sz)) == 0
+    ws = torch.empty(sz.value + 256, dtype=torch.uint8, device=b.dev)
+    off = (-ws.data_ptr()) % 256
+    mixed = dev_bf16(b.mixed0, b.dev)
+    cf.cf_moe_grouped_swiglu_forward_fp8(b.d["hq"], b.d["hd"], b.d["rw"], b.d["counts"], b.d["offsets"], b.d["idx"],
+                                         b.d["wg"], b.d["wgd"], b.d["wu"], b.d["wud"], b.d["wd"], b.d["wdd"], mixed,
+                                         b.rows, b.H, b.Ie, b.E, b.total, ws.data_ptr() + off, sz.value, stream())
+    torch.cuda.synchronize()
+    return bf16_bits(mixed)
+
+
+def check_stages(b: Bank, r, experts=None, sample=None):
+    E, H, Ie = b.E, b.H, b.Ie
+    cidx = b.compact_index()
+    assert np.array_equal(r["cidx"], cidx)                                     # permutation indices: bit-exact
+    # per-token quantize of the GPU's own activations: bit-exact
+    wq, ws_, wd_ = orc.quantize_rows(r["act"])
+    assert np.array_equal(r["actq"], wq) and np.array_equal(r["a_s"], ws_) and np.array_equal(r["a_d"], wd_)
+    # weighted unpermute of the GPU's own expert outputs: bit-exact, experts applied in ascending order
+    mixed = b.mixed0
+    for e in range(E):
+        n, o = int(b.counts[e]), int(b.offsets[e])
+        mixed = orc.moe_scatter_accumulate(mixed, r["y"][o:o + n], b.rw, b.idx[e, :n], e)
+    assert np.array_equal(r["mixed"], mixed)
+    # GEMM stages against the double reference, per expert (optionally on a sample of each expert's rows)
+    for e in (range(E) if experts is None else experts):
+        n, o = int(b.counts[e]), int(b.offsets[e])
+        if n == 0:
+            continue
+        sel = np.arange(n) if sample is None or n <= sample else np.sort(np.random.default_rng(e).choice(n, sample, replace=False))
+        rows = b.idx[e, :n][sel]
+        A, sa = b.hq[rows], b.hd[rows]
+        gref, _ = orc.gemm_nt_ref(A, b.wg[e * Ie:(e + 1) * Ie], sa, b.wgd[e * Ie:(e + 1) * Ie], scale_mode=1, want_abs=False)
+        uref, _ = orc.gemm_nt_ref(A, b.wu[e * Ie:(e + 1) * Ie], sa, b.wud[e * Ie:(e + 1) * Ie], scale_mode=1, want_abs=False)
+        exact = silu_ref(gref, uref)
+        got = orc.bf16_to_f32(r["act"][o:o + n][sel]).astype(np.float64)
+        rel = np.sqrt(((got - exact) ** 2).sum() / (exact ** 2).sum())
+        assert rel <= 4e-3, (e, rel)                                           # three bf16 roundings, as in the dense fused test
+        yref, yabs = orc.gemm_nt_ref(r["actq"][o:o + n][sel], b.wd[e * H:(e + 1) * H], r["a_d"][o:o + n][sel],
+                                     b.wdd[e * H:(e + 1) * H], scale_mode=1)
+        orc.assert_gemm_close(orc.bf16_to_f32(r["y"][o:o + n][sel]).astype(np.float64), yref, yabs, what=f"down expert {e}")
+
+
+@pytest.mark.parametrize("rows,E,k,H,Ie,zero", [(600, 5, 2, 256, 384, None), (300, 4, 2, 256, 256, 2), (1500, 3, 1, 512, 640, None), (40, 8, 3, 256, 256, None)])
+def test_grouped_bank_small(cf, dev, rows, E, k, H, Ie, zero):
+    case(f"grouped swiglu bank rows={rows} E={E} k={k} H={H} Ie={Ie}")
+    b = Bank(dev, rows, E, k, H, Ie, seed=rows + E, zero_expert=zero)
+    r = run_stages(cf, b)
+    check_stages(b, r)
+    assert np.array_equal(run_fused(cf, b), r["mixed"])                        # the one-call form is the same computation
+
+
+def test_grouped_gemm_leaves_rows_of_other_experts_alone(cf, dev):
+    case("grouped gemm write footprint")
+    b = Bank(dev, 700, 6, 2, 256, 256, seed=9)
+    r = run_stages(cf, b)
+    # every compact row was written exactly by its expert: rows are a permutation, no zero rows left behind
+    assert np.all((r["act"] != 0).any(axis=1)) and np.all((r["y"] != 0).any(axis=1))
+
+
+def test_config5_full_size(cf, dev):
+    """16384 tokens, hidden 2048, 64 experts, top-6, expert width 1408."""
+    case("config 5 full size")
+    b = Bank(dev, 16384, 64, 6, 2048, 1408, seed=5)
+    assert b.counts.sum() == 98304
+    r = run_stages(cf, b)
+    check_stages(b, r, experts=[0, 31, 63], sample=24)
+    assert np.array_equal(run_fused(cf, b), r["mixed"])

@@ -8,6 +8,8 @@
 // order by a scan instead of atomics.
 #include "common.hpp"
 
+#include <mutex>
+
 namespace cf {
 namespace {
 
@@ -326,6 +328,103 @@ __global__ __launch_bounds__(kThreads) void k_unpermute(uint16_t* __restrict__ m
     }
 }
 
+// ---- grouped GELU expert bank, reference semantics ------------------------------------------
+// mixed[row] += w * fc_out(gelu(fc_in(hidden[row]))) for every selected (expert,row): operands are
+// dequantised with per-tensor descales, the exact-erf GELU output stays in fp32 (it is not
+// re-quantised), products are accumulated in fp32, and the result is added to the bf16 output with a
+// 32-bit compare-and-swap on the word holding it.  One workgroup per (expert, tile of 16 rows);
+// workgroups past an expert's row count leave at once.  This is the correctness form the reference
+// keeps beside its tensor-core path; the fast path for expert banks is the grouped SwiGLU pipeline.
+constexpr int kGeluRows = 16;
+constexpr int kGeluChunk = 128;
+
+__device__ __forceinline__ void atomic_add_bf16(uint16_t* addr, float v) {
+    const uintptr_t a = reinterpret_cast<uintptr_t>(addr);
+    auto* word = reinterpret_cast<unsigned int*>(a & ~static_cast<uintptr_t>(3));
+    const unsigned shift = (a & 2) ? 16u : 0u;
+    unsigned old = *word;
+    while (true) {
+        const unsigned assumed = old;
+        const float cur = bf16_to_f32(static_cast<uint16_t>((assumed >> shift) & 0xffffu));
+        const unsigned next = (assumed & ~(0xffffu << shift)) | (static_cast<unsigned>(f32_to_bf16(cur + v)) << shift);
+        old = atomicCAS(word, assumed, next);
+        if (old == assumed) return;
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void k_grouped_gelu_fp8(const uint8_t* __restrict__ hidden, const float* __restrict__ fcin_descale,
+                                                               int fcin_is_e5m2, const float* __restrict__ route_weights,
+                                                               const int* __restrict__ counts, const int* __restrict__ row_indices,
+                                                               const uint8_t* __restrict__ fc_in_w, const float* __restrict__ fc_in_descale,
+                                                               const uint8_t* __restrict__ fc_out_w, const float* __restrict__ fc_out_descale,
+                                                               uint16_t* __restrict__ mixed, int rows, int H, int Ie, int E,
+                                                               int tiles_per_expert) {
+    extern __shared__ float sh[];
+    float* sh_chunk = sh;                                  // [kGeluRows][kGeluChunk]
+    float* sh_act = sh + kGeluRows * kGeluChunk;           // [kGeluRows][Ie]
+    const int e = blockIdx.x / tiles_per_expert, tile = blockIdx.x % tiles_per_expert;
+    const int first = tile * kGeluRows, n_active = counts[e];
+    if (first >= n_active) return;
+    const int n_rows = min(kGeluRows, n_active - first);
+    const int* my_rows = row_indices + static_cast<size_t>(e) * rows + first;
+    const float d_in = *fcin_descale, d_win = *fc_in_descale, d_wout = *fc_out_descale;
+    const uint8_t* w_in = fc_in_w + static_cast<size_t>(e) * H * Ie;
+    const uint8_t* w_out = fc_out_w + static_cast<size_t>(e) * Ie * H;
+
+    // fc_in: 256 output columns per pass, K in chunks of 128 staged (dequantised) through LDS
+    for (int j0 = 0; j0 < Ie; j0 += kThreads) {
+        const int j = j0 + threadIdx.x;
+        float accum[kGeluRows];
+#pragma unroll
+        for (int r = 0; r < kGeluRows; ++r) accum[r] = 0.0f;
+        for (int k0 = 0; k0 < H; k0 += kGeluChunk) {
+            const int kt = min(kGeluChunk, H - k0);
+            __syncthreads();
+            for (int i = threadIdx.x; i < n_rows * kt; i += kThreads) {
+                const int r = i / kt, k = i % kt;
+                const uint8_t b = hidden[static_cast<size_t>(my_rows[r]) * H + k0 + k];
+                sh_chunk[r * kGeluChunk + k] = (fcin_is_e5m2 ? e5m2_to_f32(b) : e4m3_to_f32(b)) * d_in;
+            }
+            __syncthreads();
+            if (j < Ie) {
+                const uint8_t* wr = w_in + static_cast<size_t>(j) * H + k0;
+                for (int k = 0; k < kt; ++k) {
+                    const float wv = e4m3_to_f32(wr[k]) * d_win;
+#pragma unroll
+                    for (int r = 0; r < kGeluRows; ++r) accum[r] = __builtin_fmaf(sh_chunk[r * kGeluChunk + k], wv, accum[r]);
+                }
+            }
+        }
+        if (j < Ie) {
+#pragma unroll
+            for (int r = 0; r < kGeluRows; ++r) {
+                const float v = accum[r];
+                sh_act[r * Ie + j] = 0.5f * v * (1.0f + erff(v * 0.7071067811865476f));
+            }
+        }
+    }
+    __syncthreads();
+    // fc_out: activations are resident in LDS
+    for (int h0 = 0; h0 < H; h0 += kThreads) {
+        const int h = h0 + threadIdx.x;
+        if (h >= H) continue;
+        float accum[kGeluRows];
+#pragma unroll
+        for (int r = 0; r < kGeluRows; ++r) accum[r] = 0.0f;
+        const uint8_t* wr = w_out + static_cast<size_t>(h) * Ie;
+        for (int k = 0; k < Ie; ++k) {
+            const float wv = e4m3_to_f32(wr[k]) * d_wout;
+#pragma unroll
+            for (int r = 0; r < kGeluRows; ++r) accum[r] = __builtin_fmaf(sh_act[r * Ie + k], wv, accum[r]);
+        }
+        for (int r = 0; r < n_rows; ++r) {
+            const int row = my_rows[r];
+            const float rw = route_weights[static_cast<size_t>(row) * E + e];
+            atomic_add_bf16(mixed + static_cast<size_t>(row) * H + h, rw * accum[r]);
+        }
+    }
+}
+
 unsigned grid_for(size_t items) {
     const size_t b = (items + kThreads - 1) / kThreads;
     return static_cast<unsigned>(b < 1 ? 1 : (b > 8192 ? 8192 : b));
@@ -527,6 +626,35 @@ int cf_moe_grouped_swiglu_forward_fp8(const void* d_hidden_e4m3, const float* d_
     if (rc) return rc;
     return cf_moe_unpermute_weighted_bf16(d_mixed, y, d_route_weights, d_counts, d_offsets, d_row_indices, rows,
                                           num_experts, H, stream);
+}
+
+int cf_moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_fcin_descale, int fcin_is_e5m2,
+                                      const float* d_route_weights, const int* d_counts, const int* d_offsets,
+                                      const int* d_row_indices, const void* d_fc_in_w, const float* d_fc_in_descale,
+                                      const void* d_fc_out_w, const float* d_fc_out_descale, uint16_t* d_mixed, int rows,
+                                      int H, int Ie, int num_experts, int total_selected_rows, cf_stream_t stream) {
+    (void)d_offsets;               // as in the reference, the tiled form needs neither
+    (void)total_selected_rows;
+    if (rows < 0 || H < 0 || Ie < 0 || num_experts < 0) return CF_ERR_INVALID_ARG;
+    if (rows == 0 || num_experts == 0 || H == 0 || Ie == 0) return CF_OK;
+    if (!d_hidden || !d_fcin_descale || !d_route_weights || !d_counts || !d_row_indices || !d_fc_in_w || !d_fc_in_descale ||
+        !d_fc_out_w || !d_fc_out_descale || !d_mixed)
+        return CF_ERR_INVALID_ARG;
+    const size_t smem = sizeof(float) * static_cast<size_t>(kGeluRows) * (kGeluChunk + Ie);
+    if (smem > 160 * 1024) return CF_ERR_UNSUPPORTED;
+    static std::once_flag once;
+    static hipError_t attr_err = hipSuccess;
+    std::call_once(once, [] {
+        attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_grouped_gelu_fp8),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    });
+    if (attr_err != hipSuccess) return static_cast<int>(attr_err);
+    const int tiles_per_expert = (rows + kGeluRows - 1) / kGeluRows;
+    k_grouped_gelu_fp8<<<num_experts * tiles_per_expert, kThreads, smem, as_stream(stream)>>>(
+        static_cast<const uint8_t*>(d_hidden), d_fcin_descale, fcin_is_e5m2, d_route_weights, d_counts, d_row_indices,
+        static_cast<const uint8_t*>(d_fc_in_w), d_fc_in_descale, static_cast<const uint8_t*>(d_fc_out_w), d_fc_out_descale,
+        d_mixed, rows, H, Ie, num_experts, tiles_per_expert);
+    return launch_status();
 }
 
 }  // extern "C"

@@ -296,6 +296,21 @@ int cf_moe_grouped_swiglu_forward_fp8(const void* d_hidden_e4m3, const float* d_
                                       int total_selected_rows, void* d_workspace,
                                       size_t workspace_bytes, cf_stream_t stream);
 
+/* moe_grouped_expert_forward_fp8, kernels.hpp:400-423, kernels/moe.cu:1063-1127 (kernel :950-1060):
+ * mixed[row] += w[row,e] * fc_out_e(gelu(fc_in_e(hidden[row]))) for every selected (expert,row);
+ * per-tensor device descales, exact-erf GELU kept in fp32 (not re-quantised), bf16 accumulation
+ * by compare-and-swap, so the last bit of d_mixed depends on arrival order as in the reference.
+ * fc_in_w [E,Ie,H], fc_out_w [E,H,Ie] E4M3; hidden E4M3 or E5M2.  d_offsets and
+ * total_selected_rows are accepted and unused, as in the reference. */
+int cf_moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_fcin_descale,
+                                      int fcin_is_e5m2, const float* d_route_weights,
+                                      const int* d_counts, const int* d_offsets,
+                                      const int* d_row_indices, const void* d_fc_in_w,
+                                      const float* d_fc_in_descale, const void* d_fc_out_w,
+                                      const float* d_fc_out_descale, uint16_t* d_mixed, int rows,
+                                      int H, int Ie, int num_experts, int total_selected_rows,
+                                      cf_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

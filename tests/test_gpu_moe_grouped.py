@@ -142,3 +142,41 @@ def test_config5_full_size(cf, dev):
     r = run_stages(cf, b)
     check_stages(b, r, experts=[0, 31, 63], sample=24)
     assert np.array_equal(run_fused(cf, b), r["mixed"])
+
+
+@pytest.mark.parametrize("rows,E,k,H,Ie,e5m2", [(90, 4, 2, 96, 72, False), (300, 6, 3, 256, 300, True), (33, 3, 3, 40, 1408, False)])
+def test_grouped_gelu_expert_bank_reference_form(cf, dev, rows, E, k, H, Ie, e5m2):
+    """moe_grouped_expert_forward_fp8: per-tensor descales, float GELU intermediate, bf16 CAS accumulate."""
+    case(f"grouped gelu bank rows={rows} E={E} k={k} H={H} Ie={Ie} e5m2={e5m2}")
+    rng = np.random.default_rng(rows + Ie)
+    x = rng.standard_normal((rows, H)).astype(np.float32)
+    fmax = 57344.0 if e5m2 else 448.0
+    sx = np.float32(fmax) / np.abs(x).max()
+    hq = (orc.e5m2_satfinite if e5m2 else orc.e4m3_satfinite)(x * sx)
+    win = (0.05 * rng.standard_normal((E, Ie, H))).astype(np.float32)
+    wout = (0.05 * rng.standard_normal((E, H, Ie))).astype(np.float32)
+    s_in, s_out = np.float32(448.0) / np.abs(win).max(), np.float32(448.0) / np.abs(wout).max()
+    winq, woutq = orc.e4m3_satfinite(win * s_in), orc.e4m3_satfinite(wout * s_out)
+    d_h, d_in, d_out = np.float32(1) / sx, np.float32(1) / s_in, np.float32(1) / s_out
+    rw = orc.moe_topk_route(rng.standard_normal((rows, E)).astype(np.float32), k)
+    counts, idx = orc.moe_build_expert_row_lists(rw)
+    mixed0 = orc.bf16_from_f32(rng.standard_normal((rows, H)).astype(np.float32))
+    mixed = dev_bf16(mixed0, dev)
+    sc = lambda v: torch.tensor([v], dtype=torch.float32, device=dev)
+    cf.cf_moe_grouped_expert_forward_fp8(dev_arr(hq, dev), sc(d_h), int(e5m2), dev_arr(rw, dev), dev_arr(counts, dev), None,
+                                         dev_arr(idx, dev), dev_arr(winq, dev), sc(d_in), dev_arr(woutq, dev), sc(d_out),
+                                         mixed, rows, H, Ie, E, rows * k, stream())
+    torch.cuda.synchronize()
+    start = orc.bf16_to_f32(mixed0).astype(np.float64)
+    ref = orc.moe_grouped_expert_forward_fp8_ref(hq, d_h, e5m2, rw, counts, idx, winq, d_in, woutq, d_out, start)
+    got = orc.bf16_to_f32(bf16_bits(mixed)).astype(np.float64)
+    rel = np.sqrt(((got - ref) ** 2).sum() / (ref ** 2).sum())
+    assert rel <= 4e-3, rel
+    # every one of the k accumulations rounds the running value to bf16 (relative 2^-9 each), and the running value
+    # can exceed both end points when contributions cancel: bound it by start, result and the typical contribution
+    typical = np.sqrt(((ref - start) ** 2).mean())
+    bound = (k + 1) * 2.0 ** -8 * (np.abs(start) + np.abs(ref) + 2.0 * typical)
+    assert np.all(np.abs(got - ref) <= bound)
+    # rows routed to no expert keep their value
+    untouched = ~(rw > 0).any(axis=1)
+    assert np.array_equal(bf16_bits(mixed)[untouched], mixed0[untouched])

@@ -36,7 +36,7 @@ constexpr int kLdsBytes = 2 * kStageBytes;        // double buffered: 128 KiB
 constexpr int kXcds = 8;
 
 enum { EPI_NONE = 0, EPI_BIAS = 1, EPI_SILU_GATE = 2, EPI_ACCUM_F32 = 3, EPI_ACCUM_BF16 = 4 };
-enum { SCALE_TENSOR = 0, SCALE_ROWCOL = 1 };
+enum { SCALE_TENSOR = 0, SCALE_ROWCOL = 1, SCALE_BLOCK = 2 };
 
 struct GemmArgs {
     int M, N, K;                 // N = output columns
@@ -312,6 +312,152 @@ void k_gemm_nt(const GemmArgs p) {
 }
 
 
+// ---- block-scaled kernel: activation scales per 1 x 128 K-group, weight scales per 128 x 128 block ----
+// Workgroup tile 128 x 256 x 128, four wavefronts 2 x 2, each 64 x 128 = 4 x 2 MFMA tiles.  One K-tile
+// is exactly one scale group, so each K-tile is multiplied into a zeroed set of partial accumulators
+// (128 registers) and then promoted into the running sum with the group's factor
+// sa[m, kt] * sb[n / 128, kt] on the vector ALU (another 128 registers).  Register-staged loads,
+// double-buffered LDS, one barrier per K-tile; K is zero-padded up to a multiple of 128.
+constexpr int BSM = 128;                                   // rows per workgroup
+constexpr int kBlkX = BSM * BK, kBlkW = BN * BK;           // 16 KiB + 32 KiB per stage
+constexpr int kBlkStage = kBlkX + kBlkW;
+constexpr int kBlkLds = 2 * kBlkStage;                     // 96 KiB
+
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void k_gemm_nt_block(const GemmArgs p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    // plain order with 8-row groups: the block-scaled shapes are modest and L2 resident
+    const int tile_m = blockIdx.x % p.tiles_m, tile_n = blockIdx.x / p.tiles_m;
+    const int m0 = tile_m * BSM, n0 = tile_n * BN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int kb = (p.K + BK - 1) / BK;                    // scale groups along K
+
+    const int r0 = tid >> 3, c = tid & 7;
+    const int lds_w = r0 * BK + ((c ^ swz(r0)) << 4);
+    const uint8_t* xsrc[4];
+    const uint8_t* wsrc[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) xsrc[i] = p.A + static_cast<size_t>(min(m0 + r0 + 32 * i, p.M - 1)) * p.lda + c * 16;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) wsrc[i] = p.B + static_cast<size_t>(min(n0 + r0 + 32 * i, p.N - 1)) * p.ldb + c * 16;
+    uint4 xr[4], wr[8];
+    auto fetch = [&](int k0) {
+        const bool live = k0 + c * 16 < p.K;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) xr[i] = live ? *reinterpret_cast<const uint4*>(xsrc[i] + k0) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) wr[i] = live ? *reinterpret_cast<const uint4*>(wsrc[i] + k0) : make_uint4(0, 0, 0, 0);
+    };
+    auto stash = [&](int stage) {
+        uint8_t* xs = smem + stage * kBlkStage + lds_w;
+        uint8_t* ws = xs + kBlkX;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4*>(xs + i * 32 * BK) = xr[i];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) *reinterpret_cast<uint4*>(ws + i * 32 * BK) = wr[i];
+    };
+
+    const int frow = lane & 31, khalf = lane >> 5, fs = swz(frow);
+    int rd[2][2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) rd[s][j] = frow * BK + (((s * 4 + khalf * 2 + j) ^ fs) << 4);
+    const int x_base = wm * 64 * BK, w_base = kBlkX + wn * 128 * BK;
+
+    v16f sum[4][2];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sum[a][b][r] = 0.0f;
+
+    // this lane's two output rows and this wave's weight block row
+    int mrow[2];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) mrow[b] = min(m0 + wm * 64 + b * 32 + (lane & 31), p.M - 1);
+    const int nblk = min(n0 + wn * 128, p.N - 1) / 128;
+
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    for (int kt = 0; kt < kb; ++kt) {
+        const int stage = kt & 1;
+        const bool more = kt + 1 < kb;
+        if (more) fetch((kt + 1) * BK);
+        // the group's factors: issued before the MFMAs so they have landed when the promotion needs them
+        const float sbv = p.sb[static_cast<size_t>(nblk) * kb + kt];
+        float f[2];
+#pragma unroll
+        for (int b = 0; b < 2; ++b) f[b] = p.sa[static_cast<size_t>(mrow[b]) * kb + kt] * sbv;
+        const uint8_t* st = smem + stage * kBlkStage;
+        v16f part[4][2];
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            v8i wf[4], xf[2];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const uint4 w0 = *reinterpret_cast<const uint4*>(st + w_base + t * 32 * BK + rd[s][0]);
+                const uint4 w1 = *reinterpret_cast<const uint4*>(st + w_base + t * 32 * BK + rd[s][1]);
+                wf[t] = v8i{(int)w0.x, (int)w0.y, (int)w0.z, (int)w0.w, (int)w1.x, (int)w1.y, (int)w1.z, (int)w1.w};
+            }
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const uint4 x0 = *reinterpret_cast<const uint4*>(st + x_base + t * 32 * BK + rd[s][0]);
+                const uint4 x1 = *reinterpret_cast<const uint4*>(st + x_base + t * 32 * BK + rd[s][1]);
+                xf[t] = v8i{(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w, (int)x1.x, (int)x1.y, (int)x1.z, (int)x1.w};
+            }
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+#pragma unroll
+                for (int b = 0; b < 2; ++b) {
+                    v16f cin;
+                    if (s == 0) {
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) cin[r] = 0.0f;
+                    } else {
+                        cin = part[a][b];
+                    }
+                    part[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[a], xf[b], cin, 0, 0, 0, 0, 0, 0);
+                }
+        }
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sum[a][b][r] = __builtin_fmaf(part[a][b][r], f[b], sum[a][b][r]);
+        if (more) stash(stage ^ 1);
+        __syncthreads();
+    }
+
+    // epilogue: the sums are already scaled; lane holds four consecutive columns per quad
+    const bool vec_ok = (p.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.C) & 7u) == 0);
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+        const int m = m0 + wm * 64 + b * 32 + (lane & 31);
+        if (m >= p.M) continue;
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int n = n0 + wn * 128 + a * 32 + g * 8 + khalf * 4;
+                uint16_t* crow = p.C + static_cast<size_t>(m) * p.ldc + n;
+                const uint32_t o01 = pack_bf16x2_hw(sum[a][b][g * 4 + 0], sum[a][b][g * 4 + 1]);
+                const uint32_t o23 = pack_bf16x2_hw(sum[a][b][g * 4 + 2], sum[a][b][g * 4 + 3]);
+                if (vec_ok && n + 3 < p.N) {
+                    *reinterpret_cast<uint2*>(crow) = make_uint2(o01, o23);
+                } else {
+                    const uint16_t o[4] = {(uint16_t)(o01 & 0xffffu), (uint16_t)(o01 >> 16), (uint16_t)(o23 & 0xffffu), (uint16_t)(o23 >> 16)};
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) if (n + q < p.N) crow[q] = o[q];
+                }
+            }
+    }
+}
+
 // ---- ring kernel: direct-to-LDS copies into five 32 KiB slots --------------------------------
 // Needs K % 128 == 0 and K >= 256.  global_load_lds_dwordx4 copies 16 bytes per lane from global
 // memory straight into LDS (lane l lands at base + 16*l): no staging registers, and eight lanes
@@ -546,6 +692,19 @@ __global__ __launch_bounds__(256) void k_gemm_nt_naive(const GemmArgs p, int fmt
     const uint8_t* a = p.A + static_cast<size_t>(m) * p.lda;
     const uint8_t* b = p.B + static_cast<size_t>(n) * p.ldb;
     const uint8_t* b2 = epi == EPI_SILU_GATE ? p.B2 + static_cast<size_t>(n) * p.ldb : nullptr;
+    if (scale_mode == SCALE_BLOCK) {
+        // per 128-group partial sums, each promoted with its own factor
+        const int kb = (p.K + 127) / 128;
+        float total = 0.0f;
+        for (int g = 0; g < kb; ++g) {
+            float part = 0.0f;
+            for (int k = g * 128; k < min(p.K, g * 128 + 128); ++k)
+                part = __builtin_fmaf((fmt & 1) ? e5m2_to_f32(a[k]) : e4m3_to_f32(a[k]), e4m3_to_f32(b[k]), part);
+            total = __builtin_fmaf(part, p.sa[static_cast<size_t>(m) * kb + g] * p.sb[static_cast<size_t>(n / 128) * kb + g], total);
+        }
+        p.C[static_cast<size_t>(m) * p.ldc + n] = f32_to_bf16(total);
+        return;
+    }
     float acc = 0.0f, acc2 = 0.0f;
     for (int k = 0; k < p.K; ++k) {
         const float av = (fmt & 1) ? e5m2_to_f32(a[k]) : e4m3_to_f32(a[k]);
@@ -641,8 +800,9 @@ int gemm_nt(GemmArgs p, int fmt, int epi, int scale_mode, int force_naive, cf_st
     if (p.M < 0 || p.N < 0 || p.K < 0) return CF_ERR_INVALID_ARG;
     if (p.M == 0 || p.N == 0) return CF_OK;
     if (!p.A || !p.B || !(epi == EPI_ACCUM_F32 ? (void*)p.Cf : (void*)p.C) || !p.sa || !p.sb) return CF_ERR_INVALID_ARG;
-    if (epi < EPI_NONE || epi > EPI_ACCUM_BF16 || scale_mode < SCALE_TENSOR || scale_mode > SCALE_ROWCOL)
+    if (epi < EPI_NONE || epi > EPI_ACCUM_BF16 || scale_mode < SCALE_TENSOR || scale_mode > SCALE_BLOCK)
         return CF_ERR_INVALID_ARG;
+    if (scale_mode == SCALE_BLOCK && (epi != EPI_NONE || fmt != 0)) return CF_ERR_UNSUPPORTED;
     if (epi == EPI_BIAS && !p.bias) return CF_ERR_INVALID_ARG;
     if (epi == EPI_SILU_GATE && (!p.B2 || !p.sb2)) return CF_ERR_INVALID_ARG;
     if (p.lda < p.K || p.ldb < p.K || p.ldc < p.N) return CF_ERR_INVALID_ARG;
@@ -652,6 +812,19 @@ int gemm_nt(GemmArgs p, int fmt, int epi, int scale_mode, int force_naive, cf_st
     if (force_naive || !tiled_ok) {
         const long long total = static_cast<long long>(p.M) * p.N;
         k_gemm_nt_naive<<<static_cast<unsigned>((total + 255) / 256), 256, 0, st>>>(p, fmt, epi, scale_mode);
+        return launch_status();
+    }
+    if (scale_mode == SCALE_BLOCK) {
+        static std::once_flag once;
+        static hipError_t attr_err = hipSuccess;
+        std::call_once(once, [] {
+            attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_nt_block),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, kBlkLds);
+        });
+        if (attr_err != hipSuccess) return static_cast<int>(attr_err);
+        p.tiles_m = (p.M + BSM - 1) / BSM;
+        p.tiles_n = (p.N + BN - 1) / BN;
+        k_gemm_nt_block<<<p.tiles_m * p.tiles_n, kThreads, kBlkLds, st>>>(p);
         return launch_status();
     }
     const int out_bn = epi == EPI_SILU_GATE ? BN / 2 : BN;

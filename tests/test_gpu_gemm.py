@@ -191,3 +191,164 @@ def test_gemm_argument_errors(cf, dev):
     assert cf.raw_cf_fp8_gemm_nt_bf16(1, 1, 16, None, 16, 0, s.data_ptr(), a.data_ptr(), s.data_ptr(), c.data_ptr(), 1, None) == -1
     assert cf.raw_cf_fp8_gemm_nt_bf16(1, 1, 16, a.data_ptr(), 8, 0, s.data_ptr(), a.data_ptr(), s.data_ptr(), c.data_ptr(), 1, None) == -1
     assert cf.raw_cf_fp8_gemm_nt_bf16(0, 1, 16, a.data_ptr(), 16, 0, s.data_ptr(), a.data_ptr(), s.data_ptr(), c.data_ptr(), 1, None) == 0
+
+
+# ---- backward-pass GEMMs (benchmark config 4) ------------------------------------------------
+def run_accum(cf, dev, A, B, sa, sb, C0, *, a_e5m2, b_e5m2, flags=0, bf16_out=False, ldc=None):
+    M, K = A.shape
+    N = B.shape[0]
+    ldc = N if ldc is None else ldc
+    s = lambda v: torch.tensor([v], dtype=torch.float32, device=dev)
+    if bf16_out:
+        C = dev_bf16(orc.bf16_from_f32(C0.astype(np.float32)), dev)
+        assert a_e5m2 is False and b_e5m2 is True
+        cf.cf_fp8_gemm_tn_accum_bf16(M, N, K, dev_arr(A, dev), s(sa), dev_arr(B, dev), s(sb), C, ldc, stream())
+        torch.cuda.synchronize()
+        return orc.bf16_to_f32(bf16_bits(C)).astype(np.float64)
+    C = torch.from_numpy(C0.astype(np.float32)).to(dev)
+    cf.cf_fp8_gemm_nt_accum_f32_ex(M, N, K, dev_arr(A, dev), K, int(a_e5m2), s(sa), dev_arr(B, dev), K, int(b_e5m2), s(sb),
+                                   C, ldc, flags, stream())
+    torch.cuda.synchronize()
+    return host(C).astype(np.float64)
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (300, 200, 384), (512, 1024, 2048), (130, 260, 80)])
+@pytest.mark.parametrize("flags", [0, NAIVE])
+def test_wgrad_tn_accumulate_f32(cf, dev, M, N, K, flags):
+    """dW[M,N] fp32 += X^T[M,K](E4M3) . dY^T[N,K](E5M2)^T, beta = 1 (lt_gemm_fp8_tn_accum_f32)."""
+    case(f"wgrad accumulate f32 {M}x{N}x{K} flags={flags}")
+    rng = np.random.default_rng(M + N + K + flags)
+    Xt, sx = rand_fp8(rng, (M, K))
+    dYt, sy = rand_fp8(rng, (N, K), e5m2=True, sigma=1e-3)
+    C0 = rng.standard_normal((M, N)) * 1e-3
+    ref, absdot = orc.gemm_nt_ref(Xt, dYt, [sx], [sy], b_e5m2=True)
+    got = run_accum(cf, dev, Xt, dYt, sx, sy, C0, a_e5m2=False, b_e5m2=True, flags=flags)
+    want = C0.astype(np.float32).astype(np.float64) + ref
+    # fp32 output: relative L2 against the unrounded reference, elementwise within the accumulation allowance
+    rel = np.sqrt(((got - want) ** 2).sum() / (want ** 2).sum())
+    assert rel <= 1e-3, rel
+    acc = orc.ACC_FP32 if flags else orc.ACC_MFMA
+    assert np.all(np.abs(got - want) <= acc * absdot + 2.0 ** -22 * (np.abs(want) + np.abs(C0)))
+    if flags == 0 and K % 128 == 0:
+        # the named entry point is the same kernel
+        C = torch.from_numpy(C0.astype(np.float32)).to(dev)
+        s = lambda v: torch.tensor([v], dtype=torch.float32, device=dev)
+        cf.cf_fp8_gemm_tn_accum_f32(M, N, K, dev_arr(Xt, dev), s(sx), dev_arr(dYt, dev), s(sy), C, N, stream())
+        torch.cuda.synchronize()
+        assert np.array_equal(host(C).astype(np.float64), got)
+
+
+def test_wgrad_tn_accumulate_bf16(cf, dev):
+    case("wgrad accumulate bf16")
+    rng = np.random.default_rng(77)
+    M, N, K = 300, 260, 512
+    Xt, sx = rand_fp8(rng, (M, K))
+    dYt, sy = rand_fp8(rng, (N, K), e5m2=True, sigma=1e-3)
+    ref, absdot = orc.gemm_nt_ref(Xt, dYt, [sx], [sy], b_e5m2=True)
+    C0 = rng.standard_normal((M, N)) * np.abs(ref).mean()
+    got = run_accum(cf, dev, Xt, dYt, sx, sy, C0, a_e5m2=False, b_e5m2=True, bf16_out=True)
+    want = orc.bf16_to_f32(orc.bf16_from_f32(C0.astype(np.float32))).astype(np.float64) + ref
+    assert np.all(np.abs(got - want) <= 1.01 * orc.bf16_ulp(want) / 2 + orc.ACC_MFMA * absdot)
+
+
+def test_config4_backward_shapes_sampled(cf, dev):
+    """dgrad: dY[8192,14336] E5M2 (per-tensor, ~N(0,1e-3)) . W[4096,14336] E4M3 -> bf16 [8192,4096];
+    wgrad: dY^T[14336... as X^T[14336,8192] E4M3 . dY^T[4096,8192] E5M2 accumulated into fp32 [14336,4096]."""
+    case("config 4 backward, full size")
+    g = torch.Generator(device=dev).manual_seed(4)
+    M, N, K = 8192, 4096, 14336
+    dy = (torch.randn((M, K), generator=g, device=dev) * 1e-3).to(torch.bfloat16)
+    w = (torch.randn((N, K), generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    sc = lambda: torch.zeros(1, device=dev)
+    amax, s_dy, d_dy, s_w, d_w = sc(), sc(), sc(), sc(), sc()
+    dyq = torch.empty((M, K), dtype=torch.uint8, device=dev); wq = torch.empty((N, K), dtype=torch.uint8, device=dev)
+    cf.cf_fp8_amax_bf16(dy, dy.numel(), amax, stream()); cf.cf_fp8_scale_from_amax(amax, 57344.0, s_dy, d_dy, stream())
+    cf.cf_fp8_quantize_e5m2(dy, dyq, s_dy, dy.numel(), stream())
+    cf.cf_fp8_amax_bf16(w, w.numel(), amax, stream()); cf.cf_fp8_scale_from_amax(amax, 448.0, s_w, d_w, stream())
+    cf.cf_fp8_quantize_e4m3(w, wq, s_w, w.numel(), stream())
+    dx = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+    cf.cf_fp8_gemm_nt_bf16(M, N, K, dyq, K, 1, d_dy, wq, d_w, dx, N, stream())
+    torch.cuda.synchronize()
+    assert host(amax)[0] > 0 and np.array_equal(host(dyq), orc.quantize_e5m2(bf16_bits(dy), host(s_dy)[0]))
+    rows = np.sort(np.random.default_rng(2).choice(M, 32, replace=False)); ridx = torch.from_numpy(rows).to(dev)
+    ref, absdot = orc.gemm_nt_ref(host(dyq[ridx]), host(wq), host(d_dy), host(d_w), a_e5m2=True)
+    orc.assert_gemm_close(orc.bf16_to_f32(bf16_bits(dx[ridx])).astype(np.float64), ref, absdot, what="config 4 dgrad")
+    del dx, w, wq
+    # wgrad: M=14336, N=4096, K=8192, both operands K-contiguous (pre-transposed); dY^T via the byte transpose
+    Mw, Nw, Kw = 14336, 4096, 8192
+    x = torch.randn((Kw, Mw), generator=g, device=dev).to(torch.bfloat16)          # swiglu_out [tokens, I]
+    s_x, d_x = sc(), sc()
+    cf.cf_fp8_amax_bf16(x, x.numel(), amax, stream()); cf.cf_fp8_scale_from_amax(amax, 448.0, s_x, d_x, stream())
+    act8 = torch.empty((Kw, Mw), dtype=torch.uint8, device=dev); snap = torch.empty((Mw, Kw), dtype=torch.uint8, device=dev)
+    cf.cf_fp8_quant_and_transpose_e4m3(x, act8, snap, s_x, Kw, Mw, stream())          # X^T [14336, 8192]
+    dyh = (torch.randn((Kw, Nw), generator=g, device=dev) * 1e-3).to(torch.bfloat16)  # dY [tokens, H]
+    cf.cf_fp8_amax_bf16(dyh, dyh.numel(), amax, stream()); cf.cf_fp8_scale_from_amax(amax, 57344.0, s_dy, d_dy, stream())
+    dyhq = torch.empty((Kw, Nw), dtype=torch.uint8, device=dev); dyt = torch.empty((Nw, Kw), dtype=torch.uint8, device=dev)
+    cf.cf_fp8_quantize_e5m2(dyh, dyhq, s_dy, dyh.numel(), stream())
+    cf.cf_transpose_u8(dyhq, dyt, Kw, Nw, stream())                                   # dY^T [4096, 8192]
+    dW = torch.full((Mw, Nw), 0.125, device=dev)
+    cf.cf_fp8_gemm_tn_accum_f32(Mw, Nw, Kw, snap, d_x, dyt, d_dy, dW, Nw, stream())
+    torch.cuda.synchronize()
+    assert torch.equal(snap, act8.t()) and torch.equal(dyt, dyhq.t())                 # the transposes are permutations
+    rows = np.sort(np.random.default_rng(3).choice(Mw, 32, replace=False)); ridx = torch.from_numpy(rows).to(dev)
+    ref, absdot = orc.gemm_nt_ref(host(snap[ridx]), host(dyt), host(d_x), host(d_dy), b_e5m2=True)
+    got = host(dW[ridx]).astype(np.float64)
+    want = 0.125 + ref
+    assert np.sqrt(((got - want) ** 2).sum() / (want ** 2).sum()) <= 1e-3
+    assert np.all(np.abs(got - want) <= orc.ACC_MFMA * absdot + 2.0 ** -22 * (np.abs(want) + 0.125))
+
+
+# ---- block-scaled GEMM (benchmark config 3) ----------------------------------------------------
+BLOCK = 2
+
+
+def block_quant_gpu(cf, dev, x_bf16, kind):
+    rows, K = x_bf16.shape
+    kb = (K + 127) // 128
+    q = torch.empty((rows, K), dtype=torch.uint8, device=dev)
+    shape = (rows, kb) if kind == "1x128" else ((rows + 127) // 128, kb)
+    s = torch.empty(shape, device=dev); d = torch.empty(shape, device=dev)
+    fn = cf.cf_fp8_quantize_block_1x128 if kind == "1x128" else cf.cf_fp8_quantize_block_128x128
+    fn(x_bf16, rows, K, q, s, d, stream())
+    return q, s, d
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 256, 128), (256, 256, 256), (300, 200, 384), (130, 260, 208), (64, 512, 1024)])
+@pytest.mark.parametrize("flags", [0, NAIVE])
+def test_gemm_block_scaled(cf, dev, M, N, K, flags):
+    case(f"gemm block-scaled {M}x{N}x{K} flags={flags}")
+    rng = np.random.default_rng(M * 3 + N + K)
+    xb = orc.bf16_from_f32((rng.standard_normal((M, K)) * np.exp(rng.standard_normal((M, 1)))).astype(np.float32))
+    wb = orc.bf16_from_f32((0.02 * rng.standard_normal((N, K))).astype(np.float32))
+    xq, xs, xd = block_quant_gpu(cf, dev, dev_bf16(xb, dev), "1x128")
+    wq, ws, wd = block_quant_gpu(cf, dev, dev_bf16(wb, dev), "128x128")
+    C = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=dev)
+    cf.cf_fp8_gemm_nt_bf16_ex(M, N, K, xq, K, 0, xd, wq, K, wd, BLOCK, EPI_NONE, None, None, None, C, N, flags, stream())
+    torch.cuda.synchronize()
+    # the quantized operands and scales are bit-exact (checked in the quantize tests); reference on the same bytes
+    oq, osx, odx = orc.quantize_block_1x128(xb)
+    assert np.array_equal(host(xq), oq) and np.array_equal(host(xd), odx)
+    ref, absdot = orc.gemm_nt_ref(host(xq), host(wq), host(xd), host(wd), scale_mode=2)
+    got = orc.bf16_to_f32(bf16_bits(C)).astype(np.float64)
+    orc.assert_gemm_close(got, ref, absdot, what=f"block {M}x{N}x{K}", acc=orc.ACC_FP32 * 4 if flags else orc.ACC_MFMA)
+
+
+def test_config3_block_scaled_full_size_sampled(cf, dev):
+    """M=4096, N=7168, K=7168; activations 1x128 groups, weights 128x128 blocks, fp32 scale tensors."""
+    case("config 3 block-scaled, full size")
+    M, N, K = 4096, 7168, 7168
+    g = torch.Generator(device=dev).manual_seed(3)
+    x = torch.randn((M, K), generator=g, device=dev).to(torch.bfloat16)
+    w = (torch.randn((N, K), generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    xq, xs, xd = block_quant_gpu(cf, dev, x, "1x128")
+    wq, ws, wd = block_quant_gpu(cf, dev, w, "128x128")
+    C = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+    cf.cf_fp8_gemm_nt_bf16_ex(M, N, K, xq, K, 0, xd, wq, K, wd, BLOCK, EPI_NONE, None, None, None, C, N, 0, stream())
+    torch.cuda.synchronize()
+    rows = np.sort(np.random.default_rng(6).choice(M, 24, replace=False)); ridx = torch.from_numpy(rows).to(dev)
+    ref, absdot = orc.gemm_nt_ref(host(xq[ridx]), host(wq), host(xd[ridx]), host(wd), scale_mode=2)
+    orc.assert_gemm_close(orc.bf16_to_f32(bf16_bits(C[ridx])).astype(np.float64), ref, absdot, what="config 3 sampled rows")
+    # weight block scales against the oracle on a few blocks
+    wb = bf16_bits(w[:256, :256])
+    oq, _, od = orc.quantize_block_128x128(wb)
+    assert np.array_equal(host(wq[:256, :256]), oq) and np.array_equal(host(wd[:2, :2]), od)

@@ -150,7 +150,13 @@ __device__ __forceinline__ float stable_sigmoid(float x) {
 }
 
 // ---- host-side launch helpers ----------------------------------------------
-inline hipStream_t as_stream(cf_stream_t s) { return static_cast<hipStream_t>(s); }
+// Every entry point converts its stream argument before it launches anything; that is also where an
+// error left behind by an earlier, unrelated runtime call of the process (an event query that was not
+// ready, say) is discarded, so that launch_status() reports this library's launches only.
+inline hipStream_t as_stream(cf_stream_t s) {
+    (void)hipGetLastError();
+    return static_cast<hipStream_t>(s);
+}
 inline int launch_status() {
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? CF_OK : static_cast<int>(e);

@@ -72,6 +72,10 @@ class Lib:
             raise RuntimeError(
                 f"{path} is missing: build the HIP library first (python -c 'import __graft_entry__ as g; g.build()'). "
                 "There is no CPU fallback.")
+        # PyTorch ships its own copy of the HIP runtime.  Whichever copy is loaded first serves the whole process
+        # (same SONAME), and a process must not end up with two: import torch first so the tensors this harness
+        # passes in and the kernels of the library share one runtime.
+        import torch  # noqa: F401
         self._dll = ctypes.CDLL(str(path))
         self.decls = parse_header()
         for name, (ret, args) in self.decls.items():

@@ -311,6 +311,54 @@ int cf_moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_fcin_
                                       int H, int Ie, int num_experts, int total_selected_rows,
                                       cf_stream_t stream);
 
+/* ---- slot state machines (host logic of src/trainer.cu over the entry points above) ------- */
+
+/* One delayed-scaling activation / gradient call site: ActSlot, src/trainer.cu:3247-3279.  The host
+ * object holds the flags (init, calib_remaining, calib_commit_pending, fp8_max); the device scalars
+ * (amax, scale, descale, the two snapshots, calib min/max, cursor, count, history) live in one
+ * caller-owned device block of cf_act_slot_state_words(history_len) 4-byte words. */
+typedef struct cf_act_slot cf_act_slot;
+
+/* words of device state one slot needs (alloc_act_slot, src/trainer.cu:4176-4201, allocates the same scalars) */
+int cf_act_slot_state_words(int history_len);
+
+/* alloc_act_slot, src/trainer.cu:4176-4201: history, cursor, count zeroed, calib_min = 0x7f7f7f7f,
+ * calib_max = 0.  history_len is kActHistoryLen (8, src/trainer.cu:3213) in the reference and 16 in
+ * benchmark config 3; calib_calls is IDA_FP8_CALIB_CALLS (default 8, src/trainer.cu:3765-3774),
+ * type_spread_threshold is IDA_FP8_TYPE_SPREAD (default 4, src/trainer.cu:3778-3787). */
+int cf_act_slot_create(cf_act_slot** out, void* d_state, int history_len, float fp8_max,
+                       int calib_calls, float type_spread_threshold, cf_stream_t stream);
+int cf_act_slot_destroy(cf_act_slot* slot);   /* frees the host object (src/trainer.cu:4176: slots die with the arena) */
+
+/* act_fp8_type, src/trainer.cu:4728-4730: 1 when the slot writes E5M2 */
+int cf_act_slot_is_e5m2(const cf_act_slot* slot);
+
+#define CF_SLOT_AMAX 0
+#define CF_SLOT_SCALE 1
+#define CF_SLOT_DESCALE 2
+#define CF_SLOT_SCALE_SNAPSHOT 3
+#define CF_SLOT_DESCALE_SNAPSHOT 4   /* what the GEMM consuming the quantized tensor dequantizes with, src/trainer.cu:6118-6122 */
+#define CF_SLOT_HISTORY 5
+#define CF_SLOT_CURSOR 6
+#define CF_SLOT_COUNT 7
+#define CF_SLOT_CALIB_MIN 8
+#define CF_SLOT_CALIB_MAX 9
+/* device address of one of the slot's scalars (the ActSlot members of src/trainer.cu:3248-3278) */
+int cf_act_slot_device_field(const cf_act_slot* slot, int field, void** d_ptr);
+
+/* fp8_quant_act, src/trainer.cu:4732-4851: recompute (snapshot scale, no side effects); pending
+ * calibration commit (host sync, may switch the slot to E5M2); calibration and first use (exact amax);
+ * steady state (previous scale, record amax, advance the history).  The clip-debug probes of
+ * src/trainer.cu:4834-4839 are separate entry points here. */
+int cf_fp8_quant_act(cf_act_slot* slot, const uint16_t* d_x, void* d_act8, size_t n,
+                     int is_recompute, cf_stream_t stream);
+
+/* One Fp8Slot of refresh_fp8_weights, src/trainer.cu:4694-4712: (optional amax) -> scale -> fwd8 [out,in]
+ * and bwd8 [in,out], one by direct quantize and one by quantize-transpose depending on how w is stored. */
+int cf_fp8_refresh_weight(const uint16_t* d_w, void* d_fwd8, void* d_bwd8, float* d_amax,
+                          float* d_scale, float* d_descale, int in_dim, int out_dim,
+                          int stored_out_major, int recompute_amax, cf_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

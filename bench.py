@@ -75,6 +75,9 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--traffic-calibration", action="store_true",
+                    help="also run a plain 1 GiB device copy, so a rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this "
+                         "command carries a kernel of known traffic to scale the counters by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; --gpus must be 1 (no multi-GPU path is built)")
@@ -136,6 +139,14 @@ def main():
         if timed:
             e[4].record()
             marks.append(e)
+
+    if args.traffic_calibration:
+        src = torch.full((1 << 30,), 7, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)          # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         step(False)

@@ -1,0 +1,28 @@
+// Compiles and links the C++ shim against libcf_fp8.so: takes the address of every forwarded function with the
+// reference's signature (over HIP types), and checks the error mapping without touching a GPU.
+#include "ida_native_hip/kernels.hpp"
+
+#include <cstdio>
+
+using namespace ida_native;
+
+int main() {
+    void (*f1)(const bf16*, std::size_t, float*, hipStream_t) = &fp8_amax_bf16;
+    void (*f2)(const float*, float, float*, float*, hipStream_t) = &fp8_scale_from_amax;
+    void (*f3)(const bf16*, void*, const float*, std::size_t, hipStream_t) = &fp8_quantize_e4m3;
+    void (*f4)(const bf16*, void*, const float*, float*, std::size_t, hipStream_t) = &fp8_quantize_e5m2_record;
+    void (*f5)(const float*, float, float*, float*, float*, int, int*, int*, hipStream_t) = &fp8_update_delayed_scale;
+    void (*f6)(const bf16*, void*, void*, const float*, int, int, hipStream_t) = &fp8_quant_and_transpose_e4m3;
+    void (*f7)(const bf16*, const bf16*, bf16*, int, hipStream_t) = &swiglu_forward;
+    void (*f8)(float*, int, int, int, hipStream_t, float*, float*, bool) = &moe_topk_route_f32;
+    void (*f9)(int, int, int, const void*, int, bool, const float*, const void*, const float*, bf16*, int, hipStream_t) = &lt_gemm_fp8_nt;
+    void (*f10)(int, int, int, const void*, const float*, const void*, const float*, float*, int, hipStream_t) = &lt_gemm_fp8_tn_accum_f32;
+    void (*f11)(int, int, int, const void*, const float*, const void*, const float*, bf16*, int, hipStream_t) = &lt_gemm_fp8_tn_accum_f32;
+    if (!f1 || !f2 || !f3 || !f4 || !f5 || !f6 || !f7 || !f8 || !f9 || !f10 || !f11) return 1;
+    int ok = 0;
+    try { swiglu_forward(nullptr, nullptr, nullptr, -1, nullptr); } catch (const std::invalid_argument&) { ++ok; }   // kernels/activations.cu:61-72
+    try { swiglu_forward(nullptr, nullptr, nullptr, 4, nullptr); } catch (const std::invalid_argument&) { ++ok; }
+    swiglu_forward(nullptr, nullptr, nullptr, 0, nullptr);                                                           // n == 0 is a no-op
+    std::printf("shim ok %d\n", ok);
+    return ok == 2 ? 0 : 2;
+}

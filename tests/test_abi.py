@@ -39,3 +39,16 @@ def test_argument_errors_do_not_need_a_gpu(cf):
     assert cf.raw_cf_fp8_quantize_e4m3(None, None, None, 0, None) == 0
     assert cf.raw_cf_fp8_quantize_e4m3(None, None, None, 8, None) == -1
     assert cf.raw_cf_fp8_quantize_rows(None, -1, 4, 0, None, None, None, None) == -1
+
+
+def test_cpp_shim_compiles_links_and_maps_errors(tmp_path):
+    """The header-only C++ shim keeps the reference's ida_native:: signatures over HIP types."""
+    import subprocess
+    exe = tmp_path / "shim_check"
+    lib_dir = ROOT / "canopy-foundry_amd"
+    cmd = ["g++", "-std=c++17", "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include", f"-I{ROOT / 'include'}",
+           str(ROOT / "tests" / "shim_compile_check.cpp"), "-o", str(exe), f"-L{lib_dir}", "-lcf_fp8",
+           f"-Wl,-rpath,{lib_dir}", "-Wl,-rpath,/opt/rocm/lib"]
+    subprocess.run(cmd, check=True, capture_output=True)
+    out = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert out.returncode == 0 and "shim ok 2" in out.stdout, out.stderr

@@ -54,6 +54,7 @@ struct GemmArgs {
     // grouped (per-expert) form, ring kernel only; all null / 0 for a dense GEMM
     const int* tile_map;         // [0] = number of row tiles, then (expert, first row, end row) per row tile
     const int* a_row_index;      // compact row r reads A row (and its descale) a_row_index[r]; null = r
+    int a_rows;                  // rows of the A buffer (= M without a row index)
     long long b_expert_stride;   // bytes between the weight matrices of consecutive experts
     int sb_expert_stride;        // elements between the channel descales of consecutive experts
 };
@@ -459,23 +460,36 @@ void k_gemm_nt_block(const GemmArgs p) {
 }
 
 // ---- ring kernel: direct-to-LDS copies into five 32 KiB slots --------------------------------
-// Needs K % 128 == 0 and K >= 256.  global_load_lds_dwordx4 copies 16 bytes per lane from global
-// memory straight into LDS (lane l lands at base + 16*l): no staging registers, and eight lanes
-// fetch one full 128-byte line of a row (half-line requests reach only ~60% of the L2 rate).
+// Needs K % 128 == 0, K >= 256 and operands smaller than 4 GiB.  global_load_lds_dwordx4 copies
+// 16 bytes per lane from global memory straight into LDS (lane l lands at base + 16*l): no staging
+// registers, and eight lanes fetch one full 128-byte line of a row (half-line requests reach only
+// ~60% of the L2 rate).  The copies take a uniform 64-bit base (operand + K offset, scalar registers)
+// plus a 32-bit per-lane byte offset, so advancing along K costs two scalar adds per K-tile.
 // A slot holds one operand tile [256 rows][128 bytes], chunks xor-swizzled as in the staged kernel.
 // Operand tile i (X of K-tile i/2 for even i, W for odd i) lives in slot i % 5, so while K-tile kt is
 // being multiplied, K-tile kt+1 is resident or landing and the X half of kt+2 is already on its way.
+// The five slot offsets are carried as a rotating set of scalars (no division in the loop).
 //
 // A K-tile is two MFMA steps (k-halves of 64).  Step (kt,0): 16 MFMAs, the operand reads of (kt,1),
 // the 8 copies of X(kt+2).  Step (kt,1): 2 MFMAs, wait for K-tile kt+1, barrier, 14 MFMAs woven
 // with the operand reads of (kt+1,0) and the 8 copies of W(kt+2).  One barrier per 2048 MFMA cycles;
-// a copy has two to three steps (2000-3000 cycles) to land.
+// a copy has two to three steps (2000-3000 cycles) to land.  With one wavefront per SIMD an
+// instruction issues every four cycles at best, so everything between two MFMAs (64 cycles) is kept
+// to a handful of instructions.
 constexpr int kSlotBytes = BM * BK;               // 32 KiB
 constexpr int kSlots = 5;
 constexpr int kRingLds = kSlots * kSlotBytes;     // 160 KiB: all of a CU's LDS
 
 // s_waitcnt immediates: vmcnt in bits [3:0] and [15:14], expcnt [6:4] and lgkmcnt [11:8] left at no-wait
 constexpr int kWaitVm0 = 0x0f70, kWaitVm8 = 0x0f78, kWaitVm16 = 0x4f70;
+
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
 
 template <int OUT_BN>
 __device__ __forceinline__ TilePos locate_tile(const GemmArgs& p, int pos) {
@@ -501,59 +515,195 @@ __device__ __forceinline__ TilePos locate_tile(const GemmArgs& p, int pos) {
     return t;
 }
 
+// Drain of a tile.  A unit is 32 output columns: one accumulator column of the wavefront (gate and up
+// accumulators of the same columns for the SiLU-gate epilogue).  TileScales holds what the drain needs in
+// registers: the descales of this lane's four output rows, and the channel descales of the unit being
+// drained (cs[g] = the four consecutive columns of accumulator quad g); the next unit's are fetched while
+// the current one is drained, the first unit's while the tile's last MFMAs run.
+template <int EPI>
+struct TileScales {
+    float sa[4];
+    float4 cs[4];
+    float4 cs2[4];
+};
+
+template <int EPI, int SCALE>
+__device__ __forceinline__ void load_row_scales(TileScales<EPI>& s, const GemmArgs& p, const TilePos& t, int wm, int lane) {
+    if constexpr (SCALE == SCALE_ROWCOL) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const int r = min(t.m0 + wm * 128 + b * 32 + (lane & 31), t.m_end - 1);
+            s.sa[b] = p.sa[p.a_row_index ? p.a_row_index[r] : r];
+        }
+    }
+}
+template <int EPI, int SCALE>
+__device__ __forceinline__ void load_unit_scales(float4 (&cs)[4], float4 (&cs2)[4], const GemmArgs& p, const TilePos& t,
+                                                 int wn, int lane, int unit) {
+    constexpr int NT = EPI == EPI_SILU_GATE ? 2 : 4;
+    if constexpr (SCALE == SCALE_ROWCOL) {
+        // uniform base (scalar registers) + a small per-lane byte offset: no 64-bit per-lane addresses to keep alive
+        const size_t ucol = static_cast<size_t>(t.expert) * p.sb_expert_stride + t.n0 + wn * (NT * 32) + unit * 32;
+        const uint8_t* b1 = reinterpret_cast<const uint8_t*>(p.sb + ucol);
+        const uint8_t* b2 = reinterpret_cast<const uint8_t*>(EPI == EPI_SILU_GATE ? p.sb2 + ucol : p.sb);
+        const uint32_t loff = static_cast<uint32_t>(lane >> 5) * 16u;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            cs[g] = *reinterpret_cast<const float4*>(b1 + (loff + g * 32u));
+            if constexpr (EPI == EPI_SILU_GATE) cs2[g] = *reinterpret_cast<const float4*>(b2 + (loff + g * 32u));
+        }
+    }
+}
+
+// An accumulator element as a VALU operand.  The explicit AGPR read keeps the register allocator from
+// moving whole accumulator tiles into VGPRs (and from there to scratch) around the drain.
+__device__ __forceinline__ float acc_read(float a) {
+    float v;
+    asm("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
+    return v;
+}
+
+// Per unit the wavefront scales its accumulators, applies the epilogue, rounds to bf16 and parks the
+// 128 rows x 64 bytes in its own 8 KiB of a free ring slot (16-byte chunks xor-swizzled by row: two-pass
+// ds_write_b64, conflict-free ds_read_b128), then streams them out 16 bytes per lane, four lanes per
+// row, so that every store instruction writes whole 64-byte half lines.  Rows at or beyond t.m_end are
+// not stored.
+template <int EPI, int SCALE>
+__device__ __forceinline__ void drain_tile(v16f (&acc)[4][4], TileScales<EPI>& s, float s1, float s2, const GemmArgs& p,
+                                           const TilePos& t, int wm, int wn, int lane, uint8_t* stage) {
+    constexpr bool GATE = EPI == EPI_SILU_GATE;
+    constexpr int NT = GATE ? 2 : 4;
+    const int row = lane & 31, khalf = lane >> 5;
+    uint8_t* wr = stage + row * 64 + khalf * 8;
+    const int wswz = (row >> 2) & 3;
+    const int rr = lane >> 2, rc = lane & 3;
+    const uint8_t* rdp = stage + rr * 64 + ((rc ^ ((rr >> 2) & 3)) << 4);
+    const int mrow0 = t.m0 + wm * 128 + rr;
+    // stores: uniform base per unit and 16-row group (scalar registers) + this lane's byte offset
+    uint8_t* cu = reinterpret_cast<uint8_t*>(p.C + static_cast<size_t>(t.m0 + wm * 128) * p.ldc + t.n0 + wn * (NT * 32));
+    const uint32_t coff = (static_cast<uint32_t>(rr) * static_cast<uint32_t>(p.ldc) + rc * 8u) * 2u;
+    const size_t cstep = static_cast<size_t>(p.ldc) * 32;      // bytes between 16-row groups
+
+#pragma unroll
+    for (int unit = 0; unit < NT; ++unit) {
+        float4 ncs[4], ncs2[4];
+        if (unit + 1 < NT) load_unit_scales<EPI, SCALE>(ncs, ncs2, p, t, wn, lane, unit + 1);
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const float sa = SCALE == SCALE_ROWCOL ? s.sa[b] : 1.0f;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                float4 c = make_float4(s1, s1, s1, s1), u = make_float4(s2, s2, s2, s2);
+                if constexpr (SCALE == SCALE_ROWCOL) {
+                    c = s.cs[g];
+                    if constexpr (GATE) u = s.cs2[g];
+                }
+                const float c4[4] = {c.x, c.y, c.z, c.w}, u4[4] = {u.x, u.y, u.z, u.w};
+                float v[4];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    if constexpr (GATE) {
+                        // the reference rounds gate and up to bf16 before the SiLU product
+                        const float gate = round_bf16_hw(acc_read(acc[2 * unit][b][g * 4 + q]) * (sa * c4[q]));
+                        const float up = round_bf16_hw(acc_read(acc[2 * unit + 1][b][g * 4 + q]) * (sa * u4[q]));
+                        v[q] = fast_silu(gate) * up;
+                    } else {
+                        v[q] = acc_read(acc[unit][b][g * 4 + q]) * (sa * c4[q]);
+                    }
+                }
+                *reinterpret_cast<uint2*>(wr + b * 32 * 64 + ((g ^ wswz) << 4)) =
+                    make_uint2(pack_bf16x2_hw(v[0], v[1]), pack_bf16x2_hw(v[2], v[3]));
+            }
+            __builtin_amdgcn_sched_barrier(0);     // one accumulator (pair) in flight at a time: keeps the drain in few registers
+        }
+        // Stores and copies share one completion counter, and a wait on copies issued after these stores
+        // would have to sit out the whole burst.  So the K-tile still landing is waited for here, where it
+        // costs next to nothing (its copies are older than a unit's worth of drain work), and the tile
+        // that follows skips the wait of its first K-tile: the stores then have two K-tiles to complete.
+        if (unit == 0) __builtin_amdgcn_s_waitcnt(kWaitVm0);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint4 v = *reinterpret_cast<const uint4*>(rdp + i * 16 * 64);
+            if (mrow0 + i * 16 < t.m_end)
+                *reinterpret_cast<uint4*>(cu + (i * cstep + unit * 64) + coff) = v;
+        }
+        if (unit + 1 < NT) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) { s.cs[g] = ncs[g]; s.cs2[g] = ncs2[g]; }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
 // The kernel is persistent: workgroup w walks tiles w, w + grid, w + 2*grid, ... of the XCD-aware
 // order, and the copy stream simply runs on into the next tile, so only a workgroup's very first
-// K-tiles pay memory latency; the epilogue of one tile runs while the next tile's first two K-tiles land.
+// K-tiles pay memory latency.  A tile's first MFMAs take a zero C operand (no accumulator clearing),
+// its scale factors are fetched under its last MFMAs, and its drain runs while the next tile's first
+// two K-tiles land.
 template <int FMT, int EPI, int SCALE>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void k_gemm_nt_ring(const GemmArgs p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
-    constexpr int OUT_BN = EPI == EPI_SILU_GATE ? BN / 2 : BN;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    constexpr bool GATE = EPI == EPI_SILU_GATE;
+    constexpr int OUT_BN = GATE ? BN / 2 : BN;
+    // the LDS-staged drain covers these epilogues; the launcher sends such a call here only when N is a multiple
+    // of the tile's output width and C and the channel descales allow 16-byte accesses
+    constexpr bool DRAIN = EPI == EPI_NONE || EPI == EPI_SILU_GATE;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
     const int total_tiles = (p.tile_map ? p.tile_map[0] : p.tiles_m) * p.tiles_n;
     const int my_tiles = (total_tiles - static_cast<int>(blockIdx.x) + static_cast<int>(gridDim.x) - 1) / static_cast<int>(gridDim.x);
     if (my_tiles <= 0) return;        // grouped launches size the grid by an upper bound of the tile count
     const int ktiles = p.K / BK;      // >= 2, checked by the launcher
-    const int total_g = my_tiles * ktiles;          // K-tiles this workgroup multiplies, over all its tiles
+
+    float s1 = 0.0f, s2 = 0.0f;
+    if constexpr (SCALE == SCALE_TENSOR && DRAIN) {
+        s1 = p.sa[0] * p.sb[0];
+        if constexpr (GATE) s2 = p.sa[0] * p.sb2[0];
+    }
 
     // ---- global -> LDS: wave w copies rows [64w, 64w+64) of an operand tile, 8 rows per instruction ----
     const int lrow = lane >> 3, lslot = lane & 7;
-    const uint8_t* xsrc[8];
-    const uint8_t* wsrc[8];
-    auto aim = [&](int seq) {                        // point the copy stream at this workgroup's seq-th tile
+    uint32_t xoff[8], woff[8];                         // per-lane byte offsets from the operand bases
+    const uint8_t* wb = p.B;                           // weight bases of the tile the copy stream is aimed at
+    const uint8_t* wb2 = p.B2;
+    auto aim = [&](int seq) {                          // point the copy stream at this workgroup's seq-th tile
         const TilePos t = locate_tile<OUT_BN>(p, blockIdx.x + seq * gridDim.x);
-        const uint8_t* wbase = p.B + t.expert * p.b_expert_stride;
-        const uint8_t* wbase2 = EPI == EPI_SILU_GATE ? p.B2 + t.expert * p.b_expert_stride : nullptr;
+        wb = p.B + t.expert * p.b_expert_stride;
+        if constexpr (GATE) wb2 = p.B2 + t.expert * p.b_expert_stride;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int row = wave * 64 + j * 8 + lrow;
-            const int gchunk = (lslot ^ swz(row)) * 16;
+            const uint32_t gchunk = (lslot ^ swz(row)) * 16;
             int arow = min(t.m0 + row, t.m_end - 1);
             if (p.a_row_index) arow = p.a_row_index[arow];
-            xsrc[j] = p.A + static_cast<size_t>(arow) * p.lda + gchunk;
-            if constexpr (EPI == EPI_SILU_GATE) {
-                // LDS weight rows of a wave: [gate 32 | up 32 | gate 32 | up 32] over the same 64 output columns
-                const int tt = (row >> 5) & 3, w = row >> 7;
-                const int n = t.n0 + w * 64 + (tt >> 1) * 32 + (row & 31);
-                wsrc[j] = ((tt & 1) ? wbase2 : wbase) + static_cast<size_t>(min(n, p.N - 1)) * p.ldb + gchunk;
-            } else {
-                wsrc[j] = wbase + static_cast<size_t>(min(t.n0 + row, p.N - 1)) * p.ldb + gchunk;
+            xoff[j] = static_cast<uint32_t>(arow) * static_cast<uint32_t>(p.lda) + gchunk;
+            int n = t.n0 + row;
+            if constexpr (GATE) {
+                // LDS weight rows of a wave: [gate 32 | up 32 | gate 32 | up 32] over the same 64 output columns;
+                // copies j < 4 of a wave read the gate matrix, j >= 4 the up matrix
+                n = t.n0 + (row >> 7) * 64 + ((row >> 6) & 1) * 32 + (row & 31);
             }
+            woff[j] = static_cast<uint32_t>(min(n, p.N - 1)) * static_cast<uint32_t>(p.ldb) + gchunk;
         }
     };
     // The copies are issued through inline assembly: the compiler cannot tell that an LDS-DMA write
     // and a later LDS read touch different slots, and would wait for every outstanding copy before
     // each operand read.  Their completion is tracked by hand with s_waitcnt vmcnt before the barriers.
-    const uint32_t lds_wave = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(smem)) +
-                              __builtin_amdgcn_readfirstlane(wave) * (64 * BK);
-    // copy instruction j (0..7) of operand tile `op` (2*g for X, 2*g+1 for W of K-tile g of the stream),
-    // reading K offset k0 of the tile the stream is aimed at
-    auto dma_one = [&](int op, int k0, int j) {
-        const uint32_t dst = lds_wave + (op % kSlots) * kSlotBytes + j * 8 * BK;
-        const uint8_t* src = (op & 1) ? wsrc[j] + k0 : xsrc[j] + k0;
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(dst), "v"(src) : "memory");
+    uint32_t lds_wave = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(smem)) + wave * (64 * BK);
+    // copy instruction J (0..7) of an operand tile into the ring slot at byte offset `slot`
+    auto dma = [&](int slot, uint32_t voff, const uint8_t* base, auto jc) {
+        constexpr int J = decltype(jc)::value;
+        const uint32_t dst = lds_wave + slot;
+        asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3"
+                     :: "s"(dst), "n"(J * 8 * BK), "v"(voff), "s"(base) : "memory", "scc");
+    };
+    auto dma_x = [&](int slot, int k0, auto jc) { dma(slot, xoff[decltype(jc)::value], p.A + k0, jc); };
+    auto dma_w = [&](int slot, int k0, auto jc) {
+        constexpr int J = decltype(jc)::value;
+        dma(slot, woff[J], ((GATE && J >= 4) ? wb2 : wb) + k0, jc);
     };
 
     // ---- LDS -> MFMA operands ----
@@ -567,120 +717,128 @@ void k_gemm_nt_ring(const GemmArgs p) {
     const uint8_t* wrd = smem + wn * 128 * BK;
 
     v16f acc[4][4];
-    auto zero_acc = [&]() {
-#pragma unroll
-        for (int a = 0; a < 4; ++a)
-#pragma unroll
-            for (int b = 0; b < 4; ++b)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
-    };
-    zero_acc();
-
     // operand registers, two sets: k-half h of any K-tile lives in set h
     v8i wq[2][4], xq[2][4];
     auto put = [](v8i& dst, int half, const uint4 v) {
         dst[4 * half + 0] = (int)v.x; dst[4 * half + 1] = (int)v.y; dst[4 * half + 2] = (int)v.z; dst[4 * half + 3] = (int)v.w;
     };
-    // the 16 reads of (g, h) in the order its MFMAs need them: w0 x0 x1 x2 x3 w1 w2 w3, two reads each
-    auto read_one = [&](int g, int h, int i) {
-        const int xoff = ((2 * g) % kSlots) * kSlotBytes, woff = ((2 * g + 1) % kSlots) * kSlotBytes;
-        const int t = i >> 1, half = i & 1;
-        const int r = rd[h][half];
-        if (t == 0)      put(wq[h][0], half, *reinterpret_cast<const uint4*>(wrd + woff + r));
-        else if (t <= 4) put(xq[h][t - 1], half, *reinterpret_cast<const uint4*>(xrd + xoff + (t - 1) * 32 * BK + r));
-        else             put(wq[h][t - 4], half, *reinterpret_cast<const uint4*>(wrd + woff + (t - 4) * 32 * BK + r));
+    // read I (0..15) of k-half H from the X tile in slot sx and the W tile in slot sw, in the order the
+    // MFMAs need them: w0 x0 x1 x2 x3 w1 w2 w3, two reads each
+    auto read_one = [&](int sx, int sw, auto hc, auto ic) {
+        constexpr int H = decltype(hc)::value, I = decltype(ic)::value;
+        constexpr int t = I >> 1, half = I & 1;
+        const int r = rd[H][half];
+        if constexpr (t == 0)      put(wq[H][0], half, *reinterpret_cast<const uint4*>(wrd + sw + r));
+        else if constexpr (t <= 4) put(xq[H][t - 1], half, *reinterpret_cast<const uint4*>(xrd + sx + (t - 1) * 32 * BK + r));
+        else                       put(wq[H][t - 4], half, *reinterpret_cast<const uint4*>(wrd + sw + (t - 4) * 32 * BK + r));
     };
-    auto mfma_one = [&](int h, int i) {
-        const int a = i >> 2, b = i & 3;
-        acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wq[h][a], xq[h][b], acc[a][b],
-                                                                     (FMT >> 1) & 1, FMT & 1, 0, 0, 0, 0);
-    };
-
-    // prologue: K-tiles 0 and 1 of the stream in flight, tile 0 landed and visible, operands (0,0) in set 0
-    aim(0);
+    auto mfma_one = [&](auto hc, auto ic, auto first_c) {
+        constexpr int H = decltype(hc)::value, I = decltype(ic)::value;
+        constexpr int a = I >> 2, b = I & 3;
+        v16f c = acc[a][b];
+        if constexpr (decltype(first_c)::value != 0) {
 #pragma unroll
-    for (int op = 0; op < 4; ++op)
-#pragma unroll
-        for (int j = 0; j < 8; ++j) dma_one(op, (op >> 1) * BK, j);
-    __builtin_amdgcn_s_waitcnt(kWaitVm16);
-    __syncthreads();
-#pragma unroll
-    for (int i = 0; i < 16; ++i) read_one(0, 0, i);
-
-    // step (g,0): no synchronisation; COPY: start X of stream K-tile g+2 (tile-local K offset dk0)
-    auto step0 = [&](int g, int dk0, auto copy_c) {
-        constexpr bool COPY = decltype(copy_c)::value != 0;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            mfma_one(0, i);
-            read_one(g, 1, i);
-            if constexpr (COPY) {
-                if (i >= 2 && i < 10) dma_one(2 * g + 4, dk0, i - 2);
-            }
-            __builtin_amdgcn_sched_barrier(0);
+            for (int r = 0; r < 16; ++r) c[r] = 0.0f;
         }
-    };
-    // step (g,1).  MODE 0: steady (X(g+2) stays in flight, start W(g+2)); MODE 1: K-tile g+1 is the
-    // last of the stream (nothing else in flight, no copies); MODE 2: g is the last K-tile (MFMAs only).
-    auto step1 = [&](int g, int dk0, auto mode_c) {
-        constexpr int MODE = decltype(mode_c)::value;
-        mfma_one(1, 0);
-        mfma_one(1, 1);
-        __builtin_amdgcn_sched_barrier(0);
-        if constexpr (MODE != 2) {
-            __builtin_amdgcn_s_waitcnt(MODE == 0 ? kWaitVm8 : kWaitVm0);
-            __syncthreads();
-            __builtin_amdgcn_sched_barrier(0);
-        }
-#pragma unroll
-        for (int i = 2; i < 16; ++i) {
-            mfma_one(1, i);
-            if constexpr (MODE != 2) {
-                read_one(g + 1, 0, i - 2);
-                if (i >= 14) read_one(g + 1, 0, i);               // reads 14 and 15 ride with the last two MFMAs
-            }
-            if constexpr (MODE == 0) {
-                if (i >= 4 && i < 12) dma_one(2 * g + 5, dk0, i - 4);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
+        acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wq[H][a], xq[H][b], c, (FMT >> 1) & 1, FMT & 1, 0, 0, 0, 0);
     };
     using C0 = std::integral_constant<int, 0>;
     using C1 = std::integral_constant<int, 1>;
-    using C2 = std::integral_constant<int, 2>;
 
-    // copy position: two K-tiles ahead of the compute position (ktiles >= 2, so at most one tile ahead)
+    // ring slots (byte offsets) of the operand tiles around the current K-tile g:
+    // a0 = X(g), a1 = W(g), a2 = X(g+1), a3 = W(g+1), a4 = the slot X(g+2) is copied into; W(g+2) goes into a0
+    int a0 = 0, a1 = kSlotBytes, a2 = 2 * kSlotBytes, a3 = 3 * kSlotBytes, a4 = 4 * kSlotBytes;
+
+    TileScales<EPI> sc;
+
+    // One K-tile g: X(g+2) and W(g+2) are started, K-tile g+1 is waited for (unless `wait` is false: then it
+    // is known to have landed) and made visible by the barrier.  FIRST: the tile's first K-tile (zero C
+    // operand).  END: the tile's last K-tile: the operands of the next tile are read after the drain, and
+    // the drain's first scale factors are fetched here instead.
+    auto ktile = [&](auto first_c, auto end_c, int dk0, const TilePos& t, bool wait) {
+        constexpr bool END = decltype(end_c)::value != 0;
+        // step (g,0)
+        static_for<0, 16>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            mfma_one(C0{}, ic, first_c);
+            read_one(a0, a1, C1{}, ic);
+            if constexpr (i >= 2 && i < 10) dma_x(a4, dk0, std::integral_constant<int, (i >= 2 && i < 10) ? i - 2 : 0>{});
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        // step (g,1)
+        mfma_one(C1{}, C0{}, C0{});
+        mfma_one(C1{}, C1{}, C0{});
+        __builtin_amdgcn_sched_barrier(0);
+        if (wait) __builtin_amdgcn_s_waitcnt(kWaitVm8);
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<2, 16>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            mfma_one(C1{}, ic, C0{});
+            if constexpr (!END) {
+                read_one(a2, a3, C0{}, std::integral_constant<int, i - 2>{});
+                if constexpr (i >= 14) read_one(a2, a3, C0{}, ic);       // reads 14 and 15 ride with the last two MFMAs
+            }
+            if constexpr (i >= 2 && i < 10) dma_w(a0, dk0, std::integral_constant<int, (i >= 2 && i < 10) ? i - 2 : 0>{});
+            if constexpr (END && DRAIN && i == 10) {
+                load_row_scales<EPI, SCALE>(sc, p, t, wm, lane);
+                load_unit_scales<EPI, SCALE>(sc.cs, sc.cs2, p, t, wn, lane, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+    auto rotate = [&]() {
+        const int b0 = a0, b1 = a1;
+        a0 = a2; a1 = a3; a2 = a4; a3 = b0; a4 = b1;
+    };
+
+    // prologue: K-tiles 0 and 1 of the stream in flight, K-tile 0 landed and visible, operands (0,0) in set 0
+    aim(0);
+    static_for<0, 8>([&](auto jc) { dma_x(a0, 0, jc); });
+    static_for<0, 8>([&](auto jc) { dma_w(a1, 0, jc); });
+    static_for<0, 8>([&](auto jc) { dma_x(a2, BK, jc); });
+    static_for<0, 8>([&](auto jc) { dma_w(a3, BK, jc); });
+    __builtin_amdgcn_s_waitcnt(kWaitVm16);
+    __syncthreads();
+    static_for<0, 16>([&](auto ic) { read_one(a0, a1, C0{}, ic); });
+
+    // Copy position: two K-tiles ahead of the compute position (ktiles >= 2, so at most one tile ahead).
+    // Past the workgroup's last tile the stream simply re-reads that tile: the last two K-tiles then run
+    // the same code as every other one, and what they copy is never used.
     int dkt = 2 % ktiles, dseq = 2 / ktiles;
     if (dseq == 1 && my_tiles > 1) aim(1);
-    int g = 0;                                     // K-tile index in this workgroup's stream
+    auto advance_copy = [&]() {
+        if (++dkt == ktiles) {                   // the stream moves on to the next tile
+            dkt = 0;
+            if (++dseq < my_tiles) aim(dseq);
+        }
+    };
+
     for (int seq = 0; seq < my_tiles; ++seq) {
-        const bool last_tile = seq + 1 == my_tiles;
-        const int steady = last_tile ? ktiles - 2 : ktiles;
-        for (int kt = 0; kt < steady; ++kt, ++g) {
-            step0(g, dkt * BK, C1{});
-            step1(g, dkt * BK, C0{});
-            if (++dkt == ktiles) {               // the stream moves on to the next tile
-                dkt = 0;
-                if (++dseq < my_tiles) aim(dseq);
-            }
-        }
-        if (last_tile) {
-            step0(g, 0, C0{});
-            step1(g, 0, C1{});
-            step0(g + 1, 0, C0{});
-            step1(g + 1, 0, C2{});
-        }
         const TilePos t = locate_tile<OUT_BN>(p, blockIdx.x + seq * gridDim.x);
-        GemmArgs q = p;                        // the epilogue sees this tile's row bound and this expert's channel scales
-        q.M = t.m_end;
-        if (SCALE == SCALE_ROWCOL) {
-            q.sb += static_cast<size_t>(t.expert) * p.sb_expert_stride;
-            if (EPI == EPI_SILU_GATE) q.sb2 += static_cast<size_t>(t.expert) * p.sb_expert_stride;
+        // after a drain the first K-tile's successor has been waited for already
+        ktile(C1{}, C0{}, dkt * BK, t, !(DRAIN && seq > 0));
+        rotate(); advance_copy();
+        for (int kt = 1; kt + 1 < ktiles; ++kt) {
+            ktile(C0{}, C0{}, dkt * BK, t, true);
+            rotate(); advance_copy();
         }
-        epilogue<EPI, SCALE>(acc, q, t.m0, t.n0, wm, wn, lane);
-        zero_acc();
+        ktile(C0{}, C1{}, dkt * BK, t, true);
+        rotate(); advance_copy();
+        // After the rotation a4 is the slot that held W of the K-tile just finished.  Every wavefront has
+        // finished reading it (barrier of the last step) and only X of the stream's third K-tile from here
+        // is copied into it next, by this wavefront's own copies, in program order after the drain.
+        if constexpr (DRAIN) {
+            drain_tile<EPI, SCALE>(acc, sc, s1, s2, p, t, wm, wn, lane, smem + a4 + wave * (64 * BK));
+        } else {
+            GemmArgs q = p;                        // the epilogue sees this tile's row bound
+            q.M = t.m_end;
+            epilogue<EPI, SCALE>(acc, q, t.m0, t.n0, wm, wn, lane);
+        }
+        static_for<0, 16>([&](auto ic) { read_one(a0, a1, C0{}, ic); });
     }
+    // the copies started past the end of the stream must have landed before the LDS is given back
+    __builtin_amdgcn_s_waitcnt(kWaitVm0);
 }
 
 // ---- naive kernel: any shape, any alignment; also the on-device cross-check ----
@@ -745,7 +903,17 @@ int launch_tiled(const GemmArgs& p, hipStream_t st) {
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
     });
     if (attr_err != hipSuccess) return static_cast<int>(attr_err);
-    if (p.K % BK == 0 && p.K >= 2 * BK && !p.force_staged) {
+    // the ring kernel addresses operand rows by 32-bit byte offsets
+    bool ring_ok = p.K % BK == 0 && p.K >= 2 * BK && static_cast<size_t>(p.a_rows) * p.lda < (1ull << 32) &&
+                   static_cast<size_t>(p.N) * p.ldb < (1ull << 32);
+    if constexpr (EPI == EPI_NONE || EPI == EPI_SILU_GATE) {
+        // its drain writes full-width tiles with 16-byte stores and reads the channel descales as float4
+        constexpr int out_bn = EPI == EPI_SILU_GATE ? BN / 2 : BN;
+        ring_ok = ring_ok && p.N % out_bn == 0 && p.ldc % 8 == 0 && aligned16(p.C);
+        if (SCALE == SCALE_ROWCOL)
+            ring_ok = ring_ok && aligned16(p.sb) && p.sb_expert_stride % 4 == 0 && (EPI != EPI_SILU_GATE || aligned16(p.sb2));
+    }
+    if (ring_ok && !p.force_staged) {
         static std::once_flag once_ring;
         static hipError_t ring_err = hipSuccess;
         std::call_once(once_ring, [] {
@@ -807,6 +975,7 @@ int gemm_nt(GemmArgs p, int fmt, int epi, int scale_mode, int force_naive, cf_st
     if (epi == EPI_SILU_GATE && (!p.B2 || !p.sb2)) return CF_ERR_INVALID_ARG;
     if (p.lda < p.K || p.ldb < p.K || p.ldc < p.N) return CF_ERR_INVALID_ARG;
     hipStream_t st = as_stream(stream);
+    p.a_rows = p.M;
     const bool tiled_ok = p.K > 0 && p.K % 16 == 0 && p.lda % 16 == 0 && p.ldb % 16 == 0 && aligned16(p.A) &&
                           aligned16(p.B) && (epi != EPI_SILU_GATE || aligned16(p.B2));
     if (force_naive || !tiled_ok) {
@@ -912,11 +1081,11 @@ int cf_fp8_grouped_gemm_workspace_bytes(int total_rows, int num_experts, size_t*
 }
 
 int cf_fp8_grouped_gemm_nt_bf16_ex(int total_rows, int N, int K, int num_experts, const int* d_counts,
-                                   const int* d_offsets, const void* A, int lda, const int* d_a_row_index,
+                                   const int* d_offsets, const void* A, int a_rows, int lda, const int* d_a_row_index,
                                    const float* a_descale, const void* B, const float* b_descale, int scale_mode,
                                    int epilogue, const void* B_up, const float* b_up_descale, uint16_t* C, int ldc,
                                    void* d_workspace, size_t workspace_bytes, cf_stream_t stream) {
-    if (total_rows < 0 || N < 0 || K < 0 || num_experts < 0) return CF_ERR_INVALID_ARG;
+    if (total_rows < 0 || N < 0 || K < 0 || num_experts < 0 || a_rows < 0) return CF_ERR_INVALID_ARG;
     if (total_rows == 0 || N == 0 || num_experts == 0) return CF_OK;
     if (!d_counts || !d_offsets || !A || !B || !C || !a_descale || !b_descale || !d_workspace) return CF_ERR_INVALID_ARG;
     if (epilogue != EPI_NONE && epilogue != EPI_SILU_GATE) return CF_ERR_INVALID_ARG;
@@ -927,7 +1096,10 @@ int cf_fp8_grouped_gemm_nt_bf16_ex(int total_rows, int N, int K, int num_experts
     if (workspace_bytes < need || (reinterpret_cast<uintptr_t>(d_workspace) & 3u)) return CF_ERR_INVALID_ARG;
     // the grouped form runs on the ring kernel only
     if (K % BK != 0 || K < 2 * BK || lda % 16 != 0 || !aligned16(A) || !aligned16(B) ||
-        (epilogue == EPI_SILU_GATE && !aligned16(B_up)) || lda < K || ldc < N)
+        (epilogue == EPI_SILU_GATE && !aligned16(B_up)) || lda < K || ldc < N ||
+        static_cast<size_t>(a_rows) * lda >= (1ull << 32) || static_cast<size_t>(N) * K >= (1ull << 32) ||
+        N % (epilogue == EPI_SILU_GATE ? BN / 2 : BN) != 0 || ldc % 8 != 0 || !aligned16(C) || !aligned16(b_descale) ||
+        (epilogue == EPI_SILU_GATE && !aligned16(b_up_descale)))
         return CF_ERR_UNSUPPORTED;
     hipStream_t st = as_stream(stream);
     const int max_row_tiles = total_rows / BM + num_experts;
@@ -942,6 +1114,7 @@ int cf_fp8_grouped_gemm_nt_bf16_ex(int total_rows, int N, int K, int num_experts
     p.C = C; p.ldc = ldc;
     p.tile_map = tile_map;
     p.a_row_index = d_a_row_index;
+    p.a_rows = a_rows;
     p.b_expert_stride = static_cast<long long>(N) * K;
     p.sb_expert_stride = scale_mode == SCALE_ROWCOL ? N : 0;
     const int out_bn = epilogue == EPI_SILU_GATE ? BN / 2 : BN;

@@ -614,13 +614,13 @@ int cf_moe_grouped_swiglu_forward_fp8(const void* d_hidden_e4m3, const float* d_
     int rc = cf_moe_compact_row_index(d_counts, d_offsets, d_row_indices, rows, num_experts, index, stream);
     if (rc) return rc;
     // gate/up: rows gathered through the compact index (the token permute is fused into the operand fetch)
-    rc = cf_fp8_grouped_gemm_nt_bf16_ex(total_selected_rows, Ie, H, num_experts, d_counts, d_offsets, d_hidden_e4m3, H, index,
+    rc = cf_fp8_grouped_gemm_nt_bf16_ex(total_selected_rows, Ie, H, num_experts, d_counts, d_offsets, d_hidden_e4m3, rows, H, index,
                                         d_hidden_descale, d_w_gate, d_w_gate_descale, CF_SCALE_ROW_COL, CF_EPI_SILU_GATE,
                                         d_w_up, d_w_up_descale, act, Ie, base + w.tile_map, map_bytes, stream);
     if (rc) return rc;
     rc = cf_fp8_quantize_rows(act, total_selected_rows, Ie, 0, actq, act_scale, act_descale, stream);
     if (rc) return rc;
-    rc = cf_fp8_grouped_gemm_nt_bf16_ex(total_selected_rows, H, Ie, num_experts, d_counts, d_offsets, actq, Ie, nullptr,
+    rc = cf_fp8_grouped_gemm_nt_bf16_ex(total_selected_rows, H, Ie, num_experts, d_counts, d_offsets, actq, total_selected_rows, Ie, nullptr,
                                         act_descale, d_w_down, d_w_down_descale, CF_SCALE_ROW_COL, CF_EPI_NONE, nullptr,
                                         nullptr, y, H, base + w.tile_map, map_bytes, stream);
     if (rc) return rc;

@@ -57,13 +57,13 @@ def run_stages(cf, b: Bank):
     cidx = torch.full((total,), -1, dtype=torch.int32, device=dev)
     cf.cf_moe_compact_row_index(b.d["counts"], b.d["offsets"], b.d["idx"], b.rows, E, cidx, stream())
     act = torch.zeros((total, Ie), dtype=torch.bfloat16, device=dev)
-    cf.cf_fp8_grouped_gemm_nt_bf16_ex(total, Ie, H, E, b.d["counts"], b.d["offsets"], b.d["hq"], H, cidx, b.d["hd"],
+    cf.cf_fp8_grouped_gemm_nt_bf16_ex(total, Ie, H, E, b.d["counts"], b.d["offsets"], b.d["hq"], b.rows, H, cidx, b.d["hd"],
                                       b.d["wg"], b.d["wgd"], ROW_COL, EPI_SILU, b.d["wu"], b.d["wud"], act, Ie, ws, sz.value, stream())
     actq = torch.empty((total, Ie), dtype=torch.uint8, device=dev)
     a_s = torch.empty(total, device=dev); a_d = torch.empty(total, device=dev)
     cf.cf_fp8_quantize_rows(act, total, Ie, 0, actq, a_s, a_d, stream())
     y = torch.zeros((total, H), dtype=torch.bfloat16, device=dev)
-    cf.cf_fp8_grouped_gemm_nt_bf16_ex(total, H, Ie, E, b.d["counts"], b.d["offsets"], actq, Ie, None, a_d,
+    cf.cf_fp8_grouped_gemm_nt_bf16_ex(total, H, Ie, E, b.d["counts"], b.d["offsets"], actq, total, Ie, None, a_d,
                                       b.d["wd"], b.d["wdd"], ROW_COL, EPI_NONE, None, None, y, H, ws, sz.value, stream())
     mixed = dev_bf16(b.mixed0, dev)
     cf.cf_moe_unpermute_weighted_bf16(mixed, y, b.d["rw"], b.d["counts"], b.d["offsets"], b.d["idx"], b.rows, E, H, stream())

@@ -516,15 +516,16 @@ __device__ __forceinline__ TilePos locate_tile(const GemmArgs& p, int pos) {
 }
 
 // Drain of a tile.  A unit is 32 output columns: one accumulator column of the wavefront (gate and up
-// accumulators of the same columns for the SiLU-gate epilogue).  TileScales holds what the drain needs in
-// registers: the descales of this lane's four output rows, and the channel descales of the unit being
-// drained (cs[g] = the four consecutive columns of accumulator quad g); the next unit's are fetched while
-// the current one is drained, the first unit's while the tile's last MFMAs run.
+// accumulators of the same columns for the SiLU-gate epilogue); units are drained in pairs (64 columns =
+// one 128-byte line of bf16 per row).  TileScales holds what the drain needs in registers: the descales
+// of this lane's four output rows, and the channel descales of the pair being drained (cs[u][g] = the
+// four consecutive columns of accumulator quad g of unit u); the next pair's are fetched while the
+// current one is drained, the first pair's while the tile's last MFMAs run.
 template <int EPI>
 struct TileScales {
     float sa[4];
-    float4 cs[4];
-    float4 cs2[4];
+    float4 cs[2][4];
+    float4 cs2[2][4];
 };
 
 template <int EPI, int SCALE>
@@ -538,20 +539,22 @@ __device__ __forceinline__ void load_row_scales(TileScales<EPI>& s, const GemmAr
     }
 }
 template <int EPI, int SCALE>
-__device__ __forceinline__ void load_unit_scales(float4 (&cs)[4], float4 (&cs2)[4], const GemmArgs& p, const TilePos& t,
-                                                 int wn, int lane, int unit) {
-    constexpr int NT = EPI == EPI_SILU_GATE ? 2 : 4;
+__device__ __forceinline__ void load_pair_scales(float4 (&cs)[2][4], float4 (&cs2)[2][4], const GemmArgs& p, const TilePos& t,
+                                                 int wn, int lane, int pair) {
+    constexpr int NU = EPI == EPI_SILU_GATE ? 2 : 4;
     if constexpr (SCALE == SCALE_ROWCOL) {
         // uniform base (scalar registers) + a small per-lane byte offset: no 64-bit per-lane addresses to keep alive
-        const size_t ucol = static_cast<size_t>(t.expert) * p.sb_expert_stride + t.n0 + wn * (NT * 32) + unit * 32;
+        const size_t ucol = static_cast<size_t>(t.expert) * p.sb_expert_stride + t.n0 + wn * (NU * 32) + pair * 64;
         const uint8_t* b1 = reinterpret_cast<const uint8_t*>(p.sb + ucol);
         const uint8_t* b2 = reinterpret_cast<const uint8_t*>(EPI == EPI_SILU_GATE ? p.sb2 + ucol : p.sb);
         const uint32_t loff = static_cast<uint32_t>(lane >> 5) * 16u;
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            cs[g] = *reinterpret_cast<const float4*>(b1 + (loff + g * 32u));
-            if constexpr (EPI == EPI_SILU_GATE) cs2[g] = *reinterpret_cast<const float4*>(b2 + (loff + g * 32u));
-        }
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                cs[u][g] = *reinterpret_cast<const float4*>(b1 + (loff + u * 128u + g * 32u));
+                if constexpr (EPI == EPI_SILU_GATE) cs2[u][g] = *reinterpret_cast<const float4*>(b2 + (loff + u * 128u + g * 32u));
+            }
     }
 }
 
@@ -563,75 +566,91 @@ __device__ __forceinline__ float acc_read(float a) {
     return v;
 }
 
-// Per unit the wavefront scales its accumulators, applies the epilogue, rounds to bf16 and parks the
-// 128 rows x 64 bytes in its own 8 KiB of a free ring slot (16-byte chunks xor-swizzled by row: two-pass
-// ds_write_b64, conflict-free ds_read_b128), then streams them out 16 bytes per lane, four lanes per
-// row, so that every store instruction writes whole 64-byte half lines.  Rows at or beyond t.m_end are
-// not stored.
+// Per pair of units and per 64 output rows the wavefront scales its accumulators, applies the epilogue,
+// rounds to bf16 and parks the 64 rows x 128 bytes in its own 8 KiB of a free ring slot (16-byte chunks
+// xor-swizzled by row: two-pass ds_write_b64, conflict-free ds_read_b128), then streams them out 16 bytes
+// per lane, eight lanes per row, so that every store instruction writes whole 128-byte lines.  The stores
+// are non-temporal: the output is not read again here and should not displace operand tiles from L2.
+// Rows at or beyond t.m_end are not stored.
 template <int EPI, int SCALE>
 __device__ __forceinline__ void drain_tile(v16f (&acc)[4][4], TileScales<EPI>& s, float s1, float s2, const GemmArgs& p,
                                            const TilePos& t, int wm, int wn, int lane, uint8_t* stage) {
     constexpr bool GATE = EPI == EPI_SILU_GATE;
-    constexpr int NT = GATE ? 2 : 4;
+    constexpr int NU = GATE ? 2 : 4;
     const int row = lane & 31, khalf = lane >> 5;
-    uint8_t* wr = stage + row * 64 + khalf * 8;
-    const int wswz = (row >> 2) & 3;
-    const int rr = lane >> 2, rc = lane & 3;
-    const uint8_t* rdp = stage + rr * 64 + ((rc ^ ((rr >> 2) & 3)) << 4);
+    uint8_t* wr = stage + row * 128 + khalf * 8;
+    const int wswz = (row >> 1) & 7;
+    const int rr = lane >> 3, rc = lane & 7;
+    // row rr + 8 i sits at swizzle (rr >> 1) ^ 4 (i & 1): two read bases, even and odd i
+    const uint8_t* rdp0 = stage + rr * 128 + ((rc ^ (rr >> 1)) << 4);
+    const uint8_t* rdp1 = stage + rr * 128 + ((rc ^ (rr >> 1) ^ 4) << 4);
     const int mrow0 = t.m0 + wm * 128 + rr;
-    // stores: uniform base per unit and 16-row group (scalar registers) + this lane's byte offset
-    uint8_t* cu = reinterpret_cast<uint8_t*>(p.C + static_cast<size_t>(t.m0 + wm * 128) * p.ldc + t.n0 + wn * (NT * 32));
+    // stores: uniform base per pair and 8-row group (scalar registers) + this lane's byte offset
+    uint8_t* cu = reinterpret_cast<uint8_t*>(p.C + static_cast<size_t>(t.m0 + wm * 128) * p.ldc + t.n0 + wn * (NU * 32));
     const uint32_t coff = (static_cast<uint32_t>(rr) * static_cast<uint32_t>(p.ldc) + rc * 8u) * 2u;
-    const size_t cstep = static_cast<size_t>(p.ldc) * 32;      // bytes between 16-row groups
+    const size_t cstep = static_cast<size_t>(p.ldc) * 16;      // bytes between 8-row groups
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 #pragma unroll
-    for (int unit = 0; unit < NT; ++unit) {
-        float4 ncs[4], ncs2[4];
-        if (unit + 1 < NT) load_unit_scales<EPI, SCALE>(ncs, ncs2, p, t, wn, lane, unit + 1);
+    for (int pair = 0; pair < NU / 2; ++pair) {
+        float4 ncs[2][4], ncs2[2][4];
+        if (pair + 1 < NU / 2) load_pair_scales<EPI, SCALE>(ncs, ncs2, p, t, wn, lane, pair + 1);
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            const float sa = SCALE == SCALE_ROWCOL ? s.sa[b] : 1.0f;
+        for (int half = 0; half < 2; ++half) {
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                float4 c = make_float4(s1, s1, s1, s1), u = make_float4(s2, s2, s2, s2);
-                if constexpr (SCALE == SCALE_ROWCOL) {
-                    c = s.cs[g];
-                    if constexpr (GATE) u = s.cs2[g];
-                }
-                const float c4[4] = {c.x, c.y, c.z, c.w}, u4[4] = {u.x, u.y, u.z, u.w};
-                float v[4];
+            for (int bb = 0; bb < 2; ++bb) {
+                const int b = half * 2 + bb;
+                const float sa = SCALE == SCALE_ROWCOL ? s.sa[b] : 1.0f;
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    if constexpr (GATE) {
-                        // the reference rounds gate and up to bf16 before the SiLU product
-                        const float gate = round_bf16_hw(acc_read(acc[2 * unit][b][g * 4 + q]) * (sa * c4[q]));
-                        const float up = round_bf16_hw(acc_read(acc[2 * unit + 1][b][g * 4 + q]) * (sa * u4[q]));
-                        v[q] = fast_silu(gate) * up;
-                    } else {
-                        v[q] = acc_read(acc[unit][b][g * 4 + q]) * (sa * c4[q]);
+                for (int uu = 0; uu < 2; ++uu) {
+                    const int unit = pair * 2 + uu;
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        float4 c = make_float4(s1, s1, s1, s1), u = make_float4(s2, s2, s2, s2);
+                        if constexpr (SCALE == SCALE_ROWCOL) {
+                            c = s.cs[uu][g];
+                            if constexpr (GATE) u = s.cs2[uu][g];
+                        }
+                        const float c4[4] = {c.x, c.y, c.z, c.w}, u4[4] = {u.x, u.y, u.z, u.w};
+                        float v[4];
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            if constexpr (GATE) {
+                                // the reference rounds gate and up to bf16 before the SiLU product
+                                const float gate = round_bf16_hw(acc_read(acc[2 * unit][b][g * 4 + q]) * (sa * c4[q]));
+                                const float up = round_bf16_hw(acc_read(acc[2 * unit + 1][b][g * 4 + q]) * (sa * u4[q]));
+                                v[q] = fast_silu(gate) * up;
+                            } else {
+                                v[q] = acc_read(acc[unit][b][g * 4 + q]) * (sa * c4[q]);
+                            }
+                        }
+                        *reinterpret_cast<uint2*>(wr + bb * 32 * 128 + (((uu * 4 + g) ^ wswz) << 4)) =
+                            make_uint2(pack_bf16x2_hw(v[0], v[1]), pack_bf16x2_hw(v[2], v[3]));
                     }
+                    __builtin_amdgcn_sched_barrier(0);     // one accumulator (pair) in flight at a time: keeps the drain in few registers
                 }
-                *reinterpret_cast<uint2*>(wr + b * 32 * 64 + ((g ^ wswz) << 4)) =
-                    make_uint2(pack_bf16x2_hw(v[0], v[1]), pack_bf16x2_hw(v[2], v[3]));
             }
-            __builtin_amdgcn_sched_barrier(0);     // one accumulator (pair) in flight at a time: keeps the drain in few registers
-        }
-        // Stores and copies share one completion counter, and a wait on copies issued after these stores
-        // would have to sit out the whole burst.  So the K-tile still landing is waited for here, where it
-        // costs next to nothing (its copies are older than a unit's worth of drain work), and the tile
-        // that follows skips the wait of its first K-tile: the stores then have two K-tiles to complete.
-        if (unit == 0) __builtin_amdgcn_s_waitcnt(kWaitVm0);
+            // Stores and copies share one completion counter, and a wait on copies issued after these stores
+            // would have to sit out the whole burst.  So the K-tile still landing is waited for here, where it
+            // costs next to nothing (its copies are older than a quarter of the drain's work), and the tile
+            // that follows skips the wait of its first K-tile: the stores then have two K-tiles to complete.
+            if (pair == 0 && half == 0) __builtin_amdgcn_s_waitcnt(kWaitVm0);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const uint4 v = *reinterpret_cast<const uint4*>(rdp + i * 16 * 64);
-            if (mrow0 + i * 16 < t.m_end)
-                *reinterpret_cast<uint4*>(cu + (i * cstep + unit * 64) + coff) = v;
+            for (int i = 0; i < 8; ++i) {
+                const uint4 v = *reinterpret_cast<const uint4*>(((i & 1) ? rdp1 : rdp0) + i * 8 * 128);
+                if (mrow0 + half * 64 + i * 8 < t.m_end) {
+                    const u32x4 vv = {v.x, v.y, v.z, v.w};
+                    __builtin_nontemporal_store(vv, reinterpret_cast<u32x4*>(cu + ((half * 8 + i) * cstep + pair * 128) + coff));
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
-        if (unit + 1 < NT) {
+        if (pair + 1 < NU / 2) {
 #pragma unroll
-            for (int g = 0; g < 4; ++g) { s.cs[g] = ncs[g]; s.cs2[g] = ncs2[g]; }
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) { s.cs[u][g] = ncs[u][g]; s.cs2[u][g] = ncs2[u][g]; }
         }
-        __builtin_amdgcn_sched_barrier(0);
     }
 }
 
@@ -782,7 +801,7 @@ void k_gemm_nt_ring(const GemmArgs p) {
             if constexpr (i >= 2 && i < 10) dma_w(a0, dk0, std::integral_constant<int, (i >= 2 && i < 10) ? i - 2 : 0>{});
             if constexpr (END && DRAIN && i == 10) {
                 load_row_scales<EPI, SCALE>(sc, p, t, wm, lane);
-                load_unit_scales<EPI, SCALE>(sc.cs, sc.cs2, p, t, wn, lane, 0);
+                load_pair_scales<EPI, SCALE>(sc.cs, sc.cs2, p, t, wn, lane, 0);
             }
             __builtin_amdgcn_sched_barrier(0);
         });

@@ -571,8 +571,8 @@ __device__ __forceinline__ float acc_read(float a) {
 // xor-swizzled by row: two-pass ds_write_b64, conflict-free ds_read_b128), then streams them out 16 bytes
 // per lane, eight lanes per row, so that every store instruction writes whole 128-byte lines.  The stores
 // are non-temporal: the output is not read again here and should not displace operand tiles from L2.
-// Rows at or beyond t.m_end are not stored.
-template <int EPI, int SCALE>
+// RAGGED: the tile may end before its 256th row; rows at or beyond t.m_end are then not stored.
+template <int EPI, int SCALE, bool RAGGED>
 __device__ __forceinline__ void drain_tile(v16f (&acc)[4][4], TileScales<EPI>& s, float s1, float s2, const GemmArgs& p,
                                            const TilePos& t, int wm, int wn, int lane, uint8_t* stage) {
     constexpr bool GATE = EPI == EPI_SILU_GATE;
@@ -638,7 +638,7 @@ __device__ __forceinline__ void drain_tile(v16f (&acc)[4][4], TileScales<EPI>& s
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const uint4 v = *reinterpret_cast<const uint4*>(((i & 1) ? rdp1 : rdp0) + i * 8 * 128);
-                if (mrow0 + half * 64 + i * 8 < t.m_end) {
+                if (!RAGGED || mrow0 + half * 64 + i * 8 < t.m_end) {
                     const u32x4 vv = {v.x, v.y, v.z, v.w};
                     __builtin_nontemporal_store(vv, reinterpret_cast<u32x4*>(cu + ((half * 8 + i) * cstep + pair * 128) + coff));
                 }
@@ -650,6 +650,65 @@ __device__ __forceinline__ void drain_tile(v16f (&acc)[4][4], TileScales<EPI>& s
             for (int u = 0; u < 2; ++u)
 #pragma unroll
                 for (int g = 0; g < 4; ++g) { s.cs[u][g] = ncs[u][g]; s.cs2[u][g] = ncs2[u][g]; }
+        }
+    }
+}
+
+// The fp32 accumulate form (C += product, per-tensor scale s1): per pair of units and per 32 output rows
+// the scaled accumulators are parked as 32 rows x 256 bytes of fp32 (chunks xor-swizzled by row), read
+// back 16 bytes per lane, sixteen lanes per row, added to what C holds (fetched while the block is being
+// scaled) and stored: whole 128-byte lines in both directions, non-temporal both ways.
+template <bool RAGGED>
+__device__ __forceinline__ void drain_tile_accum_f32(v16f (&acc)[4][4], float s1, const GemmArgs& p, const TilePos& t,
+                                                     int wm, int wn, int lane, uint8_t* stage) {
+    const int row = lane & 31, khalf = lane >> 5;
+    uint8_t* wr = stage + row * 256;
+    const int wswz = row & 15;
+    const int rr = lane >> 4, rc = lane & 15;
+    const int mrow0 = t.m0 + wm * 128 + rr;
+    uint8_t* cu = reinterpret_cast<uint8_t*>(p.Cf + static_cast<size_t>(t.m0 + wm * 128) * p.ldc + t.n0 + wn * 128);
+    const uint32_t coff = (static_cast<uint32_t>(rr) * static_cast<uint32_t>(p.ldc) + rc * 4u) * 4u;
+    const size_t cstep = static_cast<size_t>(p.ldc) * 16;      // bytes between 4-row groups
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+#pragma unroll
+    for (int pair = 0; pair < 2; ++pair) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            f32x4 old[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                old[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                if (!RAGGED || mrow0 + b * 32 + i * 4 < t.m_end)
+                    old[i] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(cu + ((b * 8 + i) * cstep + pair * 256) + coff));
+            }
+#pragma unroll
+            for (int uu = 0; uu < 2; ++uu) {
+                const int unit = pair * 2 + uu;
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    float4 v;
+                    v.x = acc_read(acc[unit][b][g * 4 + 0]) * s1;
+                    v.y = acc_read(acc[unit][b][g * 4 + 1]) * s1;
+                    v.z = acc_read(acc[unit][b][g * 4 + 2]) * s1;
+                    v.w = acc_read(acc[unit][b][g * 4 + 3]) * s1;
+                    *reinterpret_cast<float4*>(wr + (((uu * 8 + g * 2 + khalf) ^ wswz) << 4)) = v;
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // as in drain_tile: every copy in flight is waited for before the first store, and the tile that
+            // follows skips the wait of its first K-tile
+            if (pair == 0 && b == 0) __builtin_amdgcn_s_waitcnt(kWaitVm0);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int r = i * 4 + rr;
+                const float4 v = *reinterpret_cast<const float4*>(stage + r * 256 + ((rc ^ (r & 15)) << 4));
+                if (!RAGGED || mrow0 + b * 32 + i * 4 < t.m_end) {
+                    const f32x4 o = {old[i][0] + v.x, old[i][1] + v.y, old[i][2] + v.z, old[i][3] + v.w};
+                    __builtin_nontemporal_store(o, reinterpret_cast<f32x4*>(cu + ((b * 8 + i) * cstep + pair * 256) + coff));
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 }
@@ -668,7 +727,7 @@ void k_gemm_nt_ring(const GemmArgs p) {
     constexpr int OUT_BN = GATE ? BN / 2 : BN;
     // the LDS-staged drain covers these epilogues; the launcher sends such a call here only when N is a multiple
     // of the tile's output width and C and the channel descales allow 16-byte accesses
-    constexpr bool DRAIN = EPI == EPI_NONE || EPI == EPI_SILU_GATE;
+    constexpr bool DRAIN = EPI == EPI_NONE || EPI == EPI_SILU_GATE || EPI == EPI_ACCUM_F32;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
@@ -799,7 +858,7 @@ void k_gemm_nt_ring(const GemmArgs p) {
                 if constexpr (i >= 14) read_one(a2, a3, C0{}, ic);       // reads 14 and 15 ride with the last two MFMAs
             }
             if constexpr (i >= 2 && i < 10) dma_w(a0, dk0, std::integral_constant<int, (i >= 2 && i < 10) ? i - 2 : 0>{});
-            if constexpr (END && DRAIN && i == 10) {
+            if constexpr (END && DRAIN && EPI != EPI_ACCUM_F32 && i == 10) {
                 load_row_scales<EPI, SCALE>(sc, p, t, wm, lane);
                 load_pair_scales<EPI, SCALE>(sc.cs, sc.cs2, p, t, wn, lane, 0);
             }
@@ -848,7 +907,15 @@ void k_gemm_nt_ring(const GemmArgs p) {
         // finished reading it (barrier of the last step) and only X of the stream's third K-tile from here
         // is copied into it next, by this wavefront's own copies, in program order after the drain.
         if constexpr (DRAIN) {
-            drain_tile<EPI, SCALE>(acc, sc, s1, s2, p, t, wm, wn, lane, smem + a4 + wave * (64 * BK));
+            uint8_t* stage = smem + a4 + wave * (64 * BK);
+            if constexpr (EPI == EPI_ACCUM_F32) {
+                // the drain's own loads of C are waited for by the compiler; the copies in flight are older
+                if (t.m0 + BM <= t.m_end) drain_tile_accum_f32<false>(acc, s1, p, t, wm, wn, lane, stage);
+                else                      drain_tile_accum_f32<true>(acc, s1, p, t, wm, wn, lane, stage);
+            } else {
+                if (t.m0 + BM <= t.m_end) drain_tile<EPI, SCALE, false>(acc, sc, s1, s2, p, t, wm, wn, lane, stage);
+                else                      drain_tile<EPI, SCALE, true>(acc, sc, s1, s2, p, t, wm, wn, lane, stage);
+            }
         } else {
             GemmArgs q = p;                        // the epilogue sees this tile's row bound
             q.M = t.m_end;
@@ -925,6 +992,10 @@ int launch_tiled(const GemmArgs& p, hipStream_t st) {
     // the ring kernel addresses operand rows by 32-bit byte offsets
     bool ring_ok = p.K % BK == 0 && p.K >= 2 * BK && static_cast<size_t>(p.a_rows) * p.lda < (1ull << 32) &&
                    static_cast<size_t>(p.N) * p.ldb < (1ull << 32);
+    if constexpr (EPI == EPI_ACCUM_F32) {
+        // its drain adds into full-width fp32 tiles with 16-byte accesses
+        ring_ok = ring_ok && p.N % BN == 0 && p.ldc % 4 == 0 && aligned16(p.Cf);
+    }
     if constexpr (EPI == EPI_NONE || EPI == EPI_SILU_GATE) {
         // its drain writes full-width tiles with 16-byte stores and reads the channel descales as float4
         constexpr int out_bn = EPI == EPI_SILU_GATE ? BN / 2 : BN;
@@ -967,20 +1038,34 @@ int dispatch_epi(const GemmArgs& p, int epi, int scale_mode, hipStream_t st) {
     }
 }
 
-// one thread: row tiles of every expert in expert order
-__global__ void k_build_tile_map(const int* __restrict__ counts, const int* __restrict__ offsets, int num_experts,
-                                 int max_row_tiles, int* __restrict__ tile_map) {
-    int n = 0;
-    for (int e = 0; e < num_experts; ++e) {
-        const int first = offsets[e], end = first + counts[e];
-        for (int r = first; r < end && n < max_row_tiles; r += BM) {
-            tile_map[1 + 3 * n] = e;
-            tile_map[2 + 3 * n] = r;
-            tile_map[3 + 3 * n] = min(r + BM, end);
-            ++n;
+// one wavefront: row tiles of every expert in expert order (lane = expert, prefix sum of the tile counts)
+__global__ __launch_bounds__(64) void k_build_tile_map(const int* __restrict__ counts, const int* __restrict__ offsets,
+                                                       int num_experts, int max_row_tiles, int* __restrict__ tile_map) {
+    const int lane = threadIdx.x;
+    int carry = 0;
+    for (int e0 = 0; e0 < num_experts; e0 += 64) {
+        const int e = e0 + lane;
+        const int cnt = e < num_experts ? counts[e] : 0;
+        const int first = e < num_experts ? offsets[e] : 0;
+        const int nt = (cnt + BM - 1) / BM;
+        int incl = nt;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int v = __shfl_up(incl, off, 64);
+            if (lane >= off) incl += v;
         }
+        const int base = carry + incl - nt;
+        for (int i = 0; i < nt; ++i) {
+            const int n = base + i;
+            if (n < max_row_tiles) {
+                tile_map[1 + 3 * n] = e;
+                tile_map[2 + 3 * n] = first + i * BM;
+                tile_map[3 + 3 * n] = min(first + (i + 1) * BM, first + cnt);
+            }
+        }
+        carry += __shfl(incl, 63, 64);
     }
-    tile_map[0] = n;
+    if (lane == 0) tile_map[0] = min(carry, max_row_tiles);
 }
 
 int gemm_nt(GemmArgs p, int fmt, int epi, int scale_mode, int force_naive, cf_stream_t stream) {
@@ -1123,7 +1208,7 @@ int cf_fp8_grouped_gemm_nt_bf16_ex(int total_rows, int N, int K, int num_experts
     hipStream_t st = as_stream(stream);
     const int max_row_tiles = total_rows / BM + num_experts;
     int* tile_map = static_cast<int*>(d_workspace);
-    k_build_tile_map<<<1, 1, 0, st>>>(d_counts, d_offsets, num_experts, max_row_tiles, tile_map);
+    k_build_tile_map<<<1, 64, 0, st>>>(d_counts, d_offsets, num_experts, max_row_tiles, tile_map);
     GemmArgs p{};
     p.M = total_rows; p.N = N; p.K = K;
     p.A = static_cast<const uint8_t*>(A); p.lda = lda;

@@ -49,7 +49,9 @@ def run_gemm(cf, dev, A, B, sa, sb, *, lda=None, a_e5m2=False, mode=PER_TENSOR, 
     return orc.bf16_to_f32(bf16_bits(C)).astype(np.float64)
 
 
-SHAPES = [(256, 256, 128), (512, 768, 1024), (300, 200, 144), (1, 1, 16), (33, 500, 208), (257, 129, 4096), (64, 1408, 2048)]
+# (300, 512, 512) and (770, 256, 384): persistent kernel with a ragged last row tile; (1024, 1024, 256): several tiles per workgroup, two K-tiles
+SHAPES = [(256, 256, 128), (512, 768, 1024), (300, 200, 144), (1, 1, 16), (33, 500, 208), (257, 129, 4096), (64, 1408, 2048),
+          (300, 512, 512), (770, 256, 384), (1024, 1024, 256)]
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)
@@ -95,11 +97,11 @@ def test_gemm_e5m2_activations_and_row_stride(cf, dev, flags):
     orc.assert_gemm_close(got, ref, absdot)
 
 
+@pytest.mark.parametrize("M,N,K", [(300, 260, 384), (300, 512, 384), (1100, 256, 640)])
 @pytest.mark.parametrize("flags", [0, NAIVE])
-def test_gemm_row_col_scales_and_bias(cf, dev, flags):
-    case(f"gemm row/col scales + bias flags={flags}")
+def test_gemm_row_col_scales_and_bias(cf, dev, M, N, K, flags):
+    case(f"gemm row/col scales + bias {M}x{N}x{K} flags={flags}")
     rng = np.random.default_rng(6)
-    M, N, K = 300, 260, 384
     A, _ = rand_fp8(rng, (M, K))
     B, _ = rand_fp8(rng, (N, K), sigma=0.02)
     sa = rng.uniform(0.001, 0.02, M).astype(np.float32)
@@ -114,7 +116,7 @@ def test_gemm_row_col_scales_and_bias(cf, dev, flags):
     assert np.array_equal(gotb, want)
 
 
-@pytest.mark.parametrize("M,N,K", [(256, 128, 256), (300, 200, 512), (512, 1408, 2048)])
+@pytest.mark.parametrize("M,N,K", [(256, 128, 256), (300, 200, 512), (512, 1408, 2048), (300, 256, 512), (1024, 384, 256)])
 @pytest.mark.parametrize("mode", [PER_TENSOR, ROW_COL])
 def test_gemm_fused_silu_gate(cf, dev, M, N, K, mode):
     case(f"gemm silu-gate {M}x{N}x{K} mode={mode}")
@@ -212,7 +214,7 @@ def run_accum(cf, dev, A, B, sa, sb, C0, *, a_e5m2, b_e5m2, flags=0, bf16_out=Fa
     return host(C).astype(np.float64)
 
 
-@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (300, 200, 384), (512, 1024, 2048), (130, 260, 80)])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (300, 200, 384), (512, 1024, 2048), (130, 260, 80), (300, 512, 512), (1024, 768, 256)])
 @pytest.mark.parametrize("flags", [0, NAIVE])
 def test_wgrad_tn_accumulate_f32(cf, dev, M, N, K, flags):
     """dW[M,N] fp32 += X^T[M,K](E4M3) . dY^T[N,K](E5M2)^T, beta = 1 (lt_gemm_fp8_tn_accum_f32)."""

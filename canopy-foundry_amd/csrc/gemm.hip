@@ -491,12 +491,13 @@ __device__ __forceinline__ void static_for(F&& f) {
     }
 }
 
+// row_tiles: number of row tiles in the grouped form's table (its first word), read once per workgroup
 template <int OUT_BN>
-__device__ __forceinline__ TilePos locate_tile(const GemmArgs& p, int pos) {
+__device__ __forceinline__ TilePos locate_tile(const GemmArgs& p, int pos, int row_tiles) {
     TilePos t;
     if (p.tile_map) {
         // grouped: row tiles come from the table, column tiles vary fastest so neighbours share an A tile
-        const int total = p.tile_map[0] * p.tiles_n;
+        const int total = row_tiles * p.tiles_n;
         int lin = pos;
         if (total % kXcds == 0) lin = (pos % kXcds) * (total / kXcds) + pos / kXcds;
         const int mt = lin / p.tiles_n, nt = lin - mt * p.tiles_n;
@@ -572,9 +573,9 @@ __device__ __forceinline__ float acc_read(float a) {
 // per lane, eight lanes per row, so that every store instruction writes whole 128-byte lines.  The stores
 // are non-temporal: the output is not read again here and should not displace operand tiles from L2.
 // RAGGED: the tile may end before its 256th row; rows at or beyond t.m_end are then not stored.
-template <int EPI, int SCALE, bool RAGGED>
+template <int EPI, int SCALE, bool RAGGED, class Landed>
 __device__ __forceinline__ void drain_tile(v16f (&acc)[4][4], TileScales<EPI>& s, float s1, float s2, const GemmArgs& p,
-                                           const TilePos& t, int wm, int wn, int lane, uint8_t* stage) {
+                                           const TilePos& t, int wm, int wn, int lane, uint8_t* stage, Landed&& landed) {
     constexpr bool GATE = EPI == EPI_SILU_GATE;
     constexpr int NU = GATE ? 2 : 4;
     const int row = lane & 31, khalf = lane >> 5;
@@ -634,7 +635,10 @@ __device__ __forceinline__ void drain_tile(v16f (&acc)[4][4], TileScales<EPI>& s
             // would have to sit out the whole burst.  So the K-tile still landing is waited for here, where it
             // costs next to nothing (its copies are older than a quarter of the drain's work), and the tile
             // that follows skips the wait of its first K-tile: the stores then have two K-tiles to complete.
-            if (pair == 0 && half == 0) __builtin_amdgcn_s_waitcnt(kWaitVm0);
+            if (pair == 0 && half == 0) {
+                __builtin_amdgcn_s_waitcnt(kWaitVm0);
+                landed();                      // the caller's loads that must not meet copies in flight
+            }
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const uint4 v = *reinterpret_cast<const uint4*>(((i & 1) ? rdp1 : rdp0) + i * 8 * 128);
@@ -658,9 +662,9 @@ __device__ __forceinline__ void drain_tile(v16f (&acc)[4][4], TileScales<EPI>& s
 // the scaled accumulators are parked as 32 rows x 256 bytes of fp32 (chunks xor-swizzled by row), read
 // back 16 bytes per lane, sixteen lanes per row, added to what C holds (fetched while the block is being
 // scaled) and stored: whole 128-byte lines in both directions, non-temporal both ways.
-template <bool RAGGED>
+template <bool RAGGED, class Landed>
 __device__ __forceinline__ void drain_tile_accum_f32(v16f (&acc)[4][4], float s1, const GemmArgs& p, const TilePos& t,
-                                                     int wm, int wn, int lane, uint8_t* stage) {
+                                                     int wm, int wn, int lane, uint8_t* stage, Landed&& landed) {
     const int row = lane & 31, khalf = lane >> 5;
     uint8_t* wr = stage + row * 256;
     const int wswz = row & 15;
@@ -698,7 +702,10 @@ __device__ __forceinline__ void drain_tile_accum_f32(v16f (&acc)[4][4], float s1
             }
             // as in drain_tile: every copy in flight is waited for before the first store, and the tile that
             // follows skips the wait of its first K-tile
-            if (pair == 0 && b == 0) __builtin_amdgcn_s_waitcnt(kWaitVm0);
+            if (pair == 0 && b == 0) {
+                __builtin_amdgcn_s_waitcnt(kWaitVm0);
+                landed();
+            }
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const int r = i * 4 + rr;
@@ -731,7 +738,8 @@ void k_gemm_nt_ring(const GemmArgs p) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
-    const int total_tiles = (p.tile_map ? p.tile_map[0] : p.tiles_m) * p.tiles_n;
+    const int row_tiles = p.tile_map ? p.tile_map[0] : p.tiles_m;
+    const int total_tiles = row_tiles * p.tiles_n;
     const int my_tiles = (total_tiles - static_cast<int>(blockIdx.x) + static_cast<int>(gridDim.x) - 1) / static_cast<int>(gridDim.x);
     if (my_tiles <= 0) return;        // grouped launches size the grid by an upper bound of the tile count
     const int ktiles = p.K / BK;      // >= 2, checked by the launcher
@@ -747,17 +755,30 @@ void k_gemm_nt_ring(const GemmArgs p) {
     uint32_t xoff[8], woff[8];                         // per-lane byte offsets from the operand bases
     const uint8_t* wb = p.B;                           // weight bases of the tile the copy stream is aimed at
     const uint8_t* wb2 = p.B2;
-    auto aim = [&](int seq) {                          // point the copy stream at this workgroup's seq-th tile
-        const TilePos t = locate_tile<OUT_BN>(p, blockIdx.x + seq * gridDim.x);
+    // Where a tile lives and, for the grouped form, which A rows its 256 rows gather: everything `aim` needs
+    // from memory.  Both are fetched ahead of the turn of the copy stream at points where waiting for them
+    // cannot stall the copy pipeline: the position under the last K-tile of the tile two before (consumed
+    // after that tile's drain has waited for all memory traffic), the rows inside that drain.
+    auto fetch_pos = [&](int seq, TilePos& t) { t = locate_tile<OUT_BN>(p, blockIdx.x + seq * gridDim.x, row_tiles); };
+    auto fetch_rows = [&](const TilePos& t, int (&rows)[8]) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int arow = min(t.m0 + wave * 64 + j * 8 + lrow, t.m_end - 1);
+            rows[j] = p.a_row_index ? p.a_row_index[arow] : arow;
+        }
+    };
+    auto fetch_tile = [&](int seq, TilePos& t, int (&rows)[8]) {
+        fetch_pos(seq, t);
+        fetch_rows(t, rows);
+    };
+    auto aim = [&](const TilePos& t, const int (&rows)[8]) {      // point the copy stream at a fetched tile
         wb = p.B + t.expert * p.b_expert_stride;
         if constexpr (GATE) wb2 = p.B2 + t.expert * p.b_expert_stride;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int row = wave * 64 + j * 8 + lrow;
             const uint32_t gchunk = (lslot ^ swz(row)) * 16;
-            int arow = min(t.m0 + row, t.m_end - 1);
-            if (p.a_row_index) arow = p.a_row_index[arow];
-            xoff[j] = static_cast<uint32_t>(arow) * static_cast<uint32_t>(p.lda) + gchunk;
+            xoff[j] = static_cast<uint32_t>(rows[j]) * static_cast<uint32_t>(p.lda) + gchunk;
             int n = t.n0 + row;
             if constexpr (GATE) {
                 // LDS weight rows of a wave: [gate 32 | up 32 | gate 32 | up 32] over the same 64 output columns;
@@ -833,6 +854,12 @@ void k_gemm_nt_ring(const GemmArgs p) {
     // is known to have landed) and made visible by the barrier.  FIRST: the tile's first K-tile (zero C
     // operand).  END: the tile's last K-tile: the operands of the next tile are read after the drain, and
     // the drain's first scale factors are fetched here instead.
+    // tiles of this workgroup around the one being computed: t0 = current, t1 = next, t2 = the one after;
+    // nrows = the A rows of the tile the copy stream turns to next
+    TilePos t0, t1, t2;
+    int nrows[8];
+    int fetch_seq = 0;                                 // the tile END fetches next (into t2 / nrows)
+
     auto ktile = [&](auto first_c, auto end_c, int dk0, const TilePos& t, bool wait) {
         constexpr bool END = decltype(end_c)::value != 0;
         // step (g,0)
@@ -858,6 +885,9 @@ void k_gemm_nt_ring(const GemmArgs p) {
                 if constexpr (i >= 14) read_one(a2, a3, C0{}, ic);       // reads 14 and 15 ride with the last two MFMAs
             }
             if constexpr (i >= 2 && i < 10) dma_w(a0, dk0, std::integral_constant<int, (i >= 2 && i < 10) ? i - 2 : 0>{});
+            if constexpr (END && i == 11) {
+                if (fetch_seq < my_tiles) fetch_pos(fetch_seq, t2);
+            }
             if constexpr (END && DRAIN && EPI != EPI_ACCUM_F32 && i == 10) {
                 load_row_scales<EPI, SCALE>(sc, p, t, wm, lane);
                 load_pair_scales<EPI, SCALE>(sc.cs, sc.cs2, p, t, wn, lane, 0);
@@ -870,30 +900,59 @@ void k_gemm_nt_ring(const GemmArgs p) {
         a0 = a2; a1 = a3; a2 = a4; a3 = b0; a4 = b1;
     };
 
-    // prologue: K-tiles 0 and 1 of the stream in flight, K-tile 0 landed and visible, operands (0,0) in set 0
-    aim(0);
-    static_for<0, 8>([&](auto jc) { dma_x(a0, 0, jc); });
-    static_for<0, 8>([&](auto jc) { dma_w(a1, 0, jc); });
-    static_for<0, 8>([&](auto jc) { dma_x(a2, BK, jc); });
-    static_for<0, 8>([&](auto jc) { dma_w(a3, BK, jc); });
-    __builtin_amdgcn_s_waitcnt(kWaitVm16);
-    __syncthreads();
-    static_for<0, 16>([&](auto ic) { read_one(a0, a1, C0{}, ic); });
-
     // Copy position: two K-tiles ahead of the compute position (ktiles >= 2, so at most one tile ahead).
     // Past the workgroup's last tile the stream simply re-reads that tile: the last two K-tiles then run
     // the same code as every other one, and what they copy is never used.
     int dkt = 2 % ktiles, dseq = 2 / ktiles;
-    if (dseq == 1 && my_tiles > 1) aim(1);
+    // With three or more K-tiles per tile the stream turns to tile s+1 while tile s is being computed, and
+    // (t1, nrows) were fetched under the last K-tile of tile s-1.  With two K-tiles per tile the stream is a
+    // whole tile ahead; that shape simply fetches at the turn and waits.
+    const bool ahead = ktiles > 2;
+
+    // prologue: tile 0 located and aimed at, tile 1 fetched, and all of these loads waited for before the
+    // first copy is issued (the copy pipeline must never wait on them); then K-tiles 0 and 1 of the stream
+    // in flight, K-tile 0 landed and visible, operands (0,0) in set 0
+    {
+        int rows0[8];
+        fetch_tile(0, t0, rows0);
+        aim(t0, rows0);
+        t1 = t0; t2 = t0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) nrows[j] = rows0[j];
+        if (ahead && my_tiles > 1) fetch_tile(1, t1, nrows);
+        __builtin_amdgcn_s_waitcnt(kWaitVm0);
+        static_for<0, 8>([&](auto jc) { dma_x(a0, 0, jc); });
+        static_for<0, 8>([&](auto jc) { dma_w(a1, 0, jc); });
+        static_for<0, 8>([&](auto jc) { dma_x(a2, BK, jc); });
+        static_for<0, 8>([&](auto jc) { dma_w(a3, BK, jc); });
+        if (!ahead && my_tiles > 1) {
+            fetch_tile(1, t1, rows0);
+            aim(t1, rows0);
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(kWaitVm16);
+    __syncthreads();
+    static_for<0, 16>([&](auto ic) { read_one(a0, a1, C0{}, ic); });
+
     auto advance_copy = [&]() {
         if (++dkt == ktiles) {                   // the stream moves on to the next tile
             dkt = 0;
-            if (++dseq < my_tiles) aim(dseq);
+            if (++dseq < my_tiles) {
+                if (ahead) {
+                    aim(t1, nrows);
+                } else {
+                    TilePos tt;
+                    int rr[8];
+                    fetch_tile(dseq, tt, rr);
+                    aim(tt, rr);
+                }
+            }
         }
     };
 
     for (int seq = 0; seq < my_tiles; ++seq) {
-        const TilePos t = locate_tile<OUT_BN>(p, blockIdx.x + seq * gridDim.x);
+        if (!ahead) fetch_pos(seq, t0);
+        const TilePos t = t0;
         // after a drain the first K-tile's successor has been waited for already
         ktile(C1{}, C0{}, dkt * BK, t, !(DRAIN && seq > 0));
         rotate(); advance_copy();
@@ -901,26 +960,36 @@ void k_gemm_nt_ring(const GemmArgs p) {
             ktile(C0{}, C0{}, dkt * BK, t, true);
             rotate(); advance_copy();
         }
+        fetch_seq = ahead ? seq + 2 : my_tiles;       // what the last K-tile fetches into (t2, nrows)
         ktile(C0{}, C1{}, dkt * BK, t, true);
         rotate(); advance_copy();
         // After the rotation a4 is the slot that held W of the K-tile just finished.  Every wavefront has
         // finished reading it (barrier of the last step) and only X of the stream's third K-tile from here
         // is copied into it next, by this wavefront's own copies, in program order after the drain.
+        // the rows of the tile fetched under the last K-tile: loaded inside the drain, right after its wait
+        const bool more = ahead && seq + 2 < my_tiles;
+        auto landed = [&]() { if (more) fetch_rows(t2, nrows); };
         if constexpr (DRAIN) {
             uint8_t* stage = smem + a4 + wave * (64 * BK);
             if constexpr (EPI == EPI_ACCUM_F32) {
-                // the drain's own loads of C are waited for by the compiler; the copies in flight are older
-                if (t.m0 + BM <= t.m_end) drain_tile_accum_f32<false>(acc, s1, p, t, wm, wn, lane, stage);
-                else                      drain_tile_accum_f32<true>(acc, s1, p, t, wm, wn, lane, stage);
+                if (t.m0 + BM <= t.m_end) drain_tile_accum_f32<false>(acc, s1, p, t, wm, wn, lane, stage, landed);
+                else                      drain_tile_accum_f32<true>(acc, s1, p, t, wm, wn, lane, stage, landed);
             } else {
-                if (t.m0 + BM <= t.m_end) drain_tile<EPI, SCALE, false>(acc, sc, s1, s2, p, t, wm, wn, lane, stage);
-                else                      drain_tile<EPI, SCALE, true>(acc, sc, s1, s2, p, t, wm, wn, lane, stage);
+                if (t.m0 + BM <= t.m_end) drain_tile<EPI, SCALE, false>(acc, sc, s1, s2, p, t, wm, wn, lane, stage, landed);
+                else                      drain_tile<EPI, SCALE, true>(acc, sc, s1, s2, p, t, wm, wn, lane, stage, landed);
             }
         } else {
+            landed();
             GemmArgs q = p;                        // the epilogue sees this tile's row bound
             q.M = t.m_end;
             epilogue<EPI, SCALE>(acc, q, t.m0, t.n0, wm, wn, lane);
         }
+        if (more) {
+            // the row loads are older than the drain's last stores: requiring them here waits for nothing else
+#pragma unroll
+            for (int j = 0; j < 8; ++j) asm volatile("" :: "v"(nrows[j]));
+        }
+        t0 = t1; t1 = t2;
         static_for<0, 16>([&](auto ic) { read_one(a0, a1, C0{}, ic); });
     }
     // the copies started past the end of the stream must have landed before the LDS is given back

@@ -114,9 +114,13 @@ __device__ __forceinline__ int wave_sum_i(int v) {
     return v;
 }
 
-// |x| >= 0 orders like its bit pattern, so an integer max is a float max.
+// |x| >= 0 orders like its bit pattern, so an integer max is a float max.  Thousands of atomics on one
+// address serialise in L2 (about 13 ns each), so the value is read first and the atomic is issued only by a
+// caller that would raise it: the running maximum settles after a handful of updates, and a stale read
+// merely costs a redundant atomic.
 __device__ __forceinline__ void atomic_max_nonneg(float* addr, float v) {
-    atomicMax(reinterpret_cast<int*>(addr), __float_as_int(v));
+    int* p = reinterpret_cast<int*>(addr);
+    if (__float_as_int(v) > __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(p, __float_as_int(v));
 }
 
 // ---- deterministic expf ------------------------------------------------------

@@ -69,8 +69,15 @@ __global__ __launch_bounds__(kThreads) void k_amax_bf16(const uint16_t* __restri
     const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
     size_t done = 0;
     if constexpr (VEC) {
+        // four independent 32-byte loads per lane and step: few workgroups (few atomics) still keep HBM busy
         const size_t nvec = n / kVec;
-        for (size_t i = tid; i < nvec; i += stride) local = fmaxf(local, amax16(load16(x + i * kVec)));
+        size_t i = tid;
+        for (; i + 3 * stride < nvec; i += 4 * stride) {
+            const Vec16 v0 = load16(x + i * kVec), v1 = load16(x + (i + stride) * kVec);
+            const Vec16 v2 = load16(x + (i + 2 * stride) * kVec), v3 = load16(x + (i + 3 * stride) * kVec);
+            local = fmaxf(fmaxf(local, fmaxf(amax16(v0), amax16(v1))), fmaxf(amax16(v2), amax16(v3)));
+        }
+        for (; i < nvec; i += stride) local = fmaxf(local, amax16(load16(x + i * kVec)));
         done = nvec * kVec;
     }
     for (size_t i = done + tid; i < n; i += stride) local = fmaxf(local, fabsf(bf16_to_f32(x[i])));
@@ -459,7 +466,7 @@ int cf_fp8_amax_bf16(const uint16_t* d_x, size_t n, float* d_amax, cf_stream_t s
     k_zero_f32<<<1, 1, 0, as_stream(stream)>>>(d_amax);
     if (n == 0) return launch_status();
     if (aligned16(d_x))
-        k_amax_bf16<true><<<blocks_for((n + kVec - 1) / kVec), kThreads, 0, as_stream(stream)>>>(d_x, n, d_amax);
+        k_amax_bf16<true><<<min(blocks_for((n + kVec - 1) / kVec), 1024u), kThreads, 0, as_stream(stream)>>>(d_x, n, d_amax);
     else
         k_amax_bf16<false><<<blocks_for(n), kThreads, 0, as_stream(stream)>>>(d_x, n, d_amax);
     return launch_status();

@@ -1,0 +1,194 @@
+#!/usr/bin/env python3
+"""Per-kernel timing of the FP8 hot path at the benchmark shapes, against each kernel's roofline.
+
+    python canopy-foundry_amd/kernel_bench.py [--iters 20]
+
+Every kernel is timed with events on the launch stream (median of three batches of `--iters` launches) and
+reported with its algorithmic bytes or FLOPs: HBM-bound kernels as GB/s and a fraction of 8 TB/s, GEMMs as
+TFLOP/s and a fraction of the 5.0 PFLOP/s dense FP8 MFMA peak.  Inputs are synthetic and resident in HBM.
+bench.py measures the headline step; this script covers the other entry points and shapes.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import importlib.util
+import sys
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent.parent
+HBM_PEAK = 8000.0      # GB/s
+FP8_PEAK = 5000.0      # TFLOP/s
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--iters", type=int, default=20)
+    args = ap.parse_args()
+    import torch
+    sys.path.insert(0, str(ROOT))
+    import __graft_entry__ as entry
+
+    cf = entry.load_package().lib()
+    dev = torch.device("cuda:0")
+    st = torch.cuda.current_stream().cuda_stream
+    g = torch.Generator(device=dev).manual_seed(5)
+
+    def bf16(*shape, sigma=1.0):
+        return (torch.randn(*shape, device=dev, generator=g) * sigma).to(torch.bfloat16)
+
+    def fp8(*shape, e5m2=False):
+        x = torch.randn(*shape, device=dev, generator=g)
+        if e5m2:
+            return (x * (57344.0 / x.abs().max())).to(torch.float8_e5m2).view(torch.uint8)
+        return (x * (448.0 / x.abs().max())).to(torch.float8_e4m3fn).view(torch.uint8)
+
+    def u8(*shape):
+        return torch.empty(*shape, dtype=torch.uint8, device=dev)
+
+    def f32(*shape):
+        return torch.rand(*shape, device=dev) + 0.5
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(3):
+            a = torch.cuda.Event(enable_timing=True)
+            b = torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(args.iters):
+                fn()
+            b.record()
+            torch.cuda.synchronize()
+            ts.append(a.elapsed_time(b) / args.iters)
+        return sorted(ts)[1] * 1e-3      # seconds
+
+    print(f"{'kernel':<64} {'shape':<26} {'us':>9} {'rate':>14} {'of peak':>8}")
+
+    def hbm(name, shape, nbytes, fn):
+        t = timed(fn)
+        gbps = nbytes / t / 1e9
+        print(f"{name:<64} {shape:<26} {t * 1e6:9.1f} {gbps:9.0f} GB/s {100 * gbps / HBM_PEAK:7.1f}%", flush=True)
+
+    def mfma(name, shape, flop, fn):
+        t = timed(fn)
+        tf = flop / t / 1e12
+        print(f"{name:<64} {shape:<26} {t * 1e6:9.1f} {tf:7.0f} TFLOP/s {100 * tf / FP8_PEAK:7.1f}%", flush=True)
+
+    # ---- config 2 activations / weights: quantize family -------------------------------------------
+    M, K, N = 8192, 4096, 14336
+    x = bf16(M, K)
+    n = x.numel()
+    q = u8(M, K)
+    amax = torch.zeros(1, device=dev); sc = torch.ones(1, device=dev); de = torch.ones(1, device=dev)
+    hbm("amax_bf16", f"{M}x{K}", 2.0 * n, lambda: cf.cf_fp8_amax_bf16(x, n, amax, st))
+    hbm("quantize_e4m3 (known scale)", f"{M}x{K}", 3.0 * n, lambda: cf.cf_fp8_quantize_e4m3(x, q, sc, n, st))
+    hbm("quantize_e4m3_record (previous scale + amax)", f"{M}x{K}", 3.0 * n,
+        lambda: cf.cf_fp8_quantize_e4m3_record(x, q, sc, amax, n, st))
+    hbm("quantize_e5m2 (known scale)", f"{M}x{K}", 3.0 * n, lambda: cf.cf_fp8_quantize_e5m2(x, q, sc, n, st))
+    rs = torch.empty(M, device=dev); rd = torch.empty(M, device=dev)
+    hbm("quantize_rows (per-token, one pass)", f"{M}x{K}", 3.0 * n + 8 * M, lambda: cf.cf_fp8_quantize_rows(x, M, K, 0, q, rs, rd, st))
+    h = bf16(M, N)
+    hq = u8(M, N)
+    hbm("quantize_rows (per-token, one pass)", f"{M}x{N}", 3.0 * h.numel() + 8 * M,
+        lambda: cf.cf_fp8_quantize_rows(h, M, N, 0, hq, rs, rd, st))
+    w = bf16(K, N, sigma=0.02)       # [in, out]
+    wt = u8(N, K)
+    w8 = u8(K, N)
+    hbm("quantize_transpose_e4m3 (weight refresh)", f"{K}x{N}", 3.0 * w.numel(),
+        lambda: cf.cf_fp8_quantize_transpose_e4m3(w, wt, sc, K, N, st))
+    hq2 = u8(N, M)
+    hbm("quant_and_transpose_e4m3 (dual, for wgrad)", f"{M}x{N}", 4.0 * h.numel(),
+        lambda: cf.cf_fp8_quant_and_transpose_e4m3(h, hq, hq2, sc, M, N, st))
+    dy8 = fp8(M, K, e5m2=True)
+    dyt = u8(K, M)
+    hbm("transpose_u8 (dY for wgrad)", f"{M}x{K}", 2.0 * dy8.numel(), lambda: cf.cf_transpose_u8(dy8, dyt, M, K, st))
+    gate = bf16(M, N); up = bf16(M, N); out = torch.empty_like(gate)
+    hbm("swiglu_forward (stand-alone)", f"{M}x{N}", 6.0 * gate.numel(),
+        lambda: cf.cf_swiglu_forward(gate, up, out, gate.numel(), st))
+    del gate, up, out, h, hq, hq2, w, wt, w8
+
+    # ---- config 3: block-scaled ---------------------------------------------------------------------
+    M3, N3, K3 = 4096, 7168, 7168
+    a3 = bf16(M3, K3); a3q = u8(M3, K3)
+    s3 = torch.empty(M3, K3 // 128, device=dev); d3 = torch.empty_like(s3)
+    hbm("quantize_block_1x128", f"{M3}x{K3}", 3.0 * a3.numel() + 8.0 * s3.numel(),
+        lambda: cf.cf_fp8_quantize_block_1x128(a3, M3, K3, a3q, s3, d3, st))
+    w3 = bf16(N3, K3, sigma=0.02); w3q = u8(N3, K3)
+    sw3 = torch.empty(N3 // 128, K3 // 128, device=dev); dw3 = torch.empty_like(sw3)
+    hbm("quantize_block_128x128", f"{N3}x{K3}", 3.0 * w3.numel(), lambda: cf.cf_fp8_quantize_block_128x128(w3, N3, K3, w3q, sw3, dw3, st))
+    c3 = torch.empty((M3, N3), dtype=torch.bfloat16, device=dev)
+    mfma("gemm block-scaled 1x128 / 128x128 (config 3)", f"{M3}x{N3}x{K3}", 2.0 * M3 * N3 * K3,
+         lambda: cf.cf_fp8_gemm_nt_bf16_ex(M3, N3, K3, a3q, K3, 0, d3, w3q, K3, dw3, 2, 0, None, None, None, c3, N3, 0, st))
+    del a3, a3q, w3, w3q, c3
+
+    # ---- config 2 and 4 GEMMs -----------------------------------------------------------------------
+    xq = fp8(M, K); wg = fp8(N, K); wu = fp8(N, K); wd = fp8(K, N); hq = fp8(M, N)
+    xd = f32(M); wgd = f32(N); wud = f32(N); wdd = f32(K)
+    c = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+    y = torch.empty((M, K), dtype=torch.bfloat16, device=dev)
+    mfma("gemm per-tensor, bf16 out (lt_gemm_fp8_nt form)", f"{M}x{N}x{K}", 2.0 * M * N * K,
+         lambda: cf.cf_fp8_gemm_nt_bf16(M, N, K, xq, K, 0, sc, wg, de, c, N, st))
+    mfma("gemm per-token x per-channel, bf16 out", f"{M}x{N}x{K}", 2.0 * M * N * K,
+         lambda: cf.cf_fp8_gemm_nt_bf16_ex(M, N, K, xq, K, 0, xd, wg, K, wgd, 1, 0, None, None, None, c, N, 0, st))
+    mfma("gemm gate+up fused SiLU-gate (config 2)", f"{M}x2x{N}x{K}", 4.0 * M * N * K,
+         lambda: cf.cf_fp8_gemm_nt_bf16_ex(M, N, K, xq, K, 0, xd, wg, K, wgd, 1, 2, None, wu, wud, c, N, 0, st))
+    mfma("gemm down projection (config 2)", f"{M}x{K}x{N}", 2.0 * M * N * K,
+         lambda: cf.cf_fp8_gemm_nt_bf16_ex(M, K, N, hq, N, 0, xd, wd, N, wdd, 1, 0, None, None, None, y, K, 0, st))
+    dy = fp8(M, N, e5m2=True)
+    mfma("gemm dgrad, E5M2 dY (config 4)", f"{M}x{K}x{N}", 2.0 * M * N * K,
+         lambda: cf.cf_fp8_gemm_nt_bf16(M, K, N, dy, N, 1, sc, wd, de, y, K, st))
+    xt = fp8(N, M); dyt = fp8(K, M, e5m2=True)
+    dw = torch.zeros((N, K), dtype=torch.float32, device=dev)
+    mfma("gemm wgrad, fp32 accumulate into dW (config 4)", f"{N}x{K}x{M}", 2.0 * M * N * K,
+         lambda: cf.cf_fp8_gemm_tn_accum_f32(N, K, M, xt, sc, dyt, de, dw, K, st))
+    del xq, wg, wu, wd, hq, c, y, dy, xt, dyt, dw
+
+    # ---- config 5: MoE ------------------------------------------------------------------------------
+    T, H, E, k, Ie = 16384, 2048, 64, 6, 1408
+    logits = torch.randn(T, E, device=dev, generator=g)
+    rw = logits.clone()
+    hbm("softmax + top-k route (in place)", f"{T}x{E} k={k}", 8.0 * T * E,
+        lambda: (rw.copy_(logits), cf.cf_moe_topk_route_f32(rw, T, E, k, st, None, None, 1)))
+    counts = torch.zeros(E, dtype=torch.int32, device=dev)
+    idx = torch.zeros(E * T, dtype=torch.int32, device=dev)
+    offs = torch.zeros(E, dtype=torch.int32, device=dev)
+    hbm("build_expert_row_lists", f"{T}x{E}", 4.0 * T * E + 4.0 * T * k,
+        lambda: cf.cf_moe_build_expert_row_lists(rw, counts, idx, T, E, st))
+    cf.cf_moe_expert_offsets_from_counts(counts, offs, E, st)
+    total = T * k
+    hq = fp8(T, H); hd = f32(T)
+    wg = fp8(E * Ie, H); wu = fp8(E * Ie, H); wd = fp8(E * H, Ie)
+    wgd = f32(E * Ie); wud = f32(E * Ie); wdd = f32(E * H)
+    cidx = torch.zeros(total, dtype=torch.int32, device=dev)
+    cf.cf_moe_compact_row_index(counts, offs, idx, T, E, cidx, st)
+    gathered = u8(total, H)
+    hbm("gather_rows_u8 (token permute, stand-alone)", f"{total}x{H}", 2.0 * total * H,
+        lambda: cf.cf_moe_gather_rows_u8(hq, gathered, cidx, total, H, st))
+    sz = ctypes.c_size_t(0)
+    cf.raw_cf_fp8_grouped_gemm_workspace_bytes(total, E, ctypes.byref(sz))
+    ws = u8(sz.value)
+    act = torch.empty((total, Ie), dtype=torch.bfloat16, device=dev)
+    mfma("grouped gate+up SiLU-gate, fused permute (config 5)", f"{total}x2x{Ie}x{H}", 4.0 * total * Ie * H,
+         lambda: cf.cf_fp8_grouped_gemm_nt_bf16_ex(total, Ie, H, E, counts, offs, hq, T, H, cidx, hd, wg, wgd, 1, 2, wu, wud,
+                                                   act, Ie, ws, sz.value, st))
+    actq = fp8(total, Ie); ad = f32(total)
+    yy = torch.empty((total, H), dtype=torch.bfloat16, device=dev)
+    mfma("grouped down projection (config 5)", f"{total}x{H}x{Ie}", 2.0 * total * Ie * H,
+         lambda: cf.cf_fp8_grouped_gemm_nt_bf16_ex(total, H, Ie, E, counts, offs, actq, total, Ie, None, ad, wd, wdd, 1, 0, None, None,
+                                                   yy, H, ws, sz.value, st))
+    mixed = torch.zeros((T, H), dtype=torch.bfloat16, device=dev)
+    hbm("unpermute_weighted_bf16", f"{total}x{H}", 2.0 * total * H + 4.0 * T * H,
+        lambda: cf.cf_moe_unpermute_weighted_bf16(mixed, yy, rw, counts, offs, idx, T, E, H, st))
+    sz2 = ctypes.c_size_t(0)
+    cf.raw_cf_moe_grouped_swiglu_workspace_bytes(total, E, H, Ie, ctypes.byref(sz2))
+    ws2 = u8(sz2.value)
+    mfma("grouped SwiGLU expert bank, whole pipeline (config 5)", f"T={T} E={E} k={k}", 6.0 * total * Ie * H,
+         lambda: cf.cf_moe_grouped_swiglu_forward_fp8(hq, hd, rw, counts, offs, idx, wg, wgd, wu, wud, wd, wdd, mixed, T, H, Ie, E,
+                                                      total, ws2, sz2.value, st))
+
+
+if __name__ == "__main__":
+    main()

@@ -64,14 +64,9 @@ struct TilePos { int m0, m_end, n0, expert; };
 
 __device__ __forceinline__ int swz(int row) { return (row ^ ((row >> 3) & 3)) & 7; }
 
-// Position `pos` in launch order -> (tile_m, tile_n).  Workgroups are handed to the 8 XCDs round-robin,
-// so positions with the same pos % 8 share an XCD (and its L2): each XCD gets a contiguous range of
-// tiles, walked in patches of 8 (M) x tiles_n... x 4 (N) whose operands its L2 can hold.
-__device__ __forceinline__ void tile_coords(int pos, int tiles_m, int tiles_n, int& tm, int& tn) {
-    const int total = tiles_m * tiles_n;
-    const int per_xcd = total / kXcds;
-    int t = pos;
-    if (total % kXcds == 0) t = (pos % kXcds) * per_xcd + pos / kXcds;   // ragged counts keep the plain order
+// Tile t of the walk order -> (tile_m, tile_n): patches of 8 (M) x tiles_n, row tiles varying fastest, so that
+// 32 consecutive tiles form an 8 x 4 patch whose operands an XCD's L2 can hold.
+__device__ __forceinline__ void tile_coords(int t, int tiles_m, int tiles_n, int& tm, int& tn) {
     constexpr int GM = 8;
     const int group = t / (GM * tiles_n);
     const int first_m = group * GM;
@@ -79,6 +74,12 @@ __device__ __forceinline__ void tile_coords(int pos, int tiles_m, int tiles_n, i
     const int in_group = t - group * GM * tiles_n;
     tm = first_m + in_group % gm;
     tn = in_group / gm;
+}
+// Workgroups are handed to the 8 XCDs round-robin, so launch positions with the same pos % 8 share an XCD
+// (and its L2).  One tile per workgroup: position pos works on tile (pos % 8) * (total / 8) + pos / 8 of the walk
+// order, so each XCD is given a contiguous range of tiles (ragged counts keep the plain order).
+__device__ __forceinline__ int xcd_chunked(int pos, int total) {
+    return total % kXcds == 0 ? (pos % kXcds) * (total / kXcds) + pos / kXcds : pos;
 }
 
 // ---- epilogue shared by the tiled kernels ----------------------------------------
@@ -214,7 +215,7 @@ void k_gemm_nt(const GemmArgs p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
     int tile_m, tile_n;
-    tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+    tile_coords(xcd_chunked(blockIdx.x, p.tiles_m * p.tiles_n), p.tiles_m, p.tiles_n, tile_m, tile_n);
     constexpr int OUT_BN = EPI == EPI_SILU_GATE ? BN / 2 : BN;     // output columns per workgroup
     const int m0 = tile_m * BM, n0 = tile_n * OUT_BN;
 
@@ -491,23 +492,29 @@ __device__ __forceinline__ void static_for(F&& f) {
     }
 }
 
-// row_tiles: number of row tiles in the grouped form's table (its first word), read once per workgroup
+// Tile `lin` of a workgroup's walk order -> where it lives.  Dense: the patch order of tile_coords.  Grouped:
+// the table holds, per row tile, its expert's number, row range, first row tile and row-tile count, experts back
+// to back; an expert's tiles are walked in groups of 4 column tiles with its row tiles varying fastest, so that
+// 32 consecutive tiles are (up to) 8 row tiles x 4 column tiles of one expert.
+constexpr int kMapWords = 5;
 template <int OUT_BN>
-__device__ __forceinline__ TilePos locate_tile(const GemmArgs& p, int pos, int row_tiles) {
+__device__ __forceinline__ TilePos locate_tile(const GemmArgs& p, int lin) {
     TilePos t;
     if (p.tile_map) {
-        // grouped: row tiles come from the table, column tiles vary fastest so neighbours share an A tile
-        const int total = row_tiles * p.tiles_n;
-        int lin = pos;
-        if (total % kXcds == 0) lin = (pos % kXcds) * (total / kXcds) + pos / kXcds;
-        const int mt = lin / p.tiles_n, nt = lin - mt * p.tiles_n;
-        t.expert = p.tile_map[1 + 3 * mt];
-        t.m0 = p.tile_map[2 + 3 * mt];
-        t.m_end = p.tile_map[3 + 3 * mt];
-        t.n0 = nt * OUT_BN;
+        const int* e = p.tile_map + 1 + kMapWords * (lin / p.tiles_n);
+        const int expert = e[0], row_base = e[1], row_end = e[2], first_rt = e[3], n_rt = e[4];
+        constexpr int GN = 4;
+        const int local = lin - first_rt * p.tiles_n;
+        const int g = local / (n_rt * GN);
+        const int within = local - g * n_rt * GN;
+        const int rt = within % n_rt;
+        t.expert = expert;
+        t.m0 = row_base + rt * BM;
+        t.m_end = min(t.m0 + BM, row_end);
+        t.n0 = (g * GN + within / n_rt) * OUT_BN;
     } else {
         int tile_m, tile_n;
-        tile_coords(pos, p.tiles_m, p.tiles_n, tile_m, tile_n);
+        tile_coords(lin, p.tiles_m, p.tiles_n, tile_m, tile_n);
         t.expert = 0;
         t.m0 = tile_m * BM;
         t.m_end = p.M;
@@ -738,9 +745,23 @@ void k_gemm_nt_ring(const GemmArgs p) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
-    const int row_tiles = p.tile_map ? p.tile_map[0] : p.tiles_m;
-    const int total_tiles = row_tiles * p.tiles_n;
-    const int my_tiles = (total_tiles - static_cast<int>(blockIdx.x) + static_cast<int>(gridDim.x) - 1) / static_cast<int>(gridDim.x);
+    // This workgroup's walk: workgroups go to the 8 XCDs round-robin, so with a grid that is a multiple of 8 XCD x
+    // takes the contiguous range [x * per, x * per + per) of the walk order and its workgroups stride through it
+    // together: what runs on an XCD at one time is 32 consecutive tiles.
+    const int total_tiles = (p.tile_map ? p.tile_map[0] : p.tiles_m) * p.tiles_n;
+    int my_tiles, lin0, lstep;
+    if (gridDim.x % kXcds == 0) {
+        const int per = (total_tiles + kXcds - 1) / kXcds;
+        const int x = blockIdx.x % kXcds, i = blockIdx.x / kXcds;
+        lstep = gridDim.x / kXcds;
+        const int cnt = max(0, min(per, total_tiles - x * per));
+        my_tiles = (cnt - i + lstep - 1) / lstep;
+        lin0 = x * per + i;
+    } else {
+        lstep = gridDim.x;
+        my_tiles = (total_tiles - static_cast<int>(blockIdx.x) + lstep - 1) / lstep;
+        lin0 = blockIdx.x;
+    }
     if (my_tiles <= 0) return;        // grouped launches size the grid by an upper bound of the tile count
     const int ktiles = p.K / BK;      // >= 2, checked by the launcher
 
@@ -759,7 +780,7 @@ void k_gemm_nt_ring(const GemmArgs p) {
     // from memory.  Both are fetched ahead of the turn of the copy stream at points where waiting for them
     // cannot stall the copy pipeline: the position under the last K-tile of the tile two before (consumed
     // after that tile's drain has waited for all memory traffic), the rows inside that drain.
-    auto fetch_pos = [&](int seq, TilePos& t) { t = locate_tile<OUT_BN>(p, blockIdx.x + seq * gridDim.x, row_tiles); };
+    auto fetch_pos = [&](int seq, TilePos& t) { t = locate_tile<OUT_BN>(p, lin0 + seq * lstep); };
     auto fetch_rows = [&](const TilePos& t, int (&rows)[8]) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
@@ -1107,11 +1128,12 @@ int dispatch_epi(const GemmArgs& p, int epi, int scale_mode, hipStream_t st) {
     }
 }
 
-// one wavefront: row tiles of every expert in expert order (lane = expert, prefix sum of the tile counts)
+// one wavefront: the row tiles of every expert in expert order (lane = expert, prefix sum of the tile counts);
+// each row tile's entry describes its expert: number, row range, first row tile, row-tile count
 __global__ __launch_bounds__(64) void k_build_tile_map(const int* __restrict__ counts, const int* __restrict__ offsets,
                                                        int num_experts, int max_row_tiles, int* __restrict__ tile_map) {
     const int lane = threadIdx.x;
-    int carry = 0;
+    int carry = 0, written = 0;
     for (int e0 = 0; e0 < num_experts; e0 += 64) {
         const int e = e0 + lane;
         const int cnt = e < num_experts ? counts[e] : 0;
@@ -1124,17 +1146,19 @@ __global__ __launch_bounds__(64) void k_build_tile_map(const int* __restrict__ c
             if (lane >= off) incl += v;
         }
         const int base = carry + incl - nt;
-        for (int i = 0; i < nt; ++i) {
-            const int n = base + i;
-            if (n < max_row_tiles) {
-                tile_map[1 + 3 * n] = e;
-                tile_map[2 + 3 * n] = first + i * BM;
-                tile_map[3 + 3 * n] = min(first + (i + 1) * BM, first + cnt);
+        if (base + nt <= max_row_tiles) {        // always true for counts that sum to at most the caller's total_rows
+            for (int i = 0; i < nt; ++i) {
+                int* w = tile_map + 1 + kMapWords * (base + i);
+                w[0] = e; w[1] = first; w[2] = first + cnt; w[3] = base; w[4] = nt;
             }
+            if (nt > 0) written = max(written, base + nt);
         }
         carry += __shfl(incl, 63, 64);
     }
-    if (lane == 0) tile_map[0] = min(carry, max_row_tiles);
+    // experts are written in order, so the ones that fit form a prefix: the table ends with the last of them
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) written = max(written, __shfl_xor(written, off, 64));
+    if (lane == 0) tile_map[0] = written;
 }
 
 int gemm_nt(GemmArgs p, int fmt, int epi, int scale_mode, int force_naive, cf_stream_t stream) {
@@ -1249,7 +1273,7 @@ int cf_fp8_gemm_tn_accum_bf16(int M, int N, int K, const void* Xt_e4m3, const fl
 int cf_fp8_grouped_gemm_workspace_bytes(int total_rows, int num_experts, size_t* bytes) {
     if (total_rows < 0 || num_experts < 0 || !bytes) return CF_ERR_INVALID_ARG;
     const size_t max_row_tiles = static_cast<size_t>(total_rows) / BM + static_cast<size_t>(num_experts);
-    *bytes = (1 + 3 * max_row_tiles) * sizeof(int);
+    *bytes = (1 + kMapWords * max_row_tiles) * sizeof(int);
     return CF_OK;
 }
 

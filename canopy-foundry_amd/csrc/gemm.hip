@@ -1017,6 +1017,297 @@ void k_gemm_nt_ring(const GemmArgs p) {
     __builtin_amdgcn_s_waitcnt(kWaitVm0);
 }
 
+// ---- block-scaled ring kernel ---------------------------------------------------------------
+// The block-scaled GEMM on the persistent direct-to-LDS structure.  Needs K % 128 == 0, K >= 384,
+// N % 256 == 0, operands smaller than 4 GiB, K / 128 <= 256.
+// Workgroup tile 128 x 256 x 128, four wavefronts 2 x 2, each 64 x 128 = 4 x 2 MFMA tiles.  Registers:
+// the running sums (128, VGPRs, written by the vector ALU), one K-tile's partial products (128, the MFMA
+// accumulators) and the operands (64).  A K-tile is one scale group: its partial products start from a
+// zero C operand and are folded into the sums as sum += part * (sa[m, kt] * sb[n / 128, kt]), one
+// accumulator tile at a time, woven between the MFMAs of this and the next K-tile (a tile is folded after
+// its last MFMA has finished and before the next K-tile's first MFMA overwrites it).
+// LDS: three stages of (X 16 KiB + W 32 KiB); K-tile g lives in stage g % 3, K-tiles g+1 and g+2 are resident or
+// landing, and the copies of K-tile g+3 go into stage g % 3 right after the barrier that ends its use.  The
+// activation scales of a K-tile travel with it (one 4-byte copy per row into the stage's scale row), the
+// weight-block scales of a tile (one per K-tile) are copied once per tile; the scale factors are therefore
+// read from LDS and never wait on the copy pipeline.
+constexpr int kBsX = BSM * BK;                          // 16 KiB
+constexpr int kBsW = BN * BK;                           // 32 KiB
+constexpr int kBsStage = kBsX + kBsW;                   // 48 KiB
+constexpr int kBsSa = 3 * kBsStage;                     // activation scales: 3 stages x 128 floats
+constexpr int kBsSb = kBsSa + 3 * BSM * 4;              // weight-block scales: 2 tile parities x 2 column blocks x 256 floats
+constexpr int kBsMaxKb = 256;
+constexpr int kBsLds = kBsSb + 2 * 2 * kBsMaxKb * 4;    // 153,088 bytes
+constexpr int kBsCopies = 13;                           // copy instructions per wavefront and K-tile (4 X, 8 W, 1 scales)
+constexpr int kWaitVm13 = 0x0f7d, kWaitVm26 = 0x4f7a;
+
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void k_gemm_nt_block_ring(const GemmArgs p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int ktiles = p.K / BK;          // >= 3, checked by the launcher; also the number of scale groups along K
+    const int total_tiles = p.tiles_m * p.tiles_n;
+    int my_tiles, lin0, lstep;
+    if (gridDim.x % kXcds == 0) {
+        const int per = (total_tiles + kXcds - 1) / kXcds;
+        const int x = blockIdx.x % kXcds, i = blockIdx.x / kXcds;
+        lstep = gridDim.x / kXcds;
+        const int cnt = max(0, min(per, total_tiles - x * per));
+        my_tiles = (cnt - i + lstep - 1) / lstep;
+        lin0 = x * per + i;
+    } else {
+        lstep = gridDim.x;
+        my_tiles = (total_tiles - static_cast<int>(blockIdx.x) + lstep - 1) / lstep;
+        lin0 = blockIdx.x;
+    }
+    if (my_tiles <= 0) return;
+    auto tile_at = [&](int seq, int& m0, int& n0) {
+        int tm, tn;
+        tile_coords(lin0 + seq * lstep, p.tiles_m, p.tiles_n, tm, tn);
+        m0 = tm * BSM;
+        n0 = tn * BN;
+    };
+
+    // ---- global -> LDS ----
+    const int lrow = lane >> 3, lslot = lane & 7;
+    uint32_t xoff[4], woff[8], saoff = 0;              // per-lane byte offsets
+    const uint8_t* sbsrc = nullptr;                    // the tile's row of weight-block scales (wave's column block)
+    auto aim = [&](int seq) {
+        int m0, n0;
+        tile_at(seq, m0, n0);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int row = wave * 32 + j * 8 + lrow;
+            xoff[j] = static_cast<uint32_t>(min(m0 + row, p.M - 1)) * static_cast<uint32_t>(p.lda) + (lslot ^ swz(row)) * 16;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int row = wave * 64 + j * 8 + lrow;
+            woff[j] = static_cast<uint32_t>(min(n0 + row, p.N - 1)) * static_cast<uint32_t>(p.ldb) + (lslot ^ swz(row)) * 16;
+        }
+        saoff = static_cast<uint32_t>(min(m0 + wave * 32 + (lane & 31), p.M - 1)) * static_cast<uint32_t>(ktiles) * 4u;
+        sbsrc = reinterpret_cast<const uint8_t*>(p.sb + static_cast<size_t>((n0 >> 7) + (wave & 1)) * ktiles);
+    };
+    uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(smem));
+    auto dma16 = [&](uint32_t dst, uint32_t voff, const uint8_t* base) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(voff), "s"(base) : "memory");
+    };
+    // 4-byte copies by the low 32 lanes only: lane l lands at dst + 4 l
+    auto dma4_lo32 = [&](uint32_t dst, uint32_t voff, const uint8_t* base) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_mov_b32 exec_hi, 0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2\n\ts_mov_b32 exec_hi, -1\n\ts_nop 0"
+                     :: "s"(dst), "v"(voff), "s"(base) : "memory");
+    };
+    auto dma4 = [&](uint32_t dst, uint32_t voff, const uint8_t* base) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" :: "s"(dst), "v"(voff), "s"(base) : "memory");
+    };
+    // copy J (0..12) of the K-tile at K offset k0 into stage offset `stage`
+    auto copy_one = [&](int stage, int sidx, int k0, int kt, auto jc) {
+        constexpr int J = decltype(jc)::value;
+        if constexpr (J < 4)       dma16(lds0 + stage + (wave * 32 + J * 8) * BK, xoff[J], p.A + k0);
+        else if constexpr (J < 12) dma16(lds0 + stage + kBsX + (wave * 64 + (J - 4) * 8) * BK, woff[J - 4], p.B + k0);
+        else                       dma4_lo32(lds0 + kBsSa + sidx * (BSM * 4) + wave * 128, saoff, reinterpret_cast<const uint8_t*>(p.sa + kt));
+    };
+    // the weight-block scales of the tile the stream has just turned to: up to four copies of 64 floats by waves 0 and 1
+    // (one per column block), into the half of the scale table selected by the tile's parity
+    auto copy_sb = [&](int parity) {
+        if (wave < 2) {
+            for (int c = 0; c * 64 < ktiles; ++c) {
+                const uint32_t v = static_cast<uint32_t>(min(c * 64 + lane, ktiles - 1)) * 4u;
+                dma4(lds0 + kBsSb + (parity * 2 + wave) * (kBsMaxKb * 4) + c * 256, v, sbsrc);
+            }
+        }
+    };
+
+    // ---- LDS -> MFMA operands ----
+    const int frow = lane & 31, khalf = lane >> 5, fs = swz(frow);
+    int rd[2][2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) rd[h][j] = frow * BK + (((h * 4 + khalf * 2 + j) ^ fs) << 4);
+    const uint8_t* xrd = smem + wm * 64 * BK;
+    const uint8_t* wrd = smem + kBsX + wn * 128 * BK;
+
+    v16f part[4][2];      // [weight tile][activation tile]: this K-tile's partial products (MFMA accumulators)
+    v16f sum[4][2];       // running sums, already scaled
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sum[a][b][r] = 0.0f;
+    // Operand registers: one set of the four weight tiles (a tile is re-read for the next step as soon as both
+    // MFMAs of the current step that use it have issued: three tiles ahead of its next use) and two sets of the
+    // two activation tiles (k-half h of any K-tile lives in set h).
+    v8i wq[4], xq[2][2];
+    auto put = [](v8i& dst, int half, const uint4 v) {
+        dst[4 * half + 0] = (int)v.x; dst[4 * half + 1] = (int)v.y; dst[4 * half + 2] = (int)v.z; dst[4 * half + 3] = (int)v.w;
+    };
+    auto read_w = [&](int stage, auto hc, auto ac) {       // weight tile A of k-half H from the stage at `stage`
+        constexpr int H = decltype(hc)::value, A = decltype(ac)::value;
+        put(wq[A], 0, *reinterpret_cast<const uint4*>(wrd + stage + A * 32 * BK + rd[H][0]));
+        put(wq[A], 1, *reinterpret_cast<const uint4*>(wrd + stage + A * 32 * BK + rd[H][1]));
+    };
+    auto read_x = [&](int stage, auto hc, auto bc) {       // activation tile B of k-half H
+        constexpr int H = decltype(hc)::value, B = decltype(bc)::value;
+        put(xq[H][B], 0, *reinterpret_cast<const uint4*>(xrd + stage + B * 32 * BK + rd[H][0]));
+        put(xq[H][B], 1, *reinterpret_cast<const uint4*>(xrd + stage + B * 32 * BK + rd[H][1]));
+    };
+    auto mfma_one = [&](auto hc, auto ic) {
+        constexpr int H = decltype(hc)::value, I = decltype(ic)::value;
+        constexpr int a = I >> 1, b = I & 1;
+        v16f c = part[a][b];
+        if constexpr (H == 0) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) c[r] = 0.0f;
+        }
+        part[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wq[a], xq[H][b], c, 0, 0, 0, 0, 0, 0);
+    };
+    // fold accumulator tile I of the K-tile whose factors are f[0], f[1] into the sums
+    auto fold_one = [&](const float (&f)[2], auto ic) {
+        constexpr int I = decltype(ic)::value;
+        constexpr int a = I >> 1, b = I & 1;
+        // volatile: the folds must stay woven between the MFMAs where they are written, not sink behind them
+#pragma unroll
+        for (int r = 0; r < 16; r += 4) {
+            // four reads, then four multiply-adds: no instruction waits on the one before it
+            float t0, t1, t2, t3, v0 = sum[a][b][r], v1 = sum[a][b][r + 1], v2 = sum[a][b][r + 2], v3 = sum[a][b][r + 3];
+            const float p0 = part[a][b][r], p1 = part[a][b][r + 1], p2 = part[a][b][r + 2], p3 = part[a][b][r + 3], fv = f[b];
+            asm volatile("v_accvgpr_read_b32 %4, %8\n\tv_accvgpr_read_b32 %5, %9\n\tv_accvgpr_read_b32 %6, %10\n\tv_accvgpr_read_b32 %7, %11\n\t"
+                         "v_fmac_f32 %0, %4, %12\n\tv_fmac_f32 %1, %5, %12\n\tv_fmac_f32 %2, %6, %12\n\tv_fmac_f32 %3, %7, %12"
+                         : "+v"(v0), "+v"(v1), "+v"(v2), "+v"(v3), "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3)
+                         : "a"(p0), "a"(p1), "a"(p2), "a"(p3), "v"(fv));
+            sum[a][b][r] = v0; sum[a][b][r + 1] = v1; sum[a][b][r + 2] = v2; sum[a][b][r + 3] = v3;
+        }
+    };
+    using C0 = std::integral_constant<int, 0>;
+    using C1 = std::integral_constant<int, 1>;
+
+    int s0 = 0, s1 = kBsStage, s2 = 2 * kBsStage;      // stage offsets of K-tiles g, g+1, g+2
+    int i0 = 0, i1 = 1, i2 = 2;                        // and their indices (for the scale rows)
+    float f[2] = {0.0f, 0.0f};                         // factors of the K-tile whose tiles 4..7 are still to be folded
+
+    // One K-tile g at position kt of its tile.  FOLD: tiles 4..7 of the previous K-tile are folded first (not for a
+    // tile's first K-tile).  After the barrier the copies of K-tile g+3 (K offset dk0, position dkt of its tile) start.
+    auto ktile = [&](auto fold_c, int kt, int parity, int dk0, int dkt) {
+        constexpr bool FOLD = decltype(fold_c)::value != 0;
+        // step (g,0): 8 MFMAs from a zero C, the operand reads of (g,1), folds 4..7 of K-tile g-1
+        static_for<0, 8>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            if constexpr (FOLD && i < 4) fold_one(f, std::integral_constant<int, 4 + (i < 4 ? i : 0)>{});
+            mfma_one(C0{}, ic);
+            if constexpr (i == 0) read_x(s0, C1{}, C0{});
+            if constexpr (i == 1) read_x(s0, C1{}, C1{});
+            if constexpr (i == 2 || i == 4 || i == 6) read_w(s0, C1{}, std::integral_constant<int, (i - 2) / 2>{});
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        read_w(s0, C1{}, std::integral_constant<int, 3>{});
+        // this K-tile's factors: read before the barrier, after which its scale row may be overwritten
+        const float sbv = *reinterpret_cast<const float*>(smem + kBsSb + (parity * 2 + wn) * (kBsMaxKb * 4) + kt * 4);
+        float fn[2];
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+            fn[b] = *reinterpret_cast<const float*>(smem + kBsSa + i0 * (BSM * 4) + (wm * 64 + b * 32 + (lane & 31)) * 4) * sbv;
+        // step (g,1)
+        mfma_one(C1{}, C0{});
+        mfma_one(C1{}, C1{});
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(kWaitVm13);
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        f[0] = fn[0]; f[1] = fn[1];
+        static_for<2, 8>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            mfma_one(C1{}, ic);
+            if constexpr (i == 2) read_x(s1, C0{}, C0{});
+            if constexpr (i == 3) read_x(s1, C0{}, C1{});
+            if constexpr (i == 2 || i == 4 || i == 6) read_w(s1, C0{}, std::integral_constant<int, (i - 2) / 2>{});
+            // 13 copies over six slots
+            copy_one(s0, i0, dk0, dkt, std::integral_constant<int, 2 * (i - 2)>{});
+            copy_one(s0, i0, dk0, dkt, std::integral_constant<int, 2 * (i - 2) + 1>{});
+            if constexpr (i == 7) copy_one(s0, i0, dk0, dkt, std::integral_constant<int, 12>{});
+            // folds 0..3 of this K-tile, each four MFMAs after the one that finished its tile
+            if constexpr (i >= 4) fold_one(f, std::integral_constant<int, i >= 4 ? i - 4 : 0>{});
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        read_w(s1, C0{}, std::integral_constant<int, 3>{});
+    };
+    auto rotate = [&]() {
+        const int t = s0, u = i0;
+        s0 = s1; s1 = s2; s2 = t;
+        i0 = i1; i1 = i2; i2 = u;
+    };
+
+    // prologue: K-tiles 0, 1, 2 of the stream in flight, K-tile 0 landed and visible, operands (0,0) in set 0
+    aim(0);
+    copy_sb(0);
+    static_for<0, 13>([&](auto jc) { copy_one(s0, i0, 0, 0, jc); });
+    static_for<0, 13>([&](auto jc) { copy_one(s1, i1, BK, 1, jc); });
+    static_for<0, 13>([&](auto jc) { copy_one(s2, i2, 2 * BK, 2, jc); });
+    __builtin_amdgcn_s_waitcnt(kWaitVm26);
+    __syncthreads();
+    read_x(s0, C0{}, C0{}); read_x(s0, C0{}, C1{});
+    static_for<0, 4>([&](auto ac) { read_w(s0, C0{}, ac); });
+
+    // copy position: three K-tiles ahead of the compute position (ktiles >= 3, so at most one tile ahead); past the
+    // last tile the stream re-reads that tile and what it copies is never used
+    int dkt = 3 % ktiles, dseq = 3 / ktiles;
+    if (dseq == 1) {
+        if (my_tiles > 1) aim(1);
+        copy_sb(1);
+    }
+    auto advance_copy = [&]() {
+        if (++dkt == ktiles) {
+            dkt = 0;
+            if (++dseq < my_tiles) aim(dseq);
+            copy_sb(dseq & 1);
+        }
+    };
+
+    const int khalf4 = khalf * 4;
+    const bool vec_ok = (p.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.C) & 7u) == 0);
+    for (int seq = 0; seq < my_tiles; ++seq) {
+        int m0, n0;
+        tile_at(seq, m0, n0);
+        const int parity = seq & 1;
+        ktile(C0{}, 0, parity, dkt * BK, dkt);
+        rotate(); advance_copy();
+        for (int kt = 1; kt < ktiles; ++kt) {
+            ktile(C1{}, kt, parity, dkt * BK, dkt);
+            rotate(); advance_copy();
+        }
+        // the last K-tile's tiles 4..7, then the sums leave as bf16: a lane holds four consecutive columns per quad
+        static_for<4, 8>([&](auto ic) { fold_one(f, ic); });
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            const int m = m0 + wm * 64 + b * 32 + (lane & 31);
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int n = n0 + wn * 128 + a * 32 + g * 8 + khalf4;
+                    const uint32_t o01 = pack_bf16x2_hw(sum[a][b][g * 4 + 0], sum[a][b][g * 4 + 1]);
+                    const uint32_t o23 = pack_bf16x2_hw(sum[a][b][g * 4 + 2], sum[a][b][g * 4 + 3]);
+                    if (m < p.M) {
+                        uint16_t* crow = p.C + static_cast<size_t>(m) * p.ldc + n;
+                        if (vec_ok) {
+                            *reinterpret_cast<uint2*>(crow) = make_uint2(o01, o23);
+                        } else {
+                            crow[0] = static_cast<uint16_t>(o01 & 0xffffu); crow[1] = static_cast<uint16_t>(o01 >> 16);
+                            crow[2] = static_cast<uint16_t>(o23 & 0xffffu); crow[3] = static_cast<uint16_t>(o23 >> 16);
+                        }
+                    }
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) sum[a][b][g * 4 + q] = 0.0f;
+                }
+        }
+    }
+    // the copies started past the end of the stream must have landed before the LDS is given back
+    __builtin_amdgcn_s_waitcnt(kWaitVm0);
+}
+
 // ---- naive kernel: any shape, any alignment; also the on-device cross-check ----
 // one lane per output element, fp32 accumulate in k order
 __global__ __launch_bounds__(256) void k_gemm_nt_naive(const GemmArgs p, int fmt, int epi, int scale_mode) {
@@ -1190,6 +1481,24 @@ int gemm_nt(GemmArgs p, int fmt, int epi, int scale_mode, int force_naive, cf_st
         if (attr_err != hipSuccess) return static_cast<int>(attr_err);
         p.tiles_m = (p.M + BSM - 1) / BSM;
         p.tiles_n = (p.N + BN - 1) / BN;
+        const int kb = p.K / BK;
+        const bool ring_ok = p.K % BK == 0 && kb >= 3 && kb <= kBsMaxKb && p.N % BN == 0 && !p.force_staged &&
+                             static_cast<size_t>(p.M) * p.lda < (1ull << 32) && static_cast<size_t>(p.N) * p.ldb < (1ull << 32) &&
+                             static_cast<size_t>(p.M) * kb * 4 < (1ull << 32);
+        if (ring_ok) {
+            static std::once_flag once_ring;
+            static hipError_t ring_err = hipSuccess;
+            std::call_once(once_ring, [] {
+                ring_err = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_nt_block_ring),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, kBsLds);
+            });
+            if (ring_err != hipSuccess) return static_cast<int>(ring_err);
+            const int total = p.tiles_m * p.tiles_n;
+            int grid = total < num_cus() ? total : num_cus();
+            if (grid >= kXcds) grid -= grid % kXcds;
+            k_gemm_nt_block_ring<<<grid, kThreads, kBsLds, st>>>(p);
+            return launch_status();
+        }
         k_gemm_nt_block<<<p.tiles_m * p.tiles_n, kThreads, kBlkLds, st>>>(p);
         return launch_status();
     }

@@ -315,7 +315,9 @@ def block_quant_gpu(cf, dev, x_bf16, kind):
     return q, s, d
 
 
-@pytest.mark.parametrize("M,N,K", [(128, 256, 128), (256, 256, 256), (300, 200, 384), (130, 260, 208), (64, 512, 1024)])
+# (300, 512, 640), (1000, 256, 384), (3000, 768, 512): the persistent kernel (ragged rows; three K-tiles per tile; many tiles per workgroup)
+@pytest.mark.parametrize("M,N,K", [(128, 256, 128), (256, 256, 256), (300, 200, 384), (130, 260, 208), (64, 512, 1024),
+                                   (300, 512, 640), (1000, 256, 384), (3000, 768, 512)])
 @pytest.mark.parametrize("flags", [0, NAIVE])
 def test_gemm_block_scaled(cf, dev, M, N, K, flags):
     case(f"gemm block-scaled {M}x{N}x{K} flags={flags}")

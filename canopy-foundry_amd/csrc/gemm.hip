@@ -533,7 +533,8 @@ template <int EPI>
 struct TileScales {
     float sa[4];
     float4 cs[2][4];
-    float4 cs2[2][4];
+    float4 cs2[2][4];      // up-projection descales (SiLU-gate)
+    uint2 bs[2][4];        // bf16 bias of the same columns (bias epilogue)
 };
 
 template <int EPI, int SCALE>
@@ -547,12 +548,13 @@ __device__ __forceinline__ void load_row_scales(TileScales<EPI>& s, const GemmAr
     }
 }
 template <int EPI, int SCALE>
-__device__ __forceinline__ void load_pair_scales(float4 (&cs)[2][4], float4 (&cs2)[2][4], const GemmArgs& p, const TilePos& t,
-                                                 int wn, int lane, int pair) {
+__device__ __forceinline__ void load_pair_scales(float4 (&cs)[2][4], float4 (&cs2)[2][4], uint2 (&bs)[2][4], const GemmArgs& p,
+                                                 const TilePos& t, int wn, int lane, int pair) {
     constexpr int NU = EPI == EPI_SILU_GATE ? 2 : 4;
+    // uniform bases (scalar registers) + a small per-lane byte offset: no 64-bit per-lane addresses to keep alive
+    const size_t col0 = t.n0 + wn * (NU * 32) + pair * 64;
     if constexpr (SCALE == SCALE_ROWCOL) {
-        // uniform base (scalar registers) + a small per-lane byte offset: no 64-bit per-lane addresses to keep alive
-        const size_t ucol = static_cast<size_t>(t.expert) * p.sb_expert_stride + t.n0 + wn * (NU * 32) + pair * 64;
+        const size_t ucol = static_cast<size_t>(t.expert) * p.sb_expert_stride + col0;
         const uint8_t* b1 = reinterpret_cast<const uint8_t*>(p.sb + ucol);
         const uint8_t* b2 = reinterpret_cast<const uint8_t*>(EPI == EPI_SILU_GATE ? p.sb2 + ucol : p.sb);
         const uint32_t loff = static_cast<uint32_t>(lane >> 5) * 16u;
@@ -562,6 +564,16 @@ __device__ __forceinline__ void load_pair_scales(float4 (&cs)[2][4], float4 (&cs
             for (int g = 0; g < 4; ++g) {
                 cs[u][g] = *reinterpret_cast<const float4*>(b1 + (loff + u * 128u + g * 32u));
                 if constexpr (EPI == EPI_SILU_GATE) cs2[u][g] = *reinterpret_cast<const float4*>(b2 + (loff + u * 128u + g * 32u));
+            }
+    }
+    if constexpr (EPI == EPI_BIAS) {
+        const uint8_t* bb = reinterpret_cast<const uint8_t*>(p.bias + col0);
+        const uint32_t loff = static_cast<uint32_t>(lane >> 5) * 8u;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                bs[u][g] = *reinterpret_cast<const uint2*>(bb + (loff + u * 64u + g * 16u));
             }
     }
 }
@@ -601,8 +613,12 @@ __device__ __forceinline__ void drain_tile(v16f (&acc)[4][4], TileScales<EPI>& s
 
 #pragma unroll
     for (int pair = 0; pair < NU / 2; ++pair) {
+        // the next pair's factors are fetched while this pair is drained (the bias form, short of registers, fetches
+        // them at the turn instead)
+        constexpr bool PREFETCH = EPI != EPI_BIAS;
         float4 ncs[2][4], ncs2[2][4];
-        if (pair + 1 < NU / 2) load_pair_scales<EPI, SCALE>(ncs, ncs2, p, t, wn, lane, pair + 1);
+        uint2 nbs[2][4];
+        if (PREFETCH && pair + 1 < NU / 2) load_pair_scales<EPI, SCALE>(ncs, ncs2, nbs, p, t, wn, lane, pair + 1);
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
 #pragma unroll
@@ -632,6 +648,12 @@ __device__ __forceinline__ void drain_tile(v16f (&acc)[4][4], TileScales<EPI>& s
                                 v[q] = acc_read(acc[unit][b][g * 4 + q]) * (sa * c4[q]);
                             }
                         }
+                        if constexpr (EPI == EPI_BIAS) {
+                            // bias is added to the bf16 result, as the separate kernel does
+                            const uint32_t b01 = s.bs[uu][g].x, b23 = s.bs[uu][g].y;
+                            v[0] = round_bf16_hw(v[0]) + bf16_lo(b01); v[1] = round_bf16_hw(v[1]) + bf16_hi(b01);
+                            v[2] = round_bf16_hw(v[2]) + bf16_lo(b23); v[3] = round_bf16_hw(v[3]) + bf16_hi(b23);
+                        }
                         *reinterpret_cast<uint2*>(wr + bb * 32 * 128 + (((uu * 4 + g) ^ wswz) << 4)) =
                             make_uint2(pack_bf16x2_hw(v[0], v[1]), pack_bf16x2_hw(v[2], v[3]));
                     }
@@ -657,10 +679,14 @@ __device__ __forceinline__ void drain_tile(v16f (&acc)[4][4], TileScales<EPI>& s
             __builtin_amdgcn_sched_barrier(0);
         }
         if (pair + 1 < NU / 2) {
+            if constexpr (PREFETCH) {
 #pragma unroll
-            for (int u = 0; u < 2; ++u)
+                for (int u = 0; u < 2; ++u)
 #pragma unroll
-                for (int g = 0; g < 4; ++g) { s.cs[u][g] = ncs[u][g]; s.cs2[u][g] = ncs2[u][g]; }
+                    for (int g = 0; g < 4; ++g) { s.cs[u][g] = ncs[u][g]; s.cs2[u][g] = ncs2[u][g]; }
+            } else {
+                load_pair_scales<EPI, SCALE>(s.cs, s.cs2, s.bs, p, t, wn, lane, pair + 1);
+            }
         }
     }
 }
@@ -741,7 +767,7 @@ void k_gemm_nt_ring(const GemmArgs p) {
     constexpr int OUT_BN = GATE ? BN / 2 : BN;
     // the LDS-staged drain covers these epilogues; the launcher sends such a call here only when N is a multiple
     // of the tile's output width and C and the channel descales allow 16-byte accesses
-    constexpr bool DRAIN = EPI == EPI_NONE || EPI == EPI_SILU_GATE || EPI == EPI_ACCUM_F32;
+    constexpr bool DRAIN = EPI == EPI_NONE || EPI == EPI_BIAS || EPI == EPI_SILU_GATE || EPI == EPI_ACCUM_F32;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
@@ -911,7 +937,7 @@ void k_gemm_nt_ring(const GemmArgs p) {
             }
             if constexpr (END && DRAIN && EPI != EPI_ACCUM_F32 && i == 10) {
                 load_row_scales<EPI, SCALE>(sc, p, t, wm, lane);
-                load_pair_scales<EPI, SCALE>(sc.cs, sc.cs2, p, t, wn, lane, 0);
+                load_pair_scales<EPI, SCALE>(sc.cs, sc.cs2, sc.bs, p, t, wn, lane, 0);
             }
             __builtin_amdgcn_sched_barrier(0);
         });
@@ -1377,12 +1403,13 @@ int launch_tiled(const GemmArgs& p, hipStream_t st) {
         // its drain adds into full-width fp32 tiles with 16-byte accesses
         ring_ok = ring_ok && p.N % BN == 0 && p.ldc % 4 == 0 && aligned16(p.Cf);
     }
-    if constexpr (EPI == EPI_NONE || EPI == EPI_SILU_GATE) {
+    if constexpr (EPI == EPI_NONE || EPI == EPI_BIAS || EPI == EPI_SILU_GATE) {
         // its drain writes full-width tiles with 16-byte stores and reads the channel descales as float4
         constexpr int out_bn = EPI == EPI_SILU_GATE ? BN / 2 : BN;
         ring_ok = ring_ok && p.N % out_bn == 0 && p.ldc % 8 == 0 && aligned16(p.C);
         if (SCALE == SCALE_ROWCOL)
             ring_ok = ring_ok && aligned16(p.sb) && p.sb_expert_stride % 4 == 0 && (EPI != EPI_SILU_GATE || aligned16(p.sb2));
+        if (EPI == EPI_BIAS) ring_ok = ring_ok && (reinterpret_cast<uintptr_t>(p.bias) & 7u) == 0;
     }
     if (ring_ok && !p.force_staged) {
         static std::once_flag once_ring;

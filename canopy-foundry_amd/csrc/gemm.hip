@@ -1050,8 +1050,8 @@ void k_gemm_nt_ring(const GemmArgs p) {
 // the running sums (128, VGPRs, written by the vector ALU), one K-tile's partial products (128, the MFMA
 // accumulators) and the operands (64).  A K-tile is one scale group: its partial products start from a
 // zero C operand and are folded into the sums as sum += part * (sa[m, kt] * sb[n / 128, kt]), one
-// accumulator tile at a time, woven between the MFMAs of this and the next K-tile (a tile is folded after
-// its last MFMA has finished and before the next K-tile's first MFMA overwrites it).
+// accumulator tile at a time, half a tile per MFMA, woven between the MFMAs of this and the next K-tile (a tile
+// is folded after its last MFMA has finished and before the next K-tile's first MFMA overwrites it).
 // LDS: three stages of (X 16 KiB + W 32 KiB); K-tile g lives in stage g % 3, K-tiles g+1 and g+2 are resident or
 // landing, and the copies of K-tile g+3 go into stage g % 3 right after the barrier that ends its use.  The
 // activation scales of a K-tile travel with it (one 4-byte copy per row into the stage's scale row), the
@@ -1191,13 +1191,13 @@ void k_gemm_nt_block_ring(const GemmArgs p) {
         }
         part[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wq[a], xq[H][b], c, 0, 0, 0, 0, 0, 0);
     };
-    // fold accumulator tile I of the K-tile whose factors are f[0], f[1] into the sums
-    auto fold_one = [&](const float (&f)[2], auto ic) {
-        constexpr int I = decltype(ic)::value;
+    // fold half HALF (8 of the 16 registers) of accumulator tile I of the K-tile whose factors are f[0], f[1] into the sums
+    auto fold_half = [&](const float (&f)[2], auto ic, auto hc) {
+        constexpr int I = decltype(ic)::value, HALF = decltype(hc)::value;
         constexpr int a = I >> 1, b = I & 1;
         // volatile: the folds must stay woven between the MFMAs where they are written, not sink behind them
 #pragma unroll
-        for (int r = 0; r < 16; r += 4) {
+        for (int r = HALF * 8; r < HALF * 8 + 8; r += 4) {
             // four reads, then four multiply-adds: no instruction waits on the one before it
             float t0, t1, t2, t3, v0 = sum[a][b][r], v1 = sum[a][b][r + 1], v2 = sum[a][b][r + 2], v3 = sum[a][b][r + 3];
             const float p0 = part[a][b][r], p1 = part[a][b][r + 1], p2 = part[a][b][r + 2], p3 = part[a][b][r + 3], fv = f[b];
@@ -1207,6 +1207,10 @@ void k_gemm_nt_block_ring(const GemmArgs p) {
                          : "a"(p0), "a"(p1), "a"(p2), "a"(p3), "v"(fv));
             sum[a][b][r] = v0; sum[a][b][r + 1] = v1; sum[a][b][r + 2] = v2; sum[a][b][r + 3] = v3;
         }
+    };
+    auto fold_one = [&](const float (&f)[2], auto ic) {
+        fold_half(f, ic, std::integral_constant<int, 0>{});
+        fold_half(f, ic, std::integral_constant<int, 1>{});
     };
     using C0 = std::integral_constant<int, 0>;
     using C1 = std::integral_constant<int, 1>;
@@ -1222,7 +1226,8 @@ void k_gemm_nt_block_ring(const GemmArgs p) {
         // step (g,0): 8 MFMAs from a zero C, the operand reads of (g,1), folds 4..7 of K-tile g-1
         static_for<0, 8>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
-            if constexpr (FOLD && i < 4) fold_one(f, std::integral_constant<int, 4 + (i < 4 ? i : 0)>{});
+            // half a fold per MFMA: tiles 4..7 of the previous K-tile, each finished before the MFMA that overwrites it
+            if constexpr (FOLD) fold_half(f, std::integral_constant<int, 4 + i / 2>{}, std::integral_constant<int, i % 2>{});
             mfma_one(C0{}, ic);
             if constexpr (i == 0) read_x(s0, C1{}, C0{});
             if constexpr (i == 1) read_x(s0, C1{}, C1{});
@@ -1254,8 +1259,10 @@ void k_gemm_nt_block_ring(const GemmArgs p) {
             copy_one(s0, i0, dk0, dkt, std::integral_constant<int, 2 * (i - 2)>{});
             copy_one(s0, i0, dk0, dkt, std::integral_constant<int, 2 * (i - 2) + 1>{});
             if constexpr (i == 7) copy_one(s0, i0, dk0, dkt, std::integral_constant<int, 12>{});
-            // folds 0..3 of this K-tile, each four MFMAs after the one that finished its tile
-            if constexpr (i >= 4) fold_one(f, std::integral_constant<int, i >= 4 ? i - 4 : 0>{});
+            // this K-tile's tiles 0..3: two whole folds first (the schedule is two halves short otherwise), then halves
+            if constexpr (i == 2) fold_one(f, C0{});
+            if constexpr (i == 3) fold_one(f, C1{});
+            if constexpr (i >= 4) fold_half(f, std::integral_constant<int, 2 + (i >= 4 ? (i - 4) / 2 : 0)>{}, std::integral_constant<int, i % 2>{});
             __builtin_amdgcn_sched_barrier(0);
         });
         read_w(s1, C0{}, std::integral_constant<int, 3>{});

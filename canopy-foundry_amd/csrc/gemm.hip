@@ -1046,17 +1046,19 @@ void k_gemm_nt_ring(const GemmArgs p) {
 // ---- block-scaled ring kernel ---------------------------------------------------------------
 // The block-scaled GEMM on the persistent direct-to-LDS structure.  Needs K % 128 == 0, K >= 384,
 // N % 256 == 0, operands smaller than 4 GiB, K / 128 <= 256.
-// Workgroup tile 128 x 256 x 128, four wavefronts 2 x 2, each 64 x 128 = 4 x 2 MFMA tiles.  Registers:
-// the running sums (128, VGPRs, written by the vector ALU), one K-tile's partial products (128, the MFMA
-// accumulators) and the operands (64).  A K-tile is one scale group: its partial products start from a
-// zero C operand and are folded into the sums as sum += part * (sa[m, kt] * sb[n / 128, kt]), one
-// accumulator tile at a time, half a tile per MFMA, woven between the MFMAs of this and the next K-tile (a tile
-// is folded after its last MFMA has finished and before the next K-tile's first MFMA overwrites it).
+// A K-tile is one scale group: its partial products start from a zero C operand and are folded into running
+// sums as sum += part * (sa[m, kt] * sb[n / 128, kt]).  The fold is vector-ALU work in the inner loop (one
+// multiply-add per accumulator element and K-tile), so this kernel runs TWO wavefronts per SIMD: the folds of
+// one hide behind the MFMAs of the other, and with a 256-register budget per wavefront the MFMAs write their
+// results to ordinary VGPRs, where the fold can read them (reading accumulation registers stalls while an MFMA
+// is in flight).  Workgroup tile 128 x 256 x 128, eight wavefronts 2 x 4, each 64 x 64 = 2 x 2 MFMA tiles:
+// sums 64 registers, partial products 64, two operand sets 64.
 // LDS: three stages of (X 16 KiB + W 32 KiB); K-tile g lives in stage g % 3, K-tiles g+1 and g+2 are resident or
 // landing, and the copies of K-tile g+3 go into stage g % 3 right after the barrier that ends its use.  The
 // activation scales of a K-tile travel with it (one 4-byte copy per row into the stage's scale row), the
 // weight-block scales of a tile (one per K-tile) are copied once per tile; the scale factors are therefore
 // read from LDS and never wait on the copy pipeline.
+constexpr int kBsThreads = 512;
 constexpr int kBsX = BSM * BK;                          // 16 KiB
 constexpr int kBsW = BN * BK;                           // 32 KiB
 constexpr int kBsStage = kBsX + kBsW;                   // 48 KiB
@@ -1064,15 +1066,15 @@ constexpr int kBsSa = 3 * kBsStage;                     // activation scales: 3 
 constexpr int kBsSb = kBsSa + 3 * BSM * 4;              // weight-block scales: 2 tile parities x 2 column blocks x 256 floats
 constexpr int kBsMaxKb = 256;
 constexpr int kBsLds = kBsSb + 2 * 2 * kBsMaxKb * 4;    // 153,088 bytes
-constexpr int kBsCopies = 13;                           // copy instructions per wavefront and K-tile (4 X, 8 W, 1 scales)
-constexpr int kWaitVm13 = 0x0f7d, kWaitVm26 = 0x4f7a;
+constexpr int kBsCopies = 7;                            // copy instructions per wavefront and K-tile (2 X, 4 W, 1 scales)
+constexpr int kWaitVm7 = 0x0f77, kWaitVm14 = 0x0f7e;
 
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1)))
+__global__ __launch_bounds__(kBsThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void k_gemm_nt_block_ring(const GemmArgs p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);      // 0..7
+    const int wm = wave >> 2, wn = wave & 3;
     const int ktiles = p.K / BK;          // >= 3, checked by the launcher; also the number of scale groups along K
     const int total_tiles = p.tiles_m * p.tiles_n;
     int my_tiles, lin0, lstep;
@@ -1096,44 +1098,45 @@ void k_gemm_nt_block_ring(const GemmArgs p) {
         n0 = tn * BN;
     };
 
-    // ---- global -> LDS ----
+    // ---- global -> LDS: wave w copies X rows [16w, 16w+16), W rows [32w, 32w+32), the scales of X rows [16w, 16w+16) ----
     const int lrow = lane >> 3, lslot = lane & 7;
-    uint32_t xoff[4], woff[8], saoff = 0;              // per-lane byte offsets
-    const uint8_t* sbsrc = nullptr;                    // the tile's row of weight-block scales (wave's column block)
+    uint32_t xoff[2], woff[4], saoff = 0;              // per-lane byte offsets
+    const uint8_t* sbsrc = nullptr;                    // the tile's rows of weight-block scales
     auto aim = [&](int seq) {
         int m0, n0;
         tile_at(seq, m0, n0);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int row = wave * 32 + j * 8 + lrow;
+        for (int j = 0; j < 2; ++j) {
+            const int row = wave * 16 + j * 8 + lrow;
             xoff[j] = static_cast<uint32_t>(min(m0 + row, p.M - 1)) * static_cast<uint32_t>(p.lda) + (lslot ^ swz(row)) * 16;
         }
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const int row = wave * 64 + j * 8 + lrow;
+        for (int j = 0; j < 4; ++j) {
+            const int row = wave * 32 + j * 8 + lrow;
             woff[j] = static_cast<uint32_t>(min(n0 + row, p.N - 1)) * static_cast<uint32_t>(p.ldb) + (lslot ^ swz(row)) * 16;
         }
-        saoff = static_cast<uint32_t>(min(m0 + wave * 32 + (lane & 31), p.M - 1)) * static_cast<uint32_t>(ktiles) * 4u;
+        saoff = static_cast<uint32_t>(min(m0 + wave * 16 + (lane & 15), p.M - 1)) * static_cast<uint32_t>(ktiles) * 4u;
         sbsrc = reinterpret_cast<const uint8_t*>(p.sb + static_cast<size_t>((n0 >> 7) + (wave & 1)) * ktiles);
     };
     uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(smem));
     auto dma16 = [&](uint32_t dst, uint32_t voff, const uint8_t* base) {
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(voff), "s"(base) : "memory");
     };
-    // 4-byte copies by the low 32 lanes only: lane l lands at dst + 4 l
-    auto dma4_lo32 = [&](uint32_t dst, uint32_t voff, const uint8_t* base) {
-        asm volatile("s_mov_b32 m0, %0\n\ts_mov_b32 exec_hi, 0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2\n\ts_mov_b32 exec_hi, -1\n\ts_nop 0"
+    // 4-byte copies by the low 16 lanes only: lane l lands at dst + 4 l
+    auto dma4_lo16 = [&](uint32_t dst, uint32_t voff, const uint8_t* base) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_mov_b32 exec_lo, 0xffff\n\ts_mov_b32 exec_hi, 0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2\n\t"
+                     "s_mov_b32 exec_lo, -1\n\ts_mov_b32 exec_hi, -1\n\ts_nop 0"
                      :: "s"(dst), "v"(voff), "s"(base) : "memory");
     };
     auto dma4 = [&](uint32_t dst, uint32_t voff, const uint8_t* base) {
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" :: "s"(dst), "v"(voff), "s"(base) : "memory");
     };
-    // copy J (0..12) of the K-tile at K offset k0 into stage offset `stage`
+    // copy J (0..6) of the K-tile at K offset k0 (scale group kt) into the stage at `stage` (scale row sidx)
     auto copy_one = [&](int stage, int sidx, int k0, int kt, auto jc) {
         constexpr int J = decltype(jc)::value;
-        if constexpr (J < 4)       dma16(lds0 + stage + (wave * 32 + J * 8) * BK, xoff[J], p.A + k0);
-        else if constexpr (J < 12) dma16(lds0 + stage + kBsX + (wave * 64 + (J - 4) * 8) * BK, woff[J - 4], p.B + k0);
-        else                       dma4_lo32(lds0 + kBsSa + sidx * (BSM * 4) + wave * 128, saoff, reinterpret_cast<const uint8_t*>(p.sa + kt));
+        if constexpr (J < 2)      dma16(lds0 + stage + (wave * 16 + J * 8) * BK, xoff[J], p.A + k0);
+        else if constexpr (J < 6) dma16(lds0 + stage + kBsX + (wave * 32 + (J - 2) * 8) * BK, woff[J - 2], p.B + k0);
+        else                      dma4_lo16(lds0 + kBsSa + sidx * (BSM * 4) + wave * 64, saoff, reinterpret_cast<const uint8_t*>(p.sa + kt));
     };
     // the weight-block scales of the tile the stream has just turned to: up to four copies of 64 floats by waves 0 and 1
     // (one per column block), into the half of the scale table selected by the tile's parity
@@ -1154,32 +1157,28 @@ void k_gemm_nt_block_ring(const GemmArgs p) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) rd[h][j] = frow * BK + (((h * 4 + khalf * 2 + j) ^ fs) << 4);
     const uint8_t* xrd = smem + wm * 64 * BK;
-    const uint8_t* wrd = smem + kBsX + wn * 128 * BK;
+    const uint8_t* wrd = smem + kBsX + wn * 64 * BK;
 
-    v16f part[4][2];      // [weight tile][activation tile]: this K-tile's partial products (MFMA accumulators)
-    v16f sum[4][2];       // running sums, already scaled
+    v16f part[2][2];      // [weight tile][activation tile]: this K-tile's partial products
+    v16f sum[2][2];       // running sums, already scaled
 #pragma unroll
-    for (int a = 0; a < 4; ++a)
+    for (int a = 0; a < 2; ++a)
 #pragma unroll
         for (int b = 0; b < 2; ++b)
 #pragma unroll
             for (int r = 0; r < 16; ++r) sum[a][b][r] = 0.0f;
-    // Operand registers: one set of the four weight tiles (a tile is re-read for the next step as soon as both
-    // MFMAs of the current step that use it have issued: three tiles ahead of its next use) and two sets of the
-    // two activation tiles (k-half h of any K-tile lives in set h).
-    v8i wq[4], xq[2][2];
+    v8i wq[2][2], xq[2][2];       // two operand sets: k-half h of any K-tile lives in set h
     auto put = [](v8i& dst, int half, const uint4 v) {
         dst[4 * half + 0] = (int)v.x; dst[4 * half + 1] = (int)v.y; dst[4 * half + 2] = (int)v.z; dst[4 * half + 3] = (int)v.w;
     };
-    auto read_w = [&](int stage, auto hc, auto ac) {       // weight tile A of k-half H from the stage at `stage`
-        constexpr int H = decltype(hc)::value, A = decltype(ac)::value;
-        put(wq[A], 0, *reinterpret_cast<const uint4*>(wrd + stage + A * 32 * BK + rd[H][0]));
-        put(wq[A], 1, *reinterpret_cast<const uint4*>(wrd + stage + A * 32 * BK + rd[H][1]));
-    };
-    auto read_x = [&](int stage, auto hc, auto bc) {       // activation tile B of k-half H
-        constexpr int H = decltype(hc)::value, B = decltype(bc)::value;
-        put(xq[H][B], 0, *reinterpret_cast<const uint4*>(xrd + stage + B * 32 * BK + rd[H][0]));
-        put(xq[H][B], 1, *reinterpret_cast<const uint4*>(xrd + stage + B * 32 * BK + rd[H][1]));
+    // read I (0..7) of k-half H from the stage at `stage`: w0 x0 x1 w1, two reads each
+    auto read_one = [&](int stage, auto hc, auto ic) {
+        constexpr int H = decltype(hc)::value, I = decltype(ic)::value;
+        constexpr int t = I >> 1, half = I & 1;
+        const int r = rd[H][half];
+        if constexpr (t == 0)      put(wq[H][0], half, *reinterpret_cast<const uint4*>(wrd + stage + r));
+        else if constexpr (t <= 2) put(xq[H][t - 1], half, *reinterpret_cast<const uint4*>(xrd + stage + (t - 1) * 32 * BK + r));
+        else                       put(wq[H][1], half, *reinterpret_cast<const uint4*>(wrd + stage + 32 * BK + r));
     };
     auto mfma_one = [&](auto hc, auto ic) {
         constexpr int H = decltype(hc)::value, I = decltype(ic)::value;
@@ -1189,83 +1188,79 @@ void k_gemm_nt_block_ring(const GemmArgs p) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) c[r] = 0.0f;
         }
-        part[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wq[a], xq[H][b], c, 0, 0, 0, 0, 0, 0);
+        part[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wq[H][a], xq[H][b], c, 0, 0, 0, 0, 0, 0);
     };
-    // fold half HALF (8 of the 16 registers) of accumulator tile I of the K-tile whose factors are f[0], f[1] into the sums
-    auto fold_half = [&](const float (&f)[2], auto ic, auto hc) {
-        constexpr int I = decltype(ic)::value, HALF = decltype(hc)::value;
+    // fold accumulator tile I of the K-tile whose factors are f[0], f[1] into the sums
+    auto fold_one = [&](const float (&f)[2], auto ic) {
+        constexpr int I = decltype(ic)::value;
         constexpr int a = I >> 1, b = I & 1;
-        // volatile: the folds must stay woven between the MFMAs where they are written, not sink behind them
+        // volatile: the folds must stay between the MFMAs where they are written (the producing MFMA is at least
+        // three MFMAs back there), not be gathered at the end of the loop body
+        const float fv = f[b];
 #pragma unroll
-        for (int r = HALF * 8; r < HALF * 8 + 8; r += 4) {
-            // four reads, then four multiply-adds: no instruction waits on the one before it
-            float t0, t1, t2, t3, v0 = sum[a][b][r], v1 = sum[a][b][r + 1], v2 = sum[a][b][r + 2], v3 = sum[a][b][r + 3];
-            const float p0 = part[a][b][r], p1 = part[a][b][r + 1], p2 = part[a][b][r + 2], p3 = part[a][b][r + 3], fv = f[b];
-            asm volatile("v_accvgpr_read_b32 %4, %8\n\tv_accvgpr_read_b32 %5, %9\n\tv_accvgpr_read_b32 %6, %10\n\tv_accvgpr_read_b32 %7, %11\n\t"
-                         "v_fmac_f32 %0, %4, %12\n\tv_fmac_f32 %1, %5, %12\n\tv_fmac_f32 %2, %6, %12\n\tv_fmac_f32 %3, %7, %12"
-                         : "+v"(v0), "+v"(v1), "+v"(v2), "+v"(v3), "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3)
-                         : "a"(p0), "a"(p1), "a"(p2), "a"(p3), "v"(fv));
+        for (int r = 0; r < 16; r += 8) {
+            float v0 = sum[a][b][r], v1 = sum[a][b][r + 1], v2 = sum[a][b][r + 2], v3 = sum[a][b][r + 3];
+            float v4 = sum[a][b][r + 4], v5 = sum[a][b][r + 5], v6 = sum[a][b][r + 6], v7 = sum[a][b][r + 7];
+            const float p0 = part[a][b][r], p1 = part[a][b][r + 1], p2 = part[a][b][r + 2], p3 = part[a][b][r + 3];
+            const float p4 = part[a][b][r + 4], p5 = part[a][b][r + 5], p6 = part[a][b][r + 6], p7 = part[a][b][r + 7];
+            asm volatile("v_fmac_f32 %0, %8, %16\n\tv_fmac_f32 %1, %9, %16\n\tv_fmac_f32 %2, %10, %16\n\tv_fmac_f32 %3, %11, %16\n\t"
+                         "v_fmac_f32 %4, %12, %16\n\tv_fmac_f32 %5, %13, %16\n\tv_fmac_f32 %6, %14, %16\n\tv_fmac_f32 %7, %15, %16"
+                         : "+v"(v0), "+v"(v1), "+v"(v2), "+v"(v3), "+v"(v4), "+v"(v5), "+v"(v6), "+v"(v7)
+                         : "v"(p0), "v"(p1), "v"(p2), "v"(p3), "v"(p4), "v"(p5), "v"(p6), "v"(p7), "v"(fv));
             sum[a][b][r] = v0; sum[a][b][r + 1] = v1; sum[a][b][r + 2] = v2; sum[a][b][r + 3] = v3;
+            sum[a][b][r + 4] = v4; sum[a][b][r + 5] = v5; sum[a][b][r + 6] = v6; sum[a][b][r + 7] = v7;
         }
     };
-    auto fold_one = [&](const float (&f)[2], auto ic) {
-        fold_half(f, ic, std::integral_constant<int, 0>{});
-        fold_half(f, ic, std::integral_constant<int, 1>{});
+    // the same fold in plain arithmetic, for the end of a tile, where the last MFMA has only just been issued
+    auto fold_plain = [&](const float (&f)[2], auto ic) {
+        constexpr int I = decltype(ic)::value;
+        constexpr int a = I >> 1, b = I & 1;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sum[a][b][r] = __builtin_fmaf(part[a][b][r], f[b], sum[a][b][r]);
     };
     using C0 = std::integral_constant<int, 0>;
     using C1 = std::integral_constant<int, 1>;
 
     int s0 = 0, s1 = kBsStage, s2 = 2 * kBsStage;      // stage offsets of K-tiles g, g+1, g+2
     int i0 = 0, i1 = 1, i2 = 2;                        // and their indices (for the scale rows)
-    float f[2] = {0.0f, 0.0f};                         // factors of the K-tile whose tiles 4..7 are still to be folded
+    float f[2] = {0.0f, 0.0f};                         // factors of the K-tile whose partial products are still to be folded
 
-    // One K-tile g at position kt of its tile.  FOLD: tiles 4..7 of the previous K-tile are folded first (not for a
-    // tile's first K-tile).  After the barrier the copies of K-tile g+3 (K offset dk0, position dkt of its tile) start.
+    // One K-tile g at position kt of its tile.  FOLD: the previous K-tile's partial products are folded, each tile
+    // right before the MFMA that overwrites it (not for a tile's first K-tile).  After the barrier the copies of
+    // K-tile g+3 (K offset dk0, position dkt of its tile) start.
     auto ktile = [&](auto fold_c, int kt, int parity, int dk0, int dkt) {
         constexpr bool FOLD = decltype(fold_c)::value != 0;
-        // step (g,0): 8 MFMAs from a zero C, the operand reads of (g,1), folds 4..7 of K-tile g-1
-        static_for<0, 8>([&](auto ic) {
+        // step (g,0): 4 MFMAs from a zero C, the operand reads of (g,1)
+        static_for<0, 4>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
-            // half a fold per MFMA: tiles 4..7 of the previous K-tile, each finished before the MFMA that overwrites it
-            if constexpr (FOLD) fold_half(f, std::integral_constant<int, 4 + i / 2>{}, std::integral_constant<int, i % 2>{});
+            if constexpr (FOLD) fold_one(f, ic);
             mfma_one(C0{}, ic);
-            if constexpr (i == 0) read_x(s0, C1{}, C0{});
-            if constexpr (i == 1) read_x(s0, C1{}, C1{});
-            if constexpr (i == 2 || i == 4 || i == 6) read_w(s0, C1{}, std::integral_constant<int, (i - 2) / 2>{});
+            read_one(s0, C1{}, std::integral_constant<int, 2 * i>{});
+            read_one(s0, C1{}, std::integral_constant<int, 2 * i + 1>{});
             __builtin_amdgcn_sched_barrier(0);
         });
-        read_w(s0, C1{}, std::integral_constant<int, 3>{});
         // this K-tile's factors: read before the barrier, after which its scale row may be overwritten
-        const float sbv = *reinterpret_cast<const float*>(smem + kBsSb + (parity * 2 + wn) * (kBsMaxKb * 4) + kt * 4);
-        float fn[2];
+        const float sbv = *reinterpret_cast<const float*>(smem + kBsSb + (parity * 2 + (wn >> 1)) * (kBsMaxKb * 4) + kt * 4);
 #pragma unroll
         for (int b = 0; b < 2; ++b)
-            fn[b] = *reinterpret_cast<const float*>(smem + kBsSa + i0 * (BSM * 4) + (wm * 64 + b * 32 + (lane & 31)) * 4) * sbv;
+            f[b] = *reinterpret_cast<const float*>(smem + kBsSa + i0 * (BSM * 4) + (wm * 64 + b * 32 + (lane & 31)) * 4) * sbv;
         // step (g,1)
         mfma_one(C1{}, C0{});
-        mfma_one(C1{}, C1{});
         __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_waitcnt(kWaitVm13);
+        __builtin_amdgcn_s_waitcnt(kWaitVm7);
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
-        f[0] = fn[0]; f[1] = fn[1];
-        static_for<2, 8>([&](auto ic) {
+        static_for<1, 4>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
             mfma_one(C1{}, ic);
-            if constexpr (i == 2) read_x(s1, C0{}, C0{});
-            if constexpr (i == 3) read_x(s1, C0{}, C1{});
-            if constexpr (i == 2 || i == 4 || i == 6) read_w(s1, C0{}, std::integral_constant<int, (i - 2) / 2>{});
-            // 13 copies over six slots
-            copy_one(s0, i0, dk0, dkt, std::integral_constant<int, 2 * (i - 2)>{});
-            copy_one(s0, i0, dk0, dkt, std::integral_constant<int, 2 * (i - 2) + 1>{});
-            if constexpr (i == 7) copy_one(s0, i0, dk0, dkt, std::integral_constant<int, 12>{});
-            // this K-tile's tiles 0..3: two whole folds first (the schedule is two halves short otherwise), then halves
-            if constexpr (i == 2) fold_one(f, C0{});
-            if constexpr (i == 3) fold_one(f, C1{});
-            if constexpr (i >= 4) fold_half(f, std::integral_constant<int, 2 + (i >= 4 ? (i - 4) / 2 : 0)>{}, std::integral_constant<int, i % 2>{});
+            // 8 reads and 7 copies over three slots
+            static_for<0, 3>([&](auto jc) {
+                constexpr int j = (i - 1) * 3 + decltype(jc)::value;
+                if constexpr (j < 8) read_one(s1, C0{}, std::integral_constant<int, j < 8 ? j : 0>{});
+                if constexpr (j < 7) copy_one(s0, i0, dk0, dkt, std::integral_constant<int, j < 7 ? j : 0>{});
+            });
             __builtin_amdgcn_sched_barrier(0);
         });
-        read_w(s1, C0{}, std::integral_constant<int, 3>{});
     };
     auto rotate = [&]() {
         const int t = s0, u = i0;
@@ -1276,13 +1271,12 @@ void k_gemm_nt_block_ring(const GemmArgs p) {
     // prologue: K-tiles 0, 1, 2 of the stream in flight, K-tile 0 landed and visible, operands (0,0) in set 0
     aim(0);
     copy_sb(0);
-    static_for<0, 13>([&](auto jc) { copy_one(s0, i0, 0, 0, jc); });
-    static_for<0, 13>([&](auto jc) { copy_one(s1, i1, BK, 1, jc); });
-    static_for<0, 13>([&](auto jc) { copy_one(s2, i2, 2 * BK, 2, jc); });
-    __builtin_amdgcn_s_waitcnt(kWaitVm26);
+    static_for<0, 7>([&](auto jc) { copy_one(s0, i0, 0, 0, jc); });
+    static_for<0, 7>([&](auto jc) { copy_one(s1, i1, BK, 1, jc); });
+    static_for<0, 7>([&](auto jc) { copy_one(s2, i2, 2 * BK, 2, jc); });
+    __builtin_amdgcn_s_waitcnt(kWaitVm14);
     __syncthreads();
-    read_x(s0, C0{}, C0{}); read_x(s0, C0{}, C1{});
-    static_for<0, 4>([&](auto ac) { read_w(s0, C0{}, ac); });
+    static_for<0, 8>([&](auto ic) { read_one(s0, C0{}, ic); });
 
     // copy position: three K-tiles ahead of the compute position (ktiles >= 3, so at most one tile ahead); past the
     // last tile the stream re-reads that tile and what it copies is never used
@@ -1311,16 +1305,16 @@ void k_gemm_nt_block_ring(const GemmArgs p) {
             ktile(C1{}, kt, parity, dkt * BK, dkt);
             rotate(); advance_copy();
         }
-        // the last K-tile's tiles 4..7, then the sums leave as bf16: a lane holds four consecutive columns per quad
-        static_for<4, 8>([&](auto ic) { fold_one(f, ic); });
+        // the last K-tile's partial products, then the sums leave as bf16: a lane holds four consecutive columns per quad
+        static_for<0, 4>([&](auto ic) { fold_plain(f, ic); });
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
             const int m = m0 + wm * 64 + b * 32 + (lane & 31);
 #pragma unroll
-            for (int a = 0; a < 4; ++a)
+            for (int a = 0; a < 2; ++a)
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                    const int n = n0 + wn * 128 + a * 32 + g * 8 + khalf4;
+                    const int n = n0 + wn * 64 + a * 32 + g * 8 + khalf4;
                     const uint32_t o01 = pack_bf16x2_hw(sum[a][b][g * 4 + 0], sum[a][b][g * 4 + 1]);
                     const uint32_t o23 = pack_bf16x2_hw(sum[a][b][g * 4 + 2], sum[a][b][g * 4 + 3]);
                     if (m < p.M) {
@@ -1530,7 +1524,7 @@ int gemm_nt(GemmArgs p, int fmt, int epi, int scale_mode, int force_naive, cf_st
             const int total = p.tiles_m * p.tiles_n;
             int grid = total < num_cus() ? total : num_cus();
             if (grid >= kXcds) grid -= grid % kXcds;
-            k_gemm_nt_block_ring<<<grid, kThreads, kBsLds, st>>>(p);
+            k_gemm_nt_block_ring<<<grid, kBsThreads, kBsLds, st>>>(p);
             return launch_status();
         }
         k_gemm_nt_block<<<p.tiles_m * p.tiles_n, kThreads, kBlkLds, st>>>(p);

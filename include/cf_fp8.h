@@ -136,6 +136,43 @@ int cf_swiglu_forward(const uint16_t* d_gate, const uint16_t* d_up, uint16_t* d_
 int cf_bias_add_strided_bf16(uint16_t* d_inout, const uint16_t* d_bias, int rows, int cols,
                              int row_stride, int base, cf_stream_t stream);
 
+/* ---- producers of the quantizer's input, fused with it ---------------------
+ * The reference normalises, clips and quantizes an activation in four launches
+ * (src/trainer.cu:6281-6304: rmsnorm_forward, act_row_clip, fp8_quant_act); the
+ * fused forms below give the same bytes in one pass over the row.  All of them
+ * follow the reference's reduction trees, so the bf16 results are bit-identical
+ * to the launch sequence.  Shapes: H <= 16384 and min(H, 512) a multiple of 32
+ * (the reference's full-mask shuffles are defined for whole 32-lane groups
+ * only); anything else is CF_ERR_UNSUPPORTED.  Rows move as 16-byte vectors
+ * when H % 8 == 0 and the row pointers are 16-byte aligned (fp8 rows 8-byte). */
+
+/* rmsnorm_forward, kernels.hpp:117, kernels/rmsnorm.cu:13-54,101-108.
+ * d_rms may be null.  d_out may alias d_x. */
+int cf_rmsnorm_forward(const uint16_t* d_x, const uint16_t* d_scale, uint16_t* d_out, float* d_rms,
+                       int rows, int H, float eps, cf_stream_t stream);
+/* act_row_clip in its fixed-ceiling mode, src/trainer.cu:3968-3991 (static;
+ * kernels :3822-3842, :3940-3958) without the optional statistics: rows whose
+ * L2 norm exceeds `ceiling` are scaled down to it in place; ceiling <= 0 is a
+ * no-op (:3974).  d_normsq[rows] receives the row sums of squares as the
+ * reference's scratch does; may be null. */
+int cf_act_row_clip_abs(uint16_t* d_x, int rows, int cols, float ceiling, float* d_normsq,
+                        cf_stream_t stream);
+/* rmsnorm_forward -> act_row_clip(ceiling) -> per-row quantize (cf_fp8_quantize_rows)
+ * in one launch (the sequence at src/trainer.cu:6281-6304 with per-token scales).  d_normed (the bf16 normalised, clipped row, which the
+ * reference keeps for the router and the weight gradient) and d_rms may be null. */
+int cf_rmsnorm_clip_quantize_rows(const uint16_t* d_x, const uint16_t* d_scale, int rows, int H,
+                                  float eps, float ceiling, int is_e5m2, uint16_t* d_normed,
+                                  float* d_rms, void* d_q, float* d_row_scale,
+                                  float* d_row_descale, cf_stream_t stream);
+/* rmsnorm_forward -> act_row_clip(ceiling) -> fp8_quantize_e4m3_record /
+ * _e5m2_record (kernels/fp8.cu:67-103, 310-330): quantize with *d_qscale and
+ * raise *d_amax to the tensor's maximum (the caller zeroes it, as for
+ * cf_fp8_quantize_e4m3_record). */
+int cf_rmsnorm_clip_quantize_record(const uint16_t* d_x, const uint16_t* d_scale, int rows, int H,
+                                    float eps, float ceiling, int is_e5m2, uint16_t* d_normed,
+                                    float* d_rms, void* d_q, const float* d_qscale,
+                                    float* d_amax, cf_stream_t stream);
+
 /* ---- scaled FP8 GEMM -------------------------------------------------------
  * Replaces the reference's cuBLASLt wrappers, which are static functions of
  * src/trainer.cu bound to its Fp8Ctx (handle, workspace, plan cache); the

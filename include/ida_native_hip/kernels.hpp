@@ -103,6 +103,12 @@ inline void bias_add_strided_bf16(bf16* d_inout, const bf16* d_bias, int rows, i
     CF_FWD(cf_bias_add_strided_bf16(hip_detail::u(d_inout), hip_detail::u(d_bias), rows, cols, row_stride, base, stream));
 }
 
+// ---- kernels.hpp:117-120 (kernels/rmsnorm.cu) ---------------------------------------------------------------
+inline void rmsnorm_forward(const bf16* d_x, const bf16* d_scale, bf16* d_out, float* d_rms, int rows, int H, float eps,
+                            hipStream_t stream) {
+    CF_FWD(cf_rmsnorm_forward(hip_detail::u(d_x), hip_detail::u(d_scale), hip_detail::u(d_out), d_rms, rows, H, eps, stream));
+}
+
 // ---- kernels.hpp:193, 313-317, 340-343, 361-423 (kernels/cross_entropy.cu, kernels/moe.cu) -----------------
 inline void softmax_inplace_f32(float* d_x, int rows, int cols, hipStream_t stream) {
     CF_FWD(cf_softmax_inplace_f32(d_x, rows, cols, stream));

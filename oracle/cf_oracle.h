@@ -33,6 +33,10 @@
  *                                 dense sweep (it is this build's definition of
  *                                 the router's expf; CUDA's expf bits cannot be
  *                                 obtained here: parity unpinned beyond ulp level).
+ *   rmsnorm / row clip            see cf_oracle_norm.c (closed forms, double
+ *                                 recomputation, order-sensitive crafted row;
+ *                                 summation order beyond the source text:
+ *                                 parity unpinned).
  *   GEMM references               definition from the task statement: matmul
  *                                 of the dequantised operands; special cases
  *                                 reduce to numpy matmul.  cuBLASLt's own
@@ -112,6 +116,15 @@ void orc_quantize_block_128x128(const uint16_t* x, int rows, int K,
 void orc_swiglu_forward(const uint16_t* gate, const uint16_t* up, uint16_t* out, int n);
 void orc_bias_add_strided_bf16(uint16_t* inout, const uint16_t* bias,
                                int rows, int cols, int row_stride, int base);
+
+/* ---- producers of the quantizer's input (cf_oracle_norm.c) ----------------
+ * RMSNorm forward (kernels/rmsnorm.cu:13-54,101-108) and the absolute-ceiling
+ * row clip (src/trainer.cu:3822-3842,3940-3991), both with the reference's
+ * reduction trees.  orc_rmsnorm_forward returns non-zero when min(H,512) is
+ * not a multiple of 32. */
+int  orc_rmsnorm_forward(const uint16_t* x, const uint16_t* scale, uint16_t* out, float* rms,
+                         int rows, int H, float eps);
+void orc_act_row_clip_abs(uint16_t* x, int rows, int cols, float ceiling, float* normsq);
 
 /* ---- GEMM references ----------------------------------------------------
  * scale_mode: 0 per-tensor (a_descale[1], b_descale[1])

@@ -307,6 +307,28 @@ def bias_add_strided(inout, bias, rows, cols, row_stride, base):
     return inout
 
 
+# ---- producers of the quantizer's input ----------------------------------------------
+def rmsnorm_forward(x, weight, eps=1e-6):
+    x = np.ascontiguousarray(x, dtype=np.uint16)
+    weight = np.ascontiguousarray(weight, dtype=np.uint16)
+    rows, H = x.shape
+    out = np.empty((rows, H), np.uint16)
+    rms = np.empty(rows, np.float32)
+    _o.orc_rmsnorm_forward.restype = ctypes.c_int
+    rc = _o.orc_rmsnorm_forward(_p(x), _p(weight), _p(out), _p(rms), c_i(rows), c_i(H), c_f(eps))
+    if rc != 0:
+        raise ValueError(f"orc_rmsnorm_forward: unsupported H={H}")
+    return out, rms
+
+
+def act_row_clip_abs(x, ceiling):
+    x = np.ascontiguousarray(x, dtype=np.uint16).copy()
+    rows, cols = x.shape
+    normsq = np.zeros(rows, np.float32)
+    _call("orc_act_row_clip_abs", x, c_i(rows), c_i(cols), c_f(ceiling), normsq)
+    return x, normsq
+
+
 # ---- GEMM ---------------------------------------------------------------------------
 def gemm_nt_ref(A, B, a_descale, b_descale, a_e5m2=False, b_e5m2=False, scale_mode=0, lda=None, want_abs=True):
     """A[M,K] fp8 bytes (row stride lda), B[N,K] fp8 bytes -> (ref[M,N] f64, absdot[M,N] f64)."""

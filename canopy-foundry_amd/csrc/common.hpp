@@ -76,6 +76,19 @@ __device__ __forceinline__ uint32_t cvt4_fp8(float a, float b, float c, float d)
     u = nan_fix(u, a, 0); u = nan_fix(u, b, 1); u = nan_fix(u, c, 2); u = nan_fix(u, d, 3);
     return u;
 }
+// the same for inputs known to hold no NaN
+template <bool E5M2>
+__device__ __forceinline__ uint32_t cvt4_fp8_finite(float a, float b, float c, float d) {
+    int r = 0;
+    if constexpr (E5M2) {
+        r = __builtin_amdgcn_cvt_pk_bf8_f32(fp8_clamp<true>(a), fp8_clamp<true>(b), r, false);
+        r = __builtin_amdgcn_cvt_pk_bf8_f32(fp8_clamp<true>(c), fp8_clamp<true>(d), r, true);
+    } else {
+        r = __builtin_amdgcn_cvt_pk_fp8_f32(fp8_clamp<false>(a), fp8_clamp<false>(b), r, false);
+        r = __builtin_amdgcn_cvt_pk_fp8_f32(fp8_clamp<false>(c), fp8_clamp<false>(d), r, true);
+    }
+    return static_cast<uint32_t>(r);
+}
 template <bool E5M2>
 __device__ __forceinline__ uint8_t cvt1_fp8(float a) {
     return static_cast<uint8_t>(cvt4_fp8<E5M2>(a, 0.0f, 0.0f, 0.0f) & 0xffu);
@@ -112,6 +125,22 @@ __device__ __forceinline__ int wave_sum_i(int v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
     return v;
+}
+
+// Running maximum of |bf16| over both halves of packed pairs, as integers (|x| orders like its bits; any NaN
+// ends up above the infinity pattern 0x7f80)
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pk_absmax(uint32_t acc, uint32_t pair) {
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2, acc),
+                                                                  __builtin_bit_cast(u16x2, pair & 0x7fff7fffu)));
+}
+
+// The 64-lane maximum of such an accumulator as bf16 bits: below 0x7f80 every element was finite.
+__device__ __forceinline__ int wave_absmax_bits(uint32_t acc) {
+    int m = static_cast<int>(max(acc & 0xffffu, acc >> 16));
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = max(m, __shfl_xor(m, off, kWave));
+    return m;
 }
 
 // |x| >= 0 orders like its bit pattern, so an integer max is a float max.  Thousands of atomics on one

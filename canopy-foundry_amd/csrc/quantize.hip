@@ -57,6 +57,22 @@ __device__ __forceinline__ uint4 quant16(const Vec16& v, float s) {
     return o;
 }
 
+__device__ __forceinline__ uint32_t absmax16(uint32_t acc, const Vec16& v) {
+    acc = pk_absmax(pk_absmax(pk_absmax(pk_absmax(acc, v.lo.x), v.lo.y), v.lo.z), v.lo.w);
+    return pk_absmax(pk_absmax(pk_absmax(pk_absmax(acc, v.hi.x), v.hi.y), v.hi.z), v.hi.w);
+}
+// quant16 for products known to hold no NaN
+template <bool E5M2>
+__device__ __forceinline__ uint4 quant16_finite(const Vec16& v, float s) {
+    const uint32_t w[8] = {v.lo.x, v.lo.y, v.lo.z, v.lo.w, v.hi.x, v.hi.y, v.hi.z, v.hi.w};
+    uint4 o;
+    o.x = cvt4_fp8_finite<E5M2>(bf16_lo(w[0]) * s, bf16_hi(w[0]) * s, bf16_lo(w[1]) * s, bf16_hi(w[1]) * s);
+    o.y = cvt4_fp8_finite<E5M2>(bf16_lo(w[2]) * s, bf16_hi(w[2]) * s, bf16_lo(w[3]) * s, bf16_hi(w[3]) * s);
+    o.z = cvt4_fp8_finite<E5M2>(bf16_lo(w[4]) * s, bf16_hi(w[4]) * s, bf16_lo(w[5]) * s, bf16_hi(w[5]) * s);
+    o.w = cvt4_fp8_finite<E5M2>(bf16_lo(w[6]) * s, bf16_hi(w[6]) * s, bf16_lo(w[7]) * s, bf16_hi(w[7]) * s);
+    return o;
+}
+
 // ---- amax ------------------------------------------------------------------
 // VEC: x is 16-byte aligned and the body is read as 16-element vectors; the
 // n % 16 tail and the unaligned case go through the scalar loop.
@@ -241,23 +257,84 @@ __global__ __launch_bounds__(kThreads) void k_quant_rows(const uint16_t* __restr
     const uint16_t* xr = x + static_cast<size_t>(row) * K;
     uint8_t* outr = out + static_cast<size_t>(row) * K;
     Vec16 v[MAXS];
-    float local = 0.0f;
+    uint32_t acc = 0;                 // packed integer maximum of |bf16|: one instruction per pair
 #pragma unroll
     for (int s = 0; s < MAXS; ++s) {
         const int k = (s * 64 + lane) * kVec;
         if (k < K) {
             v[s] = load16(xr + k);
-            local = fmaxf(local, amax16(v[s]));
+            acc = absmax16(acc, v[s]);
         }
     }
+    const int mbits = wave_absmax_bits(acc);
+    const bool finite = mbits < 0x7f80;
+    float m = __uint_as_float(static_cast<uint32_t>(mbits) << 16);
+    if (!finite) {                    // a float maximum ignores NaNs
+        float local = 0.0f;
+#pragma unroll
+        for (int s = 0; s < MAXS; ++s)
+            if ((s * 64 + lane) * kVec < K) local = fmaxf(local, amax16(v[s]));
+        m = wave_max(local);
+    }
     constexpr float fmax_ = E5M2 ? 57344.0f : 448.0f;
-    const float a = fmaxf(wave_max(local), 1e-12f);
+    const float a = fmaxf(m, 1e-12f);
     const float sc = fmax_ / a;
     if (lane == 0) { scale[row] = sc; descale[row] = a / fmax_; }
 #pragma unroll
     for (int s = 0; s < MAXS; ++s) {
         const int k = (s * 64 + lane) * kVec;
-        if (k < K) *reinterpret_cast<uint4*>(outr + k) = quant16<E5M2>(v[s], sc);
+        if (k < K) *reinterpret_cast<uint4*>(outr + k) = finite ? quant16_finite<E5M2>(v[s], sc) : quant16<E5M2>(v[s], sc);
+    }
+}
+
+// Long rows (4096 < K <= 16384): one workgroup of four wavefronts per row, the row still register-resident (four
+// steps per lane instead of sixteen, so twice the wavefronts fit a SIMD); the row maximum crosses the
+// wavefronts through LDS.
+template <bool E5M2>
+__global__ __launch_bounds__(kThreads) void k_quant_rows_block(const uint16_t* __restrict__ x, int K,
+                                                               uint8_t* __restrict__ out,
+                                                               float* __restrict__ scale,
+                                                               float* __restrict__ descale) {
+    constexpr int MAXS = 4;
+    __shared__ int sh_bits[kThreads / 64];
+    __shared__ float sh_max[kThreads / 64];
+    const int row = blockIdx.x, tid = threadIdx.x;
+    const uint16_t* xr = x + static_cast<size_t>(row) * K;
+    uint8_t* outr = out + static_cast<size_t>(row) * K;
+    Vec16 v[MAXS];
+    uint32_t acc = 0;
+#pragma unroll
+    for (int s = 0; s < MAXS; ++s) {
+        const int k = (s * kThreads + tid) * kVec;
+        if (k < K) {
+            v[s] = load16(xr + k);
+            acc = absmax16(acc, v[s]);
+        }
+    }
+    const int wbits = wave_absmax_bits(acc);
+    if ((tid & 63) == 0) sh_bits[tid >> 6] = wbits;
+    __syncthreads();
+    const int mbits = max(max(sh_bits[0], sh_bits[1]), max(sh_bits[2], sh_bits[3]));
+    const bool finite = mbits < 0x7f80;
+    float m = __uint_as_float(static_cast<uint32_t>(mbits) << 16);
+    if (!finite) {                    // a float maximum ignores NaNs
+        float local = 0.0f;
+#pragma unroll
+        for (int s = 0; s < MAXS; ++s)
+            if ((s * kThreads + tid) * kVec < K) local = fmaxf(local, amax16(v[s]));
+        local = wave_max(local);
+        if ((tid & 63) == 0) sh_max[tid >> 6] = local;
+        __syncthreads();
+        m = fmaxf(fmaxf(sh_max[0], sh_max[1]), fmaxf(sh_max[2], sh_max[3]));
+    }
+    constexpr float fmax_ = E5M2 ? 57344.0f : 448.0f;
+    const float a = fmaxf(m, 1e-12f);
+    const float sc = fmax_ / a;
+    if (tid == 0) { scale[row] = sc; descale[row] = a / fmax_; }
+#pragma unroll
+    for (int s = 0; s < MAXS; ++s) {
+        const int k = (s * kThreads + tid) * kVec;
+        if (k < K) *reinterpret_cast<uint4*>(outr + k) = finite ? quant16_finite<E5M2>(v[s], sc) : quant16<E5M2>(v[s], sc);
     }
 }
 
@@ -563,8 +640,8 @@ int cf_fp8_quantize_rows(const uint16_t* d_x, int rows, int K, int is_e5m2, void
         if (is_e5m2) k_quant_rows<true, 4><<<grid, kThreads, 0, st>>>(d_x, rows, K, o, d_scale, d_descale);
         else         k_quant_rows<false, 4><<<grid, kThreads, 0, st>>>(d_x, rows, K, o, d_scale, d_descale);
     } else if (vec && K <= 16 * 1024) {
-        if (is_e5m2) k_quant_rows<true, 16><<<grid, kThreads, 0, st>>>(d_x, rows, K, o, d_scale, d_descale);
-        else         k_quant_rows<false, 16><<<grid, kThreads, 0, st>>>(d_x, rows, K, o, d_scale, d_descale);
+        if (is_e5m2) k_quant_rows_block<true><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);
+        else         k_quant_rows_block<false><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);
     } else {
         if (is_e5m2) k_quant_rows_generic<true><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);
         else         k_quant_rows_generic<false><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);

@@ -90,6 +90,25 @@ def main():
     hbm("quantize_e5m2 (known scale)", f"{M}x{K}", 3.0 * n, lambda: cf.cf_fp8_quantize_e5m2(x, q, sc, n, st))
     rs = torch.empty(M, device=dev); rd = torch.empty(M, device=dev)
     hbm("quantize_rows (per-token, one pass)", f"{M}x{K}", 3.0 * n + 8 * M, lambda: cf.cf_fp8_quantize_rows(x, M, K, 0, q, rs, rd, st))
+    # producers fused with the quantize (FFN input: rmsnorm -> row clip -> per-token quantize)
+    gamma = (1.0 + 0.1 * torch.randn(K, device=dev, generator=g)).to(torch.bfloat16)
+    normed = torch.empty_like(x)
+    ceiling = 65.0            # about the median row norm after normalisation: half the rows are clipped
+    hbm("rmsnorm_forward", f"{M}x{K}", 4.0 * n, lambda: cf.cf_rmsnorm_forward(x, gamma, normed, None, M, K, 1e-6, st))
+    hbm("act_row_clip_abs (in place, half the rows clipped)", f"{M}x{K}", 3.0 * n,
+        lambda: cf.cf_act_row_clip_abs(normed, M, K, ceiling, None, st))
+
+    def unfused():
+        cf.cf_rmsnorm_forward(x, gamma, normed, None, M, K, 1e-6, st)
+        cf.cf_act_row_clip_abs(normed, M, K, ceiling, None, st)
+        cf.cf_fp8_quantize_rows(normed, M, K, 0, q, rs, rd, st)
+    hbm("rmsnorm + clip + quantize_rows, three launches", f"{M}x{K}", 5.0 * n + 8 * M, unfused)
+    hbm("rmsnorm_clip_quantize_rows (fused, keeps the bf16 row)", f"{M}x{K}", 5.0 * n + 8 * M,
+        lambda: cf.cf_rmsnorm_clip_quantize_rows(x, gamma, M, K, 1e-6, ceiling, 0, normed, None, q, rs, rd, st))
+    hbm("rmsnorm_clip_quantize_rows (fused, fp8 only)", f"{M}x{K}", 3.0 * n + 8 * M,
+        lambda: cf.cf_rmsnorm_clip_quantize_rows(x, gamma, M, K, 1e-6, ceiling, 0, None, None, q, rs, rd, st))
+    hbm("rmsnorm_clip_quantize_record (fused, per-tensor)", f"{M}x{K}", 5.0 * n,
+        lambda: cf.cf_rmsnorm_clip_quantize_record(x, gamma, M, K, 1e-6, ceiling, 0, normed, None, q, sc, amax, st))
     h = bf16(M, N)
     hq = u8(M, N)
     hbm("quantize_rows (per-token, one pass)", f"{M}x{N}", 3.0 * h.numel() + 8 * M,

@@ -172,6 +172,30 @@ def test_per_row_quantize(cf, dev, rows, K, e5m2):
     assert np.array_equal(host(out), wq)
 
 
+@pytest.mark.parametrize("K", [1024, 4096, 14336])
+@pytest.mark.parametrize("e5m2", [False, True])
+def test_per_row_quantize_with_nonfinite_elements(cf, dev, K, e5m2):
+    """Rows holding NaN or infinities: the row maximum ignores NaN, an infinite maximum gives scale 0 and
+    the products 0 x inf become NaN codes, exactly as the element-wise definition says."""
+    case(f"rows quantize non-finite K={K} e5m2={e5m2}")
+    rng = np.random.default_rng(K + int(e5m2))
+    xh = rng.standard_normal((6, K)).astype(np.float32)
+    xh[1, 5] = np.nan
+    xh[2, K - 1] = np.inf
+    xh[3, 7] = -np.inf; xh[3, 9] = np.nan
+    xh[4, :] = np.nan
+    xb = orc.bf16_from_f32(xh)
+    x = dev_bf16(xb, dev)
+    out = torch.empty((6, K), dtype=torch.uint8, device=dev)
+    s = torch.empty(6, device=dev); d = torch.empty(6, device=dev)
+    cf.cf_fp8_quantize_rows(x, 6, K, int(e5m2), out, s, d, stream())
+    torch.cuda.synchronize()
+    wq, ws, wd = orc.quantize_rows(xb, e5m2)
+    assert np.array_equal(host(s).view(np.uint32), ws.view(np.uint32))
+    assert np.array_equal(host(d).view(np.uint32), wd.view(np.uint32))
+    assert np.array_equal(host(out), wq)
+
+
 @pytest.mark.parametrize("rows,K", [(128, 128), (4, 7168), (130, 384), (37, 300), (256, 1408)])
 def test_block_scaled_quantize(cf, dev, rows, K):
     case(f"block quantize {rows}x{K}")

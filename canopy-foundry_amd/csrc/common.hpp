@@ -176,10 +176,10 @@ __device__ __forceinline__ float det_expf(float x) {
     if (ki > 127) return (p * __uint_as_float(static_cast<uint32_t>(ki + 126) << 23)) * 2.0f;
     return p * __uint_as_float(static_cast<uint32_t>(ki + 127) << 23);
 }
+// 1 / (1 + e^-x) for x >= 0, e^x / (1 + e^x) below: one exponential of -|x| and one division serve both
 __device__ __forceinline__ float stable_sigmoid(float x) {
-    if (x >= 0.0f) return 1.0f / (1.0f + det_expf(-x));
-    const float e = det_expf(x);
-    return e / (1.0f + e);
+    const float e = det_expf(-fabsf(x));
+    return (x >= 0.0f ? 1.0f : e) / (1.0f + e);
 }
 
 // ---- host-side launch helpers ----------------------------------------------

@@ -13,8 +13,8 @@ __device__ __forceinline__ uint16_t swiglu1(uint16_t g, uint16_t u) {
     return f32_to_bf16((gv * stable_sigmoid(gv)) * uv);
 }
 __device__ __forceinline__ uint32_t swiglu2(uint32_t g, uint32_t u) {
-    return static_cast<uint32_t>(swiglu1(g & 0xffffu, u & 0xffffu)) |
-           (static_cast<uint32_t>(swiglu1(g >> 16, u >> 16)) << 16);
+    const float g0 = bf16_lo(g), g1 = bf16_hi(g);
+    return pack_bf16x2_hw((g0 * stable_sigmoid(g0)) * bf16_lo(u), (g1 * stable_sigmoid(g1)) * bf16_hi(u));
 }
 
 __global__ __launch_bounds__(kThreads) void k_swiglu(const uint16_t* __restrict__ gate,

@@ -76,10 +76,14 @@ __device__ __forceinline__ uint4 quant16_finite(const Vec16& v, float s) {
 // ---- amax ------------------------------------------------------------------
 // VEC: x is 16-byte aligned and the body is read as 16-element vectors; the
 // n % 16 tail and the unaligned case go through the scalar loop.
+// Launched with up to kAmaxThreads lanes per workgroup and one workgroup per CU: every workgroup ends in an
+// atomic on the same address, and those serialise, so there should be few of them.
+constexpr int kAmaxThreads = 1024;
+constexpr unsigned kAmaxBlocks = 256;
 template <bool VEC>
-__global__ __launch_bounds__(kThreads) void k_amax_bf16(const uint16_t* __restrict__ x, size_t n,
-                                                        float* __restrict__ amax) {
-    __shared__ float sh[kThreads / 64];
+__global__ __launch_bounds__(kAmaxThreads) void k_amax_bf16(const uint16_t* __restrict__ x, size_t n,
+                                                            float* __restrict__ amax) {
+    __shared__ float sh[kAmaxThreads / 64];
     float local = 0.0f;
     const size_t tid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
@@ -543,7 +547,7 @@ int cf_fp8_amax_bf16(const uint16_t* d_x, size_t n, float* d_amax, cf_stream_t s
     k_zero_f32<<<1, 1, 0, as_stream(stream)>>>(d_amax);
     if (n == 0) return launch_status();
     if (aligned16(d_x))
-        k_amax_bf16<true><<<min(blocks_for((n + kVec - 1) / kVec), 1024u), kThreads, 0, as_stream(stream)>>>(d_x, n, d_amax);
+        k_amax_bf16<true><<<min(ceil_div((n + kVec - 1) / kVec, kAmaxThreads), kAmaxBlocks), kAmaxThreads, 0, as_stream(stream)>>>(d_x, n, d_amax);
     else
         k_amax_bf16<false><<<blocks_for(n), kThreads, 0, as_stream(stream)>>>(d_x, n, d_amax);
     return launch_status();

@@ -285,6 +285,25 @@ def test_swiglu_and_bias_add(cf, dev):
     assert np.array_equal(bf16_bits(x), orc.bias_add_strided(xb, bb, 37, 40, 96, 17))
 
 
+def test_swiglu_on_every_bf16_gate(cf, dev):
+    """All 65536 gate patterns (NaNs and infinities included) against a handful of up values."""
+    case("swiglu, every bf16 gate")
+    gate = np.tile(all_bf16_bits(), 8)
+    ups = orc.bf16_from_f32(np.array([1.0, -0.75, 0.0, 3.0e38, 1e-30, np.inf, -np.inf, np.nan], np.float32))
+    up = np.repeat(ups, 65536)
+    out = torch.empty(gate.size, dtype=torch.bfloat16, device=dev)
+    cf.cf_swiglu_forward(dev_bf16(gate, dev), dev_bf16(up, dev), out, gate.size, stream())
+    torch.cuda.synchronize()
+    got, want = bf16_bits(out), orc.swiglu_forward(gate, up)
+    # a NaN result must be a NaN; its sign and payload are not defined by the arithmetic (x86 and the GPU
+    # propagate different operands' payloads)
+    nan_w, nan_g = (want & 0x7fff) > 0x7f80, (got & 0x7fff) > 0x7f80
+    assert np.array_equal(nan_w, nan_g)
+    got, want = np.where(nan_g, 0x7fc0, got), np.where(nan_w, 0x7fc0, want)
+    bad = np.nonzero(got != want)[0]
+    assert bad.size == 0, f"{bad.size} differ; first gate {gate[bad[0]]:#06x} up {up[bad[0]]:#06x} got {got[bad[0]]:#06x} want {want[bad[0]]:#06x}"
+
+
 def test_config2_activation_quantize_full_size(cf, dev):
     """M=8192 x K=4096 bf16 ~N(0,1) with 0.1% outliers at +-40 -> E4M3 with per-token scales."""
     case("config 2 activations, full size")

@@ -30,7 +30,7 @@ FP8_PEAK_TFLOPS = 5000.0      # MI355X dense FP8 MFMA peak (published)
 HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E peak (published)
 # HBM bytes per launch of the fused gate/up GEMM from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # script, scaled by what the same counters read for a 1 GiB device copy (fetch x2.000, write x1.000):
-# 1,384,206 KiB read + 229,440 KiB written.  Not measurable from inside the process; re-measure when the kernel changes.
+# 1,384,194 KiB read + 229,423 KiB written.  Not measurable from inside the process; re-measure when the kernel changes.
 GATEUP_HBM_TRAFFIC_BYTES = (1384194 + 229423) * 1024
 
 

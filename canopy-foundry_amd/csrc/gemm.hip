@@ -691,66 +691,90 @@ __device__ __forceinline__ void drain_tile(v16f (&acc)[4][4], TileScales<EPI>& s
     }
 }
 
-// The fp32 accumulate form (C += product, per-tensor scale s1): per pair of units and per 32 output rows
-// the scaled accumulators are parked as 32 rows x 256 bytes of fp32 (chunks xor-swizzled by row), read
-// back 16 bytes per lane, sixteen lanes per row, added to what C holds (fetched while the block is being
-// scaled) and stored: whole 128-byte lines in both directions, non-temporal both ways.
-template <bool RAGGED, class Landed>
-__device__ __forceinline__ void drain_tile_accum_f32(v16f (&acc)[4][4], float s1, const GemmArgs& p, const TilePos& t,
-                                                     int wm, int wn, int lane, uint8_t* stage, Landed&& landed) {
+// The accumulate forms (C += product, per-tensor scale s1; C fp32, or bf16 with one rounding of the sum): per pair
+// of units and per 32 output rows the scaled accumulators are parked as 32 rows x 256 bytes of fp32 (chunks
+// xor-swizzled by row), read back 16 bytes per lane, sixteen lanes per row, added to what C holds (fetched while
+// the block is being scaled) and stored: whole lines in both directions (128 bytes of fp32, 64 of bf16 per
+// sixteen lanes), non-temporal both ways.
+template <bool RAGGED, bool OUT_BF16, class Landed>
+__device__ __forceinline__ void drain_tile_accum(v16f (&acc)[4][4], float s1, const GemmArgs& p, const TilePos& t,
+                                                 int wm, int wn, int lane, uint8_t* stage, Landed&& landed) {
     const int row = lane & 31, khalf = lane >> 5;
     uint8_t* wr = stage + row * 256;
     const int wswz = row & 15;
     const int rr = lane >> 4, rc = lane & 15;
     const int mrow0 = t.m0 + wm * 128 + rr;
-    uint8_t* cu = reinterpret_cast<uint8_t*>(p.Cf + static_cast<size_t>(t.m0 + wm * 128) * p.ldc + t.n0 + wn * 128);
-    const uint32_t coff = (static_cast<uint32_t>(rr) * static_cast<uint32_t>(p.ldc) + rc * 4u) * 4u;
-    const size_t cstep = static_cast<size_t>(p.ldc) * 16;      // bytes between 4-row groups
+    constexpr uint32_t ES = OUT_BF16 ? 2u : 4u;                 // bytes per element of C
+    const size_t c_first = static_cast<size_t>(t.m0 + wm * 128) * p.ldc + t.n0 + wn * 128;
+    uint8_t* cu = OUT_BF16 ? reinterpret_cast<uint8_t*>(p.C + c_first) : reinterpret_cast<uint8_t*>(p.Cf + c_first);
+    const uint32_t coff = (static_cast<uint32_t>(rr) * static_cast<uint32_t>(p.ldc) + rc * 4u) * ES;
+    const size_t cstep = static_cast<size_t>(p.ldc) * 4 * ES;   // bytes between 4-row groups
+    constexpr uint32_t pair_bytes = 64 * ES;                    // a pair of units is 64 columns
     typedef float f32x4 __attribute__((ext_vector_type(4)));
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
+    // What C holds is fetched DEPTH blocks (of 32 rows x 64 columns) ahead of its use: every fetch pays the full
+    // memory latency (all workgroups drain at the same moment), so the first blocks are requested before anything
+    // else and the later ones as the registers of the earlier ones come free.
+    using Raw = std::conditional_t<OUT_BF16, u32x2, f32x4>;
+    constexpr int DEPTH = OUT_BF16 ? 4 : 2;      // what the register budget allows beside the copy offsets
+    Raw old[DEPTH][8];
+    auto fetch_old = [&](auto kc) {
+        constexpr int k = decltype(kc)::value, pair = k >> 2, b = k & 3;
 #pragma unroll
-    for (int pair = 0; pair < 2; ++pair) {
+        for (int i = 0; i < 8; ++i) {
+            old[k % DEPTH][i] = Raw{};
+            if (!RAGGED || mrow0 + b * 32 + i * 4 < t.m_end)
+                old[k % DEPTH][i] = __builtin_nontemporal_load(reinterpret_cast<const Raw*>(cu + ((b * 8 + i) * cstep + pair * pair_bytes) + coff));
+        }
+    };
+    static_for<0, DEPTH>([&](auto kc) { fetch_old(kc); });
+
+    static_for<0, 8>([&](auto kc) {
+        constexpr int k = decltype(kc)::value, pair = k >> 2, b = k & 3;
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            f32x4 old[8];
+        for (int uu = 0; uu < 2; ++uu) {
+            const int unit = pair * 2 + uu;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                old[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-                if (!RAGGED || mrow0 + b * 32 + i * 4 < t.m_end)
-                    old[i] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(cu + ((b * 8 + i) * cstep + pair * 256) + coff));
-            }
-#pragma unroll
-            for (int uu = 0; uu < 2; ++uu) {
-                const int unit = pair * 2 + uu;
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    float4 v;
-                    v.x = acc_read(acc[unit][b][g * 4 + 0]) * s1;
-                    v.y = acc_read(acc[unit][b][g * 4 + 1]) * s1;
-                    v.z = acc_read(acc[unit][b][g * 4 + 2]) * s1;
-                    v.w = acc_read(acc[unit][b][g * 4 + 3]) * s1;
-                    *reinterpret_cast<float4*>(wr + (((uu * 8 + g * 2 + khalf) ^ wswz) << 4)) = v;
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            // as in drain_tile: every copy in flight is waited for before the first store, and the tile that
-            // follows skips the wait of its first K-tile
-            if (pair == 0 && b == 0) {
-                __builtin_amdgcn_s_waitcnt(kWaitVm0);
-                landed();
-            }
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const int r = i * 4 + rr;
-                const float4 v = *reinterpret_cast<const float4*>(stage + r * 256 + ((rc ^ (r & 15)) << 4));
-                if (!RAGGED || mrow0 + b * 32 + i * 4 < t.m_end) {
-                    const f32x4 o = {old[i][0] + v.x, old[i][1] + v.y, old[i][2] + v.z, old[i][3] + v.w};
-                    __builtin_nontemporal_store(o, reinterpret_cast<f32x4*>(cu + ((b * 8 + i) * cstep + pair * 256) + coff));
-                }
+            for (int g = 0; g < 4; ++g) {
+                float4 v;
+                v.x = acc_read(acc[unit][b][g * 4 + 0]) * s1;
+                v.y = acc_read(acc[unit][b][g * 4 + 1]) * s1;
+                v.z = acc_read(acc[unit][b][g * 4 + 2]) * s1;
+                v.w = acc_read(acc[unit][b][g * 4 + 3]) * s1;
+                *reinterpret_cast<float4*>(wr + (((uu * 8 + g * 2 + khalf) ^ wswz) << 4)) = v;
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-    }
+        // as in drain_tile: every copy in flight is waited for before the first store, and the tile that
+        // follows skips the wait of its first K-tile
+        if constexpr (k == 0) {
+            __builtin_amdgcn_s_waitcnt(kWaitVm0);
+            landed();
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int r = i * 4 + rr;
+            const float4 v = *reinterpret_cast<const float4*>(stage + r * 256 + ((rc ^ (r & 15)) << 4));
+            if (!RAGGED || mrow0 + b * 32 + i * 4 < t.m_end) {
+                uint8_t* dst = cu + ((b * 8 + i) * cstep + pair * pair_bytes) + coff;
+                const Raw c = old[k % DEPTH][i];
+                if constexpr (OUT_BF16) {
+                    const u32x2 o = {pack_bf16x2_hw(v.x + bf16_lo(c[0]), v.y + bf16_hi(c[0])),
+                                     pack_bf16x2_hw(v.z + bf16_lo(c[1]), v.w + bf16_hi(c[1]))};
+                    __builtin_nontemporal_store(o, reinterpret_cast<u32x2*>(dst));
+                } else {
+                    const f32x4 o = {c[0] + v.x, c[1] + v.y, c[2] + v.z, c[3] + v.w};
+                    __builtin_nontemporal_store(o, reinterpret_cast<f32x4*>(dst));
+                }
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (k + DEPTH < 8) {
+            fetch_old(std::integral_constant<int, (k + DEPTH < 8) ? k + DEPTH : 0>{});
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    });
 }
 
 // The kernel is persistent: workgroup w walks tiles w, w + grid, w + 2*grid, ... of the XCD-aware
@@ -767,7 +791,8 @@ void k_gemm_nt_ring(const GemmArgs p) {
     constexpr int OUT_BN = GATE ? BN / 2 : BN;
     // the LDS-staged drain covers these epilogues; the launcher sends such a call here only when N is a multiple
     // of the tile's output width and C and the channel descales allow 16-byte accesses
-    constexpr bool DRAIN = EPI == EPI_NONE || EPI == EPI_BIAS || EPI == EPI_SILU_GATE || EPI == EPI_ACCUM_F32;
+    constexpr bool ACCUM = EPI == EPI_ACCUM_F32 || EPI == EPI_ACCUM_BF16;
+    constexpr bool DRAIN = EPI == EPI_NONE || EPI == EPI_BIAS || EPI == EPI_SILU_GATE || ACCUM;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
@@ -935,7 +960,7 @@ void k_gemm_nt_ring(const GemmArgs p) {
             if constexpr (END && i == 11) {
                 if (fetch_seq < my_tiles) fetch_pos(fetch_seq, t2);
             }
-            if constexpr (END && DRAIN && EPI != EPI_ACCUM_F32 && i == 10) {
+            if constexpr (END && DRAIN && !ACCUM && i == 10) {
                 load_row_scales<EPI, SCALE>(sc, p, t, wm, lane);
                 load_pair_scales<EPI, SCALE>(sc.cs, sc.cs2, sc.bs, p, t, wn, lane, 0);
             }
@@ -1018,9 +1043,10 @@ void k_gemm_nt_ring(const GemmArgs p) {
         auto landed = [&]() { if (more) fetch_rows(t2, nrows); };
         if constexpr (DRAIN) {
             uint8_t* stage = smem + a4 + wave * (64 * BK);
-            if constexpr (EPI == EPI_ACCUM_F32) {
-                if (t.m0 + BM <= t.m_end) drain_tile_accum_f32<false>(acc, s1, p, t, wm, wn, lane, stage, landed);
-                else                      drain_tile_accum_f32<true>(acc, s1, p, t, wm, wn, lane, stage, landed);
+            if constexpr (ACCUM) {
+                constexpr bool BF = EPI == EPI_ACCUM_BF16;
+                if (t.m0 + BM <= t.m_end) drain_tile_accum<false, BF>(acc, s1, p, t, wm, wn, lane, stage, landed);
+                else                      drain_tile_accum<true, BF>(acc, s1, p, t, wm, wn, lane, stage, landed);
             } else {
                 if (t.m0 + BM <= t.m_end) drain_tile<EPI, SCALE, false>(acc, sc, s1, s2, p, t, wm, wn, lane, stage, landed);
                 else                      drain_tile<EPI, SCALE, true>(acc, sc, s1, s2, p, t, wm, wn, lane, stage, landed);
@@ -1066,7 +1092,7 @@ constexpr int kBsSa = 3 * kBsStage;                     // activation scales: 3 
 constexpr int kBsSb = kBsSa + 3 * BSM * 4;              // weight-block scales: 2 tile parities x 2 column blocks x 256 floats
 constexpr int kBsMaxKb = 256;
 constexpr int kBsLds = kBsSb + 2 * 2 * kBsMaxKb * 4;    // 153,088 bytes
-constexpr int kBsCopies = 7;                            // copy instructions per wavefront and K-tile (2 X, 4 W, 1 scales)
+// seven copy instructions per wavefront and K-tile (2 X, 4 W, 1 scales): waits leave one or two K-tiles in flight
 constexpr int kWaitVm7 = 0x0f77, kWaitVm14 = 0x0f7e;
 
 __global__ __launch_bounds__(kBsThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
@@ -1403,6 +1429,10 @@ int launch_tiled(const GemmArgs& p, hipStream_t st) {
     if constexpr (EPI == EPI_ACCUM_F32) {
         // its drain adds into full-width fp32 tiles with 16-byte accesses
         ring_ok = ring_ok && p.N % BN == 0 && p.ldc % 4 == 0 && aligned16(p.Cf);
+    }
+    if constexpr (EPI == EPI_ACCUM_BF16) {
+        // the same with 8-byte accesses to bf16 tiles
+        ring_ok = ring_ok && p.N % BN == 0 && p.ldc % 4 == 0 && (reinterpret_cast<uintptr_t>(p.C) & 7u) == 0;
     }
     if constexpr (EPI == EPI_NONE || EPI == EPI_BIAS || EPI == EPI_SILU_GATE) {
         // its drain writes full-width tiles with 16-byte stores and reads the channel descales as float4

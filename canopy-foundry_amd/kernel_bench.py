@@ -163,7 +163,10 @@ def main():
     dw = torch.zeros((N, K), dtype=torch.float32, device=dev)
     mfma("gemm wgrad, fp32 accumulate into dW (config 4)", f"{N}x{K}x{M}", 2.0 * M * N * K,
          lambda: cf.cf_fp8_gemm_tn_accum_f32(N, K, M, xt, sc, dyt, de, dw, K, st))
-    del xq, wg, wu, wd, hq, c, y, dy, xt, dyt, dw
+    dwb = torch.zeros((N, K), dtype=torch.bfloat16, device=dev)
+    mfma("gemm wgrad, bf16 accumulate into dW (config 4 shape)", f"{N}x{K}x{M}", 2.0 * M * N * K,
+         lambda: cf.cf_fp8_gemm_tn_accum_bf16(N, K, M, xt, sc, dyt, de, dwb, K, st))
+    del xq, wg, wu, wd, hq, c, y, dy, xt, dyt, dw, dwb
 
     # ---- config 5: MoE ------------------------------------------------------------------------------
     T, H, E, k, Ie = 16384, 2048, 64, 6, 1408

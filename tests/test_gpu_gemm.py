@@ -240,10 +240,11 @@ def test_wgrad_tn_accumulate_f32(cf, dev, M, N, K, flags):
         assert np.array_equal(host(C).astype(np.float64), got)
 
 
-def test_wgrad_tn_accumulate_bf16(cf, dev):
-    case("wgrad accumulate bf16")
-    rng = np.random.default_rng(77)
-    M, N, K = 300, 260, 512
+@pytest.mark.parametrize("M,N,K", [(300, 260, 512), (300, 512, 512), (1024, 768, 256), (700, 256, 1152)])
+def test_wgrad_tn_accumulate_bf16(cf, dev, M, N, K):
+    """N a multiple of 256 takes the persistent kernel (ragged last row tile included), 260 the staged one."""
+    case(f"wgrad accumulate bf16 {M}x{N}x{K}")
+    rng = np.random.default_rng(77 + M + N + K)
     Xt, sx = rand_fp8(rng, (M, K))
     dYt, sy = rand_fp8(rng, (N, K), e5m2=True, sigma=1e-3)
     ref, absdot = orc.gemm_nt_ref(Xt, dYt, [sx], [sy], b_e5m2=True)

@@ -265,53 +265,81 @@ __global__ __launch_bounds__(kThreads) void k_compact_index(const int* __restric
 // ---- fused weighted unpermute ------------------------------------------------------------
 // One workgroup per token row.  For every expert with a positive route weight, in ascending expert
 // order: mixed[row] = bf16(fma(w, y[slot], mixed[row])), slot = offsets[e] + rank of the row in the
-// expert's (ascending) row list, found by binary search.  Same arithmetic and order as one
-// scatter-accumulate launch per expert.
+// expert's (ascending) row list.  Same arithmetic and order as one scatter-accumulate launch per expert.
+// The rank is found by a 64-ary search, one wavefront per selected expert: each round is one coalesced
+// probe of 64 list entries, so a list of 4096 rows costs two memory latencies instead of twelve.
+
+// Position of `row` in the ascending list[0, cnt), or -1.  Called by a whole wavefront.
+__device__ __forceinline__ int wave_find_sorted(const int* __restrict__ list, int cnt, int row, int lane) {
+    int lo = 0, len = cnt;
+    while (len > 64) {
+        const int stride = (len + 63) >> 6;
+        const int idx = lo + lane * stride;
+        const int v = idx < lo + len ? list[idx] : 0x7fffffff;
+        const unsigned long long le = __ballot(v <= row);       // a prefix of the lanes: the list ascends
+        if (le == 0) return -1;
+        const int j = 63 - __builtin_clzll(le);
+        const int end = lo + len;
+        lo += j * stride;
+        len = min(stride, end - lo);
+    }
+    const int v = lane < len ? list[lo + lane] : 0x7fffffff;
+    const unsigned long long eq = __ballot(v == row);
+    return eq ? lo + __builtin_ctzll(eq) : -1;
+}
+
 __global__ __launch_bounds__(kThreads) void k_unpermute(uint16_t* __restrict__ mixed, const uint16_t* __restrict__ y,
                                                         const float* __restrict__ route_weights,
                                                         const int* __restrict__ counts, const int* __restrict__ offsets,
                                                         const int* __restrict__ row_indices, int rows, int E, int H) {
+    __shared__ int sl_e[64];
     __shared__ int sl_slot[64];
     __shared__ float sl_w[64];
     __shared__ int sl_n;
-    const int row = blockIdx.x, t = threadIdx.x;
+    const int row = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6;
     uint16_t* mrow = mixed + static_cast<size_t>(row) * H;
     for (int e0 = 0; e0 < E; e0 += 64) {
         if (t < 64) {
             const int e = e0 + t;
             const float w = e < E ? route_weights[static_cast<size_t>(row) * E + e] : 0.0f;
             const bool sel = w > 0.0f;
-            int slot = -1;
+            const unsigned long long m = __ballot(sel);
             if (sel) {
-                const int* list = row_indices + static_cast<size_t>(e) * rows;
-                int lo = 0, hi = counts[e] - 1;
-                while (lo <= hi) {
-                    const int mid = (lo + hi) >> 1;
-                    const int v = list[mid];
-                    if (v == row) { slot = offsets[e] + mid; break; }
-                    if (v < row) lo = mid + 1; else hi = mid - 1;
-                }
-            }
-            const bool ok = sel && slot >= 0;
-            const unsigned long long m = __ballot(ok);
-            if (ok) {
                 const int pos = __builtin_popcountll(m & ((1ull << t) - 1ull));
-                sl_slot[pos] = slot;
+                sl_e[pos] = e;
                 sl_w[pos] = w;
             }
             if (t == 0) sl_n = __builtin_popcountll(m);
         }
         __syncthreads();
         const int n = sl_n;
+        for (int i = wave; i < n; i += kThreads / 64) {
+            const int e = sl_e[i];
+            const int pos = wave_find_sorted(row_indices + static_cast<size_t>(e) * rows, counts[e], row, lane);
+            if (lane == 0) sl_slot[i] = pos < 0 ? -1 : offsets[e] + pos;     // -1: not in the expert's list, skipped
+        }
+        __syncthreads();
         if (n > 0) {
             if ((H & 7) == 0) {
                 for (int c = t; c < H / 8; c += blockDim.x) {
                     uint4 mv = reinterpret_cast<uint4*>(mrow)[c];
-                    for (int i = 0; i < n; ++i) {
-                        const uint4 yv = reinterpret_cast<const uint4*>(y + static_cast<size_t>(sl_slot[i]) * H)[c];
-                        const float w = sl_w[i];
-                        mv.x = fma2_bf16(mv.x, yv.x, w); mv.y = fma2_bf16(mv.y, yv.y, w);
-                        mv.z = fma2_bf16(mv.z, yv.z, w); mv.w = fma2_bf16(mv.w, yv.w, w);
+                    for (int i0 = 0; i0 < n; i0 += 4) {
+                        // up to four rows of y in flight at once, applied in order
+                        uint4 yv[4];
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const int slot = i0 + j < n ? sl_slot[i0 + j] : -1;
+                            yv[j] = make_uint4(0, 0, 0, 0);
+                            if (slot >= 0) yv[j] = reinterpret_cast<const uint4*>(y + static_cast<size_t>(slot) * H)[c];
+                        }
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            if (i0 + j < n && sl_slot[i0 + j] >= 0) {
+                                const float w = sl_w[i0 + j];
+                                mv.x = fma2_bf16(mv.x, yv[j].x, w); mv.y = fma2_bf16(mv.y, yv[j].y, w);
+                                mv.z = fma2_bf16(mv.z, yv[j].z, w); mv.w = fma2_bf16(mv.w, yv[j].w, w);
+                            }
+                        }
                     }
                     reinterpret_cast<uint4*>(mrow)[c] = mv;
                 }
@@ -319,7 +347,8 @@ __global__ __launch_bounds__(kThreads) void k_unpermute(uint16_t* __restrict__ m
                 for (int h = t; h < H; h += blockDim.x) {
                     float m = bf16_to_f32(mrow[h]);
                     for (int i = 0; i < n; ++i)
-                        m = bf16_to_f32(f32_to_bf16(__builtin_fmaf(sl_w[i], bf16_to_f32(y[static_cast<size_t>(sl_slot[i]) * H + h]), m)));
+                        if (sl_slot[i] >= 0)
+                            m = bf16_to_f32(f32_to_bf16(__builtin_fmaf(sl_w[i], bf16_to_f32(y[static_cast<size_t>(sl_slot[i]) * H + h]), m)));
                     mrow[h] = f32_to_bf16(m);
                 }
             }

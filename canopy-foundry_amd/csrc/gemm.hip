@@ -534,7 +534,6 @@ struct TileScales {
     float sa[4];
     float4 cs[2][4];
     float4 cs2[2][4];      // up-projection descales (SiLU-gate)
-    uint2 bs[2][4];        // bf16 bias of the same columns (bias epilogue)
 };
 
 template <int EPI, int SCALE>
@@ -548,7 +547,7 @@ __device__ __forceinline__ void load_row_scales(TileScales<EPI>& s, const GemmAr
     }
 }
 template <int EPI, int SCALE>
-__device__ __forceinline__ void load_pair_scales(float4 (&cs)[2][4], float4 (&cs2)[2][4], uint2 (&bs)[2][4], const GemmArgs& p,
+__device__ __forceinline__ void load_pair_scales(float4 (&cs)[2][4], float4 (&cs2)[2][4], const GemmArgs& p,
                                                  const TilePos& t, int wn, int lane, int pair) {
     constexpr int NU = EPI == EPI_SILU_GATE ? 2 : 4;
     // uniform bases (scalar registers) + a small per-lane byte offset: no 64-bit per-lane addresses to keep alive
@@ -564,16 +563,6 @@ __device__ __forceinline__ void load_pair_scales(float4 (&cs)[2][4], float4 (&cs
             for (int g = 0; g < 4; ++g) {
                 cs[u][g] = *reinterpret_cast<const float4*>(b1 + (loff + u * 128u + g * 32u));
                 if constexpr (EPI == EPI_SILU_GATE) cs2[u][g] = *reinterpret_cast<const float4*>(b2 + (loff + u * 128u + g * 32u));
-            }
-    }
-    if constexpr (EPI == EPI_BIAS) {
-        const uint8_t* bb = reinterpret_cast<const uint8_t*>(p.bias + col0);
-        const uint32_t loff = static_cast<uint32_t>(lane >> 5) * 8u;
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                bs[u][g] = *reinterpret_cast<const uint2*>(bb + (loff + u * 64u + g * 16u));
             }
     }
 }
@@ -610,15 +599,24 @@ __device__ __forceinline__ void drain_tile(v16f (&acc)[4][4], TileScales<EPI>& s
     const uint32_t coff = (static_cast<uint32_t>(rr) * static_cast<uint32_t>(p.ldc) + rc * 8u) * 2u;
     const size_t cstep = static_cast<size_t>(p.ldc) * 16;      // bytes between 8-row groups
     typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    // Bias is added to the bf16 result, as the separate kernel does: on the way out, where a lane holds eight
+    // consecutive columns of a row, the same eight for every row it stores.  Both pairs' bias chunks are
+    // fetched before the first store, so no wait on them has to sit out a store burst.
+    uint4 bias8[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
+    if constexpr (EPI == EPI_BIAS) {
+        const uint16_t* bcol = p.bias + t.n0 + wn * (NU * 32) + rc * 8;
+#pragma unroll
+        for (int pair = 0; pair < NU / 2; ++pair) bias8[pair] = *reinterpret_cast<const uint4*>(bcol + pair * 64);
+    }
 
 #pragma unroll
     for (int pair = 0; pair < NU / 2; ++pair) {
-        // the next pair's factors are fetched while this pair is drained (the bias form, short of registers, fetches
-        // them at the turn instead)
-        constexpr bool PREFETCH = EPI != EPI_BIAS;
+        const uint4 bv = bias8[pair];
+        const float bf[8] = {bf16_lo(bv.x), bf16_hi(bv.x), bf16_lo(bv.y), bf16_hi(bv.y),
+                             bf16_lo(bv.z), bf16_hi(bv.z), bf16_lo(bv.w), bf16_hi(bv.w)};
+        // the next pair's factors are fetched while this pair is drained
         float4 ncs[2][4], ncs2[2][4];
-        uint2 nbs[2][4];
-        if (PREFETCH && pair + 1 < NU / 2) load_pair_scales<EPI, SCALE>(ncs, ncs2, nbs, p, t, wn, lane, pair + 1);
+        if (pair + 1 < NU / 2) load_pair_scales<EPI, SCALE>(ncs, ncs2, p, t, wn, lane, pair + 1);
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
 #pragma unroll
@@ -648,12 +646,6 @@ __device__ __forceinline__ void drain_tile(v16f (&acc)[4][4], TileScales<EPI>& s
                                 v[q] = acc_read(acc[unit][b][g * 4 + q]) * (sa * c4[q]);
                             }
                         }
-                        if constexpr (EPI == EPI_BIAS) {
-                            // bias is added to the bf16 result, as the separate kernel does
-                            const uint32_t b01 = s.bs[uu][g].x, b23 = s.bs[uu][g].y;
-                            v[0] = round_bf16_hw(v[0]) + bf16_lo(b01); v[1] = round_bf16_hw(v[1]) + bf16_hi(b01);
-                            v[2] = round_bf16_hw(v[2]) + bf16_lo(b23); v[3] = round_bf16_hw(v[3]) + bf16_hi(b23);
-                        }
                         *reinterpret_cast<uint2*>(wr + bb * 32 * 128 + (((uu * 4 + g) ^ wswz) << 4)) =
                             make_uint2(pack_bf16x2_hw(v[0], v[1]), pack_bf16x2_hw(v[2], v[3]));
                     }
@@ -670,7 +662,13 @@ __device__ __forceinline__ void drain_tile(v16f (&acc)[4][4], TileScales<EPI>& s
             }
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const uint4 v = *reinterpret_cast<const uint4*>(((i & 1) ? rdp1 : rdp0) + i * 8 * 128);
+                uint4 v = *reinterpret_cast<const uint4*>(((i & 1) ? rdp1 : rdp0) + i * 8 * 128);
+                if constexpr (EPI == EPI_BIAS) {
+                    v.x = pack_bf16x2_hw(bf16_lo(v.x) + bf[0], bf16_hi(v.x) + bf[1]);
+                    v.y = pack_bf16x2_hw(bf16_lo(v.y) + bf[2], bf16_hi(v.y) + bf[3]);
+                    v.z = pack_bf16x2_hw(bf16_lo(v.z) + bf[4], bf16_hi(v.z) + bf[5]);
+                    v.w = pack_bf16x2_hw(bf16_lo(v.w) + bf[6], bf16_hi(v.w) + bf[7]);
+                }
                 if (!RAGGED || mrow0 + half * 64 + i * 8 < t.m_end) {
                     const u32x4 vv = {v.x, v.y, v.z, v.w};
                     __builtin_nontemporal_store(vv, reinterpret_cast<u32x4*>(cu + ((half * 8 + i) * cstep + pair * 128) + coff));
@@ -679,14 +677,10 @@ __device__ __forceinline__ void drain_tile(v16f (&acc)[4][4], TileScales<EPI>& s
             __builtin_amdgcn_sched_barrier(0);
         }
         if (pair + 1 < NU / 2) {
-            if constexpr (PREFETCH) {
 #pragma unroll
-                for (int u = 0; u < 2; ++u)
+            for (int u = 0; u < 2; ++u)
 #pragma unroll
-                    for (int g = 0; g < 4; ++g) { s.cs[u][g] = ncs[u][g]; s.cs2[u][g] = ncs2[u][g]; }
-            } else {
-                load_pair_scales<EPI, SCALE>(s.cs, s.cs2, s.bs, p, t, wn, lane, pair + 1);
-            }
+                for (int g = 0; g < 4; ++g) { s.cs[u][g] = ncs[u][g]; s.cs2[u][g] = ncs2[u][g]; }
         }
     }
 }
@@ -962,7 +956,7 @@ void k_gemm_nt_ring(const GemmArgs p) {
             }
             if constexpr (END && DRAIN && !ACCUM && i == 10) {
                 load_row_scales<EPI, SCALE>(sc, p, t, wm, lane);
-                load_pair_scales<EPI, SCALE>(sc.cs, sc.cs2, sc.bs, p, t, wn, lane, 0);
+                load_pair_scales<EPI, SCALE>(sc.cs, sc.cs2, p, t, wn, lane, 0);
             }
             __builtin_amdgcn_sched_barrier(0);
         });
@@ -1440,7 +1434,7 @@ int launch_tiled(const GemmArgs& p, hipStream_t st) {
         ring_ok = ring_ok && p.N % out_bn == 0 && p.ldc % 8 == 0 && aligned16(p.C);
         if (SCALE == SCALE_ROWCOL)
             ring_ok = ring_ok && aligned16(p.sb) && p.sb_expert_stride % 4 == 0 && (EPI != EPI_SILU_GATE || aligned16(p.sb2));
-        if (EPI == EPI_BIAS) ring_ok = ring_ok && (reinterpret_cast<uintptr_t>(p.bias) & 7u) == 0;
+        if (EPI == EPI_BIAS) ring_ok = ring_ok && aligned16(p.bias);
     }
     if (ring_ok && !p.force_staged) {
         static std::once_flag once_ring;

@@ -135,11 +135,11 @@ __global__ void k_scale_from_amax(const float* __restrict__ amax, float fp8_max,
     *descale = a / fp8_max;
 }
 
-__global__ void k_update_delayed_scale(const float* __restrict__ amax, float fp8_max,
-                                       float* __restrict__ scale, float* __restrict__ descale,
-                                       float* __restrict__ history, int history_len,
-                                       int* __restrict__ history_cursor, int* __restrict__ history_count) {
-    const float a = fmaxf(*amax, 1e-12f);
+// kernels/fp8.cu:105-142: ring append of max(amax, 1e-12), scale from the maximum of the entries filled so far
+__device__ __forceinline__ void delayed_scale_update(float amax, float fp8_max, float* scale, float* descale,
+                                                     float* history, int history_len, int* history_cursor,
+                                                     int* history_count) {
+    const float a = fmaxf(amax, 1e-12f);
     if (history_len <= 0) {
         *scale = fp8_max / a;
         *descale = a / fp8_max;
@@ -158,6 +158,12 @@ __global__ void k_update_delayed_scale(const float* __restrict__ amax, float fp8
     *history_count = count;
     *scale = fp8_max / hist_max;
     *descale = hist_max / fp8_max;
+}
+__global__ void k_update_delayed_scale(const float* __restrict__ amax, float fp8_max,
+                                       float* __restrict__ scale, float* __restrict__ descale,
+                                       float* __restrict__ history, int history_len,
+                                       int* __restrict__ history_cursor, int* __restrict__ history_count) {
+    delayed_scale_update(*amax, fp8_max, scale, descale, history, history_len, history_cursor, history_count);
 }
 
 __global__ void k_clip_probe(const float* __restrict__ amax, const float* __restrict__ scale,
@@ -209,6 +215,58 @@ __global__ __launch_bounds__(kThreads) void k_quant(const uint16_t* __restrict__
     if constexpr (RECORD) {
         const float m = block_max(local, sh);
         if (threadIdx.x == 0) atomic_max_nonneg(amax, m);
+    }
+}
+
+// The steady-state delayed-scaling step in one launch: quantize with the scale left by the previous call while
+// recording this tensor's amax, then the workgroup that finishes last does what the reference spreads over
+// separate launches and copies: snapshot the scale pair the quantize used, publish the amax, advance the history
+// and the scale, and leave the running maximum and the arrival counter at zero for the next call.
+struct DelayedStep {
+    float* amax; float* scale; float* descale; float* scale_snapshot; float* descale_snapshot;
+    float* history; int history_len; int* cursor; int* count;
+    float* running_amax; unsigned* arrived;     // both zero between calls
+    float fp8_max;
+};
+// Every workgroup ends in an atomic on the arrival counter, and atomics on one address serialise: one large
+// workgroup per CU (as for the amax kernel) keeps that tail to a few microseconds.
+template <bool E5M2, bool VEC>
+__global__ __launch_bounds__(kAmaxThreads) void k_quant_delayed_step(const uint16_t* __restrict__ x, uint8_t* __restrict__ out,
+                                                                     size_t n, const DelayedStep d) {
+    __shared__ float sh[kAmaxThreads / 64];
+    const float s = *d.scale;
+    float local = 0.0f;
+    const size_t tid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+    size_t done = 0;
+    if constexpr (VEC) {
+        const size_t nvec = n / kVec;
+        for (size_t i = tid; i < nvec; i += stride) {
+            const Vec16 v = load16(x + i * kVec);
+            local = fmaxf(local, amax16(v));
+            *reinterpret_cast<uint4*>(out + i * kVec) = quant16<E5M2>(v, s);
+        }
+        done = nvec * kVec;
+    }
+    for (size_t i = done + tid; i < n; i += stride) {
+        const float v = bf16_to_f32(x[i]);
+        local = fmaxf(local, fabsf(v));
+        out[i] = cvt1_fp8<E5M2>(v * s);
+    }
+    const float m = block_max(local, sh);
+    if (threadIdx.x == 0) {
+        atomic_max_nonneg(d.running_amax, m);
+        __threadfence();                                     // the maximum is visible before the arrival is
+        if (atomicAdd(d.arrived, 1u) == gridDim.x - 1) {
+            __threadfence();
+            const float amax = __hip_atomic_load(d.running_amax, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            *d.scale_snapshot = s;                           // every workgroup read the same pair at its start
+            *d.descale_snapshot = *d.descale;
+            *d.amax = amax;
+            delayed_scale_update(amax, d.fp8_max, d.scale, d.descale, d.history, d.history_len, d.cursor, d.count);
+            *d.running_amax = 0.0f;
+            *d.arrived = 0u;
+        }
     }
 }
 
@@ -598,6 +656,32 @@ int cf_fp8_quantize_f32_e5m2(const float* d_x, void* d_out, const float* d_scale
     const int vec = aligned16(d_x) && (reinterpret_cast<uintptr_t>(d_out) & 3u) == 0;
     k_quant_f32<true><<<blocks_for(vec ? (n + 3) / 4 : n), kThreads, 0, as_stream(stream)>>>(
         d_x, static_cast<uint8_t*>(d_out), d_scale, n, vec);
+    return launch_status();
+}
+
+int cf_fp8_quantize_delayed_step(const uint16_t* d_x, void* d_out, size_t n, int is_e5m2, float* d_amax, float* d_scale,
+                                 float* d_descale, float* d_scale_snapshot, float* d_descale_snapshot, float* d_history,
+                                 int history_len, int* d_history_cursor, int* d_history_count, float* d_running_amax,
+                                 unsigned int* d_arrived, cf_stream_t stream) {
+    if (!d_amax || !d_scale || !d_descale || !d_scale_snapshot || !d_descale_snapshot || !d_running_amax || !d_arrived ||
+        history_len < 0 || (history_len > 0 && (!d_history || !d_history_cursor || !d_history_count)) ||
+        (n > 0 && (!d_x || !d_out)))
+        return CF_ERR_INVALID_ARG;
+    DelayedStep d{d_amax, d_scale, d_descale, d_scale_snapshot, d_descale_snapshot, d_history, history_len,
+                  d_history_cursor, d_history_count, d_running_amax, d_arrived, is_e5m2 ? CF_E5M2_MAX : CF_E4M3_MAX};
+    auto* o = static_cast<uint8_t*>(d_out);
+    hipStream_t st = as_stream(stream);
+    // n == 0 still runs one workgroup: the state advances with an amax of zero, as the separate launches would
+    auto grid_for = [](size_t items) { return max(1u, min(ceil_div(items, kAmaxThreads), kAmaxBlocks)); };
+    if (aligned16(d_x) && aligned16(d_out)) {
+        const unsigned grid = grid_for((n + kVec - 1) / kVec);
+        if (is_e5m2) k_quant_delayed_step<true, true><<<grid, kAmaxThreads, 0, st>>>(d_x, o, n, d);
+        else         k_quant_delayed_step<false, true><<<grid, kAmaxThreads, 0, st>>>(d_x, o, n, d);
+    } else {
+        const unsigned grid = grid_for(n);
+        if (is_e5m2) k_quant_delayed_step<true, false><<<grid, kAmaxThreads, 0, st>>>(d_x, o, n, d);
+        else         k_quant_delayed_step<false, false><<<grid, kAmaxThreads, 0, st>>>(d_x, o, n, d);
+    }
     return launch_status();
 }
 

@@ -20,7 +20,9 @@ namespace cf {
 namespace {
 
 // device block layout, in 4-byte words
-enum { W_AMAX = 0, W_SCALE, W_DESCALE, W_SCALE_SNAP, W_DESCALE_SNAP, W_CALIB_MIN, W_CALIB_MAX, W_CURSOR = 8, W_COUNT = 9, W_HISTORY = 16 };
+enum { W_AMAX = 0, W_SCALE, W_DESCALE, W_SCALE_SNAP, W_DESCALE_SNAP, W_CALIB_MIN, W_CALIB_MAX, W_CURSOR = 8, W_COUNT = 9,
+       W_RUNNING_AMAX = 10, W_ARRIVED = 11,      // scratch of the one-launch steady-state step, zero between calls
+       W_HISTORY = 16 };
 
 __global__ void k_slot_init(float* st, int history_len) {
     for (int i = threadIdx.x; i < W_HISTORY + history_len; i += blockDim.x) st[i] = 0.0f;   // zero words are int 0 as well
@@ -123,9 +125,9 @@ int cf_fp8_quant_act(cf_act_slot* slot, const uint16_t* d_x, void* d_act8, size_
         }
     }
 
-    k_zero_amax<<<1, 1, 0, st>>>(d);
-    CF_TRY(launch_status());
     if (slot->calib_remaining > 0 || !slot->init) {
+        k_zero_amax<<<1, 1, 0, st>>>(d);
+        CF_TRY(launch_status());
         // exact per-call amax (no stale scale); during calibration the spread of the amax is recorded too
         CF_TRY(cf_fp8_amax_bf16(d_x, n, d + W_AMAX, stream));
         CF_TRY(cf_fp8_scale_from_amax(d + W_AMAX, slot->fp8_max, d + W_SCALE, d + W_DESCALE, stream));
@@ -139,11 +141,11 @@ int cf_fp8_quant_act(cf_act_slot* slot, const uint16_t* d_x, void* d_act8, size_
         return CF_OK;
     }
     // steady state: snapshot the pair the GEMM will dequantize with, quantize with the PREVIOUS scale while recording
-    // this tensor's amax, then advance the history
-    k_snapshot<<<1, 1, 0, st>>>(d);
-    CF_TRY(launch_status());
-    CF_TRY(quantize(slot, d_x, d_act8, d + W_SCALE, d + W_AMAX, n, stream));
-    return update_history(slot, stream);
+    // this tensor's amax, then advance the history -- one launch
+    return cf_fp8_quantize_delayed_step(d_x, d_act8, n, slot->fp8_max == CF_E5M2_MAX, d + W_AMAX, d + W_SCALE, d + W_DESCALE,
+                                        d + W_SCALE_SNAP, d + W_DESCALE_SNAP, d + W_HISTORY, slot->history_len,
+                                        reinterpret_cast<int*>(d) + W_CURSOR, reinterpret_cast<int*>(d) + W_COUNT,
+                                        d + W_RUNNING_AMAX, reinterpret_cast<unsigned int*>(d) + W_ARRIVED, stream);
 }
 
 int cf_fp8_refresh_weight(const uint16_t* d_w, void* d_fwd8, void* d_bwd8, float* d_amax, float* d_scale, float* d_descale,

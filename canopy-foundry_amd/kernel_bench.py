@@ -87,6 +87,19 @@ def main():
     hbm("quantize_e4m3 (known scale)", f"{M}x{K}", 3.0 * n, lambda: cf.cf_fp8_quantize_e4m3(x, q, sc, n, st))
     hbm("quantize_e4m3_record (previous scale + amax)", f"{M}x{K}", 3.0 * n,
         lambda: cf.cf_fp8_quantize_e4m3_record(x, q, sc, amax, n, st))
+    # delayed scaling, steady state: the reference's sequence as separate launches against the one-launch step
+    hist = torch.zeros(16, device=dev); cur = torch.zeros(1, dtype=torch.int32, device=dev); cnt = torch.zeros(1, dtype=torch.int32, device=dev)
+    ssnap = torch.ones(1, device=dev); dsnap = torch.ones(1, device=dev)
+    running = torch.zeros(1, device=dev); arrived = torch.zeros(1, dtype=torch.int32, device=dev)
+
+    def delayed_separate():
+        ssnap.copy_(sc); dsnap.copy_(de); amax.zero_()
+        cf.cf_fp8_quantize_e4m3_record(x, q, sc, amax, n, st)
+        cf.cf_fp8_update_delayed_scale(amax, 448.0, sc, de, hist, 16, cur, cnt, st)
+    hbm("delayed-scaling step: 2 copies + memset + record + update", f"{M}x{K}", 3.0 * n, delayed_separate)
+    hbm("delayed-scaling step: cf_fp8_quantize_delayed_step (1 launch)", f"{M}x{K}", 3.0 * n,
+        lambda: cf.cf_fp8_quantize_delayed_step(x, q, n, 0, amax, sc, de, ssnap, dsnap, hist, 16, cur, cnt, running, arrived, st))
+    sc.fill_(1.0); de.fill_(1.0)
     hbm("quantize_e5m2 (known scale)", f"{M}x{K}", 3.0 * n, lambda: cf.cf_fp8_quantize_e5m2(x, q, sc, n, st))
     rs = torch.empty(M, device=dev); rd = torch.empty(M, device=dev)
     hbm("quantize_rows (per-token, one pass)", f"{M}x{K}", 3.0 * n + 8 * M, lambda: cf.cf_fp8_quantize_rows(x, M, K, 0, q, rs, rd, st))

@@ -69,6 +69,20 @@ int cf_fp8_update_delayed_scale(const float* d_amax, float fp8_max, float* d_sca
                                 int* d_history_cursor, int* d_history_count,
                                 cf_stream_t stream);
 
+/* The steady-state branch of fp8_quant_act (src/trainer.cu:4811-4851) in ONE launch instead of the reference's
+ * two device-to-device copies, one memset and two kernels: quantize with *d_scale (the scale the previous call
+ * left) while recording this tensor's amax; then, inside the same kernel, the pair the quantize used goes to
+ * *d_scale_snapshot / *d_descale_snapshot (what the following GEMM dequantizes with), the amax to *d_amax, and
+ * the history, cursor, count, *d_scale and *d_descale advance as fp8_update_delayed_scale does
+ * (kernels/fp8.cu:105-142).  d_running_amax and d_arrived are two words of caller-owned device memory that
+ * must be zero before the first call; every call leaves them zero again.  Calls on one state must not overlap. */
+int cf_fp8_quantize_delayed_step(const uint16_t* d_x, void* d_out, size_t n, int is_e5m2,
+                                 float* d_amax, float* d_scale, float* d_descale,
+                                 float* d_scale_snapshot, float* d_descale_snapshot,
+                                 float* d_history, int history_len, int* d_history_cursor,
+                                 int* d_history_count, float* d_running_amax,
+                                 unsigned int* d_arrived, cf_stream_t stream);
+
 /* fp8_quantize_transpose_e4m3, kernels.hpp:1009-1010, kernels/fp8.cu:281-290.
  * w[K,N] bf16 -> out[N,K] E4M3. */
 int cf_fp8_quantize_transpose_e4m3(const uint16_t* d_w, void* d_out, const float* d_scale,

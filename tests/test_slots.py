@@ -142,3 +142,43 @@ def test_device_refresh_weight(cf, dev, in_dim, out_dim, out_major):
     torch.cuda.synchronize()
     wf2, wb2, *_ = refresh_weight(w, in_dim, out_dim, out_major, amax=np.float32(amax) * 2)
     assert np.array_equal(host(fwd), wf2) and np.array_equal(host(bwd), wb2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n,offset,history_len,e5m2", [(1 << 22, 0, 16, False), (100003, 1, 8, True), (5, 0, 0, False), (0, 0, 4, False)])
+def test_one_launch_delayed_step_equals_the_separate_launches(cf, dev, n, offset, history_len, e5m2):
+    """cf_fp8_quantize_delayed_step against snapshot copy + zeroed amax + quantize_record + update_delayed_scale,
+    every byte and every state word, over several calls (history wrap-around included)."""
+    import torch
+    from gpu_util import case, dev_bf16, host, stream
+    case(f"delayed step n={n} offset={offset} history={history_len} e5m2={e5m2}")
+    fp8_max = 57344.0 if e5m2 else 448.0
+    f32 = lambda *v: torch.tensor(v, dtype=torch.float32, device=dev)
+
+    def fresh():
+        return dict(amax=f32(0.0), scale=f32(3.5), descale=f32(1 / 3.5), ssnap=f32(0.0), dsnap=f32(0.0),
+                    hist=torch.zeros(max(history_len, 1), dtype=torch.float32, device=dev),
+                    cursor=torch.zeros(1, dtype=torch.int32, device=dev), count=torch.zeros(1, dtype=torch.int32, device=dev),
+                    running=f32(0.0), arrived=torch.zeros(1, dtype=torch.int32, device=dev))
+    a, b = fresh(), fresh()
+    rng = np.random.default_rng(n + history_len)
+    record = cf.cf_fp8_quantize_e5m2_record if e5m2 else cf.cf_fp8_quantize_e4m3_record
+    for call in range(history_len + 3):
+        xb = orc.bf16_from_f32((rng.standard_normal(n + offset) * (1.0 + call)).astype(np.float32))
+        x = dev_bf16(xb, dev)[offset:]
+        qa = torch.zeros(n + offset, dtype=torch.uint8, device=dev)[offset:]
+        qb = torch.zeros(n + offset, dtype=torch.uint8, device=dev)[offset:]
+        # the reference's sequence
+        a["ssnap"].copy_(a["scale"]); a["dsnap"].copy_(a["descale"]); a["amax"].zero_()
+        record(x, qa, a["scale"], a["amax"], n, stream())
+        cf.cf_fp8_update_delayed_scale(a["amax"], fp8_max, a["scale"], a["descale"], a["hist"], history_len, a["cursor"], a["count"], stream())
+        # one launch
+        cf.cf_fp8_quantize_delayed_step(x, qb, n, int(e5m2), b["amax"], b["scale"], b["descale"], b["ssnap"], b["dsnap"],
+                                        b["hist"], history_len, b["cursor"], b["count"], b["running"], b["arrived"], stream())
+        torch.cuda.synchronize()
+        assert torch.equal(qa, qb), f"call {call}"
+        for k in ("amax", "scale", "descale", "ssnap", "dsnap", "hist", "cursor", "count"):
+            assert torch.equal(a[k], b[k]), (call, k)
+        assert float(b["running"]) == 0.0 and int(b["arrived"]) == 0
+        if n:
+            assert host(b["amax"])[0] == orc.amax_bf16(xb[offset:])

@@ -539,10 +539,21 @@ struct TileScales {
 template <int EPI, int SCALE>
 __device__ __forceinline__ void load_row_scales(TileScales<EPI>& s, const GemmArgs& p, const TilePos& t, int wm, int lane) {
     if constexpr (SCALE == SCALE_ROWCOL) {
+        // Two complete paths: these loads are issued among the copies of the tile's last K-tile, and a wait between
+        // a row-index load and the scale load that depends on it also waits for every copy in flight.  Without a
+        // row index nothing waits; with one, the four index loads share a single wait.
+        int r[4];
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            const int r = min(t.m0 + wm * 128 + b * 32 + (lane & 31), t.m_end - 1);
-            s.sa[b] = p.sa[p.a_row_index ? p.a_row_index[r] : r];
+        for (int b = 0; b < 4; ++b) r[b] = min(t.m0 + wm * 128 + b * 32 + (lane & 31), t.m_end - 1);
+        if (p.a_row_index) {
+#pragma unroll
+            for (int b = 0; b < 4; ++b) r[b] = p.a_row_index[r[b]];
+#pragma unroll
+            for (int b = 0; b < 4; ++b) s.sa[b] = p.sa[r[b]];
+            asm volatile("; row scales through the row index" ::: "memory");      // keeps the two paths from being merged again
+        } else {
+#pragma unroll
+            for (int b = 0; b < 4; ++b) s.sa[b] = p.sa[r[b]];
         }
     }
 }

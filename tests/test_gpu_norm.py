@@ -85,7 +85,8 @@ def test_row_clip_matches_oracle(cf, dev, rows, cols):
 
 @pytest.mark.parametrize("e5m2", [False, True])
 @pytest.mark.parametrize("rows,H,clip", [(1, 64, True), (19, 512, True), (8, 776, False), (50, 2048, True), (130, 4096, True),
-                                         (130, 4096, False), (6, 5120, True), (4, 8192, True), (5, 1028, True)])
+                                         (130, 4096, False), (6, 5120, True), (7, 7168, True), (4, 8192, True), (5, 1028, True),
+                                         (3, 12288, True), (9, 1024, True)])
 def test_fused_rows_matches_the_launch_sequence(cf, dev, rows, H, clip, e5m2):
     case(f"fused norm/clip/quantize rows={rows} H={H} clip={clip} e5m2={e5m2}")
     xb, wb = make_rows(rows, H, rows * 7 + H + int(e5m2))
@@ -115,9 +116,9 @@ def test_fused_rows_matches_the_launch_sequence(cf, dev, rows, H, clip, e5m2):
 
 
 @pytest.mark.parametrize("e5m2", [False, True])
-def test_fused_record_matches_the_launch_sequence(cf, dev, e5m2):
-    rows, H = 300, 2048
-    case(f"fused norm/clip/quantize-record e5m2={e5m2}")
+@pytest.mark.parametrize("rows,H", [(300, 2048), (33, 7168), (21, 1000 * 8), (64, 4096)])
+def test_fused_record_matches_the_launch_sequence(cf, dev, rows, H, e5m2):
+    case(f"fused norm/clip/quantize-record rows={rows} H={H} e5m2={e5m2}")
     xb, wb = make_rows(rows, H, 901 + int(e5m2))
     normed0, _ = orc.rmsnorm_forward(xb, wb, EPS)
     ceiling = ceiling_for(normed0)

@@ -1,25 +1,28 @@
 // Scaled FP8 GEMM for gfx950:  C[M,N] = epilogue( (A[M,K] * sa) . (B[N,K] * sb)^T ).
 //
-// Workgroup tile 256 x 256 x 128, four wavefronts in a 2 x 2 arrangement, each
-// owning a 128 x 128 sub-tile = 4 x 4 tiles of v_mfma_f32_32x32x64_f8f6f4 with
-// fp32 accumulators (256 accumulator registers per lane, one wave per SIMD).
-// A and B tiles are staged through LDS, double buffered: while the matrix cores
-// work on stage s the next K-tile is fetched from HBM/L2 with 128-bit loads
-// into registers and written to stage s^1; one barrier per K-tile.
+// Kernels in this file, in the order a call tries them:
+//   k_gemm_nt_ring        the fast path: persistent, operand tiles copied global -> LDS without staging registers
+//                         into a ring of five 32 KiB slots, epilogue through an LDS-staged drain (plain, bias,
+//                         SiLU-gate, fp32 / bf16 accumulate; per-tensor or per-row x per-channel scales; dense or
+//                         grouped per expert).  Needs K % 128 == 0, K >= 256 and a full-width, aligned C.
+//   k_gemm_nt             the same tile with register-staged, double-buffered LDS: any K % 16 == 0, any N.
+//   k_gemm_nt_block_ring  1 x 128 / 128 x 128 block scales on the persistent structure (eight wavefronts, partial
+//                         products folded into running sums every K-tile); k_gemm_nt_block is its staged fallback.
+//   k_gemm_nt_naive       one lane per output element: any shape and alignment, and the on-device cross-check.
 //
-// LDS tile layout: [256 rows][128 bytes], the eight 16-byte chunks of a row are
-// xor-swizzled with f(row) = (row ^ (row >> 3)) & 7 (low five row bits only) so
-// both the 128-bit staging writes and the 128-bit operand reads are spread over
-// all banks.
+// Common to the tiled kernels: workgroup tile 256 x 256 x 128 (128 x 256 x 128 with block scales), wavefronts own
+// 128 x 128 (64 x 64) sub-tiles of v_mfma_f32_32x32x64_f8f6f4 tiles with fp32 accumulators, one barrier per K-tile.
 //
-// The weight operand goes to the MFMA "A" side and the activation to the "B"
-// side, so a lane ends up holding four consecutive OUTPUT COLUMNS of one output
-// row per accumulator quad: the epilogue scales, applies bias / SiLU-gate, rounds
-// to bf16 and stores 8 bytes per lane without a transpose.
+// LDS tile layout: [rows][128 bytes], the eight 16-byte chunks of a row are xor-swizzled with
+// f(row) = (row ^ (row >> 3)) & 7 (low five row bits only) so both the 16-byte writes (copies or staging stores)
+// and the 16-byte operand reads are spread over all banks.
 //
-// Workgroup -> tile mapping is XCD aware: consecutive workgroup ids go round-robin
-// to the 8 XCDs, so each XCD is given a contiguous range of tiles, walked in
-// 8 (M) x 4 (N) patches whose operands fit its own L2.
+// The weight operand goes to the MFMA "A" side and the activation to the "B" side, so a lane ends up holding four
+// consecutive OUTPUT COLUMNS of one output row per accumulator quad: the epilogue scales, applies bias / SiLU-gate
+// and rounds to bf16 without a transpose.
+//
+// Workgroup -> tile mapping is XCD aware: consecutive workgroup ids go round-robin to the 8 XCDs, so each XCD is
+// given a contiguous range of tiles, walked in 8 (M) x 4 (N) patches whose operands share its own L2.
 #include "common.hpp"
 
 #include <mutex>

@@ -28,6 +28,17 @@ __device__ __forceinline__ float block_max(float v, float* sh) {
     return sh[0];
 }
 
+// the same over per-wavefront integers (already reduced within each wavefront)
+__device__ __forceinline__ int block_max_int(int wave_value, int* sh) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0) sh[wave] = wave_value;
+    __syncthreads();
+    int m = sh[0];
+    for (int w = 1; w < (int)(blockDim.x >> 6); ++w) m = max(m, sh[w]);
+    __syncthreads();
+    return m;
+}
+
 struct Vec16 { uint4 lo, hi; };   // 16 bf16
 
 __device__ __forceinline__ Vec16 load16(const uint16_t* p) {
@@ -71,6 +82,20 @@ __device__ __forceinline__ uint4 quant16_finite(const Vec16& v, float s) {
     o.z = cvt4_fp8_finite<E5M2>(bf16_lo(w[4]) * s, bf16_hi(w[4]) * s, bf16_lo(w[5]) * s, bf16_hi(w[5]) * s);
     o.w = cvt4_fp8_finite<E5M2>(bf16_lo(w[6]) * s, bf16_hi(w[6]) * s, bf16_lo(w[7]) * s, bf16_hi(w[7]) * s);
     return o;
+}
+
+// Convert 16 elements with scale s, and (RECORD) fold their |max| into the running maxima: as bf16 bits when all
+// 16 are finite (the common case: no per-element NaN handling at all), as a float maximum otherwise.
+template <bool E5M2, bool RECORD>
+__device__ __forceinline__ uint4 quant16_track(const Vec16& v, float s, bool scale_finite, int& max_bits, float& max_f) {
+    const uint32_t acc = absmax16(0u, v);
+    const int mb = static_cast<int>(max(acc & 0xffffu, acc >> 16));
+    if (mb < 0x7f80 && scale_finite) {
+        if constexpr (RECORD) max_bits = max(max_bits, mb);
+        return quant16_finite<E5M2>(v, s);
+    }
+    if constexpr (RECORD) max_f = fmaxf(max_f, amax16(v));
+    return quant16<E5M2>(v, s);
 }
 
 // ---- amax ------------------------------------------------------------------
@@ -194,7 +219,9 @@ __global__ __launch_bounds__(kThreads) void k_quant(const uint16_t* __restrict__
                                                     float* __restrict__ amax, size_t n) {
     __shared__ float sh[kThreads / 64];
     const float s = *scale;
+    const bool s_finite = fabsf(s) < __uint_as_float(0x7f800000u);
     float local = 0.0f;
+    int local_bits = 0;
     const size_t tid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
     size_t done = 0;
@@ -202,8 +229,7 @@ __global__ __launch_bounds__(kThreads) void k_quant(const uint16_t* __restrict__
         const size_t nvec = n / kVec;
         for (size_t i = tid; i < nvec; i += stride) {
             const Vec16 v = load16(x + i * kVec);
-            if constexpr (RECORD) local = fmaxf(local, amax16(v));
-            *reinterpret_cast<uint4*>(out + i * kVec) = quant16<E5M2>(v, s);
+            *reinterpret_cast<uint4*>(out + i * kVec) = quant16_track<E5M2, RECORD>(v, s, s_finite, local_bits, local);
         }
         done = nvec * kVec;
     }
@@ -213,6 +239,7 @@ __global__ __launch_bounds__(kThreads) void k_quant(const uint16_t* __restrict__
         out[i] = cvt1_fp8<E5M2>(v * s);
     }
     if constexpr (RECORD) {
+        local = fmaxf(local, __uint_as_float(static_cast<uint32_t>(local_bits) << 16));
         const float m = block_max(local, sh);
         if (threadIdx.x == 0) atomic_max_nonneg(amax, m);
     }
@@ -235,7 +262,9 @@ __global__ __launch_bounds__(kAmaxThreads) void k_quant_delayed_step(const uint1
                                                                      size_t n, const DelayedStep d) {
     __shared__ float sh[kAmaxThreads / 64];
     const float s = *d.scale;
+    const bool s_finite = fabsf(s) < __uint_as_float(0x7f800000u);
     float local = 0.0f;
+    int local_bits = 0;
     const size_t tid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
     size_t done = 0;
@@ -243,8 +272,7 @@ __global__ __launch_bounds__(kAmaxThreads) void k_quant_delayed_step(const uint1
         const size_t nvec = n / kVec;
         for (size_t i = tid; i < nvec; i += stride) {
             const Vec16 v = load16(x + i * kVec);
-            local = fmaxf(local, amax16(v));
-            *reinterpret_cast<uint4*>(out + i * kVec) = quant16<E5M2>(v, s);
+            *reinterpret_cast<uint4*>(out + i * kVec) = quant16_track<E5M2, true>(v, s, s_finite, local_bits, local);
         }
         done = nvec * kVec;
     }
@@ -253,6 +281,7 @@ __global__ __launch_bounds__(kAmaxThreads) void k_quant_delayed_step(const uint1
         local = fmaxf(local, fabsf(v));
         out[i] = cvt1_fp8<E5M2>(v * s);
     }
+    local = fmaxf(local, __uint_as_float(static_cast<uint32_t>(local_bits) << 16));
     const float m = block_max(local, sh);
     if (threadIdx.x == 0) {
         atomic_max_nonneg(d.running_amax, m);
@@ -433,15 +462,26 @@ __global__ __launch_bounds__(kThreads) void k_quant_1x128(const uint16_t* __rest
         const bool live = i < nvec;
         Vec16 v = {};
         if (live) v = load16(x + i * kVec);
-        float m = amax16(v);
-        m = fmaxf(m, __shfl_xor(m, 1, kWave));
-        m = fmaxf(m, __shfl_xor(m, 2, kWave));
-        m = fmaxf(m, __shfl_xor(m, 4, kWave));
+        // group maximum as bf16 bits (packed integer maximum of the sign-cleared pairs); a group with a NaN or
+        // an infinity (bits >= 0x7f80) takes the float maximum, which ignores NaNs, and the NaN-restoring convert
+        const uint32_t acc = absmax16(0u, v);
+        int mb = static_cast<int>(max(acc & 0xffffu, acc >> 16));
+        mb = max(mb, __shfl_xor(mb, 1, kWave));
+        mb = max(mb, __shfl_xor(mb, 2, kWave));
+        mb = max(mb, __shfl_xor(mb, 4, kWave));
+        const bool finite = mb < 0x7f80;
+        float m = __uint_as_float(static_cast<uint32_t>(mb) << 16);
+        if (!finite) {
+            m = amax16(v);
+            m = fmaxf(m, __shfl_xor(m, 1, kWave));
+            m = fmaxf(m, __shfl_xor(m, 2, kWave));
+            m = fmaxf(m, __shfl_xor(m, 4, kWave));
+        }
         const float a = fmaxf(m, 1e-12f);
         const float sc = 448.0f / a;
         if (live) {
             if ((i & 7) == 0) { scale[i >> 3] = sc; descale[i >> 3] = a / 448.0f; }
-            *reinterpret_cast<uint4*>(out + i * kVec) = quant16<false>(v, sc);
+            *reinterpret_cast<uint4*>(out + i * kVec) = finite ? quant16_finite<false>(v, sc) : quant16<false>(v, sc);
         }
     }
 }
@@ -481,20 +521,31 @@ __global__ __launch_bounds__(kThreads) void k_quant_128x128(const uint16_t* __re
     float local = 0.0f;
     if (vec) {
         Vec16 v[4];
+        uint32_t acc = 0;
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
             const int r = r0 + p * 32 + tr;
             v[p] = Vec16{};
             if (r < rows) v[p] = load16(x + static_cast<size_t>(r) * K + k0 + tc);
-            local = fmaxf(local, amax16(v[p]));
+            acc = absmax16(acc, v[p]);
         }
-        const float a = fmaxf(block_max(local, sh), 1e-12f);
+        // block maximum as bf16 bits; blocks holding a NaN or an infinity redo it as a float maximum (NaNs ignored)
+        const int mb = block_max_int(wave_absmax_bits(acc), reinterpret_cast<int*>(sh));
+        const bool finite = mb < 0x7f80;
+        float m = __uint_as_float(static_cast<uint32_t>(mb) << 16);
+        if (!finite) {
+#pragma unroll
+            for (int p = 0; p < 4; ++p) local = fmaxf(local, amax16(v[p]));
+            m = block_max(local, sh);
+        }
+        const float a = fmaxf(m, 1e-12f);
         const float sc = 448.0f / a;
         if (threadIdx.x == 0) { scale[blockIdx.x] = sc; descale[blockIdx.x] = a / 448.0f; }
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
             const int r = r0 + p * 32 + tr;
-            if (r < rows) *reinterpret_cast<uint4*>(out + static_cast<size_t>(r) * K + k0 + tc) = quant16<false>(v[p], sc);
+            if (r < rows)
+                *reinterpret_cast<uint4*>(out + static_cast<size_t>(r) * K + k0 + tc) = finite ? quant16_finite<false>(v[p], sc) : quant16<false>(v[p], sc);
         }
     } else {
         const int klen = min(128, K - k0), rlen = min(128, rows - r0);

@@ -15,6 +15,15 @@ static inline float u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
  * benchmark uses on the host (benchmarks/ampere_fp8_fused_gemm_bench.cu:51-56);
  * NaN is kept quiet instead of carrying into the exponent, which is what the
  * device conversion __float2bfloat16 does. */
+/* CUDA's fmaxf: a NaN operand of either kind is ignored (the other operand is returned).  glibc's fmaxf
+ * returns a NaN when an operand is a SIGNALING NaN, which would reset a running maximum; all 65536 bf16
+ * patterns are legal input here, so the reductions below use this form. */
+static inline float max_ignoring_nan(float a, float b) {
+    if (b != b) return a;
+    if (a != a) return b;
+    return a > b ? a : b;
+}
+
 uint16_t orc_bf16_from_f32(float v) {
     uint32_t bits = f2u(v);
     if ((bits & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((bits >> 16) | 0x0040u);
@@ -127,7 +136,7 @@ void orc_e5m2_unpack_n(const uint8_t* in, float* out, size_t n) { for (size_t i 
  * fmaxf ignores NaN operands. */
 void orc_amax_bf16(const uint16_t* x, size_t n, float* amax) {
     float local = 0.0f;
-    for (size_t i = 0; i < n; ++i) local = fmaxf(local, fabsf(orc_bf16_to_f32(x[i])));
+    for (size_t i = 0; i < n; ++i) local = max_ignoring_nan(local, fabsf(orc_bf16_to_f32(x[i])));
     *amax = local;
 }
 
@@ -156,7 +165,7 @@ void orc_quantize_e4m3_record(const uint16_t* x, uint8_t* out, const float* scal
     float local = 0.0f;
     for (size_t i = 0; i < n; ++i) {
         const float v = orc_bf16_to_f32(x[i]);
-        local = fmaxf(local, fabsf(v));
+        local = max_ignoring_nan(local, fabsf(v));
         out[i] = orc_e4m3_satfinite(v * s);
     }
     if ((int32_t)f2u(local) > (int32_t)f2u(*amax)) *amax = local;
@@ -167,7 +176,7 @@ void orc_quantize_e5m2_record(const uint16_t* x, uint8_t* out, const float* scal
     float local = 0.0f;
     for (size_t i = 0; i < n; ++i) {
         const float v = orc_bf16_to_f32(x[i]);
-        local = fmaxf(local, fabsf(v));
+        local = max_ignoring_nan(local, fabsf(v));
         out[i] = orc_e5m2_satfinite(v * s);
     }
     if ((int32_t)f2u(local) > (int32_t)f2u(*amax)) *amax = local;
@@ -306,7 +315,7 @@ void orc_calib_minmax_update(const float* amax, float* cmin, float* cmax) {
  * descale = max(amax,1e-12) / fp8_max, code = cvt(x * scale). */
 void orc_amax_f32(const float* x, size_t n, float* amax) {
     float local = 0.0f;
-    for (size_t i = 0; i < n; ++i) local = fmaxf(local, fabsf(x[i]));
+    for (size_t i = 0; i < n; ++i) local = max_ignoring_nan(local, fabsf(x[i]));
     *amax = local;
 }
 void orc_quantize_f32_e4m3(const float* x, uint8_t* out, const float* scale, size_t n) {
@@ -352,7 +361,7 @@ void orc_quantize_block_128x128(const uint16_t* x, int rows, int K,
             for (int r = r0; r < r1; ++r) {
                 float a;
                 orc_amax_bf16(x + (size_t)r * K + k0, (size_t)len, &a);
-                amax = fmaxf(amax, a);
+                amax = max_ignoring_nan(amax, a);
             }
             orc_scale_from_amax(&amax, ORC_E4M3_MAX, &scale[si], &descale[si]);
             for (int r = r0; r < r1; ++r)

@@ -37,6 +37,33 @@ def test_hardware_convert_matches_oracle_on_every_bf16_input(cf, dev, e5m2):
 
 
 @pytest.mark.parametrize("e5m2", [False, True])
+def test_recording_quantize_on_every_bf16_input(cf, dev, e5m2):
+    """The recording form on all 65536 patterns, in an order that mixes finite and non-finite vectors: same bytes
+    as the plain form, and an amax that ignores the NaNs (here +inf, the largest non-NaN magnitude present)."""
+    case(f"record, all bf16, e5m2={e5m2}")
+    rng = np.random.default_rng(3)
+    bits = rng.permutation(np.concatenate([all_bf16_bits(), np.tile(orc.bf16_from_f32(rng.standard_normal(4096).astype(np.float32)), 64)]))
+    x = dev_bf16(bits, dev)
+    fn = cf.cf_fp8_quantize_e5m2_record if e5m2 else cf.cf_fp8_quantize_e4m3_record
+    for sc in (1.0, 37.5, 0.0, float("inf")):
+        out = torch.empty(bits.size, dtype=torch.uint8, device=dev)
+        amax = scalar(0.0, dev)
+        fn(x, out, scalar(sc, dev), amax, bits.size, stream())
+        torch.cuda.synchronize()
+        wq, wamax = orc.quantize_record(bits, np.float32(sc), np.float32(0.0), e5m2)
+        assert np.array_equal(host(out), wq), f"scale {sc}"
+        assert host(amax).view(np.uint32)[0] == np.float32(wamax).view(np.uint32), f"scale {sc}"
+    finite_only = bits[(bits & 0x7fff) < 0x7f80]
+    xf = dev_bf16(finite_only, dev)
+    out = torch.empty(finite_only.size, dtype=torch.uint8, device=dev)
+    amax = scalar(0.0, dev)
+    fn(xf, out, scalar(2.0, dev), amax, finite_only.size, stream())
+    torch.cuda.synchronize()
+    wq, wamax = orc.quantize_record(finite_only, np.float32(2.0), np.float32(0.0), e5m2)
+    assert np.array_equal(host(out), wq) and host(amax)[0] == wamax
+
+
+@pytest.mark.parametrize("e5m2", [False, True])
 def test_hardware_convert_matches_oracle_on_fp32_sweep(cf, dev, e5m2):
     # 2^26 fp32 bit patterns at stride 64 plus a random offset: every exponent, every rounding position
     case(f"fp32 sweep e5m2={e5m2}")
@@ -214,6 +241,27 @@ def test_block_scaled_quantize(cf, dev, rows, K):
     torch.cuda.synchronize()
     wq, ws, wd = orc.quantize_block_128x128(xb)
     assert np.array_equal(host(s), ws) and np.array_equal(host(d), wd) and np.array_equal(host(out), wq)
+
+
+def test_block_scaled_quantize_with_nonfinite_elements(cf, dev):
+    """Groups holding NaN or infinities take the float maximum (NaNs ignored) and the NaN-restoring convert."""
+    case("block quantize, non-finite groups")
+    rng = np.random.default_rng(21)
+    rows, K = 256, 512
+    xh = rng.standard_normal((rows, K)).astype(np.float32)
+    xh[3, 5] = np.nan; xh[3, 200] = np.inf; xh[130, 300] = -np.inf; xh[200, 129] = np.nan; xh[255, 511] = np.nan
+    xb = orc.bf16_from_f32(xh)
+    x = dev_bf16(xb, dev)
+    for fn, ofn, nscale in ((cf.cf_fp8_quantize_block_1x128, orc.quantize_block_1x128, rows * (K // 128)),
+                            (cf.cf_fp8_quantize_block_128x128, orc.quantize_block_128x128, (rows // 128) * (K // 128))):
+        out = torch.empty((rows, K), dtype=torch.uint8, device=dev)
+        s = torch.empty(nscale, device=dev); d = torch.empty(nscale, device=dev)
+        fn(x, rows, K, out, s, d, stream())
+        torch.cuda.synchronize()
+        wq, ws, wd = ofn(xb)
+        assert np.array_equal(host(s).view(np.uint32), ws.reshape(-1).view(np.uint32))
+        assert np.array_equal(host(d).view(np.uint32), wd.reshape(-1).view(np.uint32))
+        assert np.array_equal(host(out), wq)
 
 
 def test_raw_pack_path(cf, dev):

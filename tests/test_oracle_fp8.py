@@ -317,3 +317,16 @@ def test_bias_add_strided():
     want = x.copy()
     want[:, 3:7] = orc.bf16_from_f32(orc.bf16_to_f32(x[:, 3:7]) + orc.bf16_to_f32(b)[None, :])
     assert np.array_equal(out, want)
+
+
+def test_running_maximum_ignores_every_kind_of_nan():
+    """CUDA's fmaxf returns the non-NaN operand for quiet and signaling NaNs alike; a signaling NaN must not
+    reset the oracle's running maximum (glibc's fmaxf would turn it into a NaN result)."""
+    bits = np.array([0x4000, 0x7f81, 0x3f80, 0xffa0, 0x7fc0, 0xc040, 0x7fbf, 0x3e00], dtype=np.uint16)   # 2, sNaN, 1, -sNaN, qNaN, -3, sNaN, .125
+    assert orc.amax_bf16(bits) == np.float32(3.0)
+    _, amax = orc.quantize_record(bits, np.float32(1.0), np.float32(0.0))
+    assert amax == np.float32(3.0)
+    _, amax = orc.quantize_record(bits, np.float32(1.0), np.float32(0.0), e5m2=True)
+    assert amax == np.float32(3.0)
+    with_inf = np.concatenate([bits, np.array([0xff80, 0x7f85], dtype=np.uint16)])
+    assert np.isposinf(orc.amax_bf16(with_inf))

@@ -160,6 +160,9 @@ def test_transposing_kernels(cf, dev, K, N):
     rng = np.random.default_rng(K * 7 + N)
     wb = orc.bf16_from_f32(rng.standard_normal((K, N)).astype(np.float32))
     s = np.float32(448.0) / orc.amax_bf16(wb)
+    if K * N > 64:        # a few non-finite elements: those vectors take the NaN-restoring convert
+        flat = wb.reshape(-1)
+        flat[rng.integers(0, flat.size, 6)] = np.array([0x7fc0, 0xffc1, 0x7f80, 0xff80, 0x7f81, 0x7fc0], dtype=np.uint16)
     w = dev_bf16(wb, dev)
     sc = scalar(s, dev)
     q = orc.quantize_e4m3(wb, s)

@@ -187,6 +187,29 @@ int cf_rmsnorm_clip_quantize_record(const uint16_t* d_x, const uint16_t* d_scale
                                     float* d_rms, void* d_q, const float* d_qscale,
                                     float* d_amax, cf_stream_t stream);
 
+/* ---- loss head: chunked cross-entropy, fused with the quantize of its gradient ---------
+ * The FP8 head (src/trainer.cu:8015-8060) projects a chunk of rows onto the vocabulary with the NT GEMM above,
+ * runs cross-entropy forward + backward in place, and quantizes the bf16 gradient to E5M2 for the input-gradient
+ * GEMM.  exp / log run on the hardware units here, so gradients agree with a correctly rounded evaluation to one
+ * bf16 ulp (CUDA's expf / logf bits are not reproducible either). */
+
+/* cross_entropy_count_valid, kernels.hpp:571-573, kernels/cross_entropy.cu:201-219,281-287:
+ * adds the number of labels >= 0 to *d_n_valid (the caller zeroes it). */
+int cf_cross_entropy_count_valid(const int32_t* d_labels, int n, int* d_n_valid, cf_stream_t stream);
+/* cross_entropy_fwd_bwd_chunk, kernels.hpp:577-585, kernels/cross_entropy.cu:225-305:
+ * grad[r,v] = bf16((softmax(logits[r])[v] - (v == label[r])) / max(*n_valid, 1)), rows with a negative label get
+ * zeros; *d_loss_out += -log(p_label + 1e-9) / max(*n_valid, 1) per valid row.  d_grad may alias d_logits. */
+int cf_cross_entropy_fwd_bwd_chunk(const uint16_t* d_logits, const int32_t* d_labels, float* d_loss_out,
+                                   uint16_t* d_grad, int rows, int V, const int* d_n_valid,
+                                   cf_stream_t stream);
+/* The same plus what fp8_quant_act does to the gradient in its steady state (src/trainer.cu:8053,
+ * kernels/fp8.cu:86-103): d_grad8 = E5M2(bf16 gradient * *d_qscale), *d_amax raised to the gradient's
+ * maximum (the caller zeroes it).  One pass over the logits instead of four. */
+int cf_cross_entropy_fwd_bwd_chunk_quant_e5m2(const uint16_t* d_logits, const int32_t* d_labels,
+                                              float* d_loss_out, uint16_t* d_grad, void* d_grad8,
+                                              const float* d_qscale, float* d_amax, int rows, int V,
+                                              const int* d_n_valid, cf_stream_t stream);
+
 /* ---- scaled FP8 GEMM -------------------------------------------------------
  * Replaces the reference's cuBLASLt wrappers, which are static functions of
  * src/trainer.cu bound to its Fp8Ctx (handle, workspace, plan cache); the

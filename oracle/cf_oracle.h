@@ -37,6 +37,9 @@
  *                                 recomputation, order-sensitive crafted row;
  *                                 summation order beyond the source text:
  *                                 parity unpinned).
+ *   cross-entropy                 see cf_oracle_ce.c (closed forms, sum-to-zero,
+ *                                 double recomputation; libm exp/log stand in
+ *                                 for CUDA's: parity unpinned beyond 1 bf16 ulp).
  *   GEMM references               definition from the task statement: matmul
  *                                 of the dequantised operands; special cases
  *                                 reduce to numpy matmul.  cuBLASLt's own
@@ -125,6 +128,11 @@ void orc_bias_add_strided_bf16(uint16_t* inout, const uint16_t* bias,
 int  orc_rmsnorm_forward(const uint16_t* x, const uint16_t* scale, uint16_t* out, float* rms,
                          int rows, int H, float eps);
 void orc_act_row_clip_abs(uint16_t* x, int rows, int cols, float ceiling, float* normsq);
+
+/* ---- chunked cross-entropy (cf_oracle_ce.c; kernels/cross_entropy.cu:201-305) ---- */
+void orc_cross_entropy_count_valid(const int32_t* labels, int n, int* n_valid);
+void orc_cross_entropy_fwd_bwd_chunk(const uint16_t* logits, const int32_t* labels, float* loss_out,
+                                     uint16_t* grad, int rows, int V, const int* n_valid);
 
 /* ---- GEMM references ----------------------------------------------------
  * scale_mode: 0 per-tensor (a_descale[1], b_descale[1])

@@ -329,6 +329,24 @@ def act_row_clip_abs(x, ceiling):
     return x, normsq
 
 
+# ---- chunked cross-entropy -----------------------------------------------------------
+def cross_entropy_count_valid(labels):
+    labels = np.ascontiguousarray(labels, dtype=np.int32)
+    n = np.zeros(1, np.int32)
+    _call("orc_cross_entropy_count_valid", labels, c_i(labels.size), n)
+    return int(n[0])
+
+
+def cross_entropy_fwd_bwd_chunk(logits, labels, n_valid, loss_in=0.0):
+    logits = np.ascontiguousarray(logits, dtype=np.uint16)
+    labels = np.ascontiguousarray(labels, dtype=np.int32)
+    rows, V = logits.shape
+    grad = np.empty((rows, V), np.uint16)
+    loss = _f32(loss_in)
+    _call("orc_cross_entropy_fwd_bwd_chunk", logits, labels, loss, grad, c_i(rows), c_i(V), np.array([n_valid], np.int32))
+    return grad, loss[0]
+
+
 # ---- GEMM ---------------------------------------------------------------------------
 def gemm_nt_ref(A, B, a_descale, b_descale, a_e5m2=False, b_e5m2=False, scale_mode=0, lda=None, want_abs=True):
     """A[M,K] fp8 bytes (row stride lda), B[N,K] fp8 bytes -> (ref[M,N] f64, absdot[M,N] f64)."""

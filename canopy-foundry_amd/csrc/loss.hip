@@ -77,18 +77,25 @@ __global__ __launch_bounds__(kCeThreads) void k_ce_rows(const CeArgs p) {
         }
     }
     const float row_max = block_reduce(m, sh, true);
+    // exp(x - max) as exp2(x * log2e - max * log2e): one fused multiply-add per element feeds the exp2 unit
+    const float bias2 = -row_max * kLog2e;
     float s = 0.0f;
 #pragma unroll
     for (int j = 0; j < kCeMaxChunks; ++j) {
         if (tid + j * kCeThreads < nchunks) {
             const uint32_t w[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
 #pragma unroll
-            for (int k = 0; k < 4; ++k) s += fast_exp(bf16_lo(w[k]) - row_max) + fast_exp(bf16_hi(w[k]) - row_max);
+            for (int k = 0; k < 4; ++k)
+                s += __builtin_amdgcn_exp2f(__builtin_fmaf(bf16_lo(w[k]), kLog2e, bias2)) +
+                     __builtin_amdgcn_exp2f(__builtin_fmaf(bf16_hi(w[k]), kLog2e, bias2));
         }
     }
     const float inv_sum = 1.0f / block_reduce(s, sh, false);
     const float inv_n = 1.0f / static_cast<float>(max(*p.n_valid, 1));
+    const float both = inv_sum * inv_n;                  // every column but the label's: exp * (1 / sum) * (1 / n)
     const float qs = QUANT ? *p.qscale : 0.0f;
+    const bool qs_finite = fabsf(qs) < __uint_as_float(0x7f800000u);
+    const int label_chunk = label >> 3;
     float llp = 0.0f;
     uint32_t absacc = 0;
 #pragma unroll
@@ -97,19 +104,33 @@ __global__ __launch_bounds__(kCeThreads) void k_ce_rows(const CeArgs p) {
         if (c < nchunks) {
             const uint32_t w[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
             uint32_t o[4];
+            if (c != label_chunk) {
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const int e = c * 8 + 2 * k;
-                o[k] = pack_bf16x2_hw(ce_grad(bf16_lo(w[k]), row_max, inv_sum, inv_n, e == label, llp),
-                                      ce_grad(bf16_hi(w[k]), row_max, inv_sum, inv_n, e + 1 == label, llp));
+                for (int k = 0; k < 4; ++k)
+                    o[k] = pack_bf16x2_hw(__builtin_amdgcn_exp2f(__builtin_fmaf(bf16_lo(w[k]), kLog2e, bias2)) * both,
+                                          __builtin_amdgcn_exp2f(__builtin_fmaf(bf16_hi(w[k]), kLog2e, bias2)) * both);
+            } else {
+                // the chunk with the label's column: kernels/cross_entropy.cu:263-268 as written
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const int e = c * 8 + 2 * k;
+                    o[k] = pack_bf16x2_hw(ce_grad(bf16_lo(w[k]), row_max, inv_sum, inv_n, e == label, llp),
+                                          ce_grad(bf16_hi(w[k]), row_max, inv_sum, inv_n, e + 1 == label, llp));
+                }
             }
             reinterpret_cast<uint4*>(grow)[c] = make_uint4(o[0], o[1], o[2], o[3]);
             if constexpr (QUANT) {
                 // src/trainer.cu:8053: the E5M2 quantize of the bf16 gradient with the slot's previous scale, amax recorded
-                absacc = pk_absmax(pk_absmax(pk_absmax(pk_absmax(absacc, o[0]), o[1]), o[2]), o[3]);
+                const uint32_t acc8 = pk_absmax(pk_absmax(pk_absmax(pk_absmax(0u, o[0]), o[1]), o[2]), o[3]);
+                absacc = pk_absmax(absacc, acc8);        // sign bits are clear in both
                 uint2 q;
-                q.x = cvt4_fp8<true>(bf16_lo(o[0]) * qs, bf16_hi(o[0]) * qs, bf16_lo(o[1]) * qs, bf16_hi(o[1]) * qs);
-                q.y = cvt4_fp8<true>(bf16_lo(o[2]) * qs, bf16_hi(o[2]) * qs, bf16_lo(o[3]) * qs, bf16_hi(o[3]) * qs);
+                if (max(acc8 & 0xffffu, acc8 >> 16) < 0x7f80u && qs_finite) {
+                    q.x = cvt4_fp8_finite<true>(bf16_lo(o[0]) * qs, bf16_hi(o[0]) * qs, bf16_lo(o[1]) * qs, bf16_hi(o[1]) * qs);
+                    q.y = cvt4_fp8_finite<true>(bf16_lo(o[2]) * qs, bf16_hi(o[2]) * qs, bf16_lo(o[3]) * qs, bf16_hi(o[3]) * qs);
+                } else {
+                    q.x = cvt4_fp8<true>(bf16_lo(o[0]) * qs, bf16_hi(o[0]) * qs, bf16_lo(o[1]) * qs, bf16_hi(o[1]) * qs);
+                    q.y = cvt4_fp8<true>(bf16_lo(o[2]) * qs, bf16_hi(o[2]) * qs, bf16_lo(o[3]) * qs, bf16_hi(o[3]) * qs);
+                }
                 reinterpret_cast<uint2*>(qrow)[c] = q;
             }
         }

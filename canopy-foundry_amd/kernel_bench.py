@@ -181,6 +181,23 @@ def main():
          lambda: cf.cf_fp8_gemm_tn_accum_bf16(N, K, M, xt, sc, dyt, de, dwb, K, st))
     del xq, wg, wu, wd, hq, c, y, dy, xt, dyt, dw, dwb
 
+    # ---- loss head: one chunk of the fused classifier (2048 rows x 32000 logits) ----------------------------
+    CR, V = 2048, 32000
+    logits = bf16(CR, V, sigma=3.0)
+    labels = torch.randint(0, V, (CR,), device=dev, generator=g, dtype=torch.int32)
+    nvalid = torch.full((1,), CR, dtype=torch.int32, device=dev)
+    cgrad = torch.empty_like(logits); cg8 = u8(CR, V); closs = torch.zeros(1, device=dev)
+    hbm("cross_entropy_fwd_bwd_chunk (bf16 gradient)", f"{CR}x{V}", 4.0 * CR * V,
+        lambda: cf.cf_cross_entropy_fwd_bwd_chunk(logits, labels, closs, cgrad, CR, V, nvalid, st))
+
+    def ce_then_quant():
+        cf.cf_cross_entropy_fwd_bwd_chunk(logits, labels, closs, cgrad, CR, V, nvalid, st)
+        cf.cf_fp8_quantize_e5m2_record(cgrad, cg8, sc, amax, CR * V, st)
+    hbm("cross entropy, then E5M2 recording quantize (2 launches)", f"{CR}x{V}", 5.0 * CR * V, ce_then_quant)
+    hbm("cross_entropy_fwd_bwd_chunk_quant_e5m2 (fused)", f"{CR}x{V}", 5.0 * CR * V,
+        lambda: cf.cf_cross_entropy_fwd_bwd_chunk_quant_e5m2(logits, labels, closs, cgrad, cg8, sc, amax, CR, V, nvalid, st))
+    del logits, cgrad, cg8
+
     # ---- config 5: MoE ------------------------------------------------------------------------------
     T, H, E, k, Ie = 16384, 2048, 64, 6, 1408
     logits = torch.randn(T, E, device=dev, generator=g)

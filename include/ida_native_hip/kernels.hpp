@@ -109,6 +109,15 @@ inline void rmsnorm_forward(const bf16* d_x, const bf16* d_scale, bf16* d_out, f
     CF_FWD(cf_rmsnorm_forward(hip_detail::u(d_x), hip_detail::u(d_scale), hip_detail::u(d_out), d_rms, rows, H, eps, stream));
 }
 
+// ---- kernels.hpp:571-585 (kernels/cross_entropy.cu) -------------------------------------------------------
+inline void cross_entropy_count_valid(const int32_t* d_labels, int n, int* d_n_valid, hipStream_t stream) {
+    CF_FWD(cf_cross_entropy_count_valid(d_labels, n, d_n_valid, stream));
+}
+inline void cross_entropy_fwd_bwd_chunk(const bf16* d_logits, const int32_t* d_labels, float* d_loss_out, bf16* d_grad,
+                                        int rows, int V, const int* d_n_valid, hipStream_t stream) {
+    CF_FWD(cf_cross_entropy_fwd_bwd_chunk(hip_detail::u(d_logits), d_labels, d_loss_out, hip_detail::u(d_grad), rows, V, d_n_valid, stream));
+}
+
 // ---- kernels.hpp:193, 313-317, 340-343, 361-423 (kernels/cross_entropy.cu, kernels/moe.cu) -----------------
 inline void softmax_inplace_f32(float* d_x, int rows, int cols, hipStream_t stream) {
     CF_FWD(cf_softmax_inplace_f32(d_x, rows, cols, stream));

@@ -47,6 +47,14 @@ __device__ __forceinline__ float ce_grad(float logit, float row_max, float inv_s
     return (prob - (is_label ? 1.0f : 0.0f)) * inv_n;
 }
 
+// The chunk's four words as the compiler cannot relate to their earlier uses: without this it unpacks all 128
+// logits of a lane to fp32 once and keeps them live across the three passes (184 registers, two wavefronts per
+// SIMD); unpacking again in each pass costs one instruction per element and halves the register count.
+__device__ __forceinline__ void opaque_words(const uint4& v, uint32_t (&w)[4]) {
+    w[0] = v.x; w[1] = v.y; w[2] = v.z; w[3] = v.w;
+    asm volatile("" : "+v"(w[0]), "+v"(w[1]), "+v"(w[2]), "+v"(w[3]));
+}
+
 // Row in registers: V % 8 == 0, V <= 32768, 16-byte aligned rows (8-byte for the fp8 gradient).
 template <bool QUANT>
 __global__ __launch_bounds__(kCeThreads) void k_ce_rows(const CeArgs p) {
@@ -83,12 +91,14 @@ __global__ __launch_bounds__(kCeThreads) void k_ce_rows(const CeArgs p) {
 #pragma unroll
     for (int j = 0; j < kCeMaxChunks; ++j) {
         if (tid + j * kCeThreads < nchunks) {
-            const uint32_t w[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+            uint32_t w[4];
+            opaque_words(v[j], w);
 #pragma unroll
             for (int k = 0; k < 4; ++k)
                 s += __builtin_amdgcn_exp2f(__builtin_fmaf(bf16_lo(w[k]), kLog2e, bias2)) +
                      __builtin_amdgcn_exp2f(__builtin_fmaf(bf16_hi(w[k]), kLog2e, bias2));
         }
+        __builtin_amdgcn_sched_barrier(0);       // one chunk's temporaries at a time: the row itself takes 64 registers
     }
     const float inv_sum = 1.0f / block_reduce(s, sh, false);
     const float inv_n = 1.0f / static_cast<float>(max(*p.n_valid, 1));
@@ -102,7 +112,8 @@ __global__ __launch_bounds__(kCeThreads) void k_ce_rows(const CeArgs p) {
     for (int j = 0; j < kCeMaxChunks; ++j) {
         const int c = tid + j * kCeThreads;
         if (c < nchunks) {
-            const uint32_t w[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+            uint32_t w[4];
+            opaque_words(v[j], w);
             uint32_t o[4];
             if (c != label_chunk) {
 #pragma unroll
@@ -134,6 +145,7 @@ __global__ __launch_bounds__(kCeThreads) void k_ce_rows(const CeArgs p) {
                 reinterpret_cast<uint2*>(qrow)[c] = q;
             }
         }
+        __builtin_amdgcn_sched_barrier(0);
     }
     // only the lane that met the label holds a non-zero term (:269-272)
     const float g_llp = block_reduce(llp, sh, false);

@@ -227,10 +227,14 @@ __global__ __launch_bounds__(256) void k_norm_row_wave(const NormArgs p, int row
     for (int j = 0; j < J; ++j) v[j] = *reinterpret_cast<const uint4*>(p.x + base + 512 * j);
 
     auto rewrite = [&](int j, auto f) {      // v[j][i] <- bf16(f(value, i))
+        // The words are hidden from common-subexpression elimination: otherwise the fp32 values unpacked for the sum
+        // of squares stay live until here (64 more registers per lane at H = 4096); unpacking again is one
+        // instruction per element.
+        uint32_t w[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+        asm volatile("" : "+v"(w[0]), "+v"(w[1]), "+v"(w[2]), "+v"(w[3]));
         uint32_t o[4];
 #pragma unroll
-        for (int k = 0; k < 4; ++k)
-            o[k] = pack_bf16x2_hw(f(bf16_at(v[j], 2 * k), 2 * k), f(bf16_at(v[j], 2 * k + 1), 2 * k + 1));
+        for (int k = 0; k < 4; ++k) o[k] = pack_bf16x2_hw(f(bf16_lo(w[k]), 2 * k), f(bf16_hi(w[k]), 2 * k + 1));
         v[j] = make_uint4(o[0], o[1], o[2], o[3]);
     };
 

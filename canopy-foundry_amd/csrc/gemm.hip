@@ -1156,7 +1156,9 @@ void k_gemm_nt_block_ring(const GemmArgs p) {
     auto dma16 = [&](uint32_t dst, uint32_t voff, const uint8_t* base) {
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(dst), "v"(voff), "s"(base) : "memory");
     };
-    // 4-byte copies by the low 16 lanes only: lane l lands at dst + 4 l
+    // 4-byte copies by the low 16 lanes only: lane l lands at dst + 4 l.  The execution mask is narrowed and then set
+    // back to all ones inside the statement; every call site is in wavefront-uniform control flow with all 64 lanes
+    // active, so "all ones" is what it was.
     auto dma4_lo16 = [&](uint32_t dst, uint32_t voff, const uint8_t* base) {
         asm volatile("s_mov_b32 m0, %0\n\ts_mov_b32 exec_lo, 0xffff\n\ts_mov_b32 exec_hi, 0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2\n\t"
                      "s_mov_b32 exec_lo, -1\n\ts_mov_b32 exec_hi, -1\n\ts_nop 0"

@@ -158,24 +158,56 @@ __global__ __launch_bounds__(128) void k_topk_generic(float* __restrict__ scores
 __global__ __launch_bounds__(1024) void k_build_row_lists(const float* __restrict__ route_weights,
                                                           int* __restrict__ counts, int* __restrict__ row_indices,
                                                           int rows, int E) {
-    __shared__ int wave_tot[16];
+    // One workgroup per expert walks its (strided) column in super-slabs of 16 x 1024 rows: all sixteen membership
+    // loads of a lane are issued together (each is a full memory latency), the 256 per-(slab, wavefront) member
+    // counts are scanned once, and every lane then writes its members at their ranks: ascending row order.
+    __shared__ int tot[256];          // [slab][wavefront] member counts, then their exclusive prefix
+    __shared__ int wsum[4];
     __shared__ int base_sh;
     const int e = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6;
     int* out = row_indices + static_cast<size_t>(e) * rows;
     if (t == 0) base_sh = 0;
-    __syncthreads();
-    for (int r0 = 0; r0 < rows; r0 += 1024) {
-        const int row = r0 + t;
-        const bool sel = row < rows && route_weights[static_cast<size_t>(row) * E + e] > 0.0f;
-        const unsigned long long m = __ballot(sel);
-        const int rank = __builtin_popcountll(m & ((1ull << lane) - 1ull));
-        if (lane == 0) wave_tot[wave] = __builtin_popcountll(m);
+    for (int r0 = 0; r0 < rows; r0 += 16 * 1024) {
+        unsigned bits = 0;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int row = r0 + i * 1024 + t;
+            const float w = row < rows ? route_weights[static_cast<size_t>(row) * E + e] : 0.0f;
+            bits |= (w > 0.0f ? 1u : 0u) << i;
+        }
+        int rank[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const unsigned long long m = __ballot((bits >> i) & 1u);
+            rank[i] = __builtin_popcountll(m & ((1ull << lane) - 1ull));
+            if (lane == 0) tot[i * 16 + wave] = __builtin_popcountll(m);
+        }
         __syncthreads();
-        int before = base_sh;
-        for (int w = 0; w < wave; ++w) before += wave_tot[w];
-        if (sel) out[before + rank] = row;
+        // exclusive prefix of the 256 counts in (slab, wavefront) order by the first four wavefronts
+        int incl = 0, mine = 0;
+        if (t < 256) {
+            mine = tot[t];
+            incl = mine;
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const int o = __shfl_up(incl, off, kWave);
+                if (lane >= off) incl += o;
+            }
+            if (lane == 63) wsum[wave] = incl;
+        }
         __syncthreads();
-        if (t == 0) { int s = 0; for (int w = 0; w < 16; ++w) s += wave_tot[w]; base_sh += s; }
+        const int base = base_sh;
+        if (t < 256) {
+            int before = 0;
+            for (int w = 0; w < wave; ++w) before += wsum[w];
+            tot[t] = before + incl - mine;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+            if ((bits >> i) & 1u) out[base + tot[i * 16 + wave] + rank[i]] = r0 + i * 1024 + t;
+        __syncthreads();                                  // tot and base_sh are rewritten next
+        if (t == 0) base_sh = base + wsum[0] + wsum[1] + wsum[2] + wsum[3];
         __syncthreads();
     }
     if (t == 0) counts[e] = base_sh;

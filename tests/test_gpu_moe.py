@@ -109,7 +109,7 @@ def test_config5_routing_and_dispatch_full_size(cf, dev):
         assert np.array_equal(bf16_bits(mixed_d), mixed)
 
 
-@pytest.mark.parametrize("rows,E,H", [(1, 1, 1), (301, 16, 24), (1030, 7, 40), (64, 3, 5)])
+@pytest.mark.parametrize("rows,E,H", [(1, 1, 1), (301, 16, 24), (1030, 7, 40), (64, 3, 5), (40000, 5, 8), (16385, 2, 8)])
 def test_dispatch_small_and_ragged(cf, dev, rows, E, H):
     case(f"dispatch rows={rows} E={E} H={H}")
     rng = np.random.default_rng(rows + E)

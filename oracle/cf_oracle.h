@@ -29,6 +29,10 @@
  *   transposes / gathers          permutation identities on ragged shapes.
  *   softmax / top-k               tests/fixtures/moe_router_parity (JSON),
  *                                 invariants, brute force on tiny E.
+ *   grouped GELU expert bank      the reference's router-parity fixture also holds
+ *                                 hidden_gated / route_weights / weights / mixed:
+ *                                 formula reproduced in float64 to 4e-8, FP8 form
+ *                                 to quantization error (tests/golden/moe_expert_bank.json).
  *   orc_expf                      <= 2 ulp of the double-precision exp over a
  *                                 dense sweep (it is this build's definition of
  *                                 the router's expf; CUDA's expf bits cannot be

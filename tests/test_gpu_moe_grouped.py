@@ -180,3 +180,41 @@ def test_grouped_gelu_expert_bank_reference_form(cf, dev, rows, E, k, H, Ie, e5m
     # rows routed to no expert keep their value
     untouched = ~(rw > 0).any(axis=1)
     assert np.array_equal(bf16_bits(mixed)[untouched], mixed0[untouched])
+
+
+def test_grouped_gelu_expert_bank_on_the_reference_fixture(cf, dev):
+    """The expert bank of the reference's own router-parity case (tests/fixtures/moe_router_parity), operands
+    quantized to E4M3 with per-tensor scales: the kernel must land on the fixture's `mixed` minus its trunk term to
+    within the quantization error, and on the oracle's reference of the same quantized operands to bf16 rounding."""
+    import json
+    import math
+    from pathlib import Path
+    case("grouped gelu bank, reference fixture")
+    g = json.loads((Path(__file__).resolve().parent / "golden" / "moe_expert_bank.json").read_text())
+    hg, rw, mixed = np.array(g["hidden_gated"]), np.array(g["route_weights"]), np.array(g["mixed"])
+    tin, tout = np.array(g["trunk_fc_in_w"]), np.array(g["trunk_fc_out_w"])
+    ein, eout = np.array(g["expert_fc_in_w"]), np.array(g["expert_fc_out_w"])
+    B, S, H = hg.shape
+    E, Ie, _ = ein.shape
+    rows = B * S
+    erf = np.vectorize(math.erf)
+    trunk = (lambda x: 0.5 * x * (1.0 + erf(x / math.sqrt(2.0))))(hg @ tin.T) @ tout.T
+    want = (mixed - trunk).reshape(rows, H)
+    route = np.repeat(rw, S, axis=0).astype(np.float32)
+    counts, idx = orc.moe_build_expert_row_lists(route)
+
+    def q(x):
+        s, d = orc.scale_from_amax(np.float32(np.abs(x).max()), 448.0)
+        return orc.e4m3_satfinite((x.astype(np.float32) * s).astype(np.float32)).reshape(x.shape), d
+    hq, hd = q(hg.reshape(rows, H)); wiq, wid = q(ein); woq, wod = q(eout)
+    out = torch.zeros((rows, H), dtype=torch.bfloat16, device=dev)
+    sc = lambda v: torch.tensor([v], dtype=torch.float32, device=dev)
+    cf.cf_moe_grouped_expert_forward_fp8(dev_arr(hq, dev), sc(hd), 0, dev_arr(route, dev), dev_arr(counts, dev), None,
+                                         dev_arr(idx, dev), dev_arr(wiq, dev), sc(wid), dev_arr(woq, dev), sc(wod),
+                                         out, rows, H, Ie, E, int(counts.sum()), stream())
+    torch.cuda.synchronize()
+    got = orc.bf16_to_f32(bf16_bits(out)).astype(np.float64)
+    scale = np.abs(want).max()
+    assert np.abs(got - want).max() < 0.06 * scale
+    ref = orc.moe_grouped_expert_forward_fp8_ref(hq, hd, False, route, counts, idx, wiq, wid, woq, wod, np.zeros((rows, H)))
+    assert np.all(np.abs(got - ref) <= (E + 1) * 2.0 ** -8 * (np.abs(ref) + scale))

@@ -214,3 +214,50 @@ def test_grouped_gelu_expert_reference_against_numpy():
         sel = np.nonzero(rw[:, e] > 0)[0]
         want[sel] += rw[sel, e][:, None].astype(np.float64) * (gelu(h[sel] @ wi.T) @ wo.T)
     assert np.allclose(got, want, rtol=1e-12, atol=1e-12)
+
+
+def test_expert_bank_formula_against_the_reference_fixture():
+    """The reference's own router-parity case also holds the expert bank's inputs and its output `mixed`
+    (tests/fixtures/moe_router_parity).  It fixes what the grouped expert forward computes:
+    mixed = trunk(h) + sum_e w[sample, e] * fc_out_e(gelu_erf(fc_in_e(h))), weights laid out [E, Ie, H] and [E, H, Ie].
+    (1) a float64 restatement reproduces `mixed` with the exact-erf GELU and visibly not with the tanh form;
+    (2) the oracle's FP8 expert-bank reference, fed the same operands quantized to E4M3, lands on mixed - trunk to
+        within the quantization error: a transposed weight or a dropped route weight would be off by the full scale."""
+    import math
+    g = json.loads((GOLD / "moe_expert_bank.json").read_text())
+    hg, rw, mixed = np.array(g["hidden_gated"]), np.array(g["route_weights"]), np.array(g["mixed"])
+    tin, tout = np.array(g["trunk_fc_in_w"]), np.array(g["trunk_fc_out_w"])
+    ein, eout = np.array(g["expert_fc_in_w"]), np.array(g["expert_fc_out_w"])
+    B, S, H = hg.shape
+    E, Ie, _ = ein.shape
+    erf = np.vectorize(math.erf)
+    gelu_erf = lambda x: 0.5 * x * (1.0 + erf(x / math.sqrt(2.0)))
+    gelu_tanh = lambda x: 0.5 * x * (1.0 + np.tanh(math.sqrt(2.0 / math.pi) * (x + 0.044715 * x ** 3)))
+
+    def bank(act):
+        out = np.zeros_like(mixed)
+        for e in range(E):
+            out += rw[:, None, e:e + 1] * (act(hg @ ein[e].T) @ eout[e].T)
+        return out
+    trunk = gelu_erf(hg @ tin.T) @ tout.T
+    assert np.abs(trunk + bank(gelu_erf) - mixed).max() < 1e-6
+    assert np.abs(gelu_tanh(hg @ tin.T) @ tout.T + bank(gelu_tanh) - mixed).max() > 5e-5
+    want = (mixed - trunk).reshape(B * S, H)
+
+    rows = B * S
+    route = np.repeat(rw, S, axis=0).astype(np.float32)              # the route weight is per sample: every token of it
+    counts, idx = orc.moe_build_expert_row_lists(route)
+
+    def q(x):                                                        # per-tensor E4M3 as the reference's slots do
+        amax = np.float32(np.abs(x).max())
+        s, d = orc.scale_from_amax(amax, 448.0)
+        return orc.e4m3_satfinite((x.astype(np.float32) * s).astype(np.float32)).reshape(x.shape), d
+    hq, hd = q(hg.reshape(rows, H))
+    wiq, wid = q(ein)
+    woq, wod = q(eout)
+    got = orc.moe_grouped_expert_forward_fp8_ref(hq, hd, False, route, counts, idx, wiq, wid, woq, wod, np.zeros((rows, H)))
+    scale = np.abs(want).max()
+    assert np.abs(got - want).max() < 0.06 * scale, (np.abs(got - want).max(), scale)      # measured: 0.027
+    # sensitivity: the same call with the experts' weights in the wrong order misses by much more
+    wrong = orc.moe_grouped_expert_forward_fp8_ref(hq, hd, False, route, counts, idx, wiq[::-1].copy(), wid, woq, wod, np.zeros((rows, H)))
+    assert np.abs(wrong - want).max() > 0.3 * scale

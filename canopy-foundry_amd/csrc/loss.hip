@@ -160,6 +160,85 @@ __global__ __launch_bounds__(kCeThreads) void k_ce_rows(const CeArgs p) {
     }
 }
 
+// Rows longer than the register-resident form takes (V % 8 == 0, aligned): the same arithmetic with the row read
+// three times in 16-byte vectors; the second and third reads mostly come from the caches.
+template <bool QUANT>
+__global__ __launch_bounds__(kCeThreads) void k_ce_rows_stream(const CeArgs p) {
+    __shared__ float sh[kCeThreads / 64];
+    const int tid = threadIdx.x, V = p.V, nchunks = V / 8;
+    const size_t row = blockIdx.x;
+    const int label = p.labels[row];
+    uint16_t* grow = p.grad + row * V;
+    uint8_t* qrow = QUANT ? p.grad8 + row * V : nullptr;
+    if (label < 0) {
+        for (int c = tid; c < nchunks; c += kCeThreads) {
+            reinterpret_cast<uint4*>(grow)[c] = make_uint4(0, 0, 0, 0);
+            if constexpr (QUANT) reinterpret_cast<uint2*>(qrow)[c] = make_uint2(0, 0);
+        }
+        return;
+    }
+    const uint4* lrow = reinterpret_cast<const uint4*>(p.logits + row * V);
+    float m = -3.402823466e38f;
+    for (int c = tid; c < nchunks; c += kCeThreads) {
+        const uint4 v = lrow[c];
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) m = fmaxf(m, fmaxf(bf16_lo(w[k]), bf16_hi(w[k])));
+    }
+    const float row_max = block_reduce(m, sh, true);
+    const float bias2 = -row_max * kLog2e;
+    float s = 0.0f;
+    for (int c = tid; c < nchunks; c += kCeThreads) {
+        const uint4 v = lrow[c];
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            s += __builtin_amdgcn_exp2f(__builtin_fmaf(bf16_lo(w[k]), kLog2e, bias2)) +
+                 __builtin_amdgcn_exp2f(__builtin_fmaf(bf16_hi(w[k]), kLog2e, bias2));
+    }
+    const float inv_sum = 1.0f / block_reduce(s, sh, false);
+    const float inv_n = 1.0f / static_cast<float>(max(*p.n_valid, 1));
+    const float both = inv_sum * inv_n;
+    const float qs = QUANT ? *p.qscale : 0.0f;
+    const int label_chunk = label >> 3;
+    float llp = 0.0f;
+    uint32_t absacc = 0;
+    for (int c = tid; c < nchunks; c += kCeThreads) {
+        const uint4 v = lrow[c];                           // read before the (possibly aliasing) store below
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        uint32_t o[4];
+        if (c != label_chunk) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                o[k] = pack_bf16x2_hw(__builtin_amdgcn_exp2f(__builtin_fmaf(bf16_lo(w[k]), kLog2e, bias2)) * both,
+                                      __builtin_amdgcn_exp2f(__builtin_fmaf(bf16_hi(w[k]), kLog2e, bias2)) * both);
+        } else {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int e = c * 8 + 2 * k;
+                o[k] = pack_bf16x2_hw(ce_grad(bf16_lo(w[k]), row_max, inv_sum, inv_n, e == label, llp),
+                                      ce_grad(bf16_hi(w[k]), row_max, inv_sum, inv_n, e + 1 == label, llp));
+            }
+        }
+        reinterpret_cast<uint4*>(grow)[c] = make_uint4(o[0], o[1], o[2], o[3]);
+        if constexpr (QUANT) {
+            absacc = pk_absmax(pk_absmax(pk_absmax(pk_absmax(absacc, o[0]), o[1]), o[2]), o[3]);
+            uint2 q;
+            q.x = cvt4_fp8<true>(bf16_lo(o[0]) * qs, bf16_hi(o[0]) * qs, bf16_lo(o[1]) * qs, bf16_hi(o[1]) * qs);
+            q.y = cvt4_fp8<true>(bf16_lo(o[2]) * qs, bf16_hi(o[2]) * qs, bf16_lo(o[3]) * qs, bf16_hi(o[3]) * qs);
+            reinterpret_cast<uint2*>(qrow)[c] = q;
+        }
+    }
+    const float g_llp = block_reduce(llp, sh, false);
+    if (tid == 0) atomicAdd(p.loss, -g_llp * inv_n);
+    if constexpr (QUANT) {
+        int mb = wave_absmax_bits(absacc);
+        if (mb > 0x7f80) mb = 0;                           // a NaN row leaves the recorded amax to the finite rows
+        const float a = block_reduce(__uint_as_float(static_cast<uint32_t>(mb) << 16), sh, true);
+        if (tid == 0) atomic_max_nonneg(p.amax, a);
+    }
+}
+
 // Any V, any alignment: three passes over the row, as the reference does.
 template <bool QUANT>
 __global__ __launch_bounds__(kCeThreads) void k_ce_rows_generic(const CeArgs p) {
@@ -213,10 +292,11 @@ __global__ __launch_bounds__(kCeThreads) void k_count_valid(const int32_t* __res
 
 template <bool QUANT>
 int launch_ce(const CeArgs& p, int rows, hipStream_t st) {
-    const bool fast = p.V % 8 == 0 && p.V <= kCeMaxChunks * kCeThreads * 8 && aligned16(p.logits) && aligned16(p.grad) &&
-                      (!QUANT || (reinterpret_cast<uintptr_t>(p.grad8) & 7u) == 0);
-    if (fast) k_ce_rows<QUANT><<<rows, kCeThreads, 0, st>>>(p);
-    else      k_ce_rows_generic<QUANT><<<rows, kCeThreads, 0, st>>>(p);
+    const bool vec = p.V % 8 == 0 && aligned16(p.logits) && aligned16(p.grad) &&
+                     (!QUANT || (reinterpret_cast<uintptr_t>(p.grad8) & 7u) == 0);
+    if (vec && p.V <= kCeMaxChunks * kCeThreads * 8) k_ce_rows<QUANT><<<rows, kCeThreads, 0, st>>>(p);
+    else if (vec)                                    k_ce_rows_stream<QUANT><<<rows, kCeThreads, 0, st>>>(p);
+    else                                             k_ce_rows_generic<QUANT><<<rows, kCeThreads, 0, st>>>(p);
     return launch_status();
 }
 

@@ -197,6 +197,13 @@ def main():
     hbm("cross_entropy_fwd_bwd_chunk_quant_e5m2 (fused)", f"{CR}x{V}", 5.0 * CR * V,
         lambda: cf.cf_cross_entropy_fwd_bwd_chunk_quant_e5m2(logits, labels, closs, cgrad, cg8, sc, amax, CR, V, nvalid, st))
     del logits, cgrad, cg8
+    CR2, V2 = 512, 128256
+    logits = bf16(CR2, V2, sigma=3.0)
+    labels2 = torch.randint(0, V2, (CR2,), device=dev, generator=g, dtype=torch.int32)
+    cgrad = torch.empty_like(logits); cg8 = u8(CR2, V2)
+    hbm("cross_entropy_fwd_bwd_chunk_quant_e5m2 (fused, three vectorized passes)", f"{CR2}x{V2}", 5.0 * CR2 * V2,
+        lambda: cf.cf_cross_entropy_fwd_bwd_chunk_quant_e5m2(logits, labels2, closs, cgrad, cg8, sc, amax, CR2, V2, nvalid, st))
+    del logits, cgrad, cg8
 
     # ---- config 5: MoE ------------------------------------------------------------------------------
     T, H, E, k, Ie = 16384, 2048, 64, 6, 1408

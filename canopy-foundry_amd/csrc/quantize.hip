@@ -378,15 +378,14 @@ __global__ __launch_bounds__(kThreads) void k_quant_rows(const uint16_t* __restr
     }
 }
 
-// Long rows (4096 < K <= 16384): one workgroup of four wavefronts per row, the row still register-resident (four
-// steps per lane instead of sixteen, so twice the wavefronts fit a SIMD); the row maximum crosses the
+// Long rows (4096 < K <= 32768): one workgroup of four wavefronts per row, the row still register-resident (four or
+// eight steps per lane instead of sixteen or more, so more wavefronts fit a SIMD); the row maximum crosses the
 // wavefronts through LDS.
-template <bool E5M2>
+template <bool E5M2, int MAXS>      // MAXS steps of 256 lanes x 16 elements: 4 covers K <= 16384, 8 covers K <= 32768
 __global__ __launch_bounds__(kThreads) void k_quant_rows_block(const uint16_t* __restrict__ x, int K,
                                                                uint8_t* __restrict__ out,
                                                                float* __restrict__ scale,
                                                                float* __restrict__ descale) {
-    constexpr int MAXS = 4;
     __shared__ int sh_bits[kThreads / 64];
     __shared__ float sh_max[kThreads / 64];
     const int row = blockIdx.x, tid = threadIdx.x;
@@ -779,8 +778,11 @@ int cf_fp8_quantize_rows(const uint16_t* d_x, int rows, int K, int is_e5m2, void
         if (is_e5m2) k_quant_rows<true, 4><<<grid, kThreads, 0, st>>>(d_x, rows, K, o, d_scale, d_descale);
         else         k_quant_rows<false, 4><<<grid, kThreads, 0, st>>>(d_x, rows, K, o, d_scale, d_descale);
     } else if (vec && K <= 16 * 1024) {
-        if (is_e5m2) k_quant_rows_block<true><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);
-        else         k_quant_rows_block<false><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);
+        if (is_e5m2) k_quant_rows_block<true, 4><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);
+        else         k_quant_rows_block<false, 4><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);
+    } else if (vec && K <= 32 * 1024) {
+        if (is_e5m2) k_quant_rows_block<true, 8><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);
+        else         k_quant_rows_block<false, 8><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);
     } else {
         if (is_e5m2) k_quant_rows_generic<true><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);
         else         k_quant_rows_generic<false><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);

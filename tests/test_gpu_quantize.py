@@ -182,7 +182,8 @@ def test_transposing_kernels(cf, dev, K, N):
     assert np.array_equal(host(t), q.T)
 
 
-@pytest.mark.parametrize("rows,K", [(8, 4096), (5, 1024), (3, 14336), (130, 2048), (4, 1408), (7, 300), (2, 20000), (1, 16)])
+@pytest.mark.parametrize("rows,K", [(8, 4096), (5, 1024), (3, 14336), (130, 2048), (4, 1408), (7, 300), (2, 20000), (1, 16),
+                                    (5, 28672), (2, 32768), (2, 40000), (3, 20001)])
 @pytest.mark.parametrize("e5m2", [False, True])
 def test_per_row_quantize(cf, dev, rows, K, e5m2):
     case(f"rows quantize {rows}x{K} e5m2={e5m2}")

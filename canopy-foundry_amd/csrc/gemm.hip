@@ -571,6 +571,19 @@ __device__ __forceinline__ void load_pair_scales(float4 (&cs)[2][4], float4 (&cs
         const uint8_t* b1 = reinterpret_cast<const uint8_t*>(p.sb + ucol);
         const uint8_t* b2 = reinterpret_cast<const uint8_t*>(EPI == EPI_SILU_GATE ? p.sb2 + ucol : p.sb);
         const uint32_t loff = static_cast<uint32_t>(lane >> 5) * 16u;
+        if constexpr (EPI != EPI_SILU_GATE) {
+            // a last column tile that N cuts short (N % 4 == 0): factors of columns at or beyond N are not used,
+            // their loads are moved onto the last four columns
+            if (t.n0 + BN > p.N) {
+                const int lim = (p.N - 4 - static_cast<int>(t.n0 + wn * (NU * 32) + pair * 64)) * 4;
+#pragma unroll
+                for (int u = 0; u < 2; ++u)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+                        cs[u][g] = *reinterpret_cast<const float4*>(b1 + min(static_cast<int>(loff + u * 128u + g * 32u), lim));
+                return;
+            }
+        }
 #pragma unroll
         for (int u = 0; u < 2; ++u)
 #pragma unroll
@@ -618,10 +631,14 @@ __device__ __forceinline__ void drain_tile(v16f (&acc)[4][4], TileScales<EPI>& s
     // fetched before the first store, so no wait on them has to sit out a store burst.
     uint4 bias8[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
     if constexpr (EPI == EPI_BIAS) {
-        const uint16_t* bcol = p.bias + t.n0 + wn * (NU * 32) + rc * 8;
+        const int bcol = t.n0 + wn * (NU * 32) + rc * 8;
 #pragma unroll
-        for (int pair = 0; pair < NU / 2; ++pair) bias8[pair] = *reinterpret_cast<const uint4*>(bcol + pair * 64);
+        for (int pair = 0; pair < NU / 2; ++pair)
+            bias8[pair] = *reinterpret_cast<const uint4*>(p.bias + (RAGGED ? min(bcol + pair * 64, p.N - 8) : bcol + pair * 64));
     }
+    // RAGGED also covers a last column tile that N cuts short (N % 8 == 0): this lane's eight columns of a pair
+    // are stored or not as a whole
+    const int ncol0 = t.n0 + wn * (NU * 32) + rc * 8;
 
 #pragma unroll
     for (int pair = 0; pair < NU / 2; ++pair) {
@@ -683,7 +700,7 @@ __device__ __forceinline__ void drain_tile(v16f (&acc)[4][4], TileScales<EPI>& s
                     v.z = pack_bf16x2_hw(bf16_lo(v.z) + bf[4], bf16_hi(v.z) + bf[5]);
                     v.w = pack_bf16x2_hw(bf16_lo(v.w) + bf[6], bf16_hi(v.w) + bf[7]);
                 }
-                if (!RAGGED || mrow0 + half * 64 + i * 8 < t.m_end) {
+                if (!RAGGED || (mrow0 + half * 64 + i * 8 < t.m_end && ncol0 + pair * 64 < p.N)) {
                     const u32x4 vv = {v.x, v.y, v.z, v.w};
                     __builtin_nontemporal_store(vv, reinterpret_cast<u32x4*>(cu + ((half * 8 + i) * cstep + pair * 128) + coff));
                 }
@@ -1056,7 +1073,8 @@ void k_gemm_nt_ring(const GemmArgs p) {
                 if (t.m0 + BM <= t.m_end) drain_tile_accum<false, BF>(acc, s1, p, t, wm, wn, lane, stage, landed);
                 else                      drain_tile_accum<true, BF>(acc, s1, p, t, wm, wn, lane, stage, landed);
             } else {
-                if (t.m0 + BM <= t.m_end) drain_tile<EPI, SCALE, false>(acc, sc, s1, s2, p, t, wm, wn, lane, stage, landed);
+                constexpr int out_bn = EPI == EPI_SILU_GATE ? BN / 2 : BN;
+                if (t.m0 + BM <= t.m_end && t.n0 + out_bn <= p.N) drain_tile<EPI, SCALE, false>(acc, sc, s1, s2, p, t, wm, wn, lane, stage, landed);
                 else                      drain_tile<EPI, SCALE, true>(acc, sc, s1, s2, p, t, wm, wn, lane, stage, landed);
             }
         } else {
@@ -1446,8 +1464,9 @@ int launch_tiled(const GemmArgs& p, hipStream_t st) {
     }
     if constexpr (EPI == EPI_NONE || EPI == EPI_BIAS || EPI == EPI_SILU_GATE) {
         // its drain writes full-width tiles with 16-byte stores and reads the channel descales as float4
-        constexpr int out_bn = EPI == EPI_SILU_GATE ? BN / 2 : BN;
-        ring_ok = ring_ok && p.N % out_bn == 0 && p.ldc % 8 == 0 && aligned16(p.C);
+        // (N may cut the last column tile short at a multiple of 8; the fused gate/up form interleaves two weight
+        // matrices per tile and keeps whole tiles)
+        ring_ok = ring_ok && (EPI == EPI_SILU_GATE ? p.N % (BN / 2) == 0 : p.N % 8 == 0 && p.N >= 8) && p.ldc % 8 == 0 && aligned16(p.C);
         if (SCALE == SCALE_ROWCOL)
             ring_ok = ring_ok && aligned16(p.sb) && p.sb_expert_stride % 4 == 0 && (EPI != EPI_SILU_GATE || aligned16(p.sb2));
         if (EPI == EPI_BIAS) ring_ok = ring_ok && aligned16(p.bias);
@@ -1672,7 +1691,7 @@ int cf_fp8_grouped_gemm_nt_bf16_ex(int total_rows, int N, int K, int num_experts
     if (K % BK != 0 || K < 2 * BK || lda % 16 != 0 || !aligned16(A) || !aligned16(B) ||
         (epilogue == EPI_SILU_GATE && !aligned16(B_up)) || lda < K || ldc < N ||
         static_cast<size_t>(a_rows) * lda >= (1ull << 32) || static_cast<size_t>(N) * K >= (1ull << 32) ||
-        N % (epilogue == EPI_SILU_GATE ? BN / 2 : BN) != 0 || ldc % 8 != 0 || !aligned16(C) || !aligned16(b_descale) ||
+        (epilogue == EPI_SILU_GATE ? N % (BN / 2) != 0 : N % 8 != 0) || N < 8 || ldc % 8 != 0 || !aligned16(C) || !aligned16(b_descale) ||
         (epilogue == EPI_SILU_GATE && !aligned16(b_up_descale)))
         return CF_ERR_UNSUPPORTED;
     hipStream_t st = as_stream(stream);

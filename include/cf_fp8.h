@@ -330,7 +330,7 @@ int cf_fp8_grouped_gemm_workspace_bytes(int total_rows, int num_experts, size_t*
  * B is [num_experts, N, K] E4M3, b_descale [num_experts, N].  total_rows is the host-side upper
  * bound rows * top_k; counts / offsets stay on the device.  a_rows is the number of rows of d_A
  * (every row index is below it; total_rows without an index).  Needs K % 128 == 0, K >= 256,
- * N a multiple of 256 (128 with the SiLU-gate epilogue), ldc % 8 == 0, 16-byte aligned operands,
+ * N a multiple of 8 (of 128 with the SiLU-gate epilogue), ldc % 8 == 0, 16-byte aligned operands,
  * descales and C, and a_rows * lda, N * K below 2^32. */
 int cf_fp8_grouped_gemm_nt_bf16_ex(int total_rows, int N, int K, int num_experts,
                                    const int* d_counts, const int* d_offsets, const void* d_A,

@@ -49,9 +49,10 @@ def run_gemm(cf, dev, A, B, sa, sb, *, lda=None, a_e5m2=False, mode=PER_TENSOR, 
     return orc.bf16_to_f32(bf16_bits(C)).astype(np.float64)
 
 
-# (300, 512, 512) and (770, 256, 384): persistent kernel with a ragged last row tile; (1024, 1024, 256): several tiles per workgroup, two K-tiles
+# (300, 512, 512) and (770, 256, 384): persistent kernel with a ragged last row tile; (1024, 1024, 256): several tiles per workgroup, two K-tiles;
+# (300, 264, 512), (512, 1000, 384), (256, 8, 256): persistent kernel with a last column tile that N cuts short at a multiple of 8
 SHAPES = [(256, 256, 128), (512, 768, 1024), (300, 200, 144), (1, 1, 16), (33, 500, 208), (257, 129, 4096), (64, 1408, 2048),
-          (300, 512, 512), (770, 256, 384), (1024, 1024, 256)]
+          (300, 512, 512), (770, 256, 384), (1024, 1024, 256), (300, 264, 512), (512, 1000, 384), (256, 8, 256)]
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)
@@ -67,6 +68,33 @@ def test_gemm_per_tensor(cf, dev, M, N, K, flags):
     # without any allowance: only cancellation points (|ref| << sum|a b|) may exceed 2 bf16 ulps
     off = np.abs(got - ref) > 2 * orc.bf16_ulp(ref)
     assert off.mean() <= 0.03 and np.all(np.abs(ref[off]) <= 2.0 ** -9 * absdot[off])
+
+
+@pytest.mark.parametrize("epi", [EPI_NONE, EPI_BIAS])
+def test_gemm_short_last_column_tile_leaves_row_padding_alone(cf, dev, epi):
+    """N = 3 x 256 + 136 with rows of C padded to ldc > N: the persistent kernel stores whole 8-column chunks up to
+    N and nothing after it; the element-per-thread kernel is the cross-check."""
+    case(f"gemm N=904 ldc=960 epi={epi}")
+    rng = np.random.default_rng(904)
+    M, N, K, ldc = 300, 904, 512, 960
+    A, _ = rand_fp8(rng, (M, K))
+    B, _ = rand_fp8(rng, (N, K), sigma=0.02)
+    sa = rng.uniform(0.001, 0.02, M).astype(np.float32)
+    sb = rng.uniform(1e-5, 1e-4, N).astype(np.float32)
+    bias = orc.bf16_from_f32((rng.standard_normal(N) * 1e-3).astype(np.float32)) if epi == EPI_BIAS else None
+    got = run_gemm(cf, dev, A, B, sa, sb, mode=ROW_COL, epi=epi, bias=bias, ldc=ldc)
+    naive = run_gemm(cf, dev, A, B, sa, sb, mode=ROW_COL, epi=epi, bias=bias, ldc=ldc, flags=NAIVE)
+    assert np.all(np.isnan(got[:, N:])) and not np.any(np.isnan(got[:, :N]))
+    ref, absdot = orc.gemm_nt_ref(A, B, sa, sb, scale_mode=1)
+    if epi == EPI_BIAS:
+        # bias is added to the bf16-rounded product: exact given the plain result
+        plain = run_gemm(cf, dev, A, B, sa, sb, mode=ROW_COL, ldc=ldc)[:, :N]
+        want = orc.bf16_to_f32(orc.bf16_from_f32((plain + orc.bf16_to_f32(bias)[None, :].astype(np.float64)).astype(np.float32)))
+        assert np.array_equal(got[:, :N], want)
+    else:
+        orc.assert_gemm_close(got[:, :N], ref, absdot)
+    assert np.all(np.isnan(naive[:, N:]))
+    assert np.mean(got[:, :N] != naive[:, :N]) < 0.25      # two accumulation orders: mostly the same bf16 value
 
 
 def test_gemm_exact_small_integers_equals_numpy_matmul(cf, dev):
@@ -97,7 +125,7 @@ def test_gemm_e5m2_activations_and_row_stride(cf, dev, flags):
     orc.assert_gemm_close(got, ref, absdot)
 
 
-@pytest.mark.parametrize("M,N,K", [(300, 260, 384), (300, 512, 384), (1100, 256, 640)])
+@pytest.mark.parametrize("M,N,K", [(300, 260, 384), (300, 512, 384), (1100, 256, 640), (300, 264, 384), (520, 904, 640)])
 @pytest.mark.parametrize("flags", [0, NAIVE])
 def test_gemm_row_col_scales_and_bias(cf, dev, M, N, K, flags):
     case(f"gemm row/col scales + bias {M}x{N}x{K} flags={flags}")

@@ -117,7 +117,8 @@ def check_stages(b: Bank, r, experts=None, sample=None):
         orc.assert_gemm_close(orc.bf16_to_f32(r["y"][o:o + n][sel]).astype(np.float64), yref, yabs, what=f"down expert {e}")
 
 
-@pytest.mark.parametrize("rows,E,k,H,Ie,zero", [(600, 5, 2, 256, 384, None), (300, 4, 2, 256, 256, 2), (1500, 3, 1, 512, 640, None), (40, 8, 3, 256, 256, None)])
+@pytest.mark.parametrize("rows,E,k,H,Ie,zero", [(600, 5, 2, 256, 384, None), (300, 4, 2, 256, 256, 2), (1500, 3, 1, 512, 640, None), (40, 8, 3, 256, 256, None),
+                                                  (500, 4, 2, 384, 256, None), (300, 3, 2, 640, 384, None)])
 def test_grouped_bank_small(cf, dev, rows, E, k, H, Ie, zero):
     case(f"grouped swiglu bank rows={rows} E={E} k={k} H={H} Ie={Ie}")
     b = Bank(dev, rows, E, k, H, Ie, seed=rows + E, zero_expert=zero)

@@ -250,7 +250,8 @@ __device__ __forceinline__ uint32_t fma2_bf16(uint32_t m, uint32_t c, float w) {
     const float hi = __builtin_fmaf(w, bf16_hi(c), bf16_hi(m));
     return pack_bf16x2(lo, hi);
 }
-// rows of `compact` map to rows of `mixed` through row_indices (or identically when it is null)
+// rows of `compact` map to rows of `mixed` through row_indices (or identically when it is null); without route
+// weights the factor is 1 and the operation is the plain add of the backward's scatter (fma(1, c, m) = m + c)
 __global__ __launch_bounds__(kThreads) void k_scatter_accumulate(uint16_t* __restrict__ mixed,
                                                                  const uint16_t* __restrict__ compact,
                                                                  const float* __restrict__ route_weights,
@@ -263,7 +264,7 @@ __global__ __launch_bounds__(kThreads) void k_scatter_accumulate(uint16_t* __res
              i += static_cast<size_t>(gridDim.x) * blockDim.x) {
             const int r = static_cast<int>(i / vpr), c = static_cast<int>(i % vpr);
             const int row = row_indices ? row_indices[r] : r;
-            const float w = route_weights[static_cast<size_t>(row) * E + expert_idx];
+            const float w = route_weights ? route_weights[static_cast<size_t>(row) * E + expert_idx] : 1.0f;
             uint4* dst = reinterpret_cast<uint4*>(mixed + static_cast<size_t>(row) * H) + c;
             const uint4 cv = reinterpret_cast<const uint4*>(compact + static_cast<size_t>(r) * H)[c];
             uint4 mv = *dst;
@@ -277,7 +278,7 @@ __global__ __launch_bounds__(kThreads) void k_scatter_accumulate(uint16_t* __res
              i += static_cast<size_t>(gridDim.x) * blockDim.x) {
             const int r = static_cast<int>(i / H), h = static_cast<int>(i % H);
             const int row = row_indices ? row_indices[r] : r;
-            const float w = route_weights[static_cast<size_t>(row) * E + expert_idx];
+            const float w = route_weights ? route_weights[static_cast<size_t>(row) * E + expert_idx] : 1.0f;
             uint16_t* dst = mixed + static_cast<size_t>(row) * H + h;
             *dst = f32_to_bf16(__builtin_fmaf(w, bf16_to_f32(compact[i]), bf16_to_f32(*dst)));
         }
@@ -320,6 +321,9 @@ __device__ __forceinline__ int wave_find_sorted(const int* __restrict__ list, in
     return eq ? lo + __builtin_ctzll(eq) : -1;
 }
 
+// UNIT: every selected expert's row is added with factor 1 (the backward's scatter-add); the route weights
+// then only say which experts selected the row.
+template <bool UNIT>
 __global__ __launch_bounds__(kThreads) void k_unpermute(uint16_t* __restrict__ mixed, const uint16_t* __restrict__ y,
                                                         const float* __restrict__ route_weights,
                                                         const int* __restrict__ counts, const int* __restrict__ offsets,
@@ -339,7 +343,7 @@ __global__ __launch_bounds__(kThreads) void k_unpermute(uint16_t* __restrict__ m
             if (sel) {
                 const int pos = __builtin_popcountll(m & ((1ull << t) - 1ull));
                 sl_e[pos] = e;
-                sl_w[pos] = w;
+                sl_w[pos] = UNIT ? 1.0f : w;
             }
             if (t == 0) sl_n = __builtin_popcountll(m);
         }
@@ -616,8 +620,32 @@ int cf_moe_unpermute_weighted_bf16(uint16_t* d_mixed, const uint16_t* d_compact_
     if (rows == 0 || num_experts == 0 || H == 0) return CF_OK;
     if (!d_mixed || !d_compact_out || !d_route_weights || !d_counts || !d_offsets || !d_row_indices) return CF_ERR_INVALID_ARG;
     if ((H & 7) == 0 && !(aligned16(d_mixed) && aligned16(d_compact_out))) return CF_ERR_UNSUPPORTED;
-    k_unpermute<<<rows, kThreads, 0, as_stream(stream)>>>(d_mixed, d_compact_out, d_route_weights, d_counts, d_offsets,
-                                                          d_row_indices, rows, num_experts, H);
+    k_unpermute<false><<<rows, kThreads, 0, as_stream(stream)>>>(d_mixed, d_compact_out, d_route_weights, d_counts, d_offsets,
+                                                                 d_row_indices, rows, num_experts, H);
+    return launch_status();
+}
+
+int cf_moe_scatter_add_rows_bf16(uint16_t* d_dst_full, const uint16_t* d_src_compact, const int* d_row_indices, int n_rows,
+                                 int H, cf_stream_t stream) {
+    if (n_rows < 0 || H < 0) return CF_ERR_INVALID_ARG;
+    if (n_rows == 0 || H == 0) return CF_OK;
+    if (!d_dst_full || !d_src_compact || !d_row_indices) return CF_ERR_INVALID_ARG;
+    const int vec = H % 8 == 0 && aligned16(d_dst_full) && aligned16(d_src_compact);
+    const size_t items = static_cast<size_t>(n_rows) * (vec ? H / 8 : H);
+    k_scatter_accumulate<<<grid_for(items), kThreads, 0, as_stream(stream)>>>(d_dst_full, d_src_compact, nullptr, d_row_indices,
+                                                                              n_rows, 0, 1, H, vec);
+    return launch_status();
+}
+
+int cf_moe_unpermute_add_bf16(uint16_t* d_dst_full, const uint16_t* d_src_compact, const float* d_route_weights,
+                              const int* d_counts, const int* d_offsets, const int* d_row_indices, int rows,
+                              int num_experts, int H, cf_stream_t stream) {
+    if (rows < 0 || num_experts < 0 || H < 0) return CF_ERR_INVALID_ARG;
+    if (rows == 0 || num_experts == 0 || H == 0) return CF_OK;
+    if (!d_dst_full || !d_src_compact || !d_route_weights || !d_counts || !d_offsets || !d_row_indices) return CF_ERR_INVALID_ARG;
+    if ((H & 7) == 0 && !(aligned16(d_dst_full) && aligned16(d_src_compact))) return CF_ERR_UNSUPPORTED;
+    k_unpermute<true><<<rows, kThreads, 0, as_stream(stream)>>>(d_dst_full, d_src_compact, d_route_weights, d_counts, d_offsets,
+                                                                d_row_indices, rows, num_experts, H);
     return launch_status();
 }
 

@@ -248,6 +248,33 @@ def main():
          lambda: cf.cf_moe_grouped_swiglu_forward_fp8(hq, hd, rw, counts, offs, idx, wg, wgd, wu, wud, wd, wdd, mixed, T, H, Ie, E,
                                                       total, ws2, sz2.value, st))
 
+    # ---- the selected-expert backward's custom kernels at the same size --------------------------------
+    dmixed = bf16(T, H)
+    eout = bf16(total, H)
+    dlog = torch.empty((T, E), dtype=torch.float32, device=dev)
+    # per slot: reads a row of expert_out, writes the gradient row over it and 4 bytes; the rows of d_mixed are
+    # counted once (each is used by k slots and the repeats come from cache)
+    hbm("grouped route grad (row dot + weighted gather, all experts)", f"{total}x{H}", 4.0 * total * H + 2.0 * T * H + 4.0 * T * E,
+        lambda: cf.cf_moe_grouped_route_grad_bf16(dmixed, eout, dlog, rw, counts, offs, idx, T, E, H, st))
+    hcounts = counts.cpu().tolist(); hoffs = offs.cpu().tolist(); idx2 = idx.view(E, T)
+
+    def per_expert():
+        # the reference's sequence: two launches per expert (src/trainer.cu:7722-7725)
+        for e in range(E):
+            n_e = hcounts[e]
+            if n_e == 0:
+                continue
+            slot = eout[hoffs[e]:hoffs[e] + n_e]
+            cf.cf_moe_row_dot_selected_bf16(dmixed, slot, dlog, idx2[e], n_e, H, E, e, st)
+            cf.cf_moe_gather_scale_rows_bf16(dmixed, slot, rw, idx2[e], n_e, e, E, H, st)
+    hbm("  the same as two launches per expert", f"{total}x{H}", 4.0 * total * H + 2.0 * T * H + 4.0 * T * E, per_expert)
+    dhid = torch.zeros((T, H), dtype=torch.bfloat16, device=dev)
+    hbm("unpermute_add_bf16 (scatter-add, all experts)", f"{total}x{H}", 2.0 * total * H + 4.0 * T * H,
+        lambda: cf.cf_moe_unpermute_add_bf16(dhid, yy, rw, counts, offs, idx, T, E, H, st))
+    pre = bf16(total, Ie); gpost = bf16(total, Ie, sigma=0.01); gpre = torch.empty_like(pre)
+    hbm("gelu_forward_bf16", f"{total}x{Ie}", 4.0 * total * Ie, lambda: cf.cf_gelu_forward_bf16(pre, gpre, total * Ie, st))
+    hbm("gelu_backward_bf16", f"{total}x{Ie}", 6.0 * total * Ie, lambda: cf.cf_gelu_backward_bf16(pre, gpost, gpre, total * Ie, st))
+
 
 if __name__ == "__main__":
     main()

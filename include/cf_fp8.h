@@ -354,6 +354,49 @@ int cf_moe_unpermute_weighted_bf16(uint16_t* d_mixed, const uint16_t* d_compact_
                                    const int* d_offsets, const int* d_row_indices, int rows,
                                    int num_experts, int H, cf_stream_t stream);
 
+/* ---- MoE expert-bank backward with the forward's routes (src/trainer.cu:7654-7741) --------
+ * The custom kernels of the selected-expert backward; its bf16 GEMMs are BLAS calls in the
+ * reference (gemm_bf16 / gemm_bf16_tn_f32) and stay BLAS calls. */
+
+/* gelu_forward, kernels.hpp:334, kernels/moe.cu:510-521: out = bf16(0.5 x (1 + erf(x / sqrt 2))). */
+int cf_gelu_forward_bf16(const uint16_t* d_x, uint16_t* d_out, size_t n, cf_stream_t stream);
+/* gelu_backward, kernels/moe.cu:1148-1167: grad_pre = bf16(grad_post * (Phi(pre) + pre phi(pre))). */
+int cf_gelu_backward_bf16(const uint16_t* d_pre, const uint16_t* d_grad_post, uint16_t* d_grad_pre,
+                          size_t n, cf_stream_t stream);
+
+/* moe_row_dot_selected_bf16, kernels/moe.cu:623-645,740-748:
+ * out[row_indices[i] * out_stride + out_col] = dot(a_full[row_indices[i]], b_compact[i]), summed in the
+ * reference's order (min(H, 256) strided partial sums, then a halving tree). */
+int cf_moe_row_dot_selected_bf16(const uint16_t* d_a_full, const uint16_t* d_b_compact, float* d_out,
+                                 const int* d_row_indices, int n_rows, int H, int out_stride,
+                                 int out_col, cf_stream_t stream);
+/* moe_gather_scale_rows_bf16, kernels/moe.cu:646-660,750-758:
+ * dst[i, h] = bf16(w[row_indices[i], expert_idx] * src[row_indices[i], h]). */
+int cf_moe_gather_scale_rows_bf16(const uint16_t* d_src, uint16_t* d_dst, const float* d_route_weights,
+                                  const int* d_row_indices, int n_rows, int expert_idx,
+                                  int num_experts, int H, cf_stream_t stream);
+/* moe_scatter_add_rows_bf16, kernels/moe.cu:661-674,760-767:
+ * dst_full[row_indices[i], h] = bf16(dst_full + src_compact[i, h]). */
+int cf_moe_scatter_add_rows_bf16(uint16_t* d_dst_full, const uint16_t* d_src_compact,
+                                 const int* d_row_indices, int n_rows, int H, cf_stream_t stream);
+
+/* The two per-expert launches moe_row_dot_selected_bf16 + moe_gather_scale_rows_bf16 of every
+ * expert (src/trainer.cu:7722-7725) in one launch over the forward's saved lists:
+ *   grad_route_weights[row, e] = dot(grad_mixed[row], expert_out[slot])   (0 where e did not select row)
+ *   expert_out[slot]           = bf16(route_weights[row, e] * grad_mixed[row])   (in place)
+ * slot = offsets[e] + position of row in expert e's list; expert_out is [sum counts, H]. */
+int cf_moe_grouped_route_grad_bf16(const uint16_t* d_grad_mixed, uint16_t* d_expert_out,
+                                   float* d_grad_route_weights, const float* d_route_weights,
+                                   const int* d_counts, const int* d_offsets, const int* d_row_indices,
+                                   int rows, int num_experts, int H, cf_stream_t stream);
+/* All per-expert moe_scatter_add_rows_bf16 launches (src/trainer.cu:7739-7740) in one: experts
+ * in ascending order per token row, one bf16 rounding per expert; the route weights only mark
+ * which experts selected a row.  Same layout rules as cf_moe_unpermute_weighted_bf16. */
+int cf_moe_unpermute_add_bf16(uint16_t* d_dst_full, const uint16_t* d_src_compact,
+                              const float* d_route_weights, const int* d_counts, const int* d_offsets,
+                              const int* d_row_indices, int rows, int num_experts, int H,
+                              cf_stream_t stream);
+
 /* The grouped SwiGLU expert bank of benchmark config 5 (the FP8 form of the expert loop in
  * moe_expert_bank_forward, src/trainer.cu:6876-6934, with the SwiGLU experts of
  * moe_generic_forward, src/trainer.cu:6510-6529): permute -> gate/up GEMM with fused SiLU gate

@@ -151,6 +151,27 @@ inline void moe_scatter_accumulate_rows_bf16(bf16* d_mixed, const bf16* d_compac
     CF_FWD(cf_moe_scatter_accumulate_rows_bf16(hip_detail::u(d_mixed), hip_detail::u(d_compact), d_route_weights,
                                                d_row_indices, n_rows, expert_idx, num_experts, H, stream));
 }
+// ---- kernels.hpp:334, kernels/moe.cu:623-674,740-767,1148-1167: the selected-expert backward's kernels ------
+inline void gelu_forward(const bf16* d_x, bf16* d_out, std::size_t n, hipStream_t stream) {
+    CF_FWD(cf_gelu_forward_bf16(hip_detail::u(d_x), hip_detail::u(d_out), n, stream));
+}
+inline void gelu_backward(const bf16* d_pre, const bf16* d_grad_post, bf16* d_grad_pre, std::size_t n, hipStream_t stream) {
+    CF_FWD(cf_gelu_backward_bf16(hip_detail::u(d_pre), hip_detail::u(d_grad_post), hip_detail::u(d_grad_pre), n, stream));
+}
+inline void moe_row_dot_selected_bf16(const bf16* d_a_full, const bf16* d_b_compact, float* d_out, const int* d_row_indices,
+                                      int n_rows, int H, int out_stride, int out_col, hipStream_t stream) {
+    CF_FWD(cf_moe_row_dot_selected_bf16(hip_detail::u(d_a_full), hip_detail::u(d_b_compact), d_out, d_row_indices, n_rows, H,
+                                        out_stride, out_col, stream));
+}
+inline void moe_gather_scale_rows_bf16(const bf16* d_src, bf16* d_dst, const float* d_route_weights, const int* d_row_indices,
+                                       int n_rows, int expert_idx, int num_experts, int H, hipStream_t stream) {
+    CF_FWD(cf_moe_gather_scale_rows_bf16(hip_detail::u(d_src), hip_detail::u(d_dst), d_route_weights, d_row_indices, n_rows,
+                                         expert_idx, num_experts, H, stream));
+}
+inline void moe_scatter_add_rows_bf16(bf16* d_dst_full, const bf16* d_src_compact, const int* d_row_indices, int n_rows, int H,
+                                      hipStream_t stream) {
+    CF_FWD(cf_moe_scatter_add_rows_bf16(hip_detail::u(d_dst_full), hip_detail::u(d_src_compact), d_row_indices, n_rows, H, stream));
+}
 inline void moe_expert_offsets_from_counts(const int* d_counts, int* d_offsets, int num_experts, hipStream_t stream) {
     CF_FWD(cf_moe_expert_offsets_from_counts(d_counts, d_offsets, num_experts, stream));
 }

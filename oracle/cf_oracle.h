@@ -44,6 +44,10 @@
  *   cross-entropy                 see cf_oracle_ce.c (closed forms, sum-to-zero,
  *                                 double recomputation; libm exp/log stand in
  *                                 for CUDA's: parity unpinned beyond 1 bf16 ulp).
+ *   MoE backward helpers          see cf_oracle_moe_bwd.c (exact-product row dot
+ *                                 with the reference's summation tree, closed
+ *                                 forms; libm erff / expf stand in for CUDA's in
+ *                                 the GELU pair: parity unpinned beyond 1 bf16 ulp).
  *   GEMM references               definition from the task statement: matmul
  *                                 of the dequantised operands; special cases
  *                                 reduce to numpy matmul.  cuBLASLt's own
@@ -137,6 +141,16 @@ void orc_act_row_clip_abs(uint16_t* x, int rows, int cols, float ceiling, float*
 void orc_cross_entropy_count_valid(const int32_t* labels, int n, int* n_valid);
 void orc_cross_entropy_fwd_bwd_chunk(const uint16_t* logits, const int32_t* labels, float* loss_out,
                                      uint16_t* grad, int rows, int V, const int* n_valid);
+
+/* ---- MoE expert-bank backward helpers (cf_oracle_moe_bwd.c; kernels/moe.cu:510-521,623-674,1148-1167) ---- */
+void orc_gelu_forward_bf16(const uint16_t* x, uint16_t* out, size_t n);
+void orc_gelu_backward_bf16(const uint16_t* pre, const uint16_t* d_post, uint16_t* d_pre, size_t n);
+void orc_moe_row_dot_selected_bf16(const uint16_t* a_full, const uint16_t* b_compact, float* out,
+                                   const int* row_indices, int n_rows, int H, int out_stride, int out_col);
+void orc_moe_gather_scale_rows_bf16(const uint16_t* src, uint16_t* dst, const float* route_weights,
+                                    const int* row_indices, int n_rows, int expert_idx, int num_experts, int H);
+void orc_moe_scatter_add_rows_bf16(uint16_t* dst_full, const uint16_t* src_compact, const int* row_indices,
+                                   int n_rows, int H);
 
 /* ---- GEMM references ----------------------------------------------------
  * scale_mode: 0 per-tensor (a_descale[1], b_descale[1])

@@ -492,6 +492,51 @@ def moe_scatter_accumulate(mixed, compact, route_weights, row_indices, expert_id
     return mixed
 
 
+# ---- MoE expert-bank backward helpers -------------------------------------------------
+def gelu_forward(x):
+    x = np.ascontiguousarray(x, dtype=np.uint16)
+    out = np.empty_like(x)
+    _call("orc_gelu_forward_bf16", x, out, c_sz(x.size))
+    return out
+
+
+def gelu_backward(pre, d_post):
+    pre = np.ascontiguousarray(pre, dtype=np.uint16)
+    d_post = np.ascontiguousarray(d_post, dtype=np.uint16)
+    out = np.empty_like(pre)
+    _call("orc_gelu_backward_bf16", pre, d_post, out, c_sz(pre.size))
+    return out
+
+
+def moe_row_dot_selected(a_full, b_compact, out, row_indices, out_col):
+    """out is [rows, out_stride] float32; returns a copy with column out_col filled at the listed rows."""
+    a_full = np.ascontiguousarray(a_full, dtype=np.uint16)
+    b_compact = np.ascontiguousarray(b_compact, dtype=np.uint16)
+    out = np.ascontiguousarray(out, dtype=np.float32).copy()
+    ri = np.ascontiguousarray(row_indices, dtype=np.int32)
+    _call("orc_moe_row_dot_selected_bf16", a_full, b_compact, out, ri, c_i(ri.size), c_i(a_full.shape[1]),
+          c_i(out.shape[1]), c_i(out_col))
+    return out
+
+
+def moe_gather_scale_rows(src, route_weights, row_indices, expert_idx):
+    src = np.ascontiguousarray(src, dtype=np.uint16)
+    rw = np.ascontiguousarray(route_weights, dtype=np.float32)
+    ri = np.ascontiguousarray(row_indices, dtype=np.int32)
+    dst = np.empty((ri.size, src.shape[1]), np.uint16)
+    _call("orc_moe_gather_scale_rows_bf16", src, dst, rw, ri, c_i(ri.size), c_i(expert_idx), c_i(rw.shape[1]),
+          c_i(src.shape[1]))
+    return dst
+
+
+def moe_scatter_add_rows(dst_full, src_compact, row_indices):
+    dst_full = np.ascontiguousarray(dst_full, dtype=np.uint16).copy()
+    src_compact = np.ascontiguousarray(src_compact, dtype=np.uint16)
+    ri = np.ascontiguousarray(row_indices, dtype=np.int32)
+    _call("orc_moe_scatter_add_rows_bf16", dst_full, src_compact, ri, c_i(ri.size), c_i(dst_full.shape[1]))
+    return dst_full
+
+
 def moe_scale_accumulate(mixed, term, route_weights, expert_idx):
     mixed = np.ascontiguousarray(mixed, dtype=np.uint16).copy()
     term = np.ascontiguousarray(term, dtype=np.uint16)

@@ -321,6 +321,85 @@ __device__ __forceinline__ int wave_find_sorted(const int* __restrict__ list, in
     return eq ? lo + __builtin_ctzll(eq) : -1;
 }
 
+// mixed row += the n listed rows of y, in list order, one bf16 rounding per row (slot < 0: skipped)
+__device__ __forceinline__ void combine_rows(uint16_t* __restrict__ mrow, const uint16_t* __restrict__ y, int H, int n,
+                                             const int* sl_slot, const float* sl_w, int t) {
+    if ((H & 7) == 0) {
+        for (int c = t; c < H / 8; c += blockDim.x) {
+            uint4 mv = reinterpret_cast<uint4*>(mrow)[c];
+            for (int i0 = 0; i0 < n; i0 += 4) {
+                // up to four rows of y in flight at once, applied in order
+                uint4 yv[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int slot = i0 + j < n ? sl_slot[i0 + j] : -1;
+                    yv[j] = make_uint4(0, 0, 0, 0);
+                    if (slot >= 0) yv[j] = reinterpret_cast<const uint4*>(y + static_cast<size_t>(slot) * H)[c];
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if (i0 + j < n && sl_slot[i0 + j] >= 0) {
+                        const float w = sl_w[i0 + j];
+                        mv.x = fma2_bf16(mv.x, yv[j].x, w); mv.y = fma2_bf16(mv.y, yv[j].y, w);
+                        mv.z = fma2_bf16(mv.z, yv[j].z, w); mv.w = fma2_bf16(mv.w, yv[j].w, w);
+                    }
+                }
+            }
+            reinterpret_cast<uint4*>(mrow)[c] = mv;
+        }
+    } else {
+        for (int h = t; h < H; h += blockDim.x) {
+            float m = bf16_to_f32(mrow[h]);
+            for (int i = 0; i < n; ++i)
+                if (sl_slot[i] >= 0)
+                    m = bf16_to_f32(f32_to_bf16(__builtin_fmaf(sl_w[i], bf16_to_f32(y[static_cast<size_t>(sl_slot[i]) * H + h]), m)));
+            mrow[h] = f32_to_bf16(m);
+        }
+    }
+}
+
+// The same with the slots read from a table slot_index[row, e] (filled by k_slot_index for the selected pairs):
+// no search, so a row's critical path is one load of its weights and slots, then the gathers.
+template <bool UNIT>
+__global__ __launch_bounds__(kThreads) void k_unpermute_indexed(uint16_t* __restrict__ mixed, const uint16_t* __restrict__ y,
+                                                                const float* __restrict__ route_weights,
+                                                                const int* __restrict__ slot_index, int E, int H) {
+    __shared__ int sl_slot[64];
+    __shared__ float sl_w[64];
+    __shared__ int sl_n;
+    const int row = blockIdx.x, t = threadIdx.x;
+    uint16_t* mrow = mixed + static_cast<size_t>(row) * H;
+    for (int e0 = 0; e0 < E; e0 += 64) {
+        if (t < 64) {
+            const int e = e0 + t;
+            const float w = e < E ? route_weights[static_cast<size_t>(row) * E + e] : 0.0f;
+            const bool sel = w > 0.0f;
+            const int slot = sel ? slot_index[static_cast<size_t>(row) * E + e] : -1;
+            const unsigned long long m = __ballot(sel);
+            if (sel) {
+                const int pos = __builtin_popcountll(m & ((1ull << t) - 1ull));
+                sl_slot[pos] = slot;
+                sl_w[pos] = UNIT ? 1.0f : w;
+            }
+            if (t == 0) sl_n = __builtin_popcountll(m);
+        }
+        __syncthreads();
+        const int n = sl_n;
+        if (n > 0) combine_rows(mrow, y, H, n, sl_slot, sl_w, t);
+        __syncthreads();
+    }
+}
+
+// slot_index[row, e] = offsets[e] + s for every entry s of expert e's list; other cells are left as they are
+__global__ __launch_bounds__(kThreads) void k_slot_index(const int* __restrict__ counts, const int* __restrict__ offsets,
+                                                         const int* __restrict__ row_indices, int rows, int E,
+                                                         int* __restrict__ slot_index) {
+    const int e = blockIdx.y;
+    const int n = counts[e], base = offsets[e];
+    for (int s = blockIdx.x * blockDim.x + threadIdx.x; s < n; s += gridDim.x * blockDim.x)
+        slot_index[static_cast<size_t>(row_indices[static_cast<size_t>(e) * rows + s]) * E + e] = base + s;
+}
+
 // UNIT: every selected expert's row is added with factor 1 (the backward's scatter-add); the route weights
 // then only say which experts selected the row.
 template <bool UNIT>
@@ -355,40 +434,7 @@ __global__ __launch_bounds__(kThreads) void k_unpermute(uint16_t* __restrict__ m
             if (lane == 0) sl_slot[i] = pos < 0 ? -1 : offsets[e] + pos;     // -1: not in the expert's list, skipped
         }
         __syncthreads();
-        if (n > 0) {
-            if ((H & 7) == 0) {
-                for (int c = t; c < H / 8; c += blockDim.x) {
-                    uint4 mv = reinterpret_cast<uint4*>(mrow)[c];
-                    for (int i0 = 0; i0 < n; i0 += 4) {
-                        // up to four rows of y in flight at once, applied in order
-                        uint4 yv[4];
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            const int slot = i0 + j < n ? sl_slot[i0 + j] : -1;
-                            yv[j] = make_uint4(0, 0, 0, 0);
-                            if (slot >= 0) yv[j] = reinterpret_cast<const uint4*>(y + static_cast<size_t>(slot) * H)[c];
-                        }
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            if (i0 + j < n && sl_slot[i0 + j] >= 0) {
-                                const float w = sl_w[i0 + j];
-                                mv.x = fma2_bf16(mv.x, yv[j].x, w); mv.y = fma2_bf16(mv.y, yv[j].y, w);
-                                mv.z = fma2_bf16(mv.z, yv[j].z, w); mv.w = fma2_bf16(mv.w, yv[j].w, w);
-                            }
-                        }
-                    }
-                    reinterpret_cast<uint4*>(mrow)[c] = mv;
-                }
-            } else {
-                for (int h = t; h < H; h += blockDim.x) {
-                    float m = bf16_to_f32(mrow[h]);
-                    for (int i = 0; i < n; ++i)
-                        if (sl_slot[i] >= 0)
-                            m = bf16_to_f32(f32_to_bf16(__builtin_fmaf(sl_w[i], bf16_to_f32(y[static_cast<size_t>(sl_slot[i]) * H + h]), m)));
-                    mrow[h] = f32_to_bf16(m);
-                }
-            }
-        }
+        if (n > 0) combine_rows(mrow, y, H, n, sl_slot, sl_w, t);
         __syncthreads();
     }
 }
@@ -649,9 +695,35 @@ int cf_moe_unpermute_add_bf16(uint16_t* d_dst_full, const uint16_t* d_src_compac
     return launch_status();
 }
 
+int cf_moe_build_slot_index(const int* d_counts, const int* d_offsets, const int* d_row_indices, int rows, int num_experts,
+                            int* d_slot_index, cf_stream_t stream) {
+    if (rows < 0 || num_experts < 0) return CF_ERR_INVALID_ARG;
+    if (rows == 0 || num_experts == 0) return CF_OK;
+    if (!d_counts || !d_offsets || !d_row_indices || !d_slot_index) return CF_ERR_INVALID_ARG;
+    const dim3 grid(ceil_div(static_cast<size_t>(rows), kThreads * 4), num_experts);
+    k_slot_index<<<grid, kThreads, 0, as_stream(stream)>>>(d_counts, d_offsets, d_row_indices, rows, num_experts, d_slot_index);
+    return launch_status();
+}
+
+int cf_moe_unpermute_indexed_bf16(uint16_t* d_mixed, const uint16_t* d_compact_out, const float* d_route_weights,
+                                  const int* d_slot_index, int rows, int num_experts, int H, int unit_weights,
+                                  cf_stream_t stream) {
+    if (rows < 0 || num_experts < 0 || H < 0) return CF_ERR_INVALID_ARG;
+    if (rows == 0 || num_experts == 0 || H == 0) return CF_OK;
+    if (!d_mixed || !d_compact_out || !d_route_weights || !d_slot_index) return CF_ERR_INVALID_ARG;
+    if ((H & 7) == 0 && !(aligned16(d_mixed) && aligned16(d_compact_out))) return CF_ERR_UNSUPPORTED;
+    if (unit_weights)
+        k_unpermute_indexed<true><<<rows, kThreads, 0, as_stream(stream)>>>(d_mixed, d_compact_out, d_route_weights, d_slot_index,
+                                                                            num_experts, H);
+    else
+        k_unpermute_indexed<false><<<rows, kThreads, 0, as_stream(stream)>>>(d_mixed, d_compact_out, d_route_weights, d_slot_index,
+                                                                             num_experts, H);
+    return launch_status();
+}
+
 // ---- grouped SwiGLU expert bank -----------------------------------------------------------------
 namespace {
-struct SwigluWs { size_t tile_map, index, act, actq, act_scale, act_descale, y, total; };
+struct SwigluWs { size_t tile_map, index, act, actq, act_scale, act_descale, y, slot, slot_bytes, total; };
 SwigluWs swiglu_layout(int total_rows, int num_experts, int H, int Ie) {
     auto up = [](size_t v) { return (v + 255) & ~static_cast<size_t>(255); };
     SwigluWs w{};
@@ -665,6 +737,11 @@ SwigluWs swiglu_layout(int total_rows, int num_experts, int H, int Ie) {
     w.act_scale = off; off = up(off + sizeof(float) * static_cast<size_t>(total_rows));
     w.act_descale = off; off = up(off + sizeof(float) * static_cast<size_t>(total_rows));
     w.y = off; off = up(off + 2 * static_cast<size_t>(total_rows) * H);
+    // the (row, expert) -> slot table of the unpermute: rows <= total_rows whenever every row selects an expert;
+    // a caller with more rows than that, or a table beyond 64 MiB, gets the searching unpermute instead
+    w.slot_bytes = sizeof(int) * static_cast<size_t>(total_rows) * num_experts;
+    if (w.slot_bytes > (64u << 20)) w.slot_bytes = 0;
+    w.slot = off; off = up(off + w.slot_bytes);
     w.total = off;
     return w;
 }
@@ -713,6 +790,12 @@ int cf_moe_grouped_swiglu_forward_fp8(const void* d_hidden_e4m3, const float* d_
                                         act_descale, d_w_down, d_w_down_descale, CF_SCALE_ROW_COL, CF_EPI_NONE, nullptr,
                                         nullptr, y, H, base + w.tile_map, map_bytes, stream);
     if (rc) return rc;
+    if (sizeof(int) * static_cast<size_t>(rows) * num_experts <= w.slot_bytes) {
+        int* slot = reinterpret_cast<int*>(base + w.slot);
+        rc = cf_moe_build_slot_index(d_counts, d_offsets, d_row_indices, rows, num_experts, slot, stream);
+        if (rc) return rc;
+        return cf_moe_unpermute_indexed_bf16(d_mixed, y, d_route_weights, slot, rows, num_experts, H, 0, stream);
+    }
     return cf_moe_unpermute_weighted_bf16(d_mixed, y, d_route_weights, d_counts, d_offsets, d_row_indices, rows,
                                           num_experts, H, stream);
 }

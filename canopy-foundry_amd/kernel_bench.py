@@ -241,6 +241,10 @@ def main():
     mixed = torch.zeros((T, H), dtype=torch.bfloat16, device=dev)
     hbm("unpermute_weighted_bf16", f"{total}x{H}", 2.0 * total * H + 4.0 * T * H,
         lambda: cf.cf_moe_unpermute_weighted_bf16(mixed, yy, rw, counts, offs, idx, T, E, H, st))
+    slot = torch.empty((T, E), dtype=torch.int32, device=dev)
+    hbm("build_slot_index", f"{T}x{E}", 8.0 * total, lambda: cf.cf_moe_build_slot_index(counts, offs, idx, T, E, slot, st))
+    hbm("unpermute_indexed_bf16 (slot table instead of the search)", f"{total}x{H}", 2.0 * total * H + 4.0 * T * H,
+        lambda: cf.cf_moe_unpermute_indexed_bf16(mixed, yy, rw, slot, T, E, H, 0, st))
     sz2 = ctypes.c_size_t(0)
     cf.raw_cf_moe_grouped_swiglu_workspace_bytes(total, E, H, Ie, ctypes.byref(sz2))
     ws2 = u8(sz2.value)

@@ -397,6 +397,18 @@ int cf_moe_unpermute_add_bf16(uint16_t* d_dst_full, const uint16_t* d_src_compac
                               const int* d_row_indices, int rows, int num_experts, int H,
                               cf_stream_t stream);
 
+/* The unpermute without the search: cf_moe_build_slot_index writes
+ * slot_index[row, e] = offsets[e] + position of row in expert e's list for every listed pair
+ * ([rows, num_experts] ints; other cells are not touched and not read), once per routing;
+ * cf_moe_unpermute_indexed_bf16 is then cf_moe_unpermute_weighted_bf16 (unit_weights = 0,
+ * kernels/moe.cu:730-738) or cf_moe_unpermute_add_bf16 (unit_weights = 1, kernels/moe.cu:760-767)
+ * with the same results.  No ordering requirement on the lists. */
+int cf_moe_build_slot_index(const int* d_counts, const int* d_offsets, const int* d_row_indices,
+                            int rows, int num_experts, int* d_slot_index, cf_stream_t stream);
+int cf_moe_unpermute_indexed_bf16(uint16_t* d_mixed, const uint16_t* d_compact_out,
+                                  const float* d_route_weights, const int* d_slot_index, int rows,
+                                  int num_experts, int H, int unit_weights, cf_stream_t stream);
+
 /* The grouped SwiGLU expert bank of benchmark config 5 (the FP8 form of the expert loop in
  * moe_expert_bank_forward, src/trainer.cu:6876-6934, with the SwiGLU experts of
  * moe_generic_forward, src/trainer.cu:6510-6529): permute -> gate/up GEMM with fused SiLU gate

@@ -191,6 +191,41 @@ def test_grouped_scatter_add_equals_the_per_expert_launches(cf, dev, rows, E, k,
     assert np.array_equal(bf16_bits(dfull), want)
 
 
+@pytest.mark.parametrize("rows,E,k,H", [(600, 5, 2, 256), (300, 70, 4, 1000), (1000, 16, 3, 2048), (16384, 64, 6, 2048)])
+@pytest.mark.parametrize("unit", [0, 1])
+def test_indexed_unpermute_equals_the_searching_one(cf, dev, rows, E, k, H, unit):
+    """The slot table is the search's answer computed once: both forms must agree bit for bit, weighted
+    (forward) and with unit factors (backward scatter-add)."""
+    case(f"indexed unpermute rows={rows} E={E} k={k} H={H} unit={unit}")
+    r = Routes(dev, rows, E, k, H, seed=rows + E + unit)
+    full = bf(np.random.default_rng(2).standard_normal((rows, H)))
+    y = dev_bf16(r.expert_out, dev)
+    a, b = dev_bf16(full, dev), dev_bf16(full, dev)
+    slot = torch.full((rows, E), -12345, dtype=torch.int32, device=dev)
+    cf.cf_moe_build_slot_index(r.d["counts"], r.d["offsets"], r.d["idx"], rows, E, slot, stream())
+    cf.cf_moe_unpermute_indexed_bf16(a, y, r.d["rw"], slot, rows, E, H, unit, stream())
+    if unit:
+        cf.cf_moe_unpermute_add_bf16(b, y, r.d["rw"], r.d["counts"], r.d["offsets"], r.d["idx"], rows, E, H, stream())
+    else:
+        cf.cf_moe_unpermute_weighted_bf16(b, y, r.d["rw"], r.d["counts"], r.d["offsets"], r.d["idx"], rows, E, H, stream())
+    torch.cuda.synchronize()
+    assert np.array_equal(bf16_bits(a), bf16_bits(b))
+    # the table itself: listed pairs hold their slot, every other cell is untouched
+    hs = host(slot)
+    want = np.full((rows, E), -12345, np.int32)
+    for e in range(E):
+        n = int(r.counts[e])
+        want[r.idx[e, :n], e] = r.offsets[e] + np.arange(n)
+    assert np.array_equal(hs, want)
+    if rows <= 1000:
+        ref = full
+        for e in range(E):
+            n, o = int(r.counts[e]), int(r.offsets[e])
+            ref = (orc.moe_scatter_add_rows(ref, r.expert_out[o:o + n], r.idx[e, :n]) if unit else
+                   orc.moe_scatter_accumulate(ref, r.expert_out[o:o + n], r.rw, r.idx[e, :n], e))
+        assert np.array_equal(bf16_bits(a), ref)
+
+
 def test_route_grad_config5_size(cf, dev):
     """16384 tokens, hidden 2048, 64 experts, top-6: the full-size launch against the oracle on three experts
     and through the identity sum_e w[row, e] * d_w[row, e] = dot(d_mixed[row], sum_e w expert_out) per row."""

@@ -194,6 +194,14 @@ inline int launch_status() {
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? CF_OK : static_cast<int>(e);
 }
+// The grouped GEMM behind cf_fp8_grouped_gemm_nt_bf16_ex, for callers inside the library that run several
+// projections over one routing: build_map = false reuses the tile table an earlier call left in d_workspace.
+int grouped_gemm_nt_bf16(int total_rows, int N, int K, int num_experts, const int* d_counts, const int* d_offsets,
+                         const void* A, int a_rows, int lda, const int* d_a_row_index, const float* a_descale,
+                         const void* B, const float* b_descale, int scale_mode, int epilogue, const void* B_up,
+                         const float* b_up_descale, uint16_t* C, int ldc, void* d_workspace, size_t workspace_bytes,
+                         bool build_map, cf_stream_t stream);
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline unsigned ceil_div(size_t a, size_t b) { return static_cast<unsigned>((a + b - 1) / b); }
 

@@ -1678,6 +1678,20 @@ int cf_fp8_grouped_gemm_nt_bf16_ex(int total_rows, int N, int K, int num_experts
                                    const float* a_descale, const void* B, const float* b_descale, int scale_mode,
                                    int epilogue, const void* B_up, const float* b_up_descale, uint16_t* C, int ldc,
                                    void* d_workspace, size_t workspace_bytes, cf_stream_t stream) {
+    return cf::grouped_gemm_nt_bf16(total_rows, N, K, num_experts, d_counts, d_offsets, A, a_rows, lda, d_a_row_index, a_descale, B,
+                                    b_descale, scale_mode, epilogue, B_up, b_up_descale, C, ldc, d_workspace, workspace_bytes,
+                                    true, stream);
+}
+
+}  // extern "C"
+
+// build_map = false: d_workspace already holds the tile table of these counts and offsets (an earlier call of
+// the same routing on the same stream built it)
+int cf::grouped_gemm_nt_bf16(int total_rows, int N, int K, int num_experts, const int* d_counts, const int* d_offsets,
+                             const void* A, int a_rows, int lda, const int* d_a_row_index, const float* a_descale,
+                             const void* B, const float* b_descale, int scale_mode, int epilogue, const void* B_up,
+                             const float* b_up_descale, uint16_t* C, int ldc, void* d_workspace, size_t workspace_bytes,
+                             bool build_map, cf_stream_t stream) {
     if (total_rows < 0 || N < 0 || K < 0 || num_experts < 0 || a_rows < 0) return CF_ERR_INVALID_ARG;
     if (total_rows == 0 || N == 0 || num_experts == 0) return CF_OK;
     if (!d_counts || !d_offsets || !A || !B || !C || !a_descale || !b_descale || !d_workspace) return CF_ERR_INVALID_ARG;
@@ -1697,7 +1711,7 @@ int cf_fp8_grouped_gemm_nt_bf16_ex(int total_rows, int N, int K, int num_experts
     hipStream_t st = as_stream(stream);
     const int max_row_tiles = total_rows / BM + num_experts;
     int* tile_map = static_cast<int*>(d_workspace);
-    k_build_tile_map<<<1, 64, 0, st>>>(d_counts, d_offsets, num_experts, max_row_tiles, tile_map);
+    if (build_map) k_build_tile_map<<<1, 64, 0, st>>>(d_counts, d_offsets, num_experts, max_row_tiles, tile_map);
     GemmArgs p{};
     p.M = total_rows; p.N = N; p.K = K;
     p.A = static_cast<const uint8_t*>(A); p.lda = lda;
@@ -1720,6 +1734,8 @@ int cf_fp8_grouped_gemm_nt_bf16_ex(int total_rows, int N, int K, int num_experts
     return epilogue == EPI_SILU_GATE ? launch_tiled<0, EPI_SILU_GATE, SCALE_ROWCOL>(p, st)
                                      : launch_tiled<0, EPI_NONE, SCALE_ROWCOL>(p, st);
 }
+
+extern "C" {
 
 // Cross-check form of the accumulate GEMMs: any format pair, optional naive kernel.
 int cf_fp8_gemm_nt_accum_f32_ex(int M, int N, int K, const void* A, int lda, int a_is_e5m2, const float* a_descale,

@@ -288,11 +288,14 @@ __global__ __launch_bounds__(kThreads) void k_scatter_accumulate(uint16_t* __res
 // ---- compact row index: the row lists of all experts back to back --------------------
 __global__ __launch_bounds__(kThreads) void k_compact_index(const int* __restrict__ counts, const int* __restrict__ offsets,
                                                             const int* __restrict__ row_indices, int rows,
-                                                            int* __restrict__ compact) {
+                                                            int* __restrict__ compact, int* __restrict__ slot_index, int E) {
     const int e = blockIdx.y;
     const int n = counts[e], base = offsets[e];
-    for (int s = blockIdx.x * blockDim.x + threadIdx.x; s < n; s += gridDim.x * blockDim.x)
-        compact[base + s] = row_indices[static_cast<size_t>(e) * rows + s];
+    for (int s = blockIdx.x * blockDim.x + threadIdx.x; s < n; s += gridDim.x * blockDim.x) {
+        const int row = row_indices[static_cast<size_t>(e) * rows + s];
+        compact[base + s] = row;
+        if (slot_index) slot_index[static_cast<size_t>(row) * E + e] = base + s;      // the inverse, for the unpermute
+    }
 }
 
 // ---- fused weighted unpermute ------------------------------------------------------------
@@ -655,7 +658,8 @@ int cf_moe_compact_row_index(const int* d_counts, const int* d_offsets, const in
     if (rows == 0 || num_experts == 0) return CF_OK;
     if (!d_counts || !d_offsets || !d_row_indices || !d_compact_index) return CF_ERR_INVALID_ARG;
     dim3 grid(ceil_div(rows, kThreads) < 16 ? ceil_div(rows, kThreads) : 16, num_experts);
-    k_compact_index<<<grid, kThreads, 0, as_stream(stream)>>>(d_counts, d_offsets, d_row_indices, rows, d_compact_index);
+    k_compact_index<<<grid, kThreads, 0, as_stream(stream)>>>(d_counts, d_offsets, d_row_indices, rows, d_compact_index, nullptr,
+                                                              num_experts);
     return launch_status();
 }
 
@@ -777,7 +781,14 @@ int cf_moe_grouped_swiglu_forward_fp8(const void* d_hidden_e4m3, const float* d_
     auto* y = reinterpret_cast<uint16_t*>(base + w.y);
     size_t map_bytes = 0;
     cf_fp8_grouped_gemm_workspace_bytes(total_selected_rows, num_experts, &map_bytes);
-    int rc = cf_moe_compact_row_index(d_counts, d_offsets, d_row_indices, rows, num_experts, index, stream);
+    // the compact index for the gather and, when the workspace holds it, its inverse for the unpermute: one launch
+    const bool indexed = sizeof(int) * static_cast<size_t>(rows) * num_experts <= w.slot_bytes;
+    int* slot = indexed ? reinterpret_cast<int*>(base + w.slot) : nullptr;
+    {
+        const dim3 grid(ceil_div(rows, kThreads) < 16 ? ceil_div(rows, kThreads) : 16, num_experts);
+        k_compact_index<<<grid, kThreads, 0, as_stream(stream)>>>(d_counts, d_offsets, d_row_indices, rows, index, slot, num_experts);
+    }
+    int rc = launch_status();
     if (rc) return rc;
     // gate/up: rows gathered through the compact index (the token permute is fused into the operand fetch)
     rc = cf_fp8_grouped_gemm_nt_bf16_ex(total_selected_rows, Ie, H, num_experts, d_counts, d_offsets, d_hidden_e4m3, rows, H, index,
@@ -786,16 +797,12 @@ int cf_moe_grouped_swiglu_forward_fp8(const void* d_hidden_e4m3, const float* d_
     if (rc) return rc;
     rc = cf_fp8_quantize_rows(act, total_selected_rows, Ie, 0, actq, act_scale, act_descale, stream);
     if (rc) return rc;
-    rc = cf_fp8_grouped_gemm_nt_bf16_ex(total_selected_rows, H, Ie, num_experts, d_counts, d_offsets, actq, total_selected_rows, Ie, nullptr,
-                                        act_descale, d_w_down, d_w_down_descale, CF_SCALE_ROW_COL, CF_EPI_NONE, nullptr,
-                                        nullptr, y, H, base + w.tile_map, map_bytes, stream);
+    // same routing, same tile table
+    rc = grouped_gemm_nt_bf16(total_selected_rows, H, Ie, num_experts, d_counts, d_offsets, actq, total_selected_rows, Ie, nullptr,
+                              act_descale, d_w_down, d_w_down_descale, CF_SCALE_ROW_COL, CF_EPI_NONE, nullptr, nullptr, y, H,
+                              base + w.tile_map, map_bytes, false, stream);
     if (rc) return rc;
-    if (sizeof(int) * static_cast<size_t>(rows) * num_experts <= w.slot_bytes) {
-        int* slot = reinterpret_cast<int*>(base + w.slot);
-        rc = cf_moe_build_slot_index(d_counts, d_offsets, d_row_indices, rows, num_experts, slot, stream);
-        if (rc) return rc;
-        return cf_moe_unpermute_indexed_bf16(d_mixed, y, d_route_weights, slot, rows, num_experts, H, 0, stream);
-    }
+    if (indexed) return cf_moe_unpermute_indexed_bf16(d_mixed, y, d_route_weights, slot, rows, num_experts, H, 0, stream);
     return cf_moe_unpermute_weighted_bf16(d_mixed, y, d_route_weights, d_counts, d_offsets, d_row_indices, rows,
                                           num_experts, H, stream);
 }

@@ -36,6 +36,11 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
     return static_cast<uint32_t>(f32_to_bf16(lo)) | (static_cast<uint32_t>(f32_to_bf16(hi)) << 16);
 }
 
+// Exact-erf GELU in fp32 (gelu_forward_kernel, kernels/moe.cu:510-517 of the reference), and the same on a packed bf16 pair with
+// one rounding of each result to bf16.
+__device__ __forceinline__ float gelu_fwd(float v) { return 0.5f * v * (1.0f + erff(v * 0.7071067811865476f)); }
+__device__ __forceinline__ uint32_t gelu2(uint32_t pair) { return pack_bf16x2(gelu_fwd(bf16_lo(pair)), gelu_fwd(bf16_hi(pair))); }
+
 // Two floats -> packed bf16 pair on gfx950's v_cvt_pk_bf16_f32 (round to nearest even).
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
@@ -195,12 +200,13 @@ inline int launch_status() {
     return e == hipSuccess ? CF_OK : static_cast<int>(e);
 }
 // The grouped GEMM behind cf_fp8_grouped_gemm_nt_bf16_ex, for callers inside the library that run several
-// projections over one routing: build_map = false reuses the tile table an earlier call left in d_workspace.
+// projections over one routing: build_map = false reuses the tile table an earlier call left in d_workspace;
+// a_is_e5m2 takes E5M2 activations (plain epilogue only).
 int grouped_gemm_nt_bf16(int total_rows, int N, int K, int num_experts, const int* d_counts, const int* d_offsets,
                          const void* A, int a_rows, int lda, const int* d_a_row_index, const float* a_descale,
                          const void* B, const float* b_descale, int scale_mode, int epilogue, const void* B_up,
                          const float* b_up_descale, uint16_t* C, int ldc, void* d_workspace, size_t workspace_bytes,
-                         bool build_map, cf_stream_t stream);
+                         bool build_map, int a_is_e5m2, cf_stream_t stream);
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline unsigned ceil_div(size_t a, size_t b) { return static_cast<unsigned>((a + b - 1) / b); }

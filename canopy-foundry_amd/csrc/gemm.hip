@@ -1680,19 +1680,20 @@ int cf_fp8_grouped_gemm_nt_bf16_ex(int total_rows, int N, int K, int num_experts
                                    void* d_workspace, size_t workspace_bytes, cf_stream_t stream) {
     return cf::grouped_gemm_nt_bf16(total_rows, N, K, num_experts, d_counts, d_offsets, A, a_rows, lda, d_a_row_index, a_descale, B,
                                     b_descale, scale_mode, epilogue, B_up, b_up_descale, C, ldc, d_workspace, workspace_bytes,
-                                    true, stream);
+                                    true, 0, stream);
 }
 
 }  // extern "C"
 
 // build_map = false: d_workspace already holds the tile table of these counts and offsets (an earlier call of
-// the same routing on the same stream built it)
+// the same routing on the same stream built it); a_is_e5m2: the activations are E5M2 (plain epilogue only)
 int cf::grouped_gemm_nt_bf16(int total_rows, int N, int K, int num_experts, const int* d_counts, const int* d_offsets,
                              const void* A, int a_rows, int lda, const int* d_a_row_index, const float* a_descale,
                              const void* B, const float* b_descale, int scale_mode, int epilogue, const void* B_up,
                              const float* b_up_descale, uint16_t* C, int ldc, void* d_workspace, size_t workspace_bytes,
-                             bool build_map, cf_stream_t stream) {
+                             bool build_map, int a_is_e5m2, cf_stream_t stream) {
     if (total_rows < 0 || N < 0 || K < 0 || num_experts < 0 || a_rows < 0) return CF_ERR_INVALID_ARG;
+    if (a_is_e5m2 && epilogue != EPI_NONE) return CF_ERR_UNSUPPORTED;
     if (total_rows == 0 || N == 0 || num_experts == 0) return CF_OK;
     if (!d_counts || !d_offsets || !A || !B || !C || !a_descale || !b_descale || !d_workspace) return CF_ERR_INVALID_ARG;
     if (epilogue != EPI_NONE && epilogue != EPI_SILU_GATE) return CF_ERR_INVALID_ARG;
@@ -1731,6 +1732,7 @@ int cf::grouped_gemm_nt_bf16(int total_rows, int N, int K, int num_experts, cons
         // per-tensor descales: one device scalar per expert for the weights
         return CF_ERR_UNSUPPORTED;
     }
+    if (a_is_e5m2) return launch_tiled<1, EPI_NONE, SCALE_ROWCOL>(p, st);
     return epilogue == EPI_SILU_GATE ? launch_tiled<0, EPI_SILU_GATE, SCALE_ROWCOL>(p, st)
                                      : launch_tiled<0, EPI_NONE, SCALE_ROWCOL>(p, st);
 }

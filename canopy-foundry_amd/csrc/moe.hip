@@ -539,6 +539,129 @@ __global__ __launch_bounds__(kThreads) void k_grouped_gelu_fp8(const uint8_t* __
     }
 }
 
+// ---- the same bank on the matrix cores -----------------------------------------------------------
+// Same arithmetic contract (GELU output kept beyond bf16, nothing re-quantised, compare-and-swap accumulation), for
+// H % 128 == 0 and Ie % 64 == 0.  One workgroup per (expert, 16 rows), four wavefronts:
+//   fc_in   v_mfma_f32_16x16x128_f8f6f4 on the fp8 bytes as they are (products of fp8 values are exact in the fp32
+//           accumulator; the two per-tensor descales multiply the sum).  The 16 hidden rows sit in LDS, weight rows
+//           come from L2 as 32-byte runs per lane.
+//   GELU    in fp32 on the accumulator, split into a bf16 head and a bf16 remainder (together 16 significand bits,
+//           relative error 2^-17) and parked in LDS.
+//   fc_out  v_mfma_f32_16x16x32_bf16 twice per step (head and remainder) against the E4M3 weights widened to bf16,
+//           which is exact.  A lane fetches 16 weight bytes at once and uses them as two k-blocks of 8; the activation
+//           reads follow the same order, and a sum does not care which k a lane group holds.
+// Weights go to the "A" side, so a lane ends with 4 neighbouring output columns of one token row.
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+constexpr int kMfmaRows = 16;
+
+__device__ __forceinline__ v8bf e4m3x8_to_bf16(uint32_t a, uint32_t b) {
+    const f32x2_t p0 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(a), false), p1 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(a), true);
+    const f32x2_t p2 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(b), false), p3 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(b), true);
+    auto pair = [](f32x2_t p) { return (__float_as_uint(p[0]) >> 16) | (__float_as_uint(p[1]) & 0xffff0000u); };
+    const v4u w = {pair(p0), pair(p1), pair(p2), pair(p3)};
+    return __builtin_bit_cast(v8bf, w);
+}
+
+// two neighbouring bf16 values += (v0, v1), one rounding each, by compare-and-swap on their word
+__device__ __forceinline__ void atomic_add_bf16x2(unsigned* word, float v0, float v1) {
+    unsigned old = *word;
+    while (true) {
+        const unsigned assumed = old;
+        const unsigned next = pack_bf16x2(bf16_lo(assumed) + v0, bf16_hi(assumed) + v1);
+        old = atomicCAS(word, assumed, next);
+        if (old == assumed) return;
+    }
+}
+
+template <bool E5M2>
+__global__ __launch_bounds__(kThreads) void k_grouped_gelu_fp8_mfma(const uint8_t* __restrict__ hidden, const float* __restrict__ fcin_descale,
+                                                                    const float* __restrict__ route_weights, const int* __restrict__ counts,
+                                                                    const int* __restrict__ row_indices, const uint8_t* __restrict__ fc_in_w,
+                                                                    const float* __restrict__ fc_in_descale, const uint8_t* __restrict__ fc_out_w,
+                                                                    const float* __restrict__ fc_out_descale, uint16_t* __restrict__ mixed,
+                                                                    int rows, int H, int Ie, int E, int tiles_per_expert) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    const int hs = H + 16;                          // hidden row stride in bytes: neighbouring rows 16 bytes apart in the banks
+    const int as = Ie + 8;                          // activation row stride in elements, likewise
+    uint8_t* sh_hidden = smem;                                                        // [16][hs] fp8
+    uint16_t* sh_hi = reinterpret_cast<uint16_t*>(smem + kMfmaRows * hs);             // [16][as] bf16 head of gelu
+    uint16_t* sh_lo = sh_hi + kMfmaRows * as;                                         // [16][as] bf16 remainder
+    const int e = blockIdx.x / tiles_per_expert, tile = blockIdx.x % tiles_per_expert;
+    const int first = tile * kMfmaRows, n_active = counts[e];
+    if (first >= n_active) return;
+    const int n_rows = min(kMfmaRows, n_active - first);
+    const int* my_rows = row_indices + static_cast<size_t>(e) * rows + first;
+    const uint8_t* w_in = fc_in_w + static_cast<size_t>(e) * H * Ie;
+    const uint8_t* w_out = fc_out_w + static_cast<size_t>(e) * Ie * H;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, t = lane & 15, g = lane >> 4;
+
+    // the tile's hidden rows (rows past the list's end repeat its last one; their results are dropped)
+    const int vec_per_row = H / 16;
+    for (int i = threadIdx.x; i < kMfmaRows * vec_per_row; i += kThreads) {
+        const int r = i / vec_per_row, c = i % vec_per_row;
+        const int src = my_rows[min(r, n_rows - 1)];
+        *reinterpret_cast<uint4*>(sh_hidden + r * hs + c * 16) =
+            *reinterpret_cast<const uint4*>(hidden + static_cast<size_t>(src) * H + c * 16);
+    }
+    __syncthreads();
+
+    const float s_in = *fcin_descale * *fc_in_descale;
+    for (int n0 = wave * 16; n0 < Ie; n0 += 4 * 16) {
+        v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        const uint8_t* wr = w_in + static_cast<size_t>(n0 + t) * H + 32 * g;
+        const uint8_t* hr = sh_hidden + t * hs + 32 * g;
+        for (int k0 = 0; k0 < H; k0 += 128) {
+            const uint4 w0 = *reinterpret_cast<const uint4*>(wr + k0), w1 = *reinterpret_cast<const uint4*>(wr + k0 + 16);
+            const uint4 x0 = *reinterpret_cast<const uint4*>(hr + k0), x1 = *reinterpret_cast<const uint4*>(hr + k0 + 16);
+            const v8i a = {(int)w0.x, (int)w0.y, (int)w0.z, (int)w0.w, (int)w1.x, (int)w1.y, (int)w1.z, (int)w1.w};
+            const v8i b = {(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w, (int)x1.x, (int)x1.y, (int)x1.z, (int)x1.w};
+            acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc, 0 /* weights E4M3 */, E5M2 ? 1 : 0, 0, 0, 0, 0);
+        }
+        // this lane: token row t, columns n0 + 4g .. + 3
+        uint32_t hb[4], lb[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float v = acc[r] * s_in;
+            const float act = gelu_fwd(v);
+            hb[r] = __float_as_uint(act) & 0xffff0000u;
+            lb[r] = f32_to_bf16(act - __uint_as_float(hb[r]));
+        }
+        const int at = t * as + n0 + 4 * g;
+        *reinterpret_cast<uint2*>(sh_hi + at) = make_uint2((hb[0] >> 16) | hb[1], (hb[2] >> 16) | hb[3]);
+        *reinterpret_cast<uint2*>(sh_lo + at) = make_uint2(lb[0] | (lb[1] << 16), lb[2] | (lb[3] << 16));
+    }
+    __syncthreads();
+
+    const float d_wout = *fc_out_descale;
+    for (int h0 = wave * 16; h0 < H; h0 += 4 * 16) {
+        v4f acc_hi = {0.0f, 0.0f, 0.0f, 0.0f}, acc_lo = {0.0f, 0.0f, 0.0f, 0.0f};
+        const uint8_t* wr = w_out + static_cast<size_t>(h0 + t) * Ie + 16 * g;
+        const uint16_t* ah = sh_hi + t * as + 16 * g;
+        const uint16_t* al = sh_lo + t * as + 16 * g;
+        for (int k0 = 0; k0 < Ie; k0 += 64) {
+            const uint4 w = *reinterpret_cast<const uint4*>(wr + k0);              // k0 + 16g .. + 15
+            const v8bf wa = e4m3x8_to_bf16(w.x, w.y), wb = e4m3x8_to_bf16(w.z, w.w);
+            const v8bf ha = *reinterpret_cast<const v8bf*>(ah + k0), hb = *reinterpret_cast<const v8bf*>(ah + k0 + 8);
+            const v8bf la = *reinterpret_cast<const v8bf*>(al + k0), lb = *reinterpret_cast<const v8bf*>(al + k0 + 8);
+            acc_hi = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, ha, acc_hi, 0, 0, 0);
+            acc_lo = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, la, acc_lo, 0, 0, 0);
+            acc_hi = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb, hb, acc_hi, 0, 0, 0);
+            acc_lo = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb, lb, acc_lo, 0, 0, 0);
+        }
+        if (t < n_rows) {
+            const int row = my_rows[t];
+            const float rw = route_weights[static_cast<size_t>(row) * E + e];
+            float v[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) v[r] = rw * ((acc_hi[r] + acc_lo[r]) * d_wout);
+            auto* word = reinterpret_cast<unsigned*>(mixed + static_cast<size_t>(row) * H + h0 + 4 * g);
+            atomic_add_bf16x2(word, v[0], v[1]);
+            atomic_add_bf16x2(word + 1, v[2], v[3]);
+        }
+    }
+}
+
 unsigned grid_for(size_t items) {
     const size_t b = (items + kThreads - 1) / kThreads;
     return static_cast<unsigned>(b < 1 ? 1 : (b > 8192 ? 8192 : b));
@@ -800,7 +923,102 @@ int cf_moe_grouped_swiglu_forward_fp8(const void* d_hidden_e4m3, const float* d_
     // same routing, same tile table
     rc = grouped_gemm_nt_bf16(total_selected_rows, H, Ie, num_experts, d_counts, d_offsets, actq, total_selected_rows, Ie, nullptr,
                               act_descale, d_w_down, d_w_down_descale, CF_SCALE_ROW_COL, CF_EPI_NONE, nullptr, nullptr, y, H,
-                              base + w.tile_map, map_bytes, false, stream);
+                              base + w.tile_map, map_bytes, false, 0, stream);
+    if (rc) return rc;
+    if (indexed) return cf_moe_unpermute_indexed_bf16(d_mixed, y, d_route_weights, slot, rows, num_experts, H, 0, stream);
+    return cf_moe_unpermute_weighted_bf16(d_mixed, y, d_route_weights, d_counts, d_offsets, d_row_indices, rows,
+                                          num_experts, H, stream);
+}
+
+// ---- grouped GELU expert bank on the matrix cores -----------------------------------------------
+// The reference's per-expert loop (gather -> FP8 GEMM -> gelu_forward -> quantize -> FP8 GEMM -> scatter-accumulate,
+// src/trainer.cu:6886-6934) for all experts at once.  The workspace is the SwiGLU bank's plus the three per-tensor
+// descales spread into the per-token / per-channel vectors the grouped GEMM reads.
+namespace {
+struct GeluWs { SwigluWs s; size_t hidden_descale, in_descale, out_descale, total; };
+GeluWs gelu_layout(int rows, int total_rows, int num_experts, int H, int Ie) {
+    auto up = [](size_t v) { return (v + 255) & ~static_cast<size_t>(255); };
+    GeluWs w{};
+    w.s = swiglu_layout(total_rows, num_experts, H, Ie);
+    size_t off = w.s.total;
+    w.hidden_descale = off; off = up(off + sizeof(float) * static_cast<size_t>(rows));
+    w.in_descale = off; off = up(off + sizeof(float) * static_cast<size_t>(num_experts) * Ie);
+    w.out_descale = off; off = up(off + sizeof(float) * static_cast<size_t>(num_experts) * H);
+    w.total = off;
+    return w;
+}
+
+__global__ __launch_bounds__(kThreads) void k_spread_descales(const float* __restrict__ a, float* __restrict__ av, size_t na,
+                                                              const float* __restrict__ b, float* __restrict__ bv, size_t nb,
+                                                              const float* __restrict__ c, float* __restrict__ cv, size_t nc) {
+    const float fa = *a, fb = *b, fc = *c;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < na + nb + nc;
+         i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+        if (i < na) av[i] = fa;
+        else if (i < na + nb) bv[i - na] = fb;
+        else cv[i - na - nb] = fc;
+    }
+}
+}  // namespace
+
+int cf_moe_grouped_gelu_workspace_bytes(int rows, int total_selected_rows, int num_experts, int H, int Ie, size_t* bytes) {
+    if (rows < 0 || total_selected_rows < 0 || num_experts < 0 || H < 0 || Ie < 0 || !bytes) return CF_ERR_INVALID_ARG;
+    *bytes = gelu_layout(rows, total_selected_rows, num_experts, H, Ie).total;
+    return CF_OK;
+}
+
+int cf_moe_grouped_gelu_forward_fp8(const void* d_hidden, const float* d_fcin_descale, int fcin_is_e5m2,
+                                    const float* d_route_weights, const int* d_counts, const int* d_offsets,
+                                    const int* d_row_indices, const void* d_fc_in_w, const float* d_fc_in_descale,
+                                    const void* d_fc_out_w, const float* d_fc_out_descale, uint16_t* d_mixed, int rows,
+                                    int H, int Ie, int num_experts, int total_selected_rows, void* d_workspace,
+                                    size_t workspace_bytes, cf_stream_t stream) {
+    if (rows < 0 || H < 0 || Ie < 0 || num_experts < 0 || total_selected_rows < 0) return CF_ERR_INVALID_ARG;
+    if (rows == 0 || num_experts == 0 || total_selected_rows == 0) return CF_OK;
+    if (!d_hidden || !d_fcin_descale || !d_route_weights || !d_counts || !d_offsets || !d_row_indices || !d_fc_in_w ||
+        !d_fc_in_descale || !d_fc_out_w || !d_fc_out_descale || !d_mixed || !d_workspace)
+        return CF_ERR_INVALID_ARG;
+    const GeluWs w = gelu_layout(rows, total_selected_rows, num_experts, H, Ie);
+    if (workspace_bytes < w.total || (reinterpret_cast<uintptr_t>(d_workspace) & 255u)) return CF_ERR_INVALID_ARG;
+    auto* base = static_cast<uint8_t*>(d_workspace);
+    int* index = reinterpret_cast<int*>(base + w.s.index);
+    auto* act = reinterpret_cast<uint16_t*>(base + w.s.act);
+    auto* actq = base + w.s.actq;
+    auto* act_scale = reinterpret_cast<float*>(base + w.s.act_scale);
+    auto* act_descale = reinterpret_cast<float*>(base + w.s.act_descale);
+    auto* y = reinterpret_cast<uint16_t*>(base + w.s.y);
+    auto* hidden_descale = reinterpret_cast<float*>(base + w.hidden_descale);
+    auto* in_descale = reinterpret_cast<float*>(base + w.in_descale);
+    auto* out_descale = reinterpret_cast<float*>(base + w.out_descale);
+    size_t map_bytes = 0;
+    cf_fp8_grouped_gemm_workspace_bytes(total_selected_rows, num_experts, &map_bytes);
+    hipStream_t st = as_stream(stream);
+    const bool indexed = sizeof(int) * static_cast<size_t>(rows) * num_experts <= w.s.slot_bytes;
+    int* slot = indexed ? reinterpret_cast<int*>(base + w.s.slot) : nullptr;
+    {
+        const dim3 grid(ceil_div(rows, kThreads) < 16 ? ceil_div(rows, kThreads) : 16, num_experts);
+        k_compact_index<<<grid, kThreads, 0, st>>>(d_counts, d_offsets, d_row_indices, rows, index, slot, num_experts);
+    }
+    int rc = launch_status();
+    if (rc) return rc;
+    {
+        const size_t na = static_cast<size_t>(rows), nb = static_cast<size_t>(num_experts) * Ie, nc = static_cast<size_t>(num_experts) * H;
+        k_spread_descales<<<grid_for(na + nb + nc), kThreads, 0, st>>>(d_fcin_descale, hidden_descale, na, d_fc_in_descale, in_descale, nb,
+                                                                      d_fc_out_descale, out_descale, nc);
+    }
+    rc = launch_status();
+    if (rc) return rc;
+    // fc_in: token rows gathered through the compact index in the operand fetch
+    rc = grouped_gemm_nt_bf16(total_selected_rows, Ie, H, num_experts, d_counts, d_offsets, d_hidden, rows, H, index, hidden_descale,
+                              d_fc_in_w, in_descale, CF_SCALE_ROW_COL, CF_EPI_NONE, nullptr, nullptr, act, Ie, base + w.s.tile_map,
+                              map_bytes, true, fcin_is_e5m2 ? 1 : 0, stream);
+    if (rc) return rc;
+    // gelu_forward and the per-token quantize in one pass over the bf16 projections
+    rc = cf_gelu_quantize_rows_e4m3(act, total_selected_rows, Ie, actq, act_scale, act_descale, stream);
+    if (rc) return rc;
+    rc = grouped_gemm_nt_bf16(total_selected_rows, H, Ie, num_experts, d_counts, d_offsets, actq, total_selected_rows, Ie, nullptr,
+                              act_descale, d_fc_out_w, out_descale, CF_SCALE_ROW_COL, CF_EPI_NONE, nullptr, nullptr, y, H,
+                              base + w.s.tile_map, map_bytes, false, 0, stream);
     if (rc) return rc;
     if (indexed) return cf_moe_unpermute_indexed_bf16(d_mixed, y, d_route_weights, slot, rows, num_experts, H, 0, stream);
     return cf_moe_unpermute_weighted_bf16(d_mixed, y, d_route_weights, d_counts, d_offsets, d_row_indices, rows,
@@ -819,6 +1037,31 @@ int cf_moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_fcin_
     if (!d_hidden || !d_fcin_descale || !d_route_weights || !d_counts || !d_row_indices || !d_fc_in_w || !d_fc_in_descale ||
         !d_fc_out_w || !d_fc_out_descale || !d_mixed)
         return CF_ERR_INVALID_ARG;
+    // the matrix-core form where the shapes are whole MFMA steps and its tile fits the LDS
+    const size_t smem_mfma = static_cast<size_t>(kMfmaRows) * (H + 16) + 4u * kMfmaRows * (static_cast<size_t>(Ie) + 8);
+    if (H % 128 == 0 && Ie % 64 == 0 && smem_mfma <= 160 * 1024 && aligned16(d_hidden) && aligned16(d_fc_in_w) &&
+        aligned16(d_fc_out_w) && (reinterpret_cast<uintptr_t>(d_mixed) & 3u) == 0) {
+        static std::once_flag once_mfma;
+        static hipError_t err_mfma = hipSuccess;
+        std::call_once(once_mfma, [] {
+            err_mfma = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_grouped_gelu_fp8_mfma<false>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (err_mfma == hipSuccess)
+                err_mfma = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_grouped_gelu_fp8_mfma<true>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        });
+        if (err_mfma != hipSuccess) return static_cast<int>(err_mfma);
+        const int tiles = (rows + kMfmaRows - 1) / kMfmaRows;
+        auto launch = [&](auto kernel) {
+            kernel<<<num_experts * tiles, kThreads, smem_mfma, as_stream(stream)>>>(
+                static_cast<const uint8_t*>(d_hidden), d_fcin_descale, d_route_weights, d_counts, d_row_indices,
+                static_cast<const uint8_t*>(d_fc_in_w), d_fc_in_descale, static_cast<const uint8_t*>(d_fc_out_w), d_fc_out_descale,
+                d_mixed, rows, H, Ie, num_experts, tiles);
+        };
+        if (fcin_is_e5m2) launch(k_grouped_gelu_fp8_mfma<true>);
+        else launch(k_grouped_gelu_fp8_mfma<false>);
+        return launch_status();
+    }
     const size_t smem = sizeof(float) * static_cast<size_t>(kGeluRows) * (kGeluChunk + Ie);
     if (smem > 160 * 1024) return CF_ERR_UNSUPPORTED;
     static std::once_flag once;

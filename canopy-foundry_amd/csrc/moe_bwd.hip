@@ -140,14 +140,12 @@ int launch_route_grad(const RouteGradArgs& p, int max_list, hipStream_t st) {
 }
 
 // ---- GELU ----------------------------------------------------------------------------------------
-__device__ __forceinline__ float gelu_fwd(float v) { return 0.5f * v * (1.0f + erff(v * 0.7071067811865476f)); }
 // `cdf + x * pdf` is one fused multiply-add in the reference's build (default contraction)
 __device__ __forceinline__ float gelu_deriv(float x) {
     const float cdf = 0.5f * (1.0f + erff(x * 0.7071067811865476f));
     const float pdf = 0.3989422804014327f * expf(-0.5f * x * x);
     return __builtin_fmaf(x, pdf, cdf);
 }
-__device__ __forceinline__ uint32_t gelu2(uint32_t pair) { return pack_bf16x2(gelu_fwd(bf16_lo(pair)), gelu_fwd(bf16_hi(pair))); }
 __device__ __forceinline__ uint32_t gelu_bwd2(uint32_t pre, uint32_t g) {
     return pack_bf16x2(bf16_lo(g) * gelu_deriv(bf16_lo(pre)), bf16_hi(g) * gelu_deriv(bf16_hi(pre)));
 }

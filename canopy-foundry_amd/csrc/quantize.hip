@@ -47,6 +47,13 @@ __device__ __forceinline__ Vec16 load16(const uint16_t* p) {
     v.hi = *reinterpret_cast<const uint4*>(p + 8);
     return v;
 }
+// the exact-erf GELU of 16 bf16 values, each result rounded to bf16 (what gelu_forward leaves in memory)
+__device__ __forceinline__ Vec16 gelu16(const Vec16& v) {
+    Vec16 g;
+    g.lo = make_uint4(gelu2(v.lo.x), gelu2(v.lo.y), gelu2(v.lo.z), gelu2(v.lo.w));
+    g.hi = make_uint4(gelu2(v.hi.x), gelu2(v.hi.y), gelu2(v.hi.z), gelu2(v.hi.w));
+    return g;
+}
 __device__ __forceinline__ float amax16(const Vec16& v) {
     const uint32_t w[8] = {v.lo.x, v.lo.y, v.lo.z, v.lo.w, v.hi.x, v.hi.y, v.hi.z, v.hi.w};
     float m = 0.0f;
@@ -337,7 +344,9 @@ __global__ __launch_bounds__(kThreads) void k_elem_clip_count(const uint16_t* __
 // One wavefront per row.  The row stays in registers between the amax pass and
 // the convert pass, so HBM sees 2 B read + 1 B written per element.
 // MAXS = register-resident steps of 64 lanes x 16 elements.
-template <bool E5M2, int MAXS>
+// GELU: the row quantized is bf16(gelu(x)), computed on the way in (the activation between an expert's two
+// projections is never written as bf16).
+template <bool E5M2, int MAXS, bool GELU = false>
 __global__ __launch_bounds__(kThreads) void k_quant_rows(const uint16_t* __restrict__ x, int rows, int K,
                                                          uint8_t* __restrict__ out,
                                                          float* __restrict__ scale,
@@ -354,6 +363,7 @@ __global__ __launch_bounds__(kThreads) void k_quant_rows(const uint16_t* __restr
         const int k = (s * 64 + lane) * kVec;
         if (k < K) {
             v[s] = load16(xr + k);
+            if constexpr (GELU) v[s] = gelu16(v[s]);
             acc = absmax16(acc, v[s]);
         }
     }
@@ -381,7 +391,7 @@ __global__ __launch_bounds__(kThreads) void k_quant_rows(const uint16_t* __restr
 // Long rows (4096 < K <= 32768): one workgroup of four wavefronts per row, the row still register-resident (four or
 // eight steps per lane instead of sixteen or more, so more wavefronts fit a SIMD); the row maximum crosses the
 // wavefronts through LDS.
-template <bool E5M2, int MAXS>      // MAXS steps of 256 lanes x 16 elements: 4 covers K <= 16384, 8 covers K <= 32768
+template <bool E5M2, int MAXS, bool GELU = false>      // MAXS steps of 256 lanes x 16 elements: 4 covers K <= 16384, 8 covers K <= 32768
 __global__ __launch_bounds__(kThreads) void k_quant_rows_block(const uint16_t* __restrict__ x, int K,
                                                                uint8_t* __restrict__ out,
                                                                float* __restrict__ scale,
@@ -398,6 +408,7 @@ __global__ __launch_bounds__(kThreads) void k_quant_rows_block(const uint16_t* _
         const int k = (s * kThreads + tid) * kVec;
         if (k < K) {
             v[s] = load16(xr + k);
+            if constexpr (GELU) v[s] = gelu16(v[s]);
             acc = absmax16(acc, v[s]);
         }
     }
@@ -429,7 +440,7 @@ __global__ __launch_bounds__(kThreads) void k_quant_rows_block(const uint16_t* _
 }
 
 // Any K, any alignment: one workgroup per row, two passes over the row.
-template <bool E5M2>
+template <bool E5M2, bool GELU = false>
 __global__ __launch_bounds__(kThreads) void k_quant_rows_generic(const uint16_t* __restrict__ x, int K,
                                                                  uint8_t* __restrict__ out,
                                                                  float* __restrict__ scale,
@@ -438,13 +449,17 @@ __global__ __launch_bounds__(kThreads) void k_quant_rows_generic(const uint16_t*
     const int row = blockIdx.x;
     const uint16_t* xr = x + static_cast<size_t>(row) * K;
     uint8_t* outr = out + static_cast<size_t>(row) * K;
+    auto value = [&](int k) {
+        const float v = bf16_to_f32(xr[k]);
+        return GELU ? bf16_to_f32(f32_to_bf16(gelu_fwd(v))) : v;
+    };
     float local = 0.0f;
-    for (int k = threadIdx.x; k < K; k += blockDim.x) local = fmaxf(local, fabsf(bf16_to_f32(xr[k])));
+    for (int k = threadIdx.x; k < K; k += blockDim.x) local = fmaxf(local, fabsf(value(k)));
     constexpr float fmax_ = E5M2 ? 57344.0f : 448.0f;
     const float a = fmaxf(block_max(local, sh), 1e-12f);
     const float sc = fmax_ / a;
     if (threadIdx.x == 0) { scale[row] = sc; descale[row] = a / fmax_; }
-    for (int k = threadIdx.x; k < K; k += blockDim.x) outr[k] = cvt1_fp8<E5M2>(bf16_to_f32(xr[k]) * sc);
+    for (int k = threadIdx.x; k < K; k += blockDim.x) outr[k] = cvt1_fp8<E5M2>(value(k) * sc);
 }
 
 // ---- 1x128 groups ------------------------------------------------------------
@@ -642,6 +657,23 @@ int launch_quant(const uint16_t* x, void* out, const float* scale, float* amax, 
     return launch_status();
 }
 
+// per-row quantize: the register-resident forms where the row fits, the two-pass form otherwise
+template <bool E5M2, bool GELU>
+int launch_quant_rows(const uint16_t* d_x, int rows, int K, void* d_out, float* d_scale, float* d_descale, cf_stream_t stream) {
+    if (rows < 0 || K < 0) return CF_ERR_INVALID_ARG;
+    if (rows == 0) return CF_OK;
+    if (!d_scale || !d_descale || (K > 0 && (!d_x || !d_out))) return CF_ERR_INVALID_ARG;
+    auto* o = static_cast<uint8_t*>(d_out);
+    hipStream_t st = as_stream(stream);
+    const bool vec = aligned16(d_x) && aligned16(d_out) && K % kVec == 0 && K > 0;
+    const unsigned grid = ceil_div(rows, kThreads / 64);
+    if (vec && K <= 4 * 1024) k_quant_rows<E5M2, 4, GELU><<<grid, kThreads, 0, st>>>(d_x, rows, K, o, d_scale, d_descale);
+    else if (vec && K <= 16 * 1024) k_quant_rows_block<E5M2, 4, GELU><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);
+    else if (vec && K <= 32 * 1024) k_quant_rows_block<E5M2, 8, GELU><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);
+    else k_quant_rows_generic<E5M2, GELU><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);
+    return launch_status();
+}
+
 }  // namespace
 }  // namespace cf
 
@@ -767,27 +799,13 @@ int cf_fp8_calib_minmax_update(const float* d_amax, float* d_cmin, float* d_cmax
 
 int cf_fp8_quantize_rows(const uint16_t* d_x, int rows, int K, int is_e5m2, void* d_out, float* d_scale,
                          float* d_descale, cf_stream_t stream) {
-    if (rows < 0 || K < 0) return CF_ERR_INVALID_ARG;
-    if (rows == 0) return CF_OK;
-    if (!d_scale || !d_descale || (K > 0 && (!d_x || !d_out))) return CF_ERR_INVALID_ARG;
-    auto* o = static_cast<uint8_t*>(d_out);
-    hipStream_t st = as_stream(stream);
-    const bool vec = aligned16(d_x) && aligned16(d_out) && K % kVec == 0 && K > 0;
-    const unsigned grid = ceil_div(rows, kThreads / 64);
-    if (vec && K <= 4 * 1024) {
-        if (is_e5m2) k_quant_rows<true, 4><<<grid, kThreads, 0, st>>>(d_x, rows, K, o, d_scale, d_descale);
-        else         k_quant_rows<false, 4><<<grid, kThreads, 0, st>>>(d_x, rows, K, o, d_scale, d_descale);
-    } else if (vec && K <= 16 * 1024) {
-        if (is_e5m2) k_quant_rows_block<true, 4><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);
-        else         k_quant_rows_block<false, 4><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);
-    } else if (vec && K <= 32 * 1024) {
-        if (is_e5m2) k_quant_rows_block<true, 8><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);
-        else         k_quant_rows_block<false, 8><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);
-    } else {
-        if (is_e5m2) k_quant_rows_generic<true><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);
-        else         k_quant_rows_generic<false><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);
-    }
-    return launch_status();
+    return is_e5m2 ? launch_quant_rows<true, false>(d_x, rows, K, d_out, d_scale, d_descale, stream)
+                   : launch_quant_rows<false, false>(d_x, rows, K, d_out, d_scale, d_descale, stream);
+}
+
+int cf_gelu_quantize_rows_e4m3(const uint16_t* d_x, int rows, int K, void* d_out, float* d_scale, float* d_descale,
+                               cf_stream_t stream) {
+    return launch_quant_rows<false, true>(d_x, rows, K, d_out, d_scale, d_descale, stream);
 }
 
 int cf_fp8_quantize_block_1x128(const uint16_t* d_x, int rows, int K, void* d_out, float* d_scale,

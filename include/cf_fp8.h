@@ -443,6 +443,33 @@ int cf_moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_fcin_
                                       int H, int Ie, int num_experts, int total_selected_rows,
                                       cf_stream_t stream);
 
+/* gelu_forward (kernels/moe.cu:510-521) followed by the per-token E4M3 quantize of its bf16
+ * output, in one pass: out = e4m3(bf16(gelu(x)) * scale[row]), scale[row] = 448 / max(amax, 1e-12)
+ * over the row of bf16(gelu(x)), descale its inverse (the formula of kernels/fp8.cu:37-39,49).
+ * Bytes and scales equal cf_gelu_forward_bf16 then cf_fp8_quantize_rows. */
+int cf_gelu_quantize_rows_e4m3(const uint16_t* d_x, int rows, int K, void* d_out, float* d_scale,
+                               float* d_descale, cf_stream_t stream);
+
+/* The FP8 expert loop of moe_expert_bank_forward (src/trainer.cu:6886-6934: moe_gather_rows_u8 ->
+ * lt_gemm_fp8_nt fc_in -> gelu_forward -> quantize -> lt_gemm_fp8_nt fc_out ->
+ * moe_scatter_accumulate_rows_bf16, once per expert behind a host synchronisation) for every expert
+ * in one call with no host round trip, on the FP8 matrix cores: same arguments as
+ * cf_moe_grouped_expert_forward_fp8 plus a workspace.  Unlike that function (and like the loop)
+ * the GELU output is rounded to bf16 and re-quantized to E4M3 before fc_out; its scale is per
+ * token row (the loop's per-expert delayed scale needs host-side slot state).  d_offsets must be
+ * the exclusive prefix sum of d_counts and total_selected_rows their sum.  H and Ie multiples of
+ * 128 and at least 256; d_workspace 256-byte aligned, cf_moe_grouped_gelu_workspace_bytes() bytes. */
+int cf_moe_grouped_gelu_workspace_bytes(int rows, int total_selected_rows, int num_experts, int H,
+                                        int Ie, size_t* bytes);
+int cf_moe_grouped_gelu_forward_fp8(const void* d_hidden, const float* d_fcin_descale,
+                                    int fcin_is_e5m2, const float* d_route_weights,
+                                    const int* d_counts, const int* d_offsets,
+                                    const int* d_row_indices, const void* d_fc_in_w,
+                                    const float* d_fc_in_descale, const void* d_fc_out_w,
+                                    const float* d_fc_out_descale, uint16_t* d_mixed, int rows,
+                                    int H, int Ie, int num_experts, int total_selected_rows,
+                                    void* d_workspace, size_t workspace_bytes, cf_stream_t stream);
+
 /* ---- slot state machines (host logic of src/trainer.cu over the entry points above) ------- */
 
 /* One delayed-scaling activation / gradient call site: ActSlot, src/trainer.cu:3247-3279.  The host

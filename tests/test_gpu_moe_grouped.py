@@ -145,7 +145,10 @@ def test_config5_full_size(cf, dev):
     assert np.array_equal(run_fused(cf, b), r["mixed"])
 
 
-@pytest.mark.parametrize("rows,E,k,H,Ie,e5m2", [(90, 4, 2, 96, 72, False), (300, 6, 3, 256, 300, True), (33, 3, 3, 40, 1408, False)])
+@pytest.mark.parametrize("rows,E,k,H,Ie,e5m2", [(90, 4, 2, 96, 72, False), (300, 6, 3, 256, 300, True), (33, 3, 3, 40, 1408, False),
+                                                 # whole MFMA steps (H % 128 == 0, Ie % 64 == 0): the matrix-core form
+                                                 (300, 6, 3, 256, 320, True), (200, 4, 2, 128, 64, False), (1000, 5, 2, 384, 448, False),
+                                                 (70, 3, 3, 2048, 1408, False)])
 def test_grouped_gelu_expert_bank_reference_form(cf, dev, rows, E, k, H, Ie, e5m2):
     """moe_grouped_expert_forward_fp8: per-tensor descales, float GELU intermediate, bf16 CAS accumulate."""
     case(f"grouped gelu bank rows={rows} E={E} k={k} H={H} Ie={Ie} e5m2={e5m2}")
@@ -219,3 +222,219 @@ def test_grouped_gelu_expert_bank_on_the_reference_fixture(cf, dev):
     assert np.abs(got - want).max() < 0.06 * scale
     ref = orc.moe_grouped_expert_forward_fp8_ref(hq, hd, False, route, counts, idx, wiq, wid, woq, wod, np.zeros((rows, H)))
     assert np.all(np.abs(got - ref) <= (E + 1) * 2.0 ** -8 * (np.abs(ref) + scale))
+
+
+# ---- the GELU expert loop on the matrix cores ----------------------------------------------------------------------
+
+@pytest.mark.parametrize("rows,K,off", [(37, 1408, 0), (9, 300, 0), (5, 8192, 0), (3, 20480, 0), (11, 256, 1), (4, 16, 0)])
+def test_gelu_quantize_rows_is_gelu_forward_then_quantize_rows(cf, dev, rows, K, off):
+    """One pass over the projections: bytes and scales equal the two launches it replaces, and equal the oracle's
+    per-row quantize of the GELU values the GPU produced (the GELU itself is pinned to one bf16 ulp elsewhere)."""
+    case(f"gelu + per-row quantize rows={rows} K={K} offset={off}")
+    rng = np.random.default_rng(rows * K)
+    x = orc.bf16_from_f32((2.5 * rng.standard_normal((rows, K))).astype(np.float32))
+    x[0, :] = 0                                                             # an all-zero row: the 1e-12 floor
+    flat = torch.zeros(rows * K + 8, dtype=torch.bfloat16, device=dev)
+    flat[off:off + rows * K] = dev_bf16(x, dev).reshape(-1)
+    dx = flat[off:off + rows * K]
+    q = torch.zeros((rows, K), dtype=torch.uint8, device=dev); s = torch.zeros(rows, device=dev); d = torch.zeros(rows, device=dev)
+    cf.cf_gelu_quantize_rows_e4m3(dx, rows, K, q, s, d, stream())
+    g = torch.zeros(rows * K, dtype=torch.bfloat16, device=dev)
+    cf.cf_gelu_forward_bf16(dx, g, rows * K, stream())
+    q2 = torch.zeros_like(q); s2 = torch.zeros_like(s); d2 = torch.zeros_like(d)
+    cf.cf_fp8_quantize_rows(g, rows, K, 0, q2, s2, d2, stream())
+    torch.cuda.synchronize()
+    assert np.array_equal(host(q), host(q2)) and np.array_equal(host(s), host(s2)) and np.array_equal(host(d), host(d2))
+    wq, ws_, wd_ = orc.quantize_rows(bf16_bits(g).reshape(rows, K))
+    assert np.array_equal(host(q), wq) and np.array_equal(host(s), ws_) and np.array_equal(host(d), wd_)
+
+
+class GeluBank:
+    """Per-tensor-scaled expert bank (the operands moe_grouped_expert_forward_fp8 takes) + routing."""
+
+    def __init__(self, dev, rows, E, k, H, Ie, seed, e5m2=False, zero_expert=None):
+        rng = np.random.default_rng(seed)
+        self.rows, self.E, self.k, self.H, self.Ie, self.e5m2, self.dev = rows, E, k, H, Ie, e5m2, dev
+        logits = rng.standard_normal((rows, E)).astype(np.float32)
+        if zero_expert is not None:
+            logits[:, zero_expert] = -50.0
+        self.rw = orc.moe_topk_route(logits, k)
+        self.counts, self.idx = orc.moe_build_expert_row_lists(self.rw)
+        self.offsets = orc.moe_expert_offsets(self.counts)
+        self.total = int(self.counts.sum())
+
+        def q(x, fmax, sat):
+            s, d = orc.scale_from_amax(np.float32(np.abs(x).max()), fmax)
+            return sat((x * s).astype(np.float32)).reshape(x.shape), np.float32(d)
+        x = rng.standard_normal((rows, H)).astype(np.float32)
+        self.hq, self.hd = q(x, 57344.0, orc.e5m2_satfinite) if e5m2 else q(x, 448.0, orc.e4m3_satfinite)
+        self.wi, self.wid = q((0.05 * rng.standard_normal((E * Ie, H))).astype(np.float32), 448.0, orc.e4m3_satfinite)
+        self.wo, self.wod = q((0.05 * rng.standard_normal((E * H, Ie))).astype(np.float32), 448.0, orc.e4m3_satfinite)
+        self.mixed0 = orc.bf16_from_f32(rng.standard_normal((rows, H)).astype(np.float32))
+        self.d = {n: dev_arr(getattr(self, n), dev) for n in ("rw", "counts", "offsets", "idx", "hq", "wi", "wo")}
+        for n in ("hd", "wid", "wod"):
+            self.d[n] = torch.tensor([getattr(self, n)], dtype=torch.float32, device=dev)
+
+
+def run_gelu_fused(cf, b: GeluBank):
+    import ctypes
+    sz = ctypes.c_size_t(0)
+    assert cf.raw_cf_moe_grouped_gelu_workspace_bytes(b.rows, b.total, b.E, b.H, b.Ie, ctypes.byref(sz)) == 0
+    ws = torch.empty(sz.value + 256, dtype=torch.uint8, device=b.dev)
+    off = (-ws.data_ptr()) % 256
+    mixed = dev_bf16(b.mixed0, b.dev)
+    cf.cf_moe_grouped_gelu_forward_fp8(b.d["hq"], b.d["hd"], int(b.e5m2), b.d["rw"], b.d["counts"], b.d["offsets"], b.d["idx"],
+                                       b.d["wi"], b.d["wid"], b.d["wo"], b.d["wod"], mixed, b.rows, b.H, b.Ie, b.E, b.total,
+                                       ws.data_ptr() + off, sz.value, stream())
+    torch.cuda.synchronize()
+    return bf16_bits(mixed)
+
+
+def run_gelu_stages(cf, b: GeluBank):
+    """The same bank through the public per-stage entry points (E4M3 hidden states), per-tensor descales spread
+    into vectors on the host."""
+    import ctypes
+    dev, E, H, Ie, total = b.dev, b.E, b.H, b.Ie, b.total
+    sz = ctypes.c_size_t(0)
+    assert cf.raw_cf_fp8_grouped_gemm_workspace_bytes(total, E, ctypes.byref(sz)) == 0
+    ws = torch.empty(sz.value, dtype=torch.uint8, device=dev)
+    full = lambda v, n: torch.full((n,), float(v), dtype=torch.float32, device=dev)
+    cidx = torch.full((total,), -1, dtype=torch.int32, device=dev)
+    cf.cf_moe_compact_row_index(b.d["counts"], b.d["offsets"], b.d["idx"], b.rows, E, cidx, stream())
+    act = torch.zeros((total, Ie), dtype=torch.bfloat16, device=dev)
+    cf.cf_fp8_grouped_gemm_nt_bf16_ex(total, Ie, H, E, b.d["counts"], b.d["offsets"], b.d["hq"], b.rows, H, cidx, full(b.hd, b.rows),
+                                      b.d["wi"], full(b.wid, E * Ie), ROW_COL, EPI_NONE, None, None, act, Ie, ws, sz.value, stream())
+    actq = torch.empty((total, Ie), dtype=torch.uint8, device=dev)
+    a_s = torch.empty(total, device=dev); a_d = torch.empty(total, device=dev)
+    cf.cf_gelu_quantize_rows_e4m3(act, total, Ie, actq, a_s, a_d, stream())
+    y = torch.zeros((total, H), dtype=torch.bfloat16, device=dev)
+    cf.cf_fp8_grouped_gemm_nt_bf16_ex(total, H, Ie, E, b.d["counts"], b.d["offsets"], actq, total, Ie, None, a_d,
+                                      b.d["wo"], full(b.wod, E * H), ROW_COL, EPI_NONE, None, None, y, H, ws, sz.value, stream())
+    mixed = dev_bf16(b.mixed0, dev)
+    cf.cf_moe_unpermute_weighted_bf16(mixed, y, b.d["rw"], b.d["counts"], b.d["offsets"], b.d["idx"], b.rows, E, H, stream())
+    torch.cuda.synchronize()
+    return dict(act=bf16_bits(act), actq=host(actq), a_d=host(a_d), y=bf16_bits(y), mixed=bf16_bits(mixed))
+
+
+def check_gelu_stages(b: GeluBank, r, experts=None, sample=None):
+    E, H, Ie = b.E, b.H, b.Ie
+    mixed = b.mixed0
+    for e in range(E):
+        n, o = int(b.counts[e]), int(b.offsets[e])
+        mixed = orc.moe_scatter_accumulate(mixed, r["y"][o:o + n], b.rw, b.idx[e, :n], e)
+    assert np.array_equal(r["mixed"], mixed)                                   # weighted unpermute: bit-exact
+    for e in (range(E) if experts is None else experts):
+        n, o = int(b.counts[e]), int(b.offsets[e])
+        if n == 0:
+            continue
+        sel = np.arange(n) if sample is None or n <= sample else np.sort(np.random.default_rng(e).choice(n, sample, replace=False))
+        rows = b.idx[e, :n][sel]
+        ref, absdot = orc.gemm_nt_ref(b.hq[rows], b.wi[e * Ie:(e + 1) * Ie], [b.hd], [b.wid], a_e5m2=b.e5m2, scale_mode=0)
+        orc.assert_gemm_close(orc.bf16_to_f32(r["act"][o:o + n][sel]).astype(np.float64), ref, absdot, what=f"fc_in expert {e}")
+        yref, yabs = orc.gemm_nt_ref(r["actq"][o:o + n][sel], b.wo[e * H:(e + 1) * H], r["a_d"][o:o + n][sel],
+                                     np.full(H, b.wod, np.float32), scale_mode=1)
+        orc.assert_gemm_close(orc.bf16_to_f32(r["y"][o:o + n][sel]).astype(np.float64), yref, yabs, what=f"fc_out expert {e}")
+
+
+def gelu_loop_ref(b: GeluBank):
+    """The reference's expert loop restated on the host from the oracle's pieces (bf16 roundings where the loop has
+    them): returns mixed as bf16 bits."""
+    mixed = b.mixed0
+    for e in range(b.E):
+        n = int(b.counts[e])
+        if n == 0:
+            continue
+        rows = b.idx[e, :n]
+        a, _ = orc.gemm_nt_ref(b.hq[rows], b.wi[e * b.Ie:(e + 1) * b.Ie], [b.hd], [b.wid], a_e5m2=b.e5m2, scale_mode=0, want_abs=False)
+        g = orc.gelu_forward(orc.bf16_from_f32(a.astype(np.float32)))
+        q, _, d = orc.quantize_rows(g)
+        y, _ = orc.gemm_nt_ref(q, b.wo[e * b.H:(e + 1) * b.H], d, np.full(b.H, b.wod, np.float32), scale_mode=1, want_abs=False)
+        mixed = orc.moe_scatter_accumulate(mixed, orc.bf16_from_f32(y.astype(np.float32)), b.rw, rows, e)
+    return mixed
+
+
+@pytest.mark.parametrize("rows,E,k,H,Ie,zero", [(600, 5, 2, 256, 384, None), (300, 4, 2, 256, 256, 2), (40, 8, 3, 384, 256, None)])
+def test_grouped_gelu_bank_on_the_matrix_cores(cf, dev, rows, E, k, H, Ie, zero):
+    case(f"grouped gelu bank (mfma) rows={rows} E={E} k={k} H={H} Ie={Ie}")
+    b = GeluBank(dev, rows, E, k, H, Ie, seed=rows + Ie, zero_expert=zero)
+    r = run_gelu_stages(cf, b)
+    check_gelu_stages(b, r)
+    got = run_gelu_fused(cf, b)
+    assert np.array_equal(got, r["mixed"])                                     # the one-call form is the same computation
+    # against the loop restated from the oracle end to end: a GELU value one bf16 ulp apart can move a quantized
+    # byte, so this is the GEMM bar on the sum rather than bit equality
+    want = orc.bf16_to_f32(gelu_loop_ref(b)).astype(np.float64)
+    g = orc.bf16_to_f32(got).astype(np.float64)
+    assert np.sqrt(((g - want) ** 2).sum() / (want ** 2).sum()) <= 4e-3
+    # and against moe_grouped_expert_forward_fp8's semantics (GELU output kept in fp32): apart by the E4M3
+    # rounding of the activations, relative 2^-4 / sqrt(3) per element
+    start = orc.bf16_to_f32(b.mixed0).astype(np.float64)
+    ref = orc.moe_grouped_expert_forward_fp8_ref(b.hq, b.hd, b.e5m2, b.rw, b.counts, b.idx, b.wi.reshape(E, Ie, H), b.wid,
+                                                 b.wo.reshape(E, H, Ie), b.wod, start)
+    assert np.sqrt(((g - ref) ** 2).sum() / ((ref - start) ** 2).sum()) <= 0.06
+    untouched = ~(b.rw > 0).any(axis=1)
+    assert np.array_equal(got[untouched], b.mixed0[untouched])
+
+
+def test_grouped_gelu_bank_e5m2_hidden_states(cf, dev):
+    case("grouped gelu bank (mfma), E5M2 hidden states")
+    b = GeluBank(dev, 500, 4, 2, 256, 384, seed=77, e5m2=True)
+    got = orc.bf16_to_f32(run_gelu_fused(cf, b)).astype(np.float64)
+    want = orc.bf16_to_f32(gelu_loop_ref(b)).astype(np.float64)
+    assert np.sqrt(((got - want) ** 2).sum() / (want ** 2).sum()) <= 4e-3
+    assert np.all(np.abs(got - want) <= (b.k + 1) * 2.0 ** -7 * (np.abs(want) + np.abs(want).mean()))
+
+
+def test_grouped_gelu_bank_config5_size(cf, dev):
+    """16384 tokens, hidden 2048, 64 experts, top-6, expert width 1408, per-tensor scales."""
+    case("grouped gelu bank (mfma), config 5 size")
+    b = GeluBank(dev, 16384, 64, 6, 2048, 1408, seed=6)
+    assert b.total == 98304
+    r = run_gelu_stages(cf, b)
+    check_gelu_stages(b, r, experts=[0, 40, 63], sample=24)
+    assert np.array_equal(run_gelu_fused(cf, b), r["mixed"])
+
+
+def test_grouped_gelu_bank_argument_errors(cf, dev):
+    case("grouped gelu bank argument checks")
+    import ctypes
+    sz = ctypes.c_size_t(0)
+    assert cf.raw_cf_moe_grouped_gelu_workspace_bytes(16, 32, 4, 256, 256, None) != 0
+    assert cf.raw_cf_moe_grouped_gelu_workspace_bytes(-1, 32, 4, 256, 256, ctypes.byref(sz)) != 0
+    b = GeluBank(dev, 64, 4, 2, 256, 256, seed=3)
+    assert cf.raw_cf_moe_grouped_gelu_workspace_bytes(b.rows, b.total, b.E, b.H, b.Ie, ctypes.byref(sz)) == 0
+    ws = torch.empty(sz.value + 256, dtype=torch.uint8, device=dev)
+    p = ws.data_ptr() + (-ws.data_ptr()) % 256
+    mixed = dev_bf16(b.mixed0, dev)
+    args = lambda wsp, nbytes, H=b.H: (b.d["hq"].data_ptr(), b.d["hd"].data_ptr(), 0, b.d["rw"].data_ptr(), b.d["counts"].data_ptr(),
+                                       b.d["offsets"].data_ptr(), b.d["idx"].data_ptr(), b.d["wi"].data_ptr(), b.d["wid"].data_ptr(),
+                                       b.d["wo"].data_ptr(), b.d["wod"].data_ptr(), mixed.data_ptr(), b.rows, H, b.Ie, b.E, b.total,
+                                       wsp, nbytes, None)
+    assert cf.raw_cf_moe_grouped_gelu_forward_fp8(*args(p, sz.value - 1)) == -1            # workspace too small
+    assert cf.raw_cf_moe_grouped_gelu_forward_fp8(*args(p + 16, sz.value)) == -1           # workspace misaligned
+    assert cf.raw_cf_moe_grouped_gelu_forward_fp8(*args(None, sz.value)) == -1
+    assert cf.raw_cf_moe_grouped_gelu_forward_fp8(*args(p, sz.value, H=200)) == -2         # K not a multiple of 128
+    torch.cuda.synchronize()
+    assert np.array_equal(bf16_bits(mixed), b.mixed0)                                      # nothing ran
+
+
+def test_grouped_gelu_expert_bank_reference_form_config5_size(cf, dev):
+    """moe_grouped_expert_forward_fp8 at 16384 tokens, hidden 2048, 64 experts, top-6, width 1408: a sample of token rows
+    against the double reference of exactly those rows."""
+    case("grouped gelu bank, reference form, config 5 size")
+    b = GeluBank(dev, 16384, 64, 6, 2048, 1408, seed=8)
+    mixed = dev_bf16(b.mixed0, dev)
+    cf.cf_moe_grouped_expert_forward_fp8(b.d["hq"], b.d["hd"], 0, b.d["rw"], b.d["counts"], None, b.d["idx"], b.d["wi"], b.d["wid"],
+                                         b.d["wo"], b.d["wod"], mixed, b.rows, b.H, b.Ie, b.E, b.total, stream())
+    torch.cuda.synchronize()
+    sel = np.sort(np.random.default_rng(1).choice(b.rows, 40, replace=False))
+    sel[0], sel[-1] = 0, b.rows - 1
+    rw = np.ascontiguousarray(b.rw[sel])
+    counts, idx = orc.moe_build_expert_row_lists(rw)
+    start = orc.bf16_to_f32(b.mixed0[sel]).astype(np.float64)
+    ref = orc.moe_grouped_expert_forward_fp8_ref(b.hq[sel], b.hd, False, rw, counts, idx, b.wi.reshape(b.E, b.Ie, b.H), b.wid,
+                                                 b.wo.reshape(b.E, b.H, b.Ie), b.wod, start)
+    got = orc.bf16_to_f32(bf16_bits(mixed)[sel]).astype(np.float64)
+    assert np.sqrt(((got - ref) ** 2).sum() / (ref ** 2).sum()) <= 4e-3
+    typical = np.sqrt(((ref - start) ** 2).mean())
+    assert np.all(np.abs(got - ref) <= (b.k + 1) * 2.0 ** -8 * (np.abs(start) + np.abs(ref) + 2.0 * typical))

@@ -447,8 +447,8 @@ __global__ __launch_bounds__(kThreads) void k_unpermute(uint16_t* __restrict__ m
 // dequantised with per-tensor descales, the exact-erf GELU output stays in fp32 (it is not
 // re-quantised), products are accumulated in fp32, and the result is added to the bf16 output with a
 // 32-bit compare-and-swap on the word holding it.  One workgroup per (expert, tile of 16 rows);
-// workgroups past an expert's row count leave at once.  This is the correctness form the reference
-// keeps beside its tensor-core path; the fast path for expert banks is the grouped SwiGLU pipeline.
+// workgroups past an expert's row count leave at once.  This fp32-FMA form follows the reference
+// kernel's loop and takes any shape; shapes made of whole MFMA steps go to k_grouped_gelu_fp8_mfma below.
 constexpr int kGeluRows = 16;
 constexpr int kGeluChunk = 128;
 
@@ -548,8 +548,9 @@ __global__ __launch_bounds__(kThreads) void k_grouped_gelu_fp8(const uint8_t* __
 //   GELU    in fp32 on the accumulator, split into a bf16 head and a bf16 remainder (together 16 significand bits,
 //           relative error 2^-17) and parked in LDS.
 //   fc_out  v_mfma_f32_16x16x32_bf16 twice per step (head and remainder) against the E4M3 weights widened to bf16,
-//           which is exact.  A lane fetches 16 weight bytes at once and uses them as two k-blocks of 8; the activation
-//           reads follow the same order, and a sum does not care which k a lane group holds.
+//           which is exact.  A lane fetches 32 weight bytes at once (the four lane groups cover a whole 128-byte line
+//           of a weight row) and uses them as four k-blocks of 8; the activation reads follow the same order, and a
+//           sum does not care which k a lane group holds.
 // Weights go to the "A" side, so a lane ends with 4 neighbouring output columns of one token row.
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
@@ -563,31 +564,42 @@ __device__ __forceinline__ v8bf e4m3x8_to_bf16(uint32_t a, uint32_t b) {
     return __builtin_bit_cast(v8bf, w);
 }
 
-// two neighbouring bf16 values += (v0, v1), one rounding each, by compare-and-swap on their word
-__device__ __forceinline__ void atomic_add_bf16x2(unsigned* word, float v0, float v1) {
-    unsigned old = *word;
+// four neighbouring bf16 values += v[0..3], one rounding each, by a 64-bit compare-and-swap; `old` is a value read
+// from the address earlier (a stale one only costs a second round)
+__device__ __forceinline__ void atomic_add_bf16x4(unsigned long long* quad, unsigned long long old, const float* v) {
     while (true) {
-        const unsigned assumed = old;
-        const unsigned next = pack_bf16x2(bf16_lo(assumed) + v0, bf16_hi(assumed) + v1);
-        old = atomicCAS(word, assumed, next);
+        const unsigned long long assumed = old;
+        const unsigned lo = static_cast<unsigned>(assumed), hi = static_cast<unsigned>(assumed >> 32);
+        const unsigned long long next = static_cast<unsigned long long>(pack_bf16x2(bf16_lo(lo) + v[0], bf16_hi(lo) + v[1])) |
+                                        (static_cast<unsigned long long>(pack_bf16x2(bf16_lo(hi) + v[2], bf16_hi(hi) + v[3])) << 32);
+        old = atomicCAS(quad, assumed, next);
         if (old == assumed) return;
     }
 }
 
+constexpr int kMfmaThreads = 512;      // eight wavefronts: two per SIMD, so one's weight fetches hide behind the other's MFMAs
+constexpr int kXcdCount = 8;
+constexpr int kMfmaDepth = 4;          // weight fetches a wavefront keeps in flight ahead of its MFMAs
+
 template <bool E5M2>
-__global__ __launch_bounds__(kThreads) void k_grouped_gelu_fp8_mfma(const uint8_t* __restrict__ hidden, const float* __restrict__ fcin_descale,
-                                                                    const float* __restrict__ route_weights, const int* __restrict__ counts,
-                                                                    const int* __restrict__ row_indices, const uint8_t* __restrict__ fc_in_w,
-                                                                    const float* __restrict__ fc_in_descale, const uint8_t* __restrict__ fc_out_w,
-                                                                    const float* __restrict__ fc_out_descale, uint16_t* __restrict__ mixed,
-                                                                    int rows, int H, int Ie, int E, int tiles_per_expert) {
+__global__ __launch_bounds__(kMfmaThreads) void k_grouped_gelu_fp8_mfma(const uint8_t* __restrict__ hidden, const float* __restrict__ fcin_descale,
+                                                                        const float* __restrict__ route_weights, const int* __restrict__ counts,
+                                                                        const int* __restrict__ row_indices, const uint8_t* __restrict__ fc_in_w,
+                                                                        const float* __restrict__ fc_in_descale, const uint8_t* __restrict__ fc_out_w,
+                                                                        const float* __restrict__ fc_out_descale, uint16_t* __restrict__ mixed,
+                                                                        int rows, int H, int Ie, int E, int tiles_per_expert) {
     extern __shared__ __align__(16) uint8_t smem[];
+    constexpr int kWaves = kMfmaThreads / 64;
     const int hs = H + 16;                          // hidden row stride in bytes: neighbouring rows 16 bytes apart in the banks
     const int as = Ie + 8;                          // activation row stride in elements, likewise
     uint8_t* sh_hidden = smem;                                                        // [16][hs] fp8
     uint16_t* sh_hi = reinterpret_cast<uint16_t*>(smem + kMfmaRows * hs);             // [16][as] bf16 head of gelu
     uint16_t* sh_lo = sh_hi + kMfmaRows * as;                                         // [16][as] bf16 remainder
-    const int e = blockIdx.x / tiles_per_expert, tile = blockIdx.x % tiles_per_expert;
+    // workgroups go round the 8 XCDs in turn: give each XCD whole experts, so one expert's weights (re-read by every
+    // 16-row tile) are served by that XCD's L2
+    const int xcd = blockIdx.x % kXcdCount, slot = blockIdx.x / kXcdCount;
+    const int e = (slot / tiles_per_expert) * kXcdCount + xcd, tile = slot % tiles_per_expert;
+    if (e >= E) return;
     const int first = tile * kMfmaRows, n_active = counts[e];
     if (first >= n_active) return;
     const int n_rows = min(kMfmaRows, n_active - first);
@@ -598,7 +610,7 @@ __global__ __launch_bounds__(kThreads) void k_grouped_gelu_fp8_mfma(const uint8_
 
     // the tile's hidden rows (rows past the list's end repeat its last one; their results are dropped)
     const int vec_per_row = H / 16;
-    for (int i = threadIdx.x; i < kMfmaRows * vec_per_row; i += kThreads) {
+    for (int i = threadIdx.x; i < kMfmaRows * vec_per_row; i += kMfmaThreads) {
         const int r = i / vec_per_row, c = i % vec_per_row;
         const int src = my_rows[min(r, n_rows - 1)];
         *reinterpret_cast<uint4*>(sh_hidden + r * hs + c * 16) =
@@ -607,16 +619,33 @@ __global__ __launch_bounds__(kThreads) void k_grouped_gelu_fp8_mfma(const uint8_
     __syncthreads();
 
     const float s_in = *fcin_descale * *fc_in_descale;
-    for (int n0 = wave * 16; n0 < Ie; n0 += 4 * 16) {
+    const int in_steps = H / 128;
+    for (int n0 = wave * 16; n0 < Ie; n0 += kWaves * 16) {
         v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
         const uint8_t* wr = w_in + static_cast<size_t>(n0 + t) * H + 32 * g;
         const uint8_t* hr = sh_hidden + t * hs + 32 * g;
-        for (int k0 = 0; k0 < H; k0 += 128) {
-            const uint4 w0 = *reinterpret_cast<const uint4*>(wr + k0), w1 = *reinterpret_cast<const uint4*>(wr + k0 + 16);
-            const uint4 x0 = *reinterpret_cast<const uint4*>(hr + k0), x1 = *reinterpret_cast<const uint4*>(hr + k0 + 16);
-            const v8i a = {(int)w0.x, (int)w0.y, (int)w0.z, (int)w0.w, (int)w1.x, (int)w1.y, (int)w1.z, (int)w1.w};
-            const v8i b = {(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w, (int)x1.x, (int)x1.y, (int)x1.z, (int)x1.w};
-            acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc, 0 /* weights E4M3 */, E5M2 ? 1 : 0, 0, 0, 0, 0);
+        uint4 w0[kMfmaDepth], w1[kMfmaDepth];
+#pragma unroll
+        for (int j = 0; j < kMfmaDepth; ++j)
+            if (j < in_steps) {
+                w0[j] = *reinterpret_cast<const uint4*>(wr + j * 128);
+                w1[j] = *reinterpret_cast<const uint4*>(wr + j * 128 + 16);
+            }
+        for (int s0 = 0; s0 < in_steps; s0 += kMfmaDepth) {
+#pragma unroll
+            for (int j = 0; j < kMfmaDepth; ++j) {
+                const int st = s0 + j;
+                if (st < in_steps) {
+                    const uint4 x0 = *reinterpret_cast<const uint4*>(hr + st * 128), x1 = *reinterpret_cast<const uint4*>(hr + st * 128 + 16);
+                    const v8i a = {(int)w0[j].x, (int)w0[j].y, (int)w0[j].z, (int)w0[j].w, (int)w1[j].x, (int)w1[j].y, (int)w1[j].z, (int)w1[j].w};
+                    const v8i b = {(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w, (int)x1.x, (int)x1.y, (int)x1.z, (int)x1.w};
+                    if (st + kMfmaDepth < in_steps) {
+                        w0[j] = *reinterpret_cast<const uint4*>(wr + (st + kMfmaDepth) * 128);
+                        w1[j] = *reinterpret_cast<const uint4*>(wr + (st + kMfmaDepth) * 128 + 16);
+                    }
+                    acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc, 0 /* weights E4M3 */, E5M2 ? 1 : 0, 0, 0, 0, 0);
+                }
+            }
         }
         // this lane: token row t, columns n0 + 4g .. + 3
         uint32_t hb[4], lb[4];
@@ -634,30 +663,62 @@ __global__ __launch_bounds__(kThreads) void k_grouped_gelu_fp8_mfma(const uint8_
     __syncthreads();
 
     const float d_wout = *fc_out_descale;
-    for (int h0 = wave * 16; h0 < H; h0 += 4 * 16) {
+    const int out_steps = Ie / 128;                 // whole 128-byte lines of a weight row; Ie % 128 == 64 leaves half a line
+    const int out_tail = out_steps * 128;
+    const bool live = t < n_rows;
+    const int row = live ? my_rows[t] : 0;
+    const float rw = live ? route_weights[static_cast<size_t>(row) * E + e] : 0.0f;
+    for (int h0 = wave * 16; h0 < H; h0 += kWaves * 16) {
         v4f acc_hi = {0.0f, 0.0f, 0.0f, 0.0f}, acc_lo = {0.0f, 0.0f, 0.0f, 0.0f};
-        const uint8_t* wr = w_out + static_cast<size_t>(h0 + t) * Ie + 16 * g;
-        const uint16_t* ah = sh_hi + t * as + 16 * g;
-        const uint16_t* al = sh_lo + t * as + 16 * g;
-        for (int k0 = 0; k0 < Ie; k0 += 64) {
-            const uint4 w = *reinterpret_cast<const uint4*>(wr + k0);              // k0 + 16g .. + 15
-            const v8bf wa = e4m3x8_to_bf16(w.x, w.y), wb = e4m3x8_to_bf16(w.z, w.w);
-            const v8bf ha = *reinterpret_cast<const v8bf*>(ah + k0), hb = *reinterpret_cast<const v8bf*>(ah + k0 + 8);
-            const v8bf la = *reinterpret_cast<const v8bf*>(al + k0), lb = *reinterpret_cast<const v8bf*>(al + k0 + 8);
-            acc_hi = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, ha, acc_hi, 0, 0, 0);
-            acc_lo = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, la, acc_lo, 0, 0, 0);
-            acc_hi = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb, hb, acc_hi, 0, 0, 0);
-            acc_lo = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb, lb, acc_lo, 0, 0, 0);
+        // the four output values this lane will add to, fetched now so the read is not waited for after the MFMAs
+        auto* quad = reinterpret_cast<unsigned long long*>(mixed + static_cast<size_t>(row) * H + h0 + 4 * g);
+        const unsigned long long before = live ? __builtin_nontemporal_load(quad) : 0ull;
+        const uint8_t* wrow = w_out + static_cast<size_t>(h0 + t) * Ie;
+        const uint8_t* wr = wrow + 32 * g;                                          // step s: k = 128 s + 32 g .. + 31
+        const uint16_t* ah = sh_hi + t * as;
+        const uint16_t* al = sh_lo + t * as;
+        // 8 weights of this lane's k run against the head and the remainder of the same 8 activations
+        auto mm = [&](uint32_t x, uint32_t y, int k) {
+            const v8bf wv = e4m3x8_to_bf16(x, y);
+            acc_hi = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, *reinterpret_cast<const v8bf*>(ah + k), acc_hi, 0, 0, 0);
+            acc_lo = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, *reinterpret_cast<const v8bf*>(al + k), acc_lo, 0, 0, 0);
+        };
+        uint4 wa[kMfmaDepth], wb[kMfmaDepth];
+#pragma unroll
+        for (int j = 0; j < kMfmaDepth; ++j)
+            if (j < out_steps) {
+                wa[j] = *reinterpret_cast<const uint4*>(wr + j * 128);
+                wb[j] = *reinterpret_cast<const uint4*>(wr + j * 128 + 16);
+            }
+        uint4 wt = {0u, 0u, 0u, 0u};
+        if (Ie & 64) wt = *reinterpret_cast<const uint4*>(wrow + out_tail + 16 * g);  // half line: k = tail + 16 g .. + 15
+        for (int s0 = 0; s0 < out_steps; s0 += kMfmaDepth) {
+#pragma unroll
+            for (int j = 0; j < kMfmaDepth; ++j) {
+                const int st = s0 + j;
+                if (st < out_steps) {
+                    const uint4 ca = wa[j], cb = wb[j];
+                    if (st + kMfmaDepth < out_steps) {
+                        wa[j] = *reinterpret_cast<const uint4*>(wr + (st + kMfmaDepth) * 128);
+                        wb[j] = *reinterpret_cast<const uint4*>(wr + (st + kMfmaDepth) * 128 + 16);
+                    }
+                    const int k = st * 128 + 32 * g;
+                    mm(ca.x, ca.y, k);
+                    mm(ca.z, ca.w, k + 8);
+                    mm(cb.x, cb.y, k + 16);
+                    mm(cb.z, cb.w, k + 24);
+                }
+            }
         }
-        if (t < n_rows) {
-            const int row = my_rows[t];
-            const float rw = route_weights[static_cast<size_t>(row) * E + e];
+        if (Ie & 64) {
+            mm(wt.x, wt.y, out_tail + 16 * g);
+            mm(wt.z, wt.w, out_tail + 16 * g + 8);
+        }
+        if (live) {
             float v[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) v[r] = rw * ((acc_hi[r] + acc_lo[r]) * d_wout);
-            auto* word = reinterpret_cast<unsigned*>(mixed + static_cast<size_t>(row) * H + h0 + 4 * g);
-            atomic_add_bf16x2(word, v[0], v[1]);
-            atomic_add_bf16x2(word + 1, v[2], v[3]);
+            atomic_add_bf16x4(quad, before, v);
         }
     }
 }
@@ -1040,7 +1101,7 @@ int cf_moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_fcin_
     // the matrix-core form where the shapes are whole MFMA steps and its tile fits the LDS
     const size_t smem_mfma = static_cast<size_t>(kMfmaRows) * (H + 16) + 4u * kMfmaRows * (static_cast<size_t>(Ie) + 8);
     if (H % 128 == 0 && Ie % 64 == 0 && smem_mfma <= 160 * 1024 && aligned16(d_hidden) && aligned16(d_fc_in_w) &&
-        aligned16(d_fc_out_w) && (reinterpret_cast<uintptr_t>(d_mixed) & 3u) == 0) {
+        aligned16(d_fc_out_w) && (reinterpret_cast<uintptr_t>(d_mixed) & 7u) == 0) {
         static std::once_flag once_mfma;
         static hipError_t err_mfma = hipSuccess;
         std::call_once(once_mfma, [] {
@@ -1053,7 +1114,7 @@ int cf_moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_fcin_
         if (err_mfma != hipSuccess) return static_cast<int>(err_mfma);
         const int tiles = (rows + kMfmaRows - 1) / kMfmaRows;
         auto launch = [&](auto kernel) {
-            kernel<<<num_experts * tiles, kThreads, smem_mfma, as_stream(stream)>>>(
+            kernel<<<kXcdCount * ((num_experts + kXcdCount - 1) / kXcdCount) * tiles, kMfmaThreads, smem_mfma, as_stream(stream)>>>(
                 static_cast<const uint8_t*>(d_hidden), d_fcin_descale, d_route_weights, d_counts, d_row_indices,
                 static_cast<const uint8_t*>(d_fc_in_w), d_fc_in_descale, static_cast<const uint8_t*>(d_fc_out_w), d_fc_out_descale,
                 d_mixed, rows, H, Ie, num_experts, tiles);

@@ -252,8 +252,8 @@ def main():
          lambda: cf.cf_moe_grouped_swiglu_forward_fp8(hq, hd, rw, counts, offs, idx, wg, wgd, wu, wud, wd, wdd, mixed, T, H, Ie, E,
                                                       total, ws2, sz2.value, st))
 
-    # the GELU expert loop (per-tensor descales): one call on the matrix cores, and the fp32 form with the
-    # reference kernel's semantics (moe_grouped_expert_forward_fp8) on the same operands
+    # the GELU expert loop (per-tensor descales): the one-call bank that re-quantizes the activations, and
+    # moe_grouped_expert_forward_fp8's contract (GELU output kept beyond bf16, 16-row tiles) on the same operands
     one = torch.full((1,), 0.01, device=dev)
     sz3 = ctypes.c_size_t(0)
     cf.raw_cf_moe_grouped_gelu_workspace_bytes(T, total, E, H, Ie, ctypes.byref(sz3))
@@ -261,11 +261,11 @@ def main():
     gq = u8(total, Ie); gs = f32(total); gd = f32(total)
     hbm("gelu_quantize_rows_e4m3 (gelu_forward + per-token quantize)", f"{total}x{Ie}", 3.0 * total * Ie,
         lambda: cf.cf_gelu_quantize_rows_e4m3(act, total, Ie, gq, gs, gd, st))
-    mfma("grouped GELU expert bank, whole pipeline, FP8 MFMA", f"T={T} E={E} k={k}", 4.0 * total * Ie * H,
+    mfma("grouped GELU expert bank, whole pipeline (re-quantizing)", f"T={T} E={E} k={k}", 4.0 * total * Ie * H,
          lambda: cf.cf_moe_grouped_gelu_forward_fp8(hq, one, 0, rw, counts, offs, idx, wg, one, wd, one, mixed, T, H, Ie, E, total,
                                                     ws3, sz3.value, st))
-    iters, args.iters = args.iters, 2
-    mfma("grouped GELU expert bank, reference form (fp32 FMA, 16-row tiles)", f"T={T} E={E} k={k}", 4.0 * total * Ie * H,
+    iters, args.iters = args.iters, 5
+    mfma("moe_grouped_expert_forward_fp8 form (fp32 GELU kept, MFMA, 16-row tiles)", f"T={T} E={E} k={k}", 4.0 * total * Ie * H,
          lambda: cf.cf_moe_grouped_expert_forward_fp8(hq, one, 0, rw, counts, offs, idx, wg, one, wd, one, mixed, T, H, Ie, E, total, st))
     args.iters = iters
     del ws3, gq

@@ -24,6 +24,7 @@ FP8_PEAK = 5000.0      # TFLOP/s
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--iters", type=int, default=20)
+    ap.add_argument("--only", default="", help="time only the rows whose name contains this text (for profiler runs)")
     args = ap.parse_args()
     import torch
     sys.path.insert(0, str(ROOT))
@@ -68,11 +69,17 @@ def main():
     print(f"{'kernel':<64} {'shape':<26} {'us':>9} {'rate':>14} {'of peak':>8}")
 
     def hbm(name, shape, nbytes, fn):
+        if args.only not in name:
+            fn()                         # later rows use what this one leaves behind
+            return
         t = timed(fn)
         gbps = nbytes / t / 1e9
         print(f"{name:<64} {shape:<26} {t * 1e6:9.1f} {gbps:9.0f} GB/s {100 * gbps / HBM_PEAK:7.1f}%", flush=True)
 
     def mfma(name, shape, flop, fn):
+        if args.only not in name:
+            fn()                         # later rows use what this one leaves behind
+            return
         t = timed(fn)
         tf = flop / t / 1e12
         print(f"{name:<64} {shape:<26} {t * 1e6:9.1f} {tf:7.0f} TFLOP/s {100 * tf / FP8_PEAK:7.1f}%", flush=True)

@@ -559,7 +559,8 @@ constexpr int kMfmaRows = 16;
 __device__ __forceinline__ v8bf e4m3x8_to_bf16(uint32_t a, uint32_t b) {
     const f32x2_t p0 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(a), false), p1 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(a), true);
     const f32x2_t p2 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(b), false), p3 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(b), true);
-    auto pair = [](f32x2_t p) { return (__float_as_uint(p[0]) >> 16) | (__float_as_uint(p[1]) & 0xffff0000u); };
+    // the upper halves of the two floats, side by side (bytes 2,3 of the first, then 2,3 of the second)
+    auto pair = [](f32x2_t p) { return __builtin_amdgcn_perm(__float_as_uint(p[1]), __float_as_uint(p[0]), 0x07060302u); };
     const v4u w = {pair(p0), pair(p1), pair(p2), pair(p3)};
     return __builtin_bit_cast(v8bf, w);
 }

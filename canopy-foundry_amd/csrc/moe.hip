@@ -580,6 +580,8 @@ __device__ __forceinline__ void atomic_add_bf16x4(unsigned long long* quad, unsi
 
 constexpr int kMfmaThreads = 512;      // eight wavefronts: two per SIMD, so one's weight fetches hide behind the other's MFMAs
 constexpr int kXcdCount = 8;
+constexpr int kMfmaOutDepth = 4;       // the same per output block in fc_out, which carries kMfmaBlocks of them
+constexpr int kMfmaBlocks = 2;         // output blocks a wavefront carries through one pass over k
 constexpr int kMfmaDepth = 4;          // weight fetches a wavefront keeps in flight ahead of its MFMAs
 
 template <bool E5M2>
@@ -669,57 +671,82 @@ __global__ __launch_bounds__(kMfmaThreads) void k_grouped_gelu_fp8_mfma(const ui
     const bool live = t < n_rows;
     const int row = live ? my_rows[t] : 0;
     const float rw = live ? route_weights[static_cast<size_t>(row) * E + e] : 0.0f;
-    for (int h0 = wave * 16; h0 < H; h0 += kWaves * 16) {
-        v4f acc_hi = {0.0f, 0.0f, 0.0f, 0.0f}, acc_lo = {0.0f, 0.0f, 0.0f, 0.0f};
-        // the four output values this lane will add to, fetched now so the read is not waited for after the MFMAs
-        auto* quad = reinterpret_cast<unsigned long long*>(mixed + static_cast<size_t>(row) * H + h0 + 4 * g);
-        const unsigned long long before = live ? __builtin_nontemporal_load(quad) : 0ull;
-        const uint8_t* wrow = w_out + static_cast<size_t>(h0 + t) * Ie;
-        const uint8_t* wr = wrow + 32 * g;                                          // step s: k = 128 s + 32 g .. + 31
-        const uint16_t* ah = sh_hi + t * as;
-        const uint16_t* al = sh_lo + t * as;
-        // 8 weights of this lane's k run against the head and the remainder of the same 8 activations
-        auto mm = [&](uint32_t x, uint32_t y, int k) {
-            const v8bf wv = e4m3x8_to_bf16(x, y);
-            acc_hi = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, *reinterpret_cast<const v8bf*>(ah + k), acc_hi, 0, 0, 0);
-            acc_lo = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, *reinterpret_cast<const v8bf*>(al + k), acc_lo, 0, 0, 0);
-        };
-        uint4 wa[kMfmaDepth], wb[kMfmaDepth];
+    const uint16_t* ah = sh_hi + t * as;
+    const uint16_t* al = sh_lo + t * as;
+    // kMfmaBlocks output blocks per pass share every activation read from LDS (the LDS port, not the MFMA, is what a
+    // pass with one block waits for).  A block past the end repeats the last one and is not written.
+    for (int h0 = wave * 16; h0 < H; h0 += kWaves * 16 * kMfmaBlocks) {
+        v4f acc_hi[kMfmaBlocks], acc_lo[kMfmaBlocks];
+        const uint8_t* wrow[kMfmaBlocks];
+        unsigned long long* quad[kMfmaBlocks];
+        unsigned long long before[kMfmaBlocks];
+        uint4 wa[kMfmaBlocks][kMfmaOutDepth], wb[kMfmaBlocks][kMfmaOutDepth], wt[kMfmaBlocks];
 #pragma unroll
-        for (int j = 0; j < kMfmaDepth; ++j)
-            if (j < out_steps) {
-                wa[j] = *reinterpret_cast<const uint4*>(wr + j * 128);
-                wb[j] = *reinterpret_cast<const uint4*>(wr + j * 128 + 16);
+        for (int b = 0; b < kMfmaBlocks; ++b) {
+            const int hb = min(h0 + b * kWaves * 16, H - 16);
+            acc_hi[b] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+            acc_lo[b] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+            // the four output values this lane will add to, fetched now so the read is not waited for after the MFMAs
+            quad[b] = reinterpret_cast<unsigned long long*>(mixed + static_cast<size_t>(row) * H + hb + 4 * g);
+            before[b] = live ? __builtin_nontemporal_load(quad[b]) : 0ull;
+            wrow[b] = w_out + static_cast<size_t>(hb + t) * Ie;
+#pragma unroll
+            for (int j = 0; j < kMfmaOutDepth; ++j)
+                if (j < out_steps) {                                                // step s: k = 128 s + 32 g .. + 31
+                    wa[b][j] = *reinterpret_cast<const uint4*>(wrow[b] + 32 * g + j * 128);
+                    wb[b][j] = *reinterpret_cast<const uint4*>(wrow[b] + 32 * g + j * 128 + 16);
+                }
+            wt[b] = make_uint4(0u, 0u, 0u, 0u);
+            if (Ie & 64) wt[b] = *reinterpret_cast<const uint4*>(wrow[b] + out_tail + 16 * g);   // half line: k = tail + 16 g .. + 15
+        }
+        // 8 weights of this lane's k run, per block, against the head and the remainder of the same 8 activations
+        auto mm = [&](const uint32_t (&x)[kMfmaBlocks], const uint32_t (&y)[kMfmaBlocks], int k) {
+            const v8bf hv = *reinterpret_cast<const v8bf*>(ah + k), lv = *reinterpret_cast<const v8bf*>(al + k);
+#pragma unroll
+            for (int b = 0; b < kMfmaBlocks; ++b) {
+                const v8bf wv = e4m3x8_to_bf16(x[b], y[b]);
+                acc_hi[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, hv, acc_hi[b], 0, 0, 0);
+                acc_lo[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, lv, acc_lo[b], 0, 0, 0);
             }
-        uint4 wt = {0u, 0u, 0u, 0u};
-        if (Ie & 64) wt = *reinterpret_cast<const uint4*>(wrow + out_tail + 16 * g);  // half line: k = tail + 16 g .. + 15
-        for (int s0 = 0; s0 < out_steps; s0 += kMfmaDepth) {
+        };
+        for (int s0 = 0; s0 < out_steps; s0 += kMfmaOutDepth) {
 #pragma unroll
-            for (int j = 0; j < kMfmaDepth; ++j) {
+            for (int j = 0; j < kMfmaOutDepth; ++j) {
                 const int st = s0 + j;
                 if (st < out_steps) {
-                    const uint4 ca = wa[j], cb = wb[j];
-                    if (st + kMfmaDepth < out_steps) {
-                        wa[j] = *reinterpret_cast<const uint4*>(wr + (st + kMfmaDepth) * 128);
-                        wb[j] = *reinterpret_cast<const uint4*>(wr + (st + kMfmaDepth) * 128 + 16);
+                    uint32_t c[8][kMfmaBlocks];
+#pragma unroll
+                    for (int b = 0; b < kMfmaBlocks; ++b) {
+                        c[0][b] = wa[b][j].x; c[1][b] = wa[b][j].y; c[2][b] = wa[b][j].z; c[3][b] = wa[b][j].w;
+                        c[4][b] = wb[b][j].x; c[5][b] = wb[b][j].y; c[6][b] = wb[b][j].z; c[7][b] = wb[b][j].w;
+                        if (st + kMfmaOutDepth < out_steps) {
+                            wa[b][j] = *reinterpret_cast<const uint4*>(wrow[b] + 32 * g + (st + kMfmaOutDepth) * 128);
+                            wb[b][j] = *reinterpret_cast<const uint4*>(wrow[b] + 32 * g + (st + kMfmaOutDepth) * 128 + 16);
+                        }
                     }
                     const int k = st * 128 + 32 * g;
-                    mm(ca.x, ca.y, k);
-                    mm(ca.z, ca.w, k + 8);
-                    mm(cb.x, cb.y, k + 16);
-                    mm(cb.z, cb.w, k + 24);
+                    mm(c[0], c[1], k);
+                    mm(c[2], c[3], k + 8);
+                    mm(c[4], c[5], k + 16);
+                    mm(c[6], c[7], k + 24);
                 }
             }
         }
         if (Ie & 64) {
-            mm(wt.x, wt.y, out_tail + 16 * g);
-            mm(wt.z, wt.w, out_tail + 16 * g + 8);
-        }
-        if (live) {
-            float v[4];
+            uint32_t c[4][kMfmaBlocks];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) v[r] = rw * ((acc_hi[r] + acc_lo[r]) * d_wout);
-            atomic_add_bf16x4(quad, before, v);
+            for (int b = 0; b < kMfmaBlocks; ++b) { c[0][b] = wt[b].x; c[1][b] = wt[b].y; c[2][b] = wt[b].z; c[3][b] = wt[b].w; }
+            mm(c[0], c[1], out_tail + 16 * g);
+            mm(c[2], c[3], out_tail + 16 * g + 8);
+        }
+#pragma unroll
+        for (int b = 0; b < kMfmaBlocks; ++b) {
+            if (live && h0 + b * kWaves * 16 < H) {
+                float v[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) v[r] = rw * ((acc_hi[b][r] + acc_lo[b][r]) * d_wout);
+                atomic_add_bf16x4(quad[b], before[b], v);
+            }
         }
     }
 }

@@ -567,13 +567,15 @@ __device__ __forceinline__ v8bf e4m3x8_to_bf16(uint32_t a, uint32_t b) {
 
 // four neighbouring bf16 values += v[0..3], one rounding each, by a 64-bit compare-and-swap; `old` is a value read
 // from the address earlier (a stale one only costs a second round)
+__device__ __forceinline__ unsigned long long add_bf16x4(unsigned long long cur, const float* v) {
+    const unsigned lo = static_cast<unsigned>(cur), hi = static_cast<unsigned>(cur >> 32);
+    return static_cast<unsigned long long>(pack_bf16x2(bf16_lo(lo) + v[0], bf16_hi(lo) + v[1])) |
+           (static_cast<unsigned long long>(pack_bf16x2(bf16_lo(hi) + v[2], bf16_hi(hi) + v[3])) << 32);
+}
 __device__ __forceinline__ void atomic_add_bf16x4(unsigned long long* quad, unsigned long long old, const float* v) {
     while (true) {
         const unsigned long long assumed = old;
-        const unsigned lo = static_cast<unsigned>(assumed), hi = static_cast<unsigned>(assumed >> 32);
-        const unsigned long long next = static_cast<unsigned long long>(pack_bf16x2(bf16_lo(lo) + v[0], bf16_hi(lo) + v[1])) |
-                                        (static_cast<unsigned long long>(pack_bf16x2(bf16_lo(hi) + v[2], bf16_hi(hi) + v[3])) << 32);
-        old = atomicCAS(quad, assumed, next);
+        old = atomicCAS(quad, assumed, add_bf16x4(assumed, v));
         if (old == assumed) return;
     }
 }
@@ -747,6 +749,221 @@ __global__ __launch_bounds__(kMfmaThreads) void k_grouped_gelu_fp8_mfma(const ui
                 for (int r = 0; r < 4; ++r) v[r] = rw * ((acc_hi[b][r] + acc_lo[b][r]) * d_wout);
                 atomic_add_bf16x4(quad[b], before[b], v);
             }
+        }
+    }
+}
+
+// ---- 32-row form ------------------------------------------------------------------------------------
+// The 16-row kernel above re-reads its expert's weights once per 16 rows, and that traffic through the L2s is what
+// it waits for.  This form takes 32 rows per workgroup (two groups of 16 token rows against every weight fetch) and
+// still keeps the GELU output at 4 bytes per element in LDS by walking Ie in chunks: fc_in + GELU for a chunk of
+// columns, then that chunk's share of fc_out added into accumulators that stay in registers across chunks: a
+// wavefront owns the output blocks wave, wave + 8, ... (H / 128 of them, at most kWideBlocks: H <= 2048), two
+// accumulators each.  Blocks are walked in pairs so an activation read from LDS feeds two blocks.  One rounding
+// per (row, expert) as before: the compare-and-swap comes after the last chunk.
+constexpr int kWideRows = 32;
+constexpr int kWideBlocks = 16;
+constexpr int kWideDepth = 2;
+
+template <bool E5M2>
+__global__ __launch_bounds__(kMfmaThreads) void k_grouped_gelu_fp8_mfma32(const uint8_t* __restrict__ hidden, const float* __restrict__ fcin_descale,
+                                                                          const float* __restrict__ route_weights, const int* __restrict__ counts,
+                                                                          const int* __restrict__ row_indices, const uint8_t* __restrict__ fc_in_w,
+                                                                          const float* __restrict__ fc_in_descale, const uint8_t* __restrict__ fc_out_w,
+                                                                          const float* __restrict__ fc_out_descale, uint16_t* __restrict__ mixed,
+                                                                          int rows, int H, int Ie, int E, int tiles_per_expert, int chunk) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    constexpr int kWaves = kMfmaThreads / 64;
+    const int hs = H + 16;                          // hidden row stride in bytes
+    const int as = chunk + 8;                       // activation row stride in elements
+    uint8_t* sh_hidden = smem;                                                        // [32][hs] fp8
+    uint16_t* sh_hi = reinterpret_cast<uint16_t*>(smem + kWideRows * hs);             // [32][as] bf16 head of gelu
+    uint16_t* sh_lo = sh_hi + kWideRows * as;                                         // [32][as] bf16 remainder
+    const int xcd = blockIdx.x % kXcdCount, slot = blockIdx.x / kXcdCount;
+    const int e = (slot / tiles_per_expert) * kXcdCount + xcd, tile = slot % tiles_per_expert;
+    if (e >= E) return;
+    const int first = tile * kWideRows, n_active = counts[e];
+    if (first >= n_active) return;
+    const int n_rows = min(kWideRows, n_active - first);
+    const int* my_rows = row_indices + static_cast<size_t>(e) * rows + first;
+    const uint8_t* w_in = fc_in_w + static_cast<size_t>(e) * H * Ie;
+    const uint8_t* w_out = fc_out_w + static_cast<size_t>(e) * Ie * H;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, t = lane & 15, g = lane >> 4;
+
+    const int vec_per_row = H / 16;
+    for (int i = threadIdx.x; i < kWideRows * vec_per_row; i += kMfmaThreads) {
+        const int r = i / vec_per_row, c = i % vec_per_row;
+        const int src = my_rows[min(r, n_rows - 1)];
+        *reinterpret_cast<uint4*>(sh_hidden + r * hs + c * 16) =
+            *reinterpret_cast<const uint4*>(hidden + static_cast<size_t>(src) * H + c * 16);
+    }
+    __syncthreads();
+
+    const float s_in = *fcin_descale * *fc_in_descale;
+    const int in_steps = H / 128;
+    const int nblk = H / 128;                       // output blocks of this wavefront
+    v4f acc[kWideBlocks][2];
+#pragma unroll
+    for (int b = 0; b < kWideBlocks; ++b) {
+        acc[b][0] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+        acc[b][1] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+
+    for (int c0 = 0; c0 < Ie; c0 += chunk) {
+        const int cw = min(chunk, Ie - c0);         // a multiple of 64
+        // ---- fc_in + GELU for columns c0 .. c0 + cw - 1 ----
+        for (int n0 = wave * 16; n0 < cw; n0 += kWaves * 16) {
+            v4f a0 = {0.0f, 0.0f, 0.0f, 0.0f}, a1 = {0.0f, 0.0f, 0.0f, 0.0f};
+            const uint8_t* wr = w_in + static_cast<size_t>(c0 + n0 + t) * H + 32 * g;
+            const uint8_t* hr0 = sh_hidden + t * hs + 32 * g;
+            const uint8_t* hr1 = hr0 + 16 * hs;
+            uint4 w0[kWideDepth], w1[kWideDepth];
+#pragma unroll
+            for (int j = 0; j < kWideDepth; ++j)
+                if (j < in_steps) {
+                    w0[j] = *reinterpret_cast<const uint4*>(wr + j * 128);
+                    w1[j] = *reinterpret_cast<const uint4*>(wr + j * 128 + 16);
+                }
+            for (int s0 = 0; s0 < in_steps; s0 += kWideDepth) {
+#pragma unroll
+                for (int j = 0; j < kWideDepth; ++j) {
+                    const int st = s0 + j;
+                    if (st < in_steps) {
+                        const v8i a = {(int)w0[j].x, (int)w0[j].y, (int)w0[j].z, (int)w0[j].w, (int)w1[j].x, (int)w1[j].y, (int)w1[j].z, (int)w1[j].w};
+                        if (st + kWideDepth < in_steps) {
+                            w0[j] = *reinterpret_cast<const uint4*>(wr + (st + kWideDepth) * 128);
+                            w1[j] = *reinterpret_cast<const uint4*>(wr + (st + kWideDepth) * 128 + 16);
+                        }
+                        const uint4 x0 = *reinterpret_cast<const uint4*>(hr0 + st * 128), x1 = *reinterpret_cast<const uint4*>(hr0 + st * 128 + 16);
+                        const uint4 y0 = *reinterpret_cast<const uint4*>(hr1 + st * 128), y1 = *reinterpret_cast<const uint4*>(hr1 + st * 128 + 16);
+                        const v8i b0 = {(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w, (int)x1.x, (int)x1.y, (int)x1.z, (int)x1.w};
+                        const v8i b1 = {(int)y0.x, (int)y0.y, (int)y0.z, (int)y0.w, (int)y1.x, (int)y1.y, (int)y1.z, (int)y1.w};
+                        a0 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b0, a0, 0, E5M2 ? 1 : 0, 0, 0, 0, 0);
+                        a1 = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b1, a1, 0, E5M2 ? 1 : 0, 0, 0, 0, 0);
+                    }
+                }
+            }
+            // this lane: token rows t and 16 + t, columns c0 + n0 + 4g .. + 3
+#pragma unroll
+            for (int tg = 0; tg < 2; ++tg) {
+                uint32_t hb[4], lb[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float act = gelu_fwd((tg ? a1[r] : a0[r]) * s_in);
+                    hb[r] = __float_as_uint(act) & 0xffff0000u;
+                    lb[r] = f32_to_bf16(act - __uint_as_float(hb[r]));
+                }
+                const int at = (tg * 16 + t) * as + n0 + 4 * g;
+                *reinterpret_cast<uint2*>(sh_hi + at) = make_uint2((hb[0] >> 16) | hb[1], (hb[2] >> 16) | hb[3]);
+                *reinterpret_cast<uint2*>(sh_lo + at) = make_uint2(lb[0] | (lb[1] << 16), lb[2] | (lb[3] << 16));
+            }
+        }
+        __syncthreads();
+
+        // ---- this chunk's share of fc_out ----
+        const int steps = cw / 128, tail = steps * 128;     // whole 128-byte runs of the chunk; cw % 128 == 64 leaves half a run
+        const uint32_t lane_row = static_cast<uint32_t>(wave * 16 + t) * static_cast<uint32_t>(Ie);
+        const uint16_t* ah0 = sh_hi + t * as;
+        const uint16_t* al0 = sh_lo + t * as;
+        const uint16_t* ah1 = ah0 + 16 * as;
+        const uint16_t* al1 = al0 + 16 * as;
+#pragma unroll
+        for (int bp = 0; bp < kWideBlocks; bp += 2) {
+            if (bp < nblk) {
+                // rows of the two blocks' weights (the second repeats the first where nblk is odd; its sums are not used)
+                // uniform base + 32-bit lane offsets: no 64-bit per-lane addresses to keep alive across the pairs
+                const int bq = bp + 1 < nblk ? bp + 1 : bp;
+                const uint8_t* wbase = w_out + c0;
+                const uint32_t oA = lane_row + static_cast<uint32_t>(kWaves * 16 * bp) * static_cast<uint32_t>(Ie);
+                const uint32_t oB = lane_row + static_cast<uint32_t>(kWaves * 16 * bq) * static_cast<uint32_t>(Ie);
+                auto ldw = [&](uint32_t off) { return *reinterpret_cast<const uint4*>(wbase + off); };
+                v4f pA0 = acc[bp][0], pA1 = acc[bp][1], pB0 = acc[bp + 1][0], pB1 = acc[bp + 1][1];
+                auto mm = [&](uint32_t xa, uint32_t ya, uint32_t xb, uint32_t yb, int k) {
+                    const v8bf wa = e4m3x8_to_bf16(xa, ya), wb = e4m3x8_to_bf16(xb, yb);
+                    const v8bf h0 = *reinterpret_cast<const v8bf*>(ah0 + k), h1 = *reinterpret_cast<const v8bf*>(ah1 + k);
+                    const v8bf l0 = *reinterpret_cast<const v8bf*>(al0 + k), l1 = *reinterpret_cast<const v8bf*>(al1 + k);
+                    pA0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, h0, pA0, 0, 0, 0);
+                    pA1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, h1, pA1, 0, 0, 0);
+                    pB0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb, h0, pB0, 0, 0, 0);
+                    pB1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb, h1, pB1, 0, 0, 0);
+                    pA0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, l0, pA0, 0, 0, 0);
+                    pA1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, l1, pA1, 0, 0, 0);
+                    pB0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb, l0, pB0, 0, 0, 0);
+                    pB1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb, l1, pB1, 0, 0, 0);
+                };
+                uint4 a0[kWideDepth], a1[kWideDepth], b0[kWideDepth], b1[kWideDepth];
+#pragma unroll
+                for (int j = 0; j < kWideDepth; ++j)
+                    if (j < steps) {                                                // step s: k = 128 s + 32 g .. + 31 of the chunk
+                        a0[j] = ldw(oA + 32 * g + j * 128);
+                        a1[j] = ldw(oA + 32 * g + j * 128 + 16);
+                        b0[j] = ldw(oB + 32 * g + j * 128);
+                        b1[j] = ldw(oB + 32 * g + j * 128 + 16);
+                    }
+                for (int s0 = 0; s0 < steps; s0 += kWideDepth) {
+#pragma unroll
+                    for (int j = 0; j < kWideDepth; ++j) {
+                        const int st = s0 + j;
+                        if (st < steps) {
+                            const uint4 ca0 = a0[j], ca1 = a1[j], cb0 = b0[j], cb1 = b1[j];
+                            if (st + kWideDepth < steps) {
+                                a0[j] = ldw(oA + 32 * g + (st + kWideDepth) * 128);
+                                a1[j] = ldw(oA + 32 * g + (st + kWideDepth) * 128 + 16);
+                                b0[j] = ldw(oB + 32 * g + (st + kWideDepth) * 128);
+                                b1[j] = ldw(oB + 32 * g + (st + kWideDepth) * 128 + 16);
+                            }
+                            const int k = st * 128 + 32 * g;
+                            mm(ca0.x, ca0.y, cb0.x, cb0.y, k);
+                            mm(ca0.z, ca0.w, cb0.z, cb0.w, k + 8);
+                            mm(ca1.x, ca1.y, cb1.x, cb1.y, k + 16);
+                            mm(ca1.z, ca1.w, cb1.z, cb1.w, k + 24);
+                        }
+                    }
+                }
+                if (cw & 64) {                                                      // half run: k = tail + 16 g .. + 15
+                    const uint4 ta = ldw(oA + tail + 16 * g);
+                    const uint4 tb = ldw(oB + tail + 16 * g);
+                    mm(ta.x, ta.y, tb.x, tb.y, tail + 16 * g);
+                    mm(ta.z, ta.w, tb.z, tb.w, tail + 16 * g + 8);
+                }
+                acc[bp][0] = pA0; acc[bp][1] = pA1; acc[bp + 1][0] = pB0; acc[bp + 1][1] = pB1;
+            }
+        }
+        __syncthreads();                            // the next chunk overwrites the activations
+    }
+
+    // ---- one compare-and-swap per (token row, 4 output columns), four in flight at a time ----
+    const float d_wout = *fc_out_descale;
+#pragma unroll
+    for (int tg = 0; tg < 2; ++tg) {
+        const int r = tg * 16 + t;
+        const bool live = r < n_rows;
+        const int row = live ? my_rows[r] : 0;
+        const float rw = live ? route_weights[static_cast<size_t>(row) * E + e] : 0.0f;
+        uint16_t* mrow = mixed + static_cast<size_t>(row) * H + 4 * g + wave * 16;
+#pragma unroll
+        for (int b0 = 0; b0 < kWideBlocks; b0 += 4) {
+            if (b0 < nblk && live) {
+                unsigned long long before[4], got[4];
+                float v[4][4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (b0 + i < nblk)
+                        before[i] = __builtin_nontemporal_load(reinterpret_cast<unsigned long long*>(mrow + (b0 + i) * kWaves * 16));
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (b0 + i < nblk) {
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) v[i][q] = rw * (acc[b0 + i][tg][q] * d_wout);
+                        got[i] = atomicCAS(reinterpret_cast<unsigned long long*>(mrow + (b0 + i) * kWaves * 16), before[i],
+                                           add_bf16x4(before[i], v[i]));
+                    }
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (b0 + i < nblk && got[i] != before[i])                     // lost a race: redo from the value found
+                        atomic_add_bf16x4(reinterpret_cast<unsigned long long*>(mrow + (b0 + i) * kWaves * 16), got[i], v[i]);
+            }
+            __builtin_amdgcn_sched_barrier(0);      // keeps the groups apart: their loads hoisted together would not fit the registers
         }
     }
 }
@@ -1126,6 +1343,39 @@ int cf_moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_fcin_
     if (!d_hidden || !d_fcin_descale || !d_route_weights || !d_counts || !d_row_indices || !d_fc_in_w || !d_fc_in_descale ||
         !d_fc_out_w || !d_fc_out_descale || !d_mixed)
         return CF_ERR_INVALID_ARG;
+    const bool mfma_ok = H % 128 == 0 && Ie % 64 == 0 && aligned16(d_hidden) && aligned16(d_fc_in_w) && aligned16(d_fc_out_w) &&
+                         (reinterpret_cast<uintptr_t>(d_mixed) & 7u) == 0;
+    // 32 rows per workgroup where the output blocks fit a wavefront's registers and LDS holds the hidden rows plus
+    // a chunk of at least 64 activation columns: Ie is walked in the fewest equal chunks that fit
+    if (mfma_ok && H <= 128 * kWideBlocks) {
+        const long long room = 160 * 1024 - static_cast<long long>(kWideRows) * (H + 16);
+        const int max_chunk = room > 0 ? static_cast<int>(((room / (4 * kWideRows)) - 8) / 64 * 64) : 0;
+        if (max_chunk >= 64) {
+            const int passes = (Ie + max_chunk - 1) / max_chunk;
+            const int chunk = ((Ie + passes - 1) / passes + 63) / 64 * 64;
+            const size_t smem32 = static_cast<size_t>(kWideRows) * (H + 16) + 4u * kWideRows * (static_cast<size_t>(chunk) + 8);
+            static std::once_flag once32;
+            static hipError_t err32 = hipSuccess;
+            std::call_once(once32, [] {
+                err32 = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_grouped_gelu_fp8_mfma32<false>),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                if (err32 == hipSuccess)
+                    err32 = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_grouped_gelu_fp8_mfma32<true>),
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            });
+            if (err32 != hipSuccess) return static_cast<int>(err32);
+            const int tiles = (rows + kWideRows - 1) / kWideRows;
+            auto launch = [&](auto kernel) {
+                kernel<<<kXcdCount * ((num_experts + kXcdCount - 1) / kXcdCount) * tiles, kMfmaThreads, smem32, as_stream(stream)>>>(
+                    static_cast<const uint8_t*>(d_hidden), d_fcin_descale, d_route_weights, d_counts, d_row_indices,
+                    static_cast<const uint8_t*>(d_fc_in_w), d_fc_in_descale, static_cast<const uint8_t*>(d_fc_out_w), d_fc_out_descale,
+                    d_mixed, rows, H, Ie, num_experts, tiles, chunk);
+            };
+            if (fcin_is_e5m2) launch(k_grouped_gelu_fp8_mfma32<true>);
+            else launch(k_grouped_gelu_fp8_mfma32<false>);
+            return launch_status();
+        }
+    }
     // the matrix-core form where the shapes are whole MFMA steps and its tile fits the LDS
     const size_t smem_mfma = static_cast<size_t>(kMfmaRows) * (H + 16) + 4u * kMfmaRows * (static_cast<size_t>(Ie) + 8);
     if (H % 128 == 0 && Ie % 64 == 0 && smem_mfma <= 160 * 1024 && aligned16(d_hidden) && aligned16(d_fc_in_w) &&

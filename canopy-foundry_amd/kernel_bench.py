@@ -272,7 +272,7 @@ def main():
          lambda: cf.cf_moe_grouped_gelu_forward_fp8(hq, one, 0, rw, counts, offs, idx, wg, one, wd, one, mixed, T, H, Ie, E, total,
                                                     ws3, sz3.value, st))
     iters, args.iters = args.iters, 5
-    mfma("moe_grouped_expert_forward_fp8 form (fp32 GELU kept, MFMA, 16-row tiles)", f"T={T} E={E} k={k}", 4.0 * total * Ie * H,
+    mfma("moe_grouped_expert_forward_fp8 form (fp32 GELU kept, MFMA)", f"T={T} E={E} k={k}", 4.0 * total * Ie * H,
          lambda: cf.cf_moe_grouped_expert_forward_fp8(hq, one, 0, rw, counts, offs, idx, wg, one, wd, one, mixed, T, H, Ie, E, total, st))
     args.iters = iters
     del ws3, gq

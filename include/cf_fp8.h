@@ -436,8 +436,9 @@ int cf_moe_grouped_swiglu_forward_fp8(const void* d_hidden_e4m3, const float* d_
  * total_selected_rows are accepted and unused, as in the reference.  With H % 128 == 0,
  * Ie % 64 == 0, 16-byte aligned operands and 8-byte aligned d_mixed the two projections run on
  * the matrix cores (fp8 MFMA for fc_in; fc_out as bf16 MFMA on a two-term bf16 split of the fp32
- * GELU output, relative error 2^-17, against the weights widened exactly); other shapes take an
- * fp32 FMA kernel.  Same contract either way. */
+ * GELU output, relative error 2^-17, against the weights widened exactly; 32 token rows per
+ * workgroup up to H = 2048, 16 beyond); other shapes take an fp32 FMA kernel.  Same contract
+ * either way. */
 int cf_moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_fcin_descale,
                                       int fcin_is_e5m2, const float* d_route_weights,
                                       const int* d_counts, const int* d_offsets,

@@ -148,7 +148,9 @@ def test_config5_full_size(cf, dev):
 @pytest.mark.parametrize("rows,E,k,H,Ie,e5m2", [(90, 4, 2, 96, 72, False), (300, 6, 3, 256, 300, True), (33, 3, 3, 40, 1408, False),
                                                  # whole MFMA steps (H % 128 == 0, Ie % 64 == 0): the matrix-core form
                                                  (300, 6, 3, 256, 320, True), (200, 4, 2, 128, 64, False), (1000, 5, 2, 384, 448, False),
-                                                 (70, 3, 3, 2048, 1408, False)])
+                                                 (70, 3, 3, 2048, 1408, False),
+                                                 # three unequal chunks of Ie in the 32-row form; H > 2048: the 16-row form
+                                                 (50, 2, 2, 2048, 1472, True), (40, 3, 2, 2304, 128, False), (90, 2, 1, 2176, 192, True)])
 def test_grouped_gelu_expert_bank_reference_form(cf, dev, rows, E, k, H, Ie, e5m2):
     """moe_grouped_expert_forward_fp8: per-tensor descales, float GELU intermediate, bf16 CAS accumulate."""
     case(f"grouped gelu bank rows={rows} E={E} k={k} H={H} Ie={Ie} e5m2={e5m2}")

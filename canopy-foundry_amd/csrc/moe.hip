@@ -466,6 +466,9 @@ __device__ __forceinline__ void atomic_add_bf16(uint16_t* addr, float v) {
     }
 }
 
+// BF16: the reference's bf16 sibling (moe_grouped_expert_forward_bf16, same scheduling): hidden and weights are bf16
+// (the byte pointers then address 2-byte elements), no descales.
+template <bool BF16>
 __global__ __launch_bounds__(kThreads) void k_grouped_gelu_fp8(const uint8_t* __restrict__ hidden, const float* __restrict__ fcin_descale,
                                                                int fcin_is_e5m2, const float* __restrict__ route_weights,
                                                                const int* __restrict__ counts, const int* __restrict__ row_indices,
@@ -481,9 +484,18 @@ __global__ __launch_bounds__(kThreads) void k_grouped_gelu_fp8(const uint8_t* __
     if (first >= n_active) return;
     const int n_rows = min(kGeluRows, n_active - first);
     const int* my_rows = row_indices + static_cast<size_t>(e) * rows + first;
-    const float d_in = *fcin_descale, d_win = *fc_in_descale, d_wout = *fc_out_descale;
-    const uint8_t* w_in = fc_in_w + static_cast<size_t>(e) * H * Ie;
-    const uint8_t* w_out = fc_out_w + static_cast<size_t>(e) * Ie * H;
+    const float d_in = BF16 ? 1.0f : *fcin_descale, d_win = BF16 ? 1.0f : *fc_in_descale, d_wout = BF16 ? 1.0f : *fc_out_descale;
+    constexpr int kElem = BF16 ? 2 : 1;
+    const uint8_t* w_in = fc_in_w + static_cast<size_t>(e) * H * Ie * kElem;
+    const uint8_t* w_out = fc_out_w + static_cast<size_t>(e) * Ie * H * kElem;
+    auto hidden_at = [&](size_t i) {
+        if constexpr (BF16) return bf16_to_f32(reinterpret_cast<const uint16_t*>(hidden)[i]);
+        else return (fcin_is_e5m2 ? e5m2_to_f32(hidden[i]) : e4m3_to_f32(hidden[i])) * d_in;
+    };
+    auto weight_at = [&](const uint8_t* w, size_t i, float d) {
+        if constexpr (BF16) return bf16_to_f32(reinterpret_cast<const uint16_t*>(w)[i]);
+        else return e4m3_to_f32(w[i]) * d;
+    };
 
     // fc_in: 256 output columns per pass, K in chunks of 128 staged (dequantised) through LDS
     for (int j0 = 0; j0 < Ie; j0 += kThreads) {
@@ -496,14 +508,13 @@ __global__ __launch_bounds__(kThreads) void k_grouped_gelu_fp8(const uint8_t* __
             __syncthreads();
             for (int i = threadIdx.x; i < n_rows * kt; i += kThreads) {
                 const int r = i / kt, k = i % kt;
-                const uint8_t b = hidden[static_cast<size_t>(my_rows[r]) * H + k0 + k];
-                sh_chunk[r * kGeluChunk + k] = (fcin_is_e5m2 ? e5m2_to_f32(b) : e4m3_to_f32(b)) * d_in;
+                sh_chunk[r * kGeluChunk + k] = hidden_at(static_cast<size_t>(my_rows[r]) * H + k0 + k);
             }
             __syncthreads();
             if (j < Ie) {
-                const uint8_t* wr = w_in + static_cast<size_t>(j) * H + k0;
+                const size_t wr = static_cast<size_t>(j) * H + k0;
                 for (int k = 0; k < kt; ++k) {
-                    const float wv = e4m3_to_f32(wr[k]) * d_win;
+                    const float wv = weight_at(w_in, wr + k, d_win);
 #pragma unroll
                     for (int r = 0; r < kGeluRows; ++r) accum[r] = __builtin_fmaf(sh_chunk[r * kGeluChunk + k], wv, accum[r]);
                 }
@@ -525,9 +536,9 @@ __global__ __launch_bounds__(kThreads) void k_grouped_gelu_fp8(const uint8_t* __
         float accum[kGeluRows];
 #pragma unroll
         for (int r = 0; r < kGeluRows; ++r) accum[r] = 0.0f;
-        const uint8_t* wr = w_out + static_cast<size_t>(h) * Ie;
+        const size_t wr = static_cast<size_t>(h) * Ie;
         for (int k = 0; k < Ie; ++k) {
-            const float wv = e4m3_to_f32(wr[k]) * d_wout;
+            const float wv = weight_at(w_out, wr + k, d_wout);
 #pragma unroll
             for (int r = 0; r < kGeluRows; ++r) accum[r] = __builtin_fmaf(sh_act[r * Ie + k], wv, accum[r]);
         }
@@ -1406,14 +1417,40 @@ int cf_moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_fcin_
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
     std::call_once(once, [] {
-        attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_grouped_gelu_fp8),
+        attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_grouped_gelu_fp8<false>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     });
     if (attr_err != hipSuccess) return static_cast<int>(attr_err);
     const int tiles_per_expert = (rows + kGeluRows - 1) / kGeluRows;
-    k_grouped_gelu_fp8<<<num_experts * tiles_per_expert, kThreads, smem, as_stream(stream)>>>(
+    k_grouped_gelu_fp8<false><<<num_experts * tiles_per_expert, kThreads, smem, as_stream(stream)>>>(
         static_cast<const uint8_t*>(d_hidden), d_fcin_descale, fcin_is_e5m2, d_route_weights, d_counts, d_row_indices,
         static_cast<const uint8_t*>(d_fc_in_w), d_fc_in_descale, static_cast<const uint8_t*>(d_fc_out_w), d_fc_out_descale,
+        d_mixed, rows, H, Ie, num_experts, tiles_per_expert);
+    return launch_status();
+}
+
+int cf_moe_grouped_expert_forward_bf16(const uint16_t* d_hidden, const float* d_route_weights, const int* d_counts,
+                                       const int* d_offsets, const int* d_row_indices, const uint16_t* d_fc_in_w,
+                                       const uint16_t* d_fc_out_w, uint16_t* d_mixed, int rows, int H, int Ie,
+                                       int num_experts, int total_selected_rows, cf_stream_t stream) {
+    (void)d_offsets;               // as in the reference, the tiled form needs neither
+    (void)total_selected_rows;
+    if (rows < 0 || H < 0 || Ie < 0 || num_experts < 0) return CF_ERR_INVALID_ARG;
+    if (rows == 0 || num_experts == 0 || H == 0 || Ie == 0) return CF_OK;
+    if (!d_hidden || !d_route_weights || !d_counts || !d_row_indices || !d_fc_in_w || !d_fc_out_w || !d_mixed) return CF_ERR_INVALID_ARG;
+    const size_t smem = sizeof(float) * static_cast<size_t>(kGeluRows) * (kGeluChunk + Ie);
+    if (smem > 160 * 1024) return CF_ERR_UNSUPPORTED;
+    static std::once_flag once;
+    static hipError_t attr_err = hipSuccess;
+    std::call_once(once, [] {
+        attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_grouped_gelu_fp8<true>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    });
+    if (attr_err != hipSuccess) return static_cast<int>(attr_err);
+    const int tiles_per_expert = (rows + kGeluRows - 1) / kGeluRows;
+    k_grouped_gelu_fp8<true><<<num_experts * tiles_per_expert, kThreads, smem, as_stream(stream)>>>(
+        reinterpret_cast<const uint8_t*>(d_hidden), nullptr, 0, d_route_weights, d_counts, d_row_indices,
+        reinterpret_cast<const uint8_t*>(d_fc_in_w), nullptr, reinterpret_cast<const uint8_t*>(d_fc_out_w), nullptr,
         d_mixed, rows, H, Ie, num_experts, tiles_per_expert);
     return launch_status();
 }

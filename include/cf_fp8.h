@@ -448,6 +448,17 @@ int cf_moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_fcin_
                                       int H, int Ie, int num_experts, int total_selected_rows,
                                       cf_stream_t stream);
 
+/* moe_grouped_expert_forward_bf16, kernels.hpp:400-407: the same device-scheduled expert bank on
+ * bf16 hidden states and bf16 weights (fc_in_w [E,Ie,H], fc_out_w [E,H,Ie]), no descales; fp32
+ * accumulation, exact-erf GELU kept in fp32, compare-and-swap accumulation into d_mixed.  The
+ * non-FP8 sibling: fp32 FMA kernel in the reference's loop form, any shape. */
+int cf_moe_grouped_expert_forward_bf16(const uint16_t* d_hidden, const float* d_route_weights,
+                                       const int* d_counts, const int* d_offsets,
+                                       const int* d_row_indices, const uint16_t* d_fc_in_w,
+                                       const uint16_t* d_fc_out_w, uint16_t* d_mixed, int rows,
+                                       int H, int Ie, int num_experts, int total_selected_rows,
+                                       cf_stream_t stream);
+
 /* gelu_forward (kernels/moe.cu:510-521) followed by the per-token E4M3 quantize of its bf16
  * output, in one pass: out = e4m3(bf16(gelu(x)) * scale[row]), scale[row] = 448 / max(amax, 1e-12)
  * over the row of bf16(gelu(x)), descale its inverse (the formula of kernels/fp8.cu:37-39,49).

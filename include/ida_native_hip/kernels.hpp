@@ -175,6 +175,14 @@ inline void moe_scatter_add_rows_bf16(bf16* d_dst_full, const bf16* d_src_compac
 inline void moe_expert_offsets_from_counts(const int* d_counts, int* d_offsets, int num_experts, hipStream_t stream) {
     CF_FWD(cf_moe_expert_offsets_from_counts(d_counts, d_offsets, num_experts, stream));
 }
+inline void moe_grouped_expert_forward_bf16(const bf16* d_hidden, const float* d_route_weights, const int* d_counts,
+                                            const int* d_offsets, const int* d_row_indices, const bf16* d_fc_in_w,
+                                            const bf16* d_fc_out_w, bf16* d_mixed, int rows, int H, int Ie, int num_experts,
+                                            int total_selected_rows, hipStream_t stream) {
+    CF_FWD(cf_moe_grouped_expert_forward_bf16(hip_detail::u(d_hidden), d_route_weights, d_counts, d_offsets, d_row_indices,
+                                              hip_detail::u(d_fc_in_w), hip_detail::u(d_fc_out_w), hip_detail::u(d_mixed), rows, H,
+                                              Ie, num_experts, total_selected_rows, stream));
+}
 inline void moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_fcin_descale, int fcin_is_e5m2,
                                            const float* d_route_weights, const int* d_counts, const int* d_offsets,
                                            const int* d_row_indices, const void* d_fc_in_w, const float* d_fc_in_descale,

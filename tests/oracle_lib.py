@@ -560,3 +560,24 @@ def moe_grouped_expert_forward_fp8_ref(hidden, fcin_descale, fcin_e5m2, route_we
           fc_in_w, c_f(fc_in_descale), np.ascontiguousarray(fc_out_w, dtype=np.uint8), c_f(fc_out_descale),
           mixed, c_i(rows), c_i(H), c_i(Ie), c_i(E), c_i(THREADS))
     return mixed
+
+
+def moe_grouped_expert_forward_bf16_ref(hidden, route_weights, counts, row_indices, fc_in_w, fc_out_w, mixed0):
+    """moe_grouped_expert_forward_bf16 (kernels/moe.cu, the bf16 sibling of the grouped FP8 expert forward) in
+    float64 numpy: per expert, its listed rows through fc_in [Ie,H], exact-erf GELU, fc_out [H,Ie], times the route
+    weight, summed into mixed.  hidden / weights are bf16 bit patterns; returns float64 [rows,H]."""
+    import math
+    erf = np.vectorize(math.erf, otypes=[np.float64])
+    x = bf16_to_f32(hidden).astype(np.float64)
+    w_in = bf16_to_f32(fc_in_w).astype(np.float64)
+    w_out = bf16_to_f32(fc_out_w).astype(np.float64)
+    rw = np.asarray(route_weights, dtype=np.float64)
+    out = np.array(mixed0, dtype=np.float64, copy=True)
+    for e in range(rw.shape[1]):
+        rows = np.asarray(row_indices)[e, : int(counts[e])]
+        if rows.size == 0:
+            continue
+        pre = x[rows] @ w_in[e].T
+        act = 0.5 * pre * (1.0 + erf(pre * 0.70710678118654752440))
+        out[rows] += rw[rows, e][:, None] * (act @ w_out[e].T)
+    return out

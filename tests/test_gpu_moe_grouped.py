@@ -440,3 +440,29 @@ def test_grouped_gelu_expert_bank_reference_form_config5_size(cf, dev):
     assert np.sqrt(((got - ref) ** 2).sum() / (ref ** 2).sum()) <= 4e-3
     typical = np.sqrt(((ref - start) ** 2).mean())
     assert np.all(np.abs(got - ref) <= (b.k + 1) * 2.0 ** -8 * (np.abs(start) + np.abs(ref) + 2.0 * typical))
+
+
+@pytest.mark.parametrize("rows,E,k,H,Ie", [(90, 4, 2, 96, 72), (300, 6, 3, 256, 320), (33, 3, 3, 40, 1408)])
+def test_grouped_gelu_expert_bank_bf16_sibling(cf, dev, rows, E, k, H, Ie):
+    """moe_grouped_expert_forward_bf16: bf16 hidden states and weights, float GELU intermediate, bf16 CAS accumulate."""
+    case(f"grouped gelu bank, bf16 sibling rows={rows} E={E} k={k} H={H} Ie={Ie}")
+    rng = np.random.default_rng(rows + Ie + 1)
+    hidden = orc.bf16_from_f32(rng.standard_normal((rows, H)).astype(np.float32))
+    win = orc.bf16_from_f32((0.05 * rng.standard_normal((E, Ie, H))).astype(np.float32))
+    wout = orc.bf16_from_f32((0.05 * rng.standard_normal((E, H, Ie))).astype(np.float32))
+    rw = orc.moe_topk_route(rng.standard_normal((rows, E)).astype(np.float32), k)
+    counts, idx = orc.moe_build_expert_row_lists(rw)
+    mixed0 = orc.bf16_from_f32(rng.standard_normal((rows, H)).astype(np.float32))
+    mixed = dev_bf16(mixed0, dev)
+    cf.cf_moe_grouped_expert_forward_bf16(dev_bf16(hidden, dev), dev_arr(rw, dev), dev_arr(counts, dev), None, dev_arr(idx, dev),
+                                          dev_bf16(win, dev), dev_bf16(wout, dev), mixed, rows, H, Ie, E, rows * k, stream())
+    torch.cuda.synchronize()
+    start = orc.bf16_to_f32(mixed0).astype(np.float64)
+    ref = orc.moe_grouped_expert_forward_bf16_ref(hidden, rw, counts, idx, win, wout, start)
+    got = orc.bf16_to_f32(bf16_bits(mixed)).astype(np.float64)
+    assert np.sqrt(((got - ref) ** 2).sum() / (ref ** 2).sum()) <= 4e-3
+    typical = np.sqrt(((ref - start) ** 2).mean())
+    assert np.all(np.abs(got - ref) <= (k + 1) * 2.0 ** -8 * (np.abs(start) + np.abs(ref) + 2.0 * typical))
+    untouched = ~(rw > 0).any(axis=1)
+    assert np.array_equal(bf16_bits(mixed)[untouched], mixed0[untouched])
+    assert cf.raw_cf_moe_grouped_expert_forward_bf16(None, None, None, None, None, None, None, None, 4, 8, 8, 2, 8, None) == -1

@@ -261,3 +261,28 @@ def test_expert_bank_formula_against_the_reference_fixture():
     # sensitivity: the same call with the experts' weights in the wrong order misses by much more
     wrong = orc.moe_grouped_expert_forward_fp8_ref(hq, hd, False, route, counts, idx, wiq[::-1].copy(), wid, woq, wod, np.zeros((rows, H)))
     assert np.abs(wrong - want).max() > 0.3 * scale
+
+
+def test_expert_bank_bf16_ref_on_the_reference_fixture():
+    """The bf16 sibling's reference against the same fixture: with the operands rounded to bf16 it lands on the
+    fixture's `mixed` minus its trunk term to bf16 rounding of the operands (2^-9 each), and a transposed expert
+    order misses by far more; with two experts' rows swapped in the lists it changes."""
+    import math
+    g = json.loads((GOLD / "moe_expert_bank.json").read_text())
+    hg, rw, mixed = np.array(g["hidden_gated"]), np.array(g["route_weights"]), np.array(g["mixed"])
+    tin, tout = np.array(g["trunk_fc_in_w"]), np.array(g["trunk_fc_out_w"])
+    ein, eout = np.array(g["expert_fc_in_w"]), np.array(g["expert_fc_out_w"])
+    B, S, H = hg.shape
+    rows = B * S
+    erf = np.vectorize(math.erf)
+    trunk = (lambda x: 0.5 * x * (1.0 + erf(x / math.sqrt(2.0))))(hg @ tin.T) @ tout.T
+    want = (mixed - trunk).reshape(rows, H)
+    route = np.repeat(rw, S, axis=0).astype(np.float32)
+    counts, idx = orc.moe_build_expert_row_lists(route)
+    b = lambda x: orc.bf16_from_f32(x.astype(np.float32))
+    got = orc.moe_grouped_expert_forward_bf16_ref(b(hg.reshape(rows, H)), route, counts, idx, b(ein), b(eout), np.zeros((rows, H)))
+    scale = np.abs(want).max()
+    assert np.abs(got - want).max() < 0.01 * scale, (np.abs(got - want).max(), scale)
+    wrong = orc.moe_grouped_expert_forward_bf16_ref(b(hg.reshape(rows, H)), route, counts, idx, b(ein)[::-1].copy(), b(eout),
+                                                    np.zeros((rows, H)))
+    assert np.abs(wrong - want).max() > 0.3 * scale

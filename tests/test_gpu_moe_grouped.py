@@ -466,3 +466,24 @@ def test_grouped_gelu_expert_bank_bf16_sibling(cf, dev, rows, E, k, H, Ie):
     untouched = ~(rw > 0).any(axis=1)
     assert np.array_equal(bf16_bits(mixed)[untouched], mixed0[untouched])
     assert cf.raw_cf_moe_grouped_expert_forward_bf16(None, None, None, None, None, None, None, None, 4, 8, 8, 2, 8, None) == -1
+
+
+@pytest.mark.parametrize("rows,E,k,H,Ie,zero", [(100, 4, 2, 256, 128, 1), (5, 3, 1, 128, 64, None), (37, 3, 2, 2304, 64, 0)])
+def test_grouped_gelu_reference_form_ragged_and_empty_experts(cf, dev, rows, E, k, H, Ie, zero):
+    """The matrix-core forms with experts nobody selects, lists shorter than one row tile, and a last tile that ends
+    inside the first group of 16 rows."""
+    case(f"grouped gelu bank, reference form, ragged rows={rows} E={E} k={k} H={H} Ie={Ie} zero={zero}")
+    b = GeluBank(dev, rows, E, k, H, Ie, seed=rows + H, zero_expert=zero)
+    if zero is not None:
+        assert b.counts[zero] == 0
+    mixed = dev_bf16(b.mixed0, dev)
+    cf.cf_moe_grouped_expert_forward_fp8(b.d["hq"], b.d["hd"], 0, b.d["rw"], b.d["counts"], None, b.d["idx"], b.d["wi"], b.d["wid"],
+                                         b.d["wo"], b.d["wod"], mixed, b.rows, b.H, b.Ie, b.E, b.total, stream())
+    torch.cuda.synchronize()
+    start = orc.bf16_to_f32(b.mixed0).astype(np.float64)
+    ref = orc.moe_grouped_expert_forward_fp8_ref(b.hq, b.hd, False, b.rw, b.counts, b.idx, b.wi.reshape(E, Ie, H), b.wid,
+                                                 b.wo.reshape(E, H, Ie), b.wod, start)
+    got = orc.bf16_to_f32(bf16_bits(mixed)).astype(np.float64)
+    assert np.sqrt(((got - ref) ** 2).sum() / (ref ** 2).sum()) <= 4e-3
+    typical = np.sqrt(((ref - start) ** 2).mean())
+    assert np.all(np.abs(got - ref) <= (k + 1) * 2.0 ** -8 * (np.abs(start) + np.abs(ref) + 2.0 * typical))

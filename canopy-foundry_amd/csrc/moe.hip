@@ -552,7 +552,7 @@ __global__ __launch_bounds__(kThreads) void k_grouped_gelu_fp8(const uint8_t* __
 
 // ---- the same bank on the matrix cores -----------------------------------------------------------
 // Same arithmetic contract (GELU output kept beyond bf16, nothing re-quantised, compare-and-swap accumulation), for
-// H % 128 == 0 and Ie % 64 == 0.  One workgroup per (expert, 16 rows), four wavefronts:
+// H % 128 == 0 and Ie % 64 == 0.  One workgroup per (expert, 16 rows), eight wavefronts:
 //   fc_in   v_mfma_f32_16x16x128_f8f6f4 on the fp8 bytes as they are (products of fp8 values are exact in the fp32
 //           accumulator; the two per-tensor descales multiply the sum).  The 16 hidden rows sit in LDS, weight rows
 //           come from L2 as 32-byte runs per lane.

@@ -979,6 +979,125 @@ __global__ __launch_bounds__(kMfmaThreads) void k_grouped_gelu_fp8_mfma32(const 
     }
 }
 
+// ---- the bf16 sibling on the matrix cores -------------------------------------------------------------
+// moe_grouped_expert_forward_bf16 in the 16-row form above: both projections are v_mfma_f32_16x16x32_bf16 (products
+// of two bf16 values are exact in the fp32 accumulator), fc_out again on the two-term split of the fp32 GELU output.
+// A 128-byte run of a weight row is 64 elements: a lane fetches 32 bytes = two k-blocks of 8.  H % 64 == 0,
+// Ie % 64 == 0.
+__global__ __launch_bounds__(kMfmaThreads) void k_grouped_gelu_bf16_mfma(const uint16_t* __restrict__ hidden, const float* __restrict__ route_weights,
+                                                                         const int* __restrict__ counts, const int* __restrict__ row_indices,
+                                                                         const uint16_t* __restrict__ fc_in_w, const uint16_t* __restrict__ fc_out_w,
+                                                                         uint16_t* __restrict__ mixed, int rows, int H, int Ie, int E,
+                                                                         int tiles_per_expert) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    constexpr int kWaves = kMfmaThreads / 64;
+    const int hs = H + 8;                           // row strides in elements: neighbouring rows 16 bytes apart in the banks
+    const int as = Ie + 8;
+    uint16_t* sh_hidden = reinterpret_cast<uint16_t*>(smem);                          // [16][hs]
+    uint16_t* sh_hi = sh_hidden + kMfmaRows * hs;                                     // [16][as] bf16 head of gelu
+    uint16_t* sh_lo = sh_hi + kMfmaRows * as;                                         // [16][as] bf16 remainder
+    const int xcd = blockIdx.x % kXcdCount, slot = blockIdx.x / kXcdCount;
+    const int e = (slot / tiles_per_expert) * kXcdCount + xcd, tile = slot % tiles_per_expert;
+    if (e >= E) return;
+    const int first = tile * kMfmaRows, n_active = counts[e];
+    if (first >= n_active) return;
+    const int n_rows = min(kMfmaRows, n_active - first);
+    const int* my_rows = row_indices + static_cast<size_t>(e) * rows + first;
+    const uint16_t* w_in = fc_in_w + static_cast<size_t>(e) * H * Ie;
+    const uint16_t* w_out = fc_out_w + static_cast<size_t>(e) * Ie * H;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, t = lane & 15, g = lane >> 4;
+
+    const int vec_per_row = H / 8;
+    for (int i = threadIdx.x; i < kMfmaRows * vec_per_row; i += kMfmaThreads) {
+        const int r = i / vec_per_row, c = i % vec_per_row;
+        const int src = my_rows[min(r, n_rows - 1)];
+        *reinterpret_cast<uint4*>(sh_hidden + r * hs + c * 8) =
+            *reinterpret_cast<const uint4*>(hidden + static_cast<size_t>(src) * H + c * 8);
+    }
+    __syncthreads();
+
+    // one projection's inner product for a block of 16 weight rows: step s covers k = 64 s + 16 g .. + 15 of this lane
+    auto load2 = [](const uint16_t* p, v8bf& a, v8bf& b) {
+        a = *reinterpret_cast<const v8bf*>(p);
+        b = *reinterpret_cast<const v8bf*>(p + 8);
+    };
+    const int in_steps = H / 64;
+    for (int n0 = wave * 16; n0 < Ie; n0 += kWaves * 16) {
+        v4f acc0 = {0.0f, 0.0f, 0.0f, 0.0f}, acc1 = {0.0f, 0.0f, 0.0f, 0.0f};
+        const uint16_t* wr = w_in + static_cast<size_t>(n0 + t) * H + 16 * g;
+        const uint16_t* hr = sh_hidden + t * hs + 16 * g;
+        v8bf wa[kMfmaDepth], wb[kMfmaDepth];
+#pragma unroll
+        for (int j = 0; j < kMfmaDepth; ++j)
+            if (j < in_steps) load2(wr + j * 64, wa[j], wb[j]);
+        for (int s0 = 0; s0 < in_steps; s0 += kMfmaDepth) {
+#pragma unroll
+            for (int j = 0; j < kMfmaDepth; ++j) {
+                const int st = s0 + j;
+                if (st < in_steps) {
+                    const v8bf ca = wa[j], cb = wb[j];
+                    if (st + kMfmaDepth < in_steps) load2(wr + (st + kMfmaDepth) * 64, wa[j], wb[j]);
+                    v8bf xa, xb;
+                    load2(hr + st * 64, xa, xb);
+                    acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ca, xa, acc0, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cb, xb, acc1, 0, 0, 0);
+                }
+            }
+        }
+        uint32_t hb[4], lb[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float act = gelu_fwd(acc0[r] + acc1[r]);
+            hb[r] = __float_as_uint(act) & 0xffff0000u;
+            lb[r] = f32_to_bf16(act - __uint_as_float(hb[r]));
+        }
+        const int at = t * as + n0 + 4 * g;
+        *reinterpret_cast<uint2*>(sh_hi + at) = make_uint2((hb[0] >> 16) | hb[1], (hb[2] >> 16) | hb[3]);
+        *reinterpret_cast<uint2*>(sh_lo + at) = make_uint2(lb[0] | (lb[1] << 16), lb[2] | (lb[3] << 16));
+    }
+    __syncthreads();
+
+    const int out_steps = Ie / 64;
+    const bool live = t < n_rows;
+    const int row = live ? my_rows[t] : 0;
+    const float rw = live ? route_weights[static_cast<size_t>(row) * E + e] : 0.0f;
+    const uint16_t* ah = sh_hi + t * as + 16 * g;
+    const uint16_t* al = sh_lo + t * as + 16 * g;
+    for (int h0 = wave * 16; h0 < H; h0 += kWaves * 16) {
+        v4f acc_hi = {0.0f, 0.0f, 0.0f, 0.0f}, acc_lo = {0.0f, 0.0f, 0.0f, 0.0f};
+        auto* quad = reinterpret_cast<unsigned long long*>(mixed + static_cast<size_t>(row) * H + h0 + 4 * g);
+        const unsigned long long before = live ? __builtin_nontemporal_load(quad) : 0ull;
+        const uint16_t* wr = w_out + static_cast<size_t>(h0 + t) * Ie + 16 * g;
+        v8bf wa[kMfmaDepth], wb[kMfmaDepth];
+#pragma unroll
+        for (int j = 0; j < kMfmaDepth; ++j)
+            if (j < out_steps) load2(wr + j * 64, wa[j], wb[j]);
+        for (int s0 = 0; s0 < out_steps; s0 += kMfmaDepth) {
+#pragma unroll
+            for (int j = 0; j < kMfmaDepth; ++j) {
+                const int st = s0 + j;
+                if (st < out_steps) {
+                    const v8bf ca = wa[j], cb = wb[j];
+                    if (st + kMfmaDepth < out_steps) load2(wr + (st + kMfmaDepth) * 64, wa[j], wb[j]);
+                    v8bf ha, hbv, la, lbv;
+                    load2(ah + st * 64, ha, hbv);
+                    load2(al + st * 64, la, lbv);
+                    acc_hi = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ca, ha, acc_hi, 0, 0, 0);
+                    acc_lo = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ca, la, acc_lo, 0, 0, 0);
+                    acc_hi = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cb, hbv, acc_hi, 0, 0, 0);
+                    acc_lo = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cb, lbv, acc_lo, 0, 0, 0);
+                }
+            }
+        }
+        if (live) {
+            float v[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) v[r] = rw * (acc_hi[r] + acc_lo[r]);
+            atomic_add_bf16x4(quad, before, v);
+        }
+    }
+}
+
 unsigned grid_for(size_t items) {
     const size_t b = (items + kThreads - 1) / kThreads;
     return static_cast<unsigned>(b < 1 ? 1 : (b > 8192 ? 8192 : b));
@@ -1438,6 +1557,22 @@ int cf_moe_grouped_expert_forward_bf16(const uint16_t* d_hidden, const float* d_
     if (rows < 0 || H < 0 || Ie < 0 || num_experts < 0) return CF_ERR_INVALID_ARG;
     if (rows == 0 || num_experts == 0 || H == 0 || Ie == 0) return CF_OK;
     if (!d_hidden || !d_route_weights || !d_counts || !d_row_indices || !d_fc_in_w || !d_fc_out_w || !d_mixed) return CF_ERR_INVALID_ARG;
+    // the matrix-core form where the shapes are whole MFMA steps and its tile fits the LDS
+    const size_t smem_mfma = 2u * kMfmaRows * (static_cast<size_t>(H) + 8) + 4u * kMfmaRows * (static_cast<size_t>(Ie) + 8);
+    if (H % 64 == 0 && Ie % 64 == 0 && smem_mfma <= 160 * 1024 && aligned16(d_hidden) && aligned16(d_fc_in_w) && aligned16(d_fc_out_w) &&
+        (reinterpret_cast<uintptr_t>(d_mixed) & 7u) == 0) {
+        static std::once_flag once_mfma;
+        static hipError_t err_mfma = hipSuccess;
+        std::call_once(once_mfma, [] {
+            err_mfma = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_grouped_gelu_bf16_mfma),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        });
+        if (err_mfma != hipSuccess) return static_cast<int>(err_mfma);
+        const int tiles = (rows + kMfmaRows - 1) / kMfmaRows;
+        k_grouped_gelu_bf16_mfma<<<kXcdCount * ((num_experts + kXcdCount - 1) / kXcdCount) * tiles, kMfmaThreads, smem_mfma, as_stream(stream)>>>(
+            d_hidden, d_route_weights, d_counts, d_row_indices, d_fc_in_w, d_fc_out_w, d_mixed, rows, H, Ie, num_experts, tiles);
+        return launch_status();
+    }
     const size_t smem = sizeof(float) * static_cast<size_t>(kGeluRows) * (kGeluChunk + Ie);
     if (smem > 160 * 1024) return CF_ERR_UNSUPPORTED;
     static std::once_flag once;

@@ -274,8 +274,11 @@ def main():
     iters, args.iters = args.iters, 5
     mfma("moe_grouped_expert_forward_fp8 form (fp32 GELU kept, MFMA)", f"T={T} E={E} k={k}", 4.0 * total * Ie * H,
          lambda: cf.cf_moe_grouped_expert_forward_fp8(hq, one, 0, rw, counts, offs, idx, wg, one, wd, one, mixed, T, H, Ie, E, total, st))
+    hb16 = bf16(T, H); wi16 = bf16(E * Ie, H, sigma=0.02); wo16 = bf16(E * H, Ie, sigma=0.02)
+    mfma("moe_grouped_expert_forward_bf16 (the bf16 sibling, MFMA)", f"T={T} E={E} k={k}", 4.0 * total * Ie * H,
+         lambda: cf.cf_moe_grouped_expert_forward_bf16(hb16, rw, counts, offs, idx, wi16, wo16, mixed, T, H, Ie, E, total, st))
     args.iters = iters
-    del ws3, gq
+    del ws3, gq, hb16, wi16, wo16
 
     # ---- the selected-expert backward's custom kernels at the same size --------------------------------
     dmixed = bf16(T, H)

@@ -451,7 +451,9 @@ int cf_moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_fcin_
 /* moe_grouped_expert_forward_bf16, kernels.hpp:400-407: the same device-scheduled expert bank on
  * bf16 hidden states and bf16 weights (fc_in_w [E,Ie,H], fc_out_w [E,H,Ie]), no descales; fp32
  * accumulation, exact-erf GELU kept in fp32, compare-and-swap accumulation into d_mixed.  The
- * non-FP8 sibling: fp32 FMA kernel in the reference's loop form, any shape. */
+ * non-FP8 sibling: bf16 MFMA for both projections when H % 64 == 0, Ie % 64 == 0, the operands are
+ * 16-byte aligned and d_mixed 8-byte aligned (16-row tiles); an fp32 FMA kernel in the reference's
+ * loop form otherwise. */
 int cf_moe_grouped_expert_forward_bf16(const uint16_t* d_hidden, const float* d_route_weights,
                                        const int* d_counts, const int* d_offsets,
                                        const int* d_row_indices, const uint16_t* d_fc_in_w,

@@ -442,7 +442,9 @@ def test_grouped_gelu_expert_bank_reference_form_config5_size(cf, dev):
     assert np.all(np.abs(got - ref) <= (b.k + 1) * 2.0 ** -8 * (np.abs(start) + np.abs(ref) + 2.0 * typical))
 
 
-@pytest.mark.parametrize("rows,E,k,H,Ie", [(90, 4, 2, 96, 72), (300, 6, 3, 256, 320), (33, 3, 3, 40, 1408)])
+@pytest.mark.parametrize("rows,E,k,H,Ie", [(90, 4, 2, 96, 72), (33, 3, 3, 40, 1408),
+                                            # H % 64 == 0 and Ie % 64 == 0: the matrix-core form
+                                            (300, 6, 3, 256, 320), (70, 3, 3, 2048, 1408), (200, 4, 2, 64, 64), (21, 5, 2, 192, 448)])
 def test_grouped_gelu_expert_bank_bf16_sibling(cf, dev, rows, E, k, H, Ie):
     """moe_grouped_expert_forward_bf16: bf16 hidden states and weights, float GELU intermediate, bf16 CAS accumulate."""
     case(f"grouped gelu bank, bf16 sibling rows={rows} E={E} k={k} H={H} Ie={Ie}")

@@ -90,3 +90,66 @@ def test_delayed_scaling_step_replays_from_a_graph(cf, dev):
         assert torch.equal(q, want_q), f"replay {i}"
         for a, b in zip(eager, captured):
             assert torch.equal(a, b), f"replay {i}"
+
+
+def test_moe_layer_replays_from_a_graph(cf, dev):
+    """Routing, row lists, offsets and both one-call expert banks (SwiGLU; GELU with re-quantized activations) in one
+    captured graph: every buffer the routing fills is consumed on the device, so a replay on new logits and new hidden
+    states must reproduce the eager run bit for bit."""
+    import ctypes
+    case("graph capture: top-k route -> row lists -> offsets -> SwiGLU bank -> GELU bank")
+    T, E, k, H, Ie = 768, 8, 2, 256, 384
+    total = T * k
+    g = torch.Generator(device=dev); g.manual_seed(23)
+    wg, wgd = fp8_weights(E * Ie, H, dev, g); wu, wud = fp8_weights(E * Ie, H, dev, g); wd, wdd = fp8_weights(E * H, Ie, dev, g)
+    one = torch.full((1,), 0.02, device=dev)
+    logits = torch.empty((T, E), device=dev)
+    rw = torch.empty((T, E), device=dev)
+    hq = torch.empty((T, H), dtype=torch.uint8, device=dev); hd = torch.empty(T, device=dev)
+    counts = torch.zeros(E, dtype=torch.int32, device=dev); offs = torch.zeros(E, dtype=torch.int32, device=dev)
+    idx = torch.zeros(E * T, dtype=torch.int32, device=dev)
+    out_swiglu = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+    out_gelu = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+    s1, s2 = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    assert cf.raw_cf_moe_grouped_swiglu_workspace_bytes(total, E, H, Ie, ctypes.byref(s1)) == 0
+    assert cf.raw_cf_moe_grouped_gelu_workspace_bytes(T, total, E, H, Ie, ctypes.byref(s2)) == 0
+    ws1 = torch.empty(s1.value + 256, dtype=torch.uint8, device=dev); p1 = ws1.data_ptr() + (-ws1.data_ptr()) % 256
+    ws2 = torch.empty(s2.value + 256, dtype=torch.uint8, device=dev); p2 = ws2.data_ptr() + (-ws2.data_ptr()) % 256
+
+    def step():
+        s = stream()
+        rw.copy_(logits)
+        out_swiglu.zero_(); out_gelu.zero_()
+        cf.cf_moe_topk_route_f32(rw, T, E, k, s, None, None, 1)
+        cf.cf_moe_build_expert_row_lists(rw, counts, idx, T, E, s)
+        cf.cf_moe_expert_offsets_from_counts(counts, offs, E, s)
+        cf.cf_moe_grouped_swiglu_forward_fp8(hq, hd, rw, counts, offs, idx, wg, wgd, wu, wud, wd, wdd, out_swiglu, T, H, Ie, E, total,
+                                             p1, s1.value, s)
+        cf.cf_moe_grouped_gelu_forward_fp8(hq, one, 0, rw, counts, offs, idx, wg, one, wd, one, out_gelu, T, H, Ie, E, total,
+                                           p2, s2.value, s)
+
+    def new_inputs(i):
+        logits.copy_(torch.randn(T, E, device=dev, generator=g))
+        x = torch.randn(T, H, device=dev, generator=g) * (1.0 + i)
+        amax = x.abs().amax(dim=1).clamp_min(1e-12)
+        hq.copy_((x * (448.0 / amax)[:, None]).to(torch.float8_e4m3fn).view(torch.uint8)); hd.copy_(amax / 448.0)
+
+    new_inputs(0); step(); torch.cuda.synchronize()                 # warm-up outside the capture
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for i in range(4):
+        new_inputs(i)
+        step()
+        torch.cuda.synchronize()
+        want = (out_swiglu.clone(), out_gelu.clone(), counts.clone(), rw.clone())
+        assert int(counts.sum()) == total
+        out_swiglu.fill_(7.0); out_gelu.fill_(7.0); counts.fill_(-1); rw.fill_(0.5)
+        scratch = torch.randn(1 << 20, device=dev).sum()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(counts, want[2]) and torch.equal(rw, want[3]), f"replay {i}"
+        assert torch.equal(out_swiglu.view(torch.int16), want[0].view(torch.int16)), f"replay {i}"
+        assert torch.equal(out_gelu.view(torch.int16), want[1].view(torch.int16)), f"replay {i}"
+        assert float(scratch) == float(scratch)

@@ -489,3 +489,18 @@ def test_grouped_gelu_reference_form_ragged_and_empty_experts(cf, dev, rows, E, 
     assert np.sqrt(((got - ref) ** 2).sum() / (ref ** 2).sum()) <= 4e-3
     typical = np.sqrt(((ref - start) ** 2).mean())
     assert np.all(np.abs(got - ref) <= (k + 1) * 2.0 ** -8 * (np.abs(start) + np.abs(ref) + 2.0 * typical))
+
+
+def test_gelu_quantize_rows_argument_errors(cf, dev):
+    case("gelu + per-row quantize argument checks")
+    z = torch.zeros(64, dtype=torch.bfloat16, device=dev)
+    q = torch.zeros(64, dtype=torch.uint8, device=dev)
+    s = torch.zeros(4, device=dev)
+    assert cf.raw_cf_gelu_quantize_rows_e4m3(None, 4, 16, q.data_ptr(), s.data_ptr(), s.data_ptr(), None) == -1
+    assert cf.raw_cf_gelu_quantize_rows_e4m3(z.data_ptr(), 4, 16, None, s.data_ptr(), s.data_ptr(), None) == -1
+    assert cf.raw_cf_gelu_quantize_rows_e4m3(z.data_ptr(), 4, 16, q.data_ptr(), None, s.data_ptr(), None) == -1
+    assert cf.raw_cf_gelu_quantize_rows_e4m3(z.data_ptr(), -1, 16, q.data_ptr(), s.data_ptr(), s.data_ptr(), None) == -1
+    assert cf.raw_cf_gelu_quantize_rows_e4m3(None, 0, 16, None, None, None, None) == 0
+    # K = 0: nothing to convert, the scales of an empty row are those of amax = 0
+    assert cf.raw_cf_gelu_quantize_rows_e4m3(None, 4, 0, None, s.data_ptr(), s.data_ptr(), None) == 0
+    torch.cuda.synchronize()

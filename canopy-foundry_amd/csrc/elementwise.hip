@@ -30,7 +30,7 @@ __global__ __launch_bounds__(kThreads) void k_swiglu(const uint16_t* __restrict_
             const uint4 u = reinterpret_cast<const uint4*>(up)[i];
             uint4 o;
             o.x = swiglu2(g.x, u.x); o.y = swiglu2(g.y, u.y); o.z = swiglu2(g.z, u.z); o.w = swiglu2(g.w, u.w);
-            reinterpret_cast<uint4*>(out)[i] = o;
+            store_stream16(reinterpret_cast<uint4*>(out) + i, o);
         }
         done = nvec * 8;
     }

@@ -129,7 +129,7 @@ __global__ __launch_bounds__(kCeThreads) void k_ce_rows(const CeArgs p) {
                                           ce_grad(bf16_hi(w[k]), row_max, inv_sum, inv_n, e + 1 == label, llp));
                 }
             }
-            reinterpret_cast<uint4*>(grow)[c] = make_uint4(o[0], o[1], o[2], o[3]);
+            store_stream16(reinterpret_cast<uint4*>(grow) + c, make_uint4(o[0], o[1], o[2], o[3]));
             if constexpr (QUANT) {
                 // src/trainer.cu:8053: the E5M2 quantize of the bf16 gradient with the slot's previous scale, amax recorded
                 const uint32_t acc8 = pk_absmax(pk_absmax(pk_absmax(pk_absmax(0u, o[0]), o[1]), o[2]), o[3]);
@@ -220,7 +220,7 @@ __global__ __launch_bounds__(kCeThreads) void k_ce_rows_stream(const CeArgs p) {
                                       ce_grad(bf16_hi(w[k]), row_max, inv_sum, inv_n, e + 1 == label, llp));
             }
         }
-        reinterpret_cast<uint4*>(grow)[c] = make_uint4(o[0], o[1], o[2], o[3]);
+        store_stream16(reinterpret_cast<uint4*>(grow) + c, make_uint4(o[0], o[1], o[2], o[3]));
         if constexpr (QUANT) {
             absacc = pk_absmax(pk_absmax(pk_absmax(pk_absmax(absacc, o[0]), o[1]), o[2]), o[3]);
             uint2 q;

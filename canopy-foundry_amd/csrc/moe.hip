@@ -227,7 +227,7 @@ __global__ __launch_bounds__(kThreads) void k_gather_rows16(const uint4* __restr
     for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total;
          i += static_cast<size_t>(gridDim.x) * blockDim.x) {
         const int r = static_cast<int>(i / vec_per_row), c = static_cast<int>(i % vec_per_row);
-        dst[i] = src[static_cast<size_t>(row_indices[r]) * vec_per_row + c];
+        store_stream16(dst + i, src[static_cast<size_t>(row_indices[r]) * vec_per_row + c]);
     }
 }
 template <typename T>
@@ -348,7 +348,7 @@ __device__ __forceinline__ void combine_rows(uint16_t* __restrict__ mrow, const 
                     }
                 }
             }
-            reinterpret_cast<uint4*>(mrow)[c] = mv;
+            store_stream16(reinterpret_cast<uint4*>(mrow) + c, mv);
         }
     } else {
         for (int h = t; h < H; h += blockDim.x) {

@@ -68,7 +68,7 @@ __global__ __launch_bounds__(kThreads) void k_route_grad_half_wave(const RouteGr
                 for (int j = 0; j < 8; ++j) part[j] = __builtin_fmaf(bf16_elem(av, j), bf16_elem(bv, j), part[j]);
             }
             if constexpr (SCALE)
-                d[s * 32] = make_uint4(scale2_bf16(av.x, w), scale2_bf16(av.y, w), scale2_bf16(av.z, w), scale2_bf16(av.w, w));
+                store_stream16(d + s * 32, make_uint4(scale2_bf16(av.x, w), scale2_bf16(av.y, w), scale2_bf16(av.z, w), scale2_bf16(av.w, w)));
         }
         if constexpr (DOT) {
             // strides 128, 64, 32, 16, 8 of the halving tree
@@ -157,9 +157,9 @@ __global__ __launch_bounds__(kThreads) void k_gelu_vec(const uint4* __restrict__
         const uint4 v = x[i];
         if constexpr (BWD) {
             const uint4 u = g[i];
-            out[i] = make_uint4(gelu_bwd2(v.x, u.x), gelu_bwd2(v.y, u.y), gelu_bwd2(v.z, u.z), gelu_bwd2(v.w, u.w));
+            store_stream16(out + i, make_uint4(gelu_bwd2(v.x, u.x), gelu_bwd2(v.y, u.y), gelu_bwd2(v.z, u.z), gelu_bwd2(v.w, u.w)));
         } else {
-            out[i] = make_uint4(gelu2(v.x), gelu2(v.y), gelu2(v.z), gelu2(v.w));
+            store_stream16(out + i, make_uint4(gelu2(v.x), gelu2(v.y), gelu2(v.z), gelu2(v.w)));
         }
     }
 }

@@ -338,7 +338,7 @@ __global__ __launch_bounds__(256) void k_norm_row_wave(const NormArgs p, int row
     }
 #pragma unroll
     for (int j = 0; j < J; ++j) {
-        if (p.normed) *reinterpret_cast<uint4*>(p.normed + base + 512 * j) = v[j];
+        if (p.normed) store_stream16(p.normed + base + 512 * j, v[j]);
         if constexpr (QMODE != Q_NONE) {
             uint2 o;
             if (finite) {     // every product is finite: no NaN code to restore
@@ -348,7 +348,7 @@ __global__ __launch_bounds__(256) void k_norm_row_wave(const NormArgs p, int row
                 o.x = cvt4_fp8<E5M2>(bf16_lo(v[j].x) * qs, bf16_hi(v[j].x) * qs, bf16_lo(v[j].y) * qs, bf16_hi(v[j].y) * qs);
                 o.y = cvt4_fp8<E5M2>(bf16_lo(v[j].z) * qs, bf16_hi(v[j].z) * qs, bf16_lo(v[j].w) * qs, bf16_hi(v[j].w) * qs);
             }
-            *reinterpret_cast<uint2*>(p.q + base + 512 * j) = o;
+            store_stream8(p.q + base + 512 * j, o);
         }
     }
 }

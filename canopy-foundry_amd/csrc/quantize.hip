@@ -236,7 +236,7 @@ __global__ __launch_bounds__(kThreads) void k_quant(const uint16_t* __restrict__
         const size_t nvec = n / kVec;
         for (size_t i = tid; i < nvec; i += stride) {
             const Vec16 v = load16(x + i * kVec);
-            *reinterpret_cast<uint4*>(out + i * kVec) = quant16_track<E5M2, RECORD>(v, s, s_finite, local_bits, local);
+            store_stream16(out + i * kVec, quant16_track<E5M2, RECORD>(v, s, s_finite, local_bits, local));
         }
         done = nvec * kVec;
     }
@@ -279,7 +279,7 @@ __global__ __launch_bounds__(kAmaxThreads) void k_quant_delayed_step(const uint1
         const size_t nvec = n / kVec;
         for (size_t i = tid; i < nvec; i += stride) {
             const Vec16 v = load16(x + i * kVec);
-            *reinterpret_cast<uint4*>(out + i * kVec) = quant16_track<E5M2, true>(v, s, s_finite, local_bits, local);
+            store_stream16(out + i * kVec, quant16_track<E5M2, true>(v, s, s_finite, local_bits, local));
         }
         done = nvec * kVec;
     }
@@ -384,7 +384,7 @@ __global__ __launch_bounds__(kThreads) void k_quant_rows(const uint16_t* __restr
 #pragma unroll
     for (int s = 0; s < MAXS; ++s) {
         const int k = (s * 64 + lane) * kVec;
-        if (k < K) *reinterpret_cast<uint4*>(outr + k) = finite ? quant16_finite<E5M2>(v[s], sc) : quant16<E5M2>(v[s], sc);
+        if (k < K) store_stream16(outr + k, finite ? quant16_finite<E5M2>(v[s], sc) : quant16<E5M2>(v[s], sc));
     }
 }
 
@@ -435,7 +435,7 @@ __global__ __launch_bounds__(kThreads) void k_quant_rows_block(const uint16_t* _
 #pragma unroll
     for (int s = 0; s < MAXS; ++s) {
         const int k = (s * kThreads + tid) * kVec;
-        if (k < K) *reinterpret_cast<uint4*>(outr + k) = finite ? quant16_finite<E5M2>(v[s], sc) : quant16<E5M2>(v[s], sc);
+        if (k < K) store_stream16(outr + k, finite ? quant16_finite<E5M2>(v[s], sc) : quant16<E5M2>(v[s], sc));
     }
 }
 
@@ -495,7 +495,7 @@ __global__ __launch_bounds__(kThreads) void k_quant_1x128(const uint16_t* __rest
         const float sc = 448.0f / a;
         if (live) {
             if ((i & 7) == 0) { scale[i >> 3] = sc; descale[i >> 3] = a / 448.0f; }
-            *reinterpret_cast<uint4*>(out + i * kVec) = finite ? quant16_finite<false>(v, sc) : quant16<false>(v, sc);
+            store_stream16(out + i * kVec, finite ? quant16_finite<false>(v, sc) : quant16<false>(v, sc));
         }
     }
 }
@@ -559,7 +559,7 @@ __global__ __launch_bounds__(kThreads) void k_quant_128x128(const uint16_t* __re
         for (int p = 0; p < 4; ++p) {
             const int r = r0 + p * 32 + tr;
             if (r < rows)
-                *reinterpret_cast<uint4*>(out + static_cast<size_t>(r) * K + k0 + tc) = finite ? quant16_finite<false>(v[p], sc) : quant16<false>(v[p], sc);
+                store_stream16(out + static_cast<size_t>(r) * K + k0 + tc, finite ? quant16_finite<false>(v[p], sc) : quant16<false>(v[p], sc));
         }
     } else {
         const int klen = min(128, K - k0), rlen = min(128, rows - r0);

@@ -70,7 +70,7 @@ __global__ __launch_bounds__(kThreads) void k_transpose_tiled(const void* __rest
     for (int i = 0; i < 8; ++i) {
         const size_t idx = static_cast<size_t>(r0 + ty * 8 + i) * C + c0 + tx * 8;
         rowb[i] = load_row8<QUANT>(in, idx, s);
-        if constexpr (DUAL) *reinterpret_cast<uint2*>(straight + idx) = rowb[i];
+        if constexpr (DUAL) store_stream8(straight + idx, rowb[i]);
     }
     // columns 0..3 come from the .x words, 4..7 from the .y words; rows 0..3 and 4..7 give the two dwords
     const bool odd = tx & 1;
@@ -93,7 +93,7 @@ __global__ __launch_bounds__(kThreads) void k_transpose_tiled(const void* __rest
     for (int p = 0; p < 4; ++p) {
         const int c = p * 32 + rr;
         const uint4 v = *reinterpret_cast<const uint4*>(&tile[c * kPitch + ((chunk ^ (c >> 4)) << 4)]);
-        *reinterpret_cast<uint4*>(outT + static_cast<size_t>(c0 + c) * R + r0 + chunk * 16) = v;
+        store_stream16(outT + static_cast<size_t>(c0 + c) * R + r0 + chunk * 16, v);
     }
 }
 

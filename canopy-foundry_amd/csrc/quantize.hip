@@ -319,7 +319,7 @@ __global__ __launch_bounds__(kThreads) void k_quant_f32(const float* __restrict_
         const size_t nvec = n / 4;
         for (size_t i = tid; i < nvec; i += stride) {
             const float4 v = reinterpret_cast<const float4*>(x)[i];
-            reinterpret_cast<uint32_t*>(out)[i] = cvt4_fp8<E5M2>(v.x * s, v.y * s, v.z * s, v.w * s);
+            __builtin_nontemporal_store(cvt4_fp8<E5M2>(v.x * s, v.y * s, v.z * s, v.w * s), reinterpret_cast<uint32_t*>(out) + i);
         }
         done = nvec * 4;
     }

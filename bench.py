@@ -131,20 +131,24 @@ def main():
     y = torch.empty((M, K), dtype=torch.bfloat16, device=dev)
 
     ev = lambda: torch.cuda.Event(enable_timing=True)
-    marks = []
+    marks = []        # timed steps: one bracket, around the dominant kernel
+    detail = []       # breakdown steps (after the timed region): a bracket around every kernel
 
-    def step(timed):
-        e = [ev() for _ in range(5)] if timed else None
-        if timed: e[0].record()
+    def step(mode):
+        """mode 0: no events; 1: events around the gate/up GEMM only; 2: events around every kernel."""
+        e = [ev() for _ in range(5)] if mode else None
+        if mode == 2: e[0].record()
         cf.cf_fp8_quantize_rows(x, M, K, 0, xq, xs, xd, st)
-        if timed: e[1].record()
+        if mode: e[1].record()
         cf.cf_fp8_gemm_nt_bf16_ex(M, N, K, xq, K, 0, xd, wgq, K, wgd, 1, 2, None, wuq, wud, h, N, 0, st)
-        if timed: e[2].record()
+        if mode: e[2].record()
         cf.cf_fp8_quantize_rows(h, M, N, 0, hq, hs, hd, st)
-        if timed: e[3].record()
+        if mode == 2: e[3].record()
         cf.cf_fp8_gemm_nt_bf16_ex(M, K, N, hq, N, 0, hd, wdq, N, wdd, 1, 0, None, None, None, y, K, 0, st)
-        if timed:
+        if mode == 2:
             e[4].record()
+            detail.append(e)
+        elif mode == 1:
             marks.append(e)
 
     if args.traffic_calibration:
@@ -156,15 +160,20 @@ def main():
         del src, dst
 
     for _ in range(args.warmup):
-        step(False)
+        step(0)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        step(True)
+        step(1)
     torch.cuda.synchronize()
     t1 = time.perf_counter()
 
     ms_per_step = (t1 - t0) * 1e3 / args.steps
+    # per-kernel breakdown: the same steps again with a bracket around every kernel, outside the timed region
+    # (each bracket costs a launch gap, which the timed steps should not pay four times over)
+    for _ in range(min(args.steps, 20)):
+        step(2)
+    torch.cuda.synchronize()
 
     def back_to_back(fn, launches=20, batches=3):
         """ms per launch of `fn` launched back to back (no other kernel, no event between the launches)."""
@@ -183,7 +192,8 @@ def main():
     # that is a quarter of a 20 us kernel)
     qx_alone_ms = back_to_back(lambda: cf.cf_fp8_quantize_rows(x, M, K, 0, xq, xs, xd, st))
     qh_alone_ms = back_to_back(lambda: cf.cf_fp8_quantize_rows(h, M, N, 0, hq, hs, hd, st))
-    seg = [sum(e[i].elapsed_time(e[i + 1]) for e in marks) / len(marks) for i in range(4)]   # ms
+    seg = [sum(e[i].elapsed_time(e[i + 1]) for e in detail) / len(detail) for i in range(4)]   # ms
+    seg[1] = sum(e[1].elapsed_time(e[2]) for e in marks) / len(marks)       # the dominant kernel: from the timed steps
     flop_gateup = 2.0 * 2.0 * M * N * K
     flop_down = 2.0 * M * K * N
     total_flop = flop_gateup + flop_down

@@ -270,6 +270,22 @@ __global__ __launch_bounds__(kAmaxThreads) void k_quant_delayed_step(const uint1
     __shared__ float sh[kAmaxThreads / 64];
     const float s = *d.scale;
     const bool s_finite = fabsf(s) < __uint_as_float(0x7f800000u);
+    // What the workgroup that arrives last needs of the slot's state is read now, by every workgroup's first lane, so
+    // that no chain of dependent loads is left for the end: the state only changes in that last step, i.e. between
+    // launches.  pre_max = the history maximum over the entries the update will look at, without the one it overwrites.
+    float pre_descale = 0.0f, pre_max = 0.0f;
+    int pre_cursor = 0, pre_count = 0;
+    if (threadIdx.x == 0) {
+        pre_descale = *d.descale;
+        if (d.history_len > 0) {
+            pre_cursor = *d.cursor;
+            pre_count = *d.count;
+            if (pre_cursor < 0 || pre_cursor >= d.history_len) pre_cursor = 0;
+            if (pre_count < d.history_len) ++pre_count;
+            for (int i = 0; i < pre_count; ++i)
+                if (i != pre_cursor) pre_max = fmaxf(pre_max, d.history[i]);
+        }
+    }
     float local = 0.0f;
     int local_bits = 0;
     const size_t tid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
@@ -297,9 +313,19 @@ __global__ __launch_bounds__(kAmaxThreads) void k_quant_delayed_step(const uint1
             __threadfence();
             const float amax = __hip_atomic_load(d.running_amax, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             *d.scale_snapshot = s;                           // every workgroup read the same pair at its start
-            *d.descale_snapshot = *d.descale;
+            *d.descale_snapshot = pre_descale;
             *d.amax = amax;
-            delayed_scale_update(amax, d.fp8_max, d.scale, d.descale, d.history, d.history_len, d.cursor, d.count);
+            // delayed_scale_update() on the state read at the start
+            const float a = fmaxf(amax, 1e-12f);
+            float hist_max = a;
+            if (d.history_len > 0) {
+                d.history[pre_cursor] = a;
+                hist_max = fmaxf(pre_cursor < pre_count ? fmaxf(pre_max, a) : pre_max, 1e-12f);
+                *d.cursor = (pre_cursor + 1) % d.history_len;
+                *d.count = pre_count;
+            }
+            *d.scale = d.fp8_max / hist_max;
+            *d.descale = hist_max / d.fp8_max;
             *d.running_amax = 0.0f;
             *d.arrived = 0u;
         }

@@ -155,13 +155,11 @@ int cf_fp8_refresh_weight(const uint16_t* d_w, void* d_fwd8, void* d_bwd8, float
     const size_t n = static_cast<size_t>(in_dim) * out_dim;
     if (recompute_amax) CF_TRY(cf_fp8_amax_bf16(d_w, n, d_amax, stream));
     CF_TRY(cf_fp8_scale_from_amax(d_amax, CF_E4M3_MAX, d_scale, d_descale, stream));
-    if (stored_out_major) {
-        // stored [out,in]: the direct quantize is the forward layout, the transposed one the backward layout
-        CF_TRY(cf_fp8_quantize_e4m3(d_w, d_fwd8, d_scale, n, stream));
-        return cf_fp8_quantize_transpose_e4m3(d_w, d_bwd8, d_scale, out_dim, in_dim, stream);
-    }
-    CF_TRY(cf_fp8_quantize_e4m3(d_w, d_bwd8, d_scale, n, stream));
-    return cf_fp8_quantize_transpose_e4m3(d_w, d_fwd8, d_scale, in_dim, out_dim, stream);
+    // Both layouts from one read of the weight (the dual quantize gives the same bytes as the reference's two
+    // kernels, fp8_quantize_e4m3 and fp8_quantize_transpose_e4m3: same scale, same conversion).
+    if (stored_out_major)   // stored [out,in]: the direct quantize is the forward layout, the transposed one the backward layout
+        return cf_fp8_quant_and_transpose_e4m3(d_w, d_fwd8, d_bwd8, d_scale, out_dim, in_dim, stream);
+    return cf_fp8_quant_and_transpose_e4m3(d_w, d_bwd8, d_fwd8, d_scale, in_dim, out_dim, stream);
 }
 
 }  // extern "C"

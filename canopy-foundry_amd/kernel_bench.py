@@ -138,6 +138,12 @@ def main():
     w8 = u8(K, N)
     hbm("quantize_transpose_e4m3 (weight refresh)", f"{K}x{N}", 3.0 * w.numel(),
         lambda: cf.cf_fp8_quantize_transpose_e4m3(w, wt, sc, K, N, st))
+    # refresh_fp8_weights for one weight: amax, scale, and the two layouts (one read for both)
+    hbm("refresh_weight: amax + scale + fwd8 and bwd8 layouts", f"{K}x{N}", 6.0 * w.numel(),
+        lambda: cf.cf_fp8_refresh_weight(w, wt, w8, amax, sc, de, K, N, 0, 1, st))
+    hbm("  the reference's sequence: amax, scale, quantize, quantize-transpose", f"{K}x{N}", 6.0 * w.numel(),
+        lambda: (cf.cf_fp8_amax_bf16(w, w.numel(), amax, st), cf.cf_fp8_scale_from_amax(amax, 448.0, sc, de, st),
+                 cf.cf_fp8_quantize_e4m3(w, w8, sc, w.numel(), st), cf.cf_fp8_quantize_transpose_e4m3(w, wt, sc, K, N, st)))
     hq2 = u8(N, M)
     hbm("quant_and_transpose_e4m3 (dual, for wgrad)", f"{M}x{N}", 4.0 * h.numel(),
         lambda: cf.cf_fp8_quant_and_transpose_e4m3(h, hq, hq2, sc, M, N, st))

@@ -14,6 +14,7 @@
 // threads 8 l .. 8 l + 7; the tree's strides 128 .. 8 are exchanges across lanes (xor 16 .. 1), 4, 2, 1 in-lane.
 // Any other H takes a workgroup of T threads per row and the tree through LDS.
 #include "common.hpp"
+#include <mutex>
 
 namespace cf {
 namespace {
@@ -172,10 +173,43 @@ __global__ __launch_bounds__(kThreads) void k_gelu_scalar(const uint16_t* __rest
     }
 }
 
+// The forward for large tensors: bf16(gelu(x)) depends on the 16 bits of x only, so a workgroup that stays on its CU
+// builds the table of all 65536 results once (128 KiB of LDS) and looks every element up; erff costs about 40 vector
+// instructions per element and is what the plain kernel waits for.  Same bits.
+constexpr int kLutThreads = 1024;
+__global__ __launch_bounds__(kLutThreads) void k_gelu_lut(const uint4* __restrict__ x, uint4* __restrict__ out, size_t nvec) {
+    extern __shared__ uint16_t lut[];
+    for (int i = threadIdx.x; i < 65536; i += kLutThreads) lut[i] = f32_to_bf16(gelu_fwd(bf16_to_f32(static_cast<uint16_t>(i))));
+    __syncthreads();
+    auto look2 = [&](uint32_t pair) { return static_cast<uint32_t>(lut[pair & 0xffffu]) | (static_cast<uint32_t>(lut[pair >> 16]) << 16); };
+    for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec; i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+        const uint4 v = x[i];
+        store_stream16(out + i, make_uint4(look2(v.x), look2(v.y), look2(v.z), look2(v.w)));
+    }
+}
+
 template <bool BWD>
 int launch_gelu(const uint16_t* x, const uint16_t* g, uint16_t* out, size_t n, hipStream_t st) {
     const bool vec = aligned16(x) && aligned16(out) && (!BWD || aligned16(g));
     const size_t nvec = vec ? n / 8 : 0;
+    if constexpr (!BWD) {
+        if (nvec >= (8u << 20)) {        // 64 Mi elements: enough to pay for one table per CU
+            static std::once_flag once;
+            static hipError_t err = hipSuccess;
+            static int cus = 256;
+            std::call_once(once, [] {
+                err = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gelu_lut), hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+                int dev = 0, c = 0;
+                if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&c, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && c > 0)
+                    cus = c;
+            });
+            if (err != hipSuccess) return static_cast<int>(err);
+            k_gelu_lut<<<cus, kLutThreads, 128 * 1024, st>>>(reinterpret_cast<const uint4*>(x), reinterpret_cast<uint4*>(out), nvec);
+            if (nvec * 8 < n)
+                k_gelu_scalar<BWD><<<static_cast<unsigned>(min(ceil_div(n - nvec * 8, kThreads), 65536u)), kThreads, 0, st>>>(x, g, out, nvec * 8, n);
+            return launch_status();
+        }
+    }
     if (nvec)
         k_gelu_vec<BWD><<<static_cast<unsigned>(min(ceil_div(nvec, kThreads), 65536u)), kThreads, 0, st>>>(
             reinterpret_cast<const uint4*>(x), reinterpret_cast<const uint4*>(g), reinterpret_cast<uint4*>(out), nvec);

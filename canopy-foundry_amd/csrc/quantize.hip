@@ -6,6 +6,7 @@
 // two 128-bit loads and one 128-bit store, a wavefront reduces with xor
 // shuffles, and a workgroup issues one atomic.
 #include "common.hpp"
+#include <mutex>
 
 namespace cf {
 namespace {
@@ -414,6 +415,61 @@ __global__ __launch_bounds__(kThreads) void k_quant_rows(const uint16_t* __restr
     }
 }
 
+// GELU + per-row quantize for many rows: the exact-erf GELU of a bf16 value is a function of its 16 bits, so a
+// workgroup that stays on its CU builds the table of all 65536 results once (128 KiB of LDS, 64 erff per lane) and then
+// looks every element up instead of evaluating erff, which is what the plain form above waits for (about 40 vector
+// instructions per element).  Same bits: the table holds bf16(gelu_fwd(x)) for every x.
+constexpr int kLutThreads = 1024;
+__global__ __launch_bounds__(kLutThreads) void k_gelu_quant_rows_lut(const uint16_t* __restrict__ x, int rows, int K,
+                                                                     uint8_t* __restrict__ out, float* __restrict__ scale,
+                                                                     float* __restrict__ descale) {
+    extern __shared__ uint16_t lut[];
+    for (int i = threadIdx.x; i < 65536; i += kLutThreads) lut[i] = f32_to_bf16(gelu_fwd(bf16_to_f32(static_cast<uint16_t>(i))));
+    __syncthreads();
+    auto look2 = [&](uint32_t pair) { return static_cast<uint32_t>(lut[pair & 0xffffu]) | (static_cast<uint32_t>(lut[pair >> 16]) << 16); };
+    constexpr int MAXS = 4;
+    const int lane = threadIdx.x & 63;
+    const int waves = gridDim.x * (kLutThreads / 64);
+    for (int row = blockIdx.x * (kLutThreads / 64) + (threadIdx.x >> 6); row < rows; row += waves) {
+        const uint16_t* xr = x + static_cast<size_t>(row) * K;
+        uint8_t* outr = out + static_cast<size_t>(row) * K;
+        Vec16 v[MAXS];
+        uint32_t acc = 0;
+#pragma unroll
+        for (int s = 0; s < MAXS; ++s) {
+            const int k = (s * 64 + lane) * kVec;
+            if (k < K) v[s] = load16(xr + k);
+        }
+#pragma unroll
+        for (int s = 0; s < MAXS; ++s) {
+            const int k = (s * 64 + lane) * kVec;
+            if (k < K) {
+                v[s].lo = make_uint4(look2(v[s].lo.x), look2(v[s].lo.y), look2(v[s].lo.z), look2(v[s].lo.w));
+                v[s].hi = make_uint4(look2(v[s].hi.x), look2(v[s].hi.y), look2(v[s].hi.z), look2(v[s].hi.w));
+                acc = absmax16(acc, v[s]);
+            }
+        }
+        const int mbits = wave_absmax_bits(acc);
+        const bool finite = mbits < 0x7f80;
+        float m = __uint_as_float(static_cast<uint32_t>(mbits) << 16);
+        if (!finite) {                    // a float maximum ignores NaNs
+            float local = 0.0f;
+#pragma unroll
+            for (int s = 0; s < MAXS; ++s)
+                if ((s * 64 + lane) * kVec < K) local = fmaxf(local, amax16(v[s]));
+            m = wave_max(local);
+        }
+        const float a = fmaxf(m, 1e-12f);
+        const float sc = 448.0f / a;
+        if (lane == 0) { scale[row] = sc; descale[row] = a / 448.0f; }
+#pragma unroll
+        for (int s = 0; s < MAXS; ++s) {
+            const int k = (s * 64 + lane) * kVec;
+            if (k < K) store_stream16(outr + k, finite ? quant16_finite<false>(v[s], sc) : quant16<false>(v[s], sc));
+        }
+    }
+}
+
 // Long rows (4096 < K <= 32768): one workgroup of four wavefronts per row, the row still register-resident (four or
 // eight steps per lane instead of sixteen or more, so more wavefronts fit a SIMD); the row maximum crosses the
 // wavefronts through LDS.
@@ -693,6 +749,25 @@ int launch_quant_rows(const uint16_t* d_x, int rows, int K, void* d_out, float* 
     hipStream_t st = as_stream(stream);
     const bool vec = aligned16(d_x) && aligned16(d_out) && K % kVec == 0 && K > 0;
     const unsigned grid = ceil_div(rows, kThreads / 64);
+    if constexpr (GELU && !E5M2) {
+        // enough rows to pay for 256 tables of 65536 entries (each costs what 64 rows of 1024 elements cost directly)
+        if (vec && K <= 4 * 1024 && static_cast<size_t>(rows) * K >= (64u << 20)) {
+            static std::once_flag once;
+            static hipError_t err = hipSuccess;
+            static int cus = 256;
+            std::call_once(once, [] {
+                err = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gelu_quant_rows_lut),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+                int dev = 0, n = 0;
+                if (hipGetDevice(&dev) == hipSuccess &&
+                    hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+                    cus = n;
+            });
+            if (err != hipSuccess) return static_cast<int>(err);
+            k_gelu_quant_rows_lut<<<cus, kLutThreads, 128 * 1024, st>>>(d_x, rows, K, o, d_scale, d_descale);
+            return launch_status();
+        }
+    }
     if (vec && K <= 4 * 1024) k_quant_rows<E5M2, 4, GELU><<<grid, kThreads, 0, st>>>(d_x, rows, K, o, d_scale, d_descale);
     else if (vec && K <= 16 * 1024) k_quant_rows_block<E5M2, 4, GELU><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);
     else if (vec && K <= 32 * 1024) k_quant_rows_block<E5M2, 8, GELU><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);

@@ -262,3 +262,22 @@ def test_argument_errors(cf, dev):
     assert cf.raw_cf_moe_gather_scale_rows_bf16(z.data_ptr(), z.data_ptr(), zf.data_ptr(), zi.data_ptr(), 1, 3, 2, 8, None) != 0
     assert cf.raw_cf_gelu_forward_bf16(None, z.data_ptr(), 4, None) != 0
     assert cf.raw_cf_gelu_forward_bf16(None, None, 0, None) == 0
+
+
+def test_gelu_forward_table_form_matches_the_plain_kernel(cf, dev):
+    """Tensors of 64 Mi elements and more take the form that looks results up in a per-workgroup table; it must give
+    the bits of the plain kernel (run here on the same data in pieces below that size), an unaligned tail included."""
+    case("gelu forward, table form")
+    n = (64 << 20) + 8 * 1000 + 3
+    g = torch.Generator(device=dev); g.manual_seed(4)
+    x = (torch.randn(n, device=dev, generator=g) * 3.0).to(torch.bfloat16)
+    x[:65536] = torch.arange(65536, device=dev, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)   # every bf16 value
+    out = torch.empty_like(x)
+    cf.cf_gelu_forward_bf16(x, out, n, stream())
+    want = torch.empty_like(x)
+    piece = 16 << 20
+    for a in range(0, n, piece):
+        m = min(piece, n - a)
+        cf.cf_gelu_forward_bf16(x[a:a + m], want[a:a + m], m, stream())
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16))

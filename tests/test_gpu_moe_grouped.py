@@ -504,3 +504,25 @@ def test_gelu_quantize_rows_argument_errors(cf, dev):
     # K = 0: nothing to convert, the scales of an empty row are those of amax = 0
     assert cf.raw_cf_gelu_quantize_rows_e4m3(None, 4, 0, None, s.data_ptr(), s.data_ptr(), None) == 0
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("rows,K", [(49152, 1408), (16384, 4096)])
+def test_gelu_quantize_rows_table_form(cf, dev, rows, K):
+    """Enough rows for the form that looks GELU up in a per-workgroup table of all 65536 bf16 values: bytes and scales
+    must equal gelu_forward followed by the per-row quantize (both pinned against the oracle elsewhere), NaN and
+    infinity rows included."""
+    case(f"gelu + per-row quantize, table form rows={rows} K={K}")
+    g = torch.Generator(device=dev); g.manual_seed(rows + K)
+    x = (torch.randn(rows, K, device=dev, generator=g) * 2.5).to(torch.bfloat16)
+    x[0, :] = 0
+    x[1, 5] = float("nan"); x[2, 7] = float("inf"); x[3, 9] = float("-inf")
+    x[4] = torch.arange(K, device=dev).to(torch.bfloat16) - K / 2                  # large magnitudes
+    q = torch.zeros((rows, K), dtype=torch.uint8, device=dev); s = torch.zeros(rows, device=dev); d = torch.zeros(rows, device=dev)
+    cf.cf_gelu_quantize_rows_e4m3(x, rows, K, q, s, d, stream())
+    y = torch.empty_like(x)
+    cf.cf_gelu_forward_bf16(x, y, rows * K, stream())
+    q2 = torch.zeros_like(q); s2 = torch.zeros_like(s); d2 = torch.zeros_like(d)
+    cf.cf_fp8_quantize_rows(y, rows, K, 0, q2, s2, d2, stream())
+    torch.cuda.synchronize()
+    assert torch.equal(q, q2)
+    assert torch.equal(s.view(torch.int32), s2.view(torch.int32)) and torch.equal(d.view(torch.int32), d2.view(torch.int32))

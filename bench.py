@@ -12,7 +12,9 @@ All inputs are resident in HBM when the timed region starts.
 Prints ONE JSON line.  `value` is the step's GEMM work (2*M*N*K for gate, up and down) divided by the
 whole step time, quantize passes included.  `roofline` describes the dominant kernel (the fused
 gate/up GEMM) from HIP events recorded around that launch inside the timed region; `cpu_baseline`
-is the reference's CPU linear-forward idiom on config 1, timed on this host.
+is the reference's CPU linear-forward idiom on config 1, timed on this host.  Extra keys: the step replayed
+from a HIP graph, a plain-copy HBM ceiling for the quantize kernels, socket power and shader clock sampled
+during the timed region.
 """
 from __future__ import annotations
 
@@ -28,52 +30,151 @@ sys.path.insert(0, str(ROOT))
 
 FP8_PEAK_TFLOPS = 5000.0      # MI355X dense FP8 MFMA peak (published)
 HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E peak (published)
-# HBM bytes per launch of the fused gate/up GEMM from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# script, scaled by what the same counters read for a 1 GiB device copy (fetch x2.000, write x1.000):
-# 1,384,194 KiB read + 229,423 KiB written.  Not measurable from inside the process; re-measure when the kernel changes.
-GATEUP_HBM_TRAFFIC_BYTES = (1384194 + 229423) * 1024
+TRAFFIC_PROFILE = ROOT / "profiles" / "mlp_config2_hbm_traffic_pmc.txt"
+GEMM_SOURCES = [ROOT / "canopy-foundry_amd" / "csrc" / "gemm.hip", ROOT / "canopy-foundry_amd" / "csrc" / "common.hpp"]
 
 
-def cpu_baseline(sample_rows=3072):
-    """A bounded sample of config 2's gate projection on the host cores: the first `sample_rows` token rows
-    against the full gate weight [14336,4096].  Per-token / per-channel amax -> E4M3 quantize (oracle
-    rounding), dequantize, then Y = dequant(X).dequant(W)^T as one scalar fp32 dot per output with the rows
-    split over threads (the loop idiom of src/cpu_trainer.cpp:306-324), bf16 output."""
+def gemm_source_hash():
+    import hashlib
+    h = hashlib.sha256()
+    for f in GEMM_SOURCES:
+        h.update(f.read_bytes())
+    return h.hexdigest()[:16]
+
+
+def gateup_hbm_traffic_bytes():
+    """HBM bytes per launch of the fused gate/up GEMM: not measurable from inside the process, so it is read from
+    the committed rocprofv3 --pmc summary (FETCH_SIZE and WRITE_SIZE runs of this script, scaled by what the same
+    counters read for a 1 GiB device copy).  The summary records the hash of the GEMM sources it was measured on;
+    when the sources have changed since, the figure would be stale and None is reported instead."""
+    try:
+        text = TRAFFIC_PROFILE.read_text()
+    except OSError:
+        return None, "profiles file missing"
+    rec = dict(l.split(":", 1) for l in text.splitlines() if l.startswith("bench."))
+    want = rec.get("bench.gemm_source_sha256_16", "").strip()
+    if want != gemm_source_hash():
+        return None, f"GEMM sources changed since the PMC run (profile {want or 'unmarked'}, now {gemm_source_hash()})"
+    return int(rec["bench.roofline.traffic_bytes"].strip()), f"profiles/{TRAFFIC_PROFILE.name}"
+
+
+class PowerSampler:
+    """Samples the GPU's socket power (hwmon power1_input, microwatts) and the current shader clock level
+    (pp_dpm_sclk) from sysfs while the timed region runs.  Both are readable by an ordinary user on the
+    MI355X boxes; where they are not, the keys are simply absent from the report."""
+
+    def __init__(self, period_s=0.004):
+        import glob
+        self.power = next(iter(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input")), None)
+        self.sclk = next(iter(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk")), None)
+        self.period, self.watts, self.mhz, self._stop, self._t = period_s, [], [], False, None
+
+    def _run(self):
+        import re
+        while not self._stop:
+            try:
+                if self.power:
+                    self.watts.append(int(open(self.power).read()) / 1e6)
+                if self.sclk:
+                    m = re.search(r"(\d+)Mhz \*", open(self.sclk).read())
+                    if m:
+                        self.mhz.append(int(m.group(1)))
+            except (OSError, ValueError):
+                pass
+            time.sleep(self.period)
+
+    def __enter__(self):
+        import threading
+        self._t = threading.Thread(target=self._run, daemon=True)
+        self._t.start()
+        return self
+
+    def __exit__(self, *a):
+        self._stop = True
+        self._t.join()
+
+    def report(self):
+        out = {}
+        if self.watts:
+            out["socket_power_w_avg"] = round(sum(self.watts) / len(self.watts), 1)
+            out["socket_power_w_max"] = round(max(self.watts), 1)
+        if self.mhz:
+            out["sclk_mhz_avg"] = round(sum(self.mhz) / len(self.mhz), 1)
+            out["sclk_mhz_min"] = min(self.mhz)
+        out["samples"] = max(len(self.watts), len(self.mhz))
+        return out
+
+
+def host_threads():
+    """(threads used, what the box reports).  The reference's parallel_for takes std::thread::hardware_concurrency();
+    the benchmark boxes export their CPU share as OMP_NUM_THREADS (16 for one GPU) and ask that pools stay within it,
+    so that is the count used when it is the smaller one; both figures are reported."""
+    hw = os.cpu_count() or 1
+    try:
+        affinity = len(os.sched_getaffinity(0))
+    except AttributeError:
+        affinity = hw
+    share = int(os.environ.get("OMP_NUM_THREADS", "0") or 0)
+    used = min(hw, affinity, share) if share > 0 else min(hw, affinity)
+    return max(1, used), {"hardware_concurrency": hw, "affinity": affinity, "omp_num_threads_env": share or None}
+
+
+def cpu_baseline(config2_rows=1024):
+    """The reference's CPU path on benchmark config 1, timed on this host: X fp32 [512,1024] ~ N(0,1), W fp32
+    [1024,1024] ~ N(0,0.02), per-tensor amax -> E4M3 scale, operands rounded through the E4M3 quantize / dequantize
+    (outside the timed span, reported separately), then the linear forward of src/cpu_trainer.cpp:306-324 with the
+    parallel_for / cpu_dot idiom of :89-108 (rows split over threads, one scalar fp32 dot in k order per output, bf16
+    output): one warm-up, best of five.  `config2_sample` adds the same loop on a bounded sample of the benchmark's own
+    workload (first rows of config 2's gate projection), one pass."""
     import numpy as np
     sys.path.insert(0, str(ROOT / "tests"))
     import oracle_lib as orc      # checker code, used here only as the reported CPU baseline
 
-    try:
-        cores = len(os.sched_getaffinity(0))
-    except AttributeError:
-        cores = os.cpu_count() or 1
-    cores = max(1, min(cores, 16))
+    threads, reported = host_threads()
     rng = np.random.default_rng(1)
-    T, K, N = sample_rows, 4096, 14336
+    T, K, N = 512, 1024, 1024
     x = rng.standard_normal((T, K), dtype=np.float32)
-    u = rng.random((T, K), dtype=np.float32)
-    x[u < 0.0005] = 40.0
-    x[u > 0.9995] = -40.0
-    del u
-    w = rng.standard_normal((N, K), dtype=np.float32)
-    w *= np.float32(0.02)
-    xb, wb = orc.bf16_from_f32(x), orc.bf16_from_f32(w)
-    del x, w
+    w = rng.standard_normal((N, K), dtype=np.float32) * np.float32(0.02)
     t0 = time.perf_counter()
-    xq, _, xd = orc.quantize_rows(xb)
-    wq, _, wd = orc.quantize_rows(wb)
-    xf = orc.e4m3_unpack(xq) * xd[:, None]
-    wf = orc.e4m3_unpack(wq) * wd[:, None]
-    t1 = time.perf_counter()
-    orc.linear_forward_f32(xf, wf, threads=cores)
-    t2 = time.perf_counter()
+    ops = []
+    for t in (x, w):
+        scale, descale = orc.scale_from_amax(orc.amax_f32(t), 448.0)
+        ops.append(orc.dequant(orc.quantize_f32_e4m3(t, scale), descale))
+    t_quant = time.perf_counter() - t0
+    orc.linear_forward_f32(ops[0], ops[1], threads=threads)          # warm-up
+    best = float("inf")
+    for _ in range(5):
+        t0 = time.perf_counter()
+        orc.linear_forward_f32(ops[0], ops[1], threads=threads)
+        best = min(best, time.perf_counter() - t0)
     flop = 2.0 * T * K * N
-    return {
-        "value": round(flop / (t2 - t0) / 1e12, 6), "unit": "TFLOP/s", "cores": cores, "kind": "port",
-        "sample": f"config 2 gate projection, first {T} of 8192 token rows x full W[14336x4096]: per-row amax + E4M3 "
-                  f"quantize + dequantize ({t1 - t0:.1f} s) and scalar fp32 linear forward on {cores} threads "
-                  f"({t2 - t1:.1f} s), one pass",
+    out = {
+        "value": round(flop / best / 1e12, 6), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+        "sample": f"config 1, whole: X[512x1024] . W[1024x1024]^T on E4M3-rounded operands, scalar fp32 linear forward on "
+                  f"{threads} threads, best of 5 after one warm-up = {best * 1e3:.2f} ms; amax + quantize + dequantize of both "
+                  f"operands (outside the timed span, one thread) {t_quant * 1e3:.1f} ms",
+        "host": reported,
     }
+    if config2_rows:
+        T2, K2, N2 = config2_rows, 4096, 14336
+        x2 = rng.standard_normal((T2, K2), dtype=np.float32)
+        u2 = rng.random((T2, K2), dtype=np.float32)
+        x2[u2 < 0.0005] = 40.0
+        x2[u2 > 0.9995] = -40.0
+        w2 = rng.standard_normal((N2, K2), dtype=np.float32) * np.float32(0.02)
+        xq, _, xd = orc.quantize_rows(orc.bf16_from_f32(x2))
+        wq, _, wd = orc.quantize_rows(orc.bf16_from_f32(w2))
+        xf = orc.e4m3_unpack(xq) * xd[:, None]
+        wf = orc.e4m3_unpack(wq) * wd[:, None]
+        t0 = time.perf_counter()
+        orc.linear_forward_f32(xf, wf, threads=threads)
+        dt = time.perf_counter() - t0
+        out["config2_sample"] = {
+            "value": round(2.0 * T2 * K2 * N2 / dt / 1e12, 6), "unit": "TFLOP/s", "cores": threads,
+            "sample": f"first {T2} of 8192 token rows x full gate weight [14336x4096], per-token / per-channel E4M3-rounded "
+                      f"operands, linear forward only, one pass = {dt:.2f} s",
+        }
+    return out
 
 
 def main():
@@ -162,11 +263,12 @@ def main():
     for _ in range(args.warmup):
         step(0)
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step(1)
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
+    with PowerSampler() as sampler:
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step(1)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
 
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     # per-kernel breakdown: the same steps again with a bracket around every kernel, outside the timed region
@@ -188,6 +290,55 @@ def main():
             ts.append(a.elapsed_time(b) / launches)
         return sorted(ts)[len(ts) // 2]
 
+    # The same four launches recorded once into a HIP graph and replayed: what the step costs without the per-launch
+    # host work and without the event brackets.  Captured on a side stream (the library launches on the stream it is
+    # given), replayed `steps` times between two synchronisations.
+    graph_ms = None
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                cs = side.cuda_stream
+                cf.cf_fp8_quantize_rows(x, M, K, 0, xq, xs, xd, cs)
+                cf.cf_fp8_gemm_nt_bf16_ex(M, N, K, xq, K, 0, xd, wgq, K, wgd, 1, 2, None, wuq, wud, h, N, 0, cs)
+                cf.cf_fp8_quantize_rows(h, M, N, 0, hq, hs, hd, cs)
+                cf.cf_fp8_gemm_nt_bf16_ex(M, K, N, hq, N, 0, hd, wdq, N, wdd, 1, 0, None, None, None, y, K, 0, cs)
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        g0 = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        graph_ms = (time.perf_counter() - g0) * 1e3 / args.steps
+    except Exception as exc:      # a capture failure must not cost the benchmark its line
+        graph_ms = None
+        graph_note = f"graph capture failed: {exc}"
+    else:
+        graph_note = "the step's four launches replayed from one captured HIP graph, same buffers, no event brackets"
+
+    # A ceiling for the two quantize kernels inside the step: a plain device copy that moves as many bytes as the H
+    # quantize (2 B read + 1 B written per element), from sources that are in no cache (five source buffers of 176 MB
+    # used in turn, more than the 256 MB memory-side cache holds), bracketed like the kernels in the step.
+    copy_bytes = int(1.5 * M * N)
+    srcs = [torch.full((copy_bytes,), i, dtype=torch.uint8, device=dev) for i in range(5)]
+    dsts = [torch.empty(copy_bytes, dtype=torch.uint8, device=dev) for _ in range(2)]
+    torch.cuda.synchronize()
+    cts = []
+    for i in range(15):
+        a, b = ev(), ev()
+        a.record()
+        dsts[i % 2].copy_(srcs[i % 5])
+        b.record()
+        torch.cuda.synchronize()
+        if i >= 5:
+            cts.append(a.elapsed_time(b))
+    copy_ms = sorted(cts)[len(cts) // 2]
+    hbm_copy_gbps = 2.0 * copy_bytes / (copy_ms * 1e-3) / 1e9
+    del srcs, dsts
+
     # outside the timed steps: the two quantize kernels on their own (the brackets inside a step include a launch gap
     # that is a quarter of a 20 us kernel)
     qx_alone_ms = back_to_back(lambda: cf.cf_fp8_quantize_rows(x, M, K, 0, xq, xs, xd, st))
@@ -206,6 +357,7 @@ def main():
     qh_gbps = qh_bytes / (seg[2] * 1e-3) / 1e9
 
     props = torch.cuda.get_device_properties(dev)
+    traffic, traffic_note = gateup_hbm_traffic_bytes()
     out = {
         "metric": "fp8_gemm_tflops_mlp_m8192_n14336_k4096_with_quantize",
         "value": round(value, 2),
@@ -245,8 +397,16 @@ def main():
         "roofline": {
             "kernel": "k_gemm_nt_ring<e4m3,silu_gate,row_col> M=8192 N=2x14336 K=4096",
             "bound": "mfma", "achieved": round(gateup_tflops, 1), "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": round(gateup_tflops / FP8_PEAK_TFLOPS, 4), "traffic": GATEUP_HBM_TRAFFIC_BYTES,
+            "frac": round(gateup_tflops / FP8_PEAK_TFLOPS, 4), "traffic": traffic,
         },
+        "traffic_source": traffic_note,
+        "hbm_achievable_gbps": round(hbm_copy_gbps, 1),
+        "hbm_achievable_note": f"plain device copy of {copy_bytes} bytes (as many bytes moved as the H quantize) from sources in "
+                               f"no cache, one event bracket per copy like the kernels in the step: {copy_ms * 1e3:.1f} us",
+        "graph_replay": {"ms_per_step": None if graph_ms is None else round(graph_ms, 4),
+                         "tflops": None if graph_ms is None else round(total_flop / (graph_ms * 1e-3) / 1e12, 2),
+                         "note": graph_note},
+        "timed_region_power": sampler.report(),
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()

@@ -192,9 +192,6 @@ __device__ __forceinline__ void epilogue(v16f (&acc)[4][4], const GemmArgs& p, i
                         }
                     }
                     const uint32_t o01 = pack_bf16x2_hw(v[0], v[1]), o23 = pack_bf16x2_hw(v[2], v[3]);
-#ifdef CF_ABLATE_STORE
-                    if (p.ldc < 0)
-#endif
                     if (vec_ok && n + 3 < p.N) {
                         *reinterpret_cast<uint2*>(crow) = make_uint2(o01, o23);
                     } else {
@@ -1699,6 +1696,9 @@ int cf::grouped_gemm_nt_bf16(int total_rows, int N, int K, int num_experts, cons
     if (epilogue != EPI_NONE && epilogue != EPI_SILU_GATE) return CF_ERR_INVALID_ARG;
     if (epilogue == EPI_SILU_GATE && (!B_up || !b_up_descale)) return CF_ERR_INVALID_ARG;
     if (scale_mode != SCALE_TENSOR && scale_mode != SCALE_ROWCOL) return CF_ERR_INVALID_ARG;
+    // per-tensor descales would need one device scalar per expert for the weights: not built.  Rejected before
+    // anything is launched, so a refused call leaves the workspace untouched.
+    if (scale_mode == SCALE_TENSOR) return CF_ERR_UNSUPPORTED;
     size_t need = 0;
     cf_fp8_grouped_gemm_workspace_bytes(total_rows, num_experts, &need);
     if (workspace_bytes < need || (reinterpret_cast<uintptr_t>(d_workspace) & 3u)) return CF_ERR_INVALID_ARG;
@@ -1728,10 +1728,6 @@ int cf::grouped_gemm_nt_bf16(int total_rows, int N, int K, int num_experts, cons
     const int out_bn = epilogue == EPI_SILU_GATE ? BN / 2 : BN;
     p.tiles_m = max_row_tiles;
     p.tiles_n = (N + out_bn - 1) / out_bn;
-    if (scale_mode == SCALE_TENSOR) {
-        // per-tensor descales: one device scalar per expert for the weights
-        return CF_ERR_UNSUPPORTED;
-    }
     if (a_is_e5m2) return launch_tiled<1, EPI_NONE, SCALE_ROWCOL>(p, st);
     return epilogue == EPI_SILU_GATE ? launch_tiled<0, EPI_SILU_GATE, SCALE_ROWCOL>(p, st)
                                      : launch_tiled<0, EPI_NONE, SCALE_ROWCOL>(p, st);

@@ -11,7 +11,9 @@
  *   - work is enqueued on `stream` (a hipStream_t passed as void*) and nothing
  *     synchronises;
  *   - bf16 tensors are passed as uint16_t*, fp8 tensors as void* / uint8_t*;
- *   - the library allocates nothing and keeps no mutable global state.
+ *   - the library allocates no device memory and keeps no mutable global
+ *     state; the only allocation is the small host object behind
+ *     cf_act_slot_create (freed by cf_act_slot_destroy).
  * The reference functions return void and throw; the C ABI returns 0 on
  * success, a positive hipError_t when the runtime reports one, or a negative
  * CF_ERR_* code for an argument the kernels cannot honour.
@@ -146,9 +148,19 @@ int cf_fp8_quantize_block_128x128(const uint16_t* d_x, int rows, int K, void* d_
  * throws std::invalid_argument, kernels/activations.cu:61-72). */
 int cf_swiglu_forward(const uint16_t* d_gate, const uint16_t* d_up, uint16_t* d_out, int n,
                       cf_stream_t stream);
+/* swiglu_backward, kernels.hpp:167-175, kernels/activations.cu:42-58, 89-106:
+ * grad_gate = bf16((grad_out * up) * silu'(gate)), grad_up = bf16(grad_out * silu(gate)).
+ * n < 0 or a null pointer with n > 0 is CF_ERR_INVALID_ARG, as the reference throws. */
+int cf_swiglu_backward(const uint16_t* d_grad_out, const uint16_t* d_gate, const uint16_t* d_up,
+                       uint16_t* d_grad_gate, uint16_t* d_grad_up, int n, cf_stream_t stream);
 /* bias_add_strided_bf16, kernels.hpp:243-247, kernels/moe.cu:349-356. */
 int cf_bias_add_strided_bf16(uint16_t* d_inout, const uint16_t* d_bias, int rows, int cols,
                              int row_stride, int base, cf_stream_t stream);
+/* col_sum_strided_bf16, kernels.hpp:255-259, kernels/moe.cu:335-348, 357-364: the bias gradient,
+ * out_accum[c] += sum over rows of in[row, base + c], the sum taken in fp32 in ascending row order
+ * from zero (the reference's order, so the bits are the reference's). */
+int cf_col_sum_strided_bf16(const uint16_t* d_in, float* d_out_accum, int rows, int cols,
+                            int row_stride, int base, cf_stream_t stream);
 
 /* ---- producers of the quantizer's input, fused with it ---------------------
  * The reference normalises, clips and quantizes an activation in four launches

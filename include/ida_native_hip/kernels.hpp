@@ -98,6 +98,15 @@ inline void fp8_update_delayed_scale(const float* d_amax, float fp8_max, float* 
 inline void swiglu_forward(const bf16* d_gate, const bf16* d_up, bf16* d_out, int N, hipStream_t stream) {
     CF_FWD(cf_swiglu_forward(hip_detail::u(d_gate), hip_detail::u(d_up), hip_detail::u(d_out), N, stream));
 }
+inline void swiglu_backward(const bf16* d_grad_out, const bf16* d_gate, const bf16* d_up, bf16* d_grad_gate,
+                            bf16* d_grad_up, int N, hipStream_t stream) {
+    CF_FWD(cf_swiglu_backward(hip_detail::u(d_grad_out), hip_detail::u(d_gate), hip_detail::u(d_up),
+                              hip_detail::u(d_grad_gate), hip_detail::u(d_grad_up), N, stream));
+}
+inline void col_sum_strided_bf16(const bf16* d_in, float* d_out_accum, int rows, int cols, int row_stride, int base,
+                                 hipStream_t stream) {
+    CF_FWD(cf_col_sum_strided_bf16(hip_detail::u(d_in), d_out_accum, rows, cols, row_stride, base, stream));
+}
 inline void bias_add_strided_bf16(bf16* d_inout, const bf16* d_bias, int rows, int cols, int row_stride, int base,
                                   hipStream_t stream) {
     CF_FWD(cf_bias_add_strided_bf16(hip_detail::u(d_inout), hip_detail::u(d_bias), rows, cols, row_stride, base, stream));

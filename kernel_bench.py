@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Per-kernel timing of the FP8 hot path at the benchmark shapes, against each kernel's roofline.
 
-    python canopy-foundry_amd/kernel_bench.py [--iters 20]
+    python kernel_bench.py [--iters 20]
 
 Every kernel is timed with events on the launch stream (median of three batches of `--iters` launches) and
 reported with its algorithmic bytes or FLOPs: HBM-bound kernels as GB/s and a fraction of 8 TB/s, GEMMs as
@@ -16,7 +16,7 @@ import importlib.util
 import sys
 from pathlib import Path
 
-ROOT = Path(__file__).resolve().parent.parent
+ROOT = Path(__file__).resolve().parent
 HBM_PEAK = 8000.0      # GB/s
 FP8_PEAK = 5000.0      # TFLOP/s
 

@@ -386,6 +386,32 @@ void orc_swiglu_forward(const uint16_t* gate, const uint16_t* up, uint16_t* out,
     }
 }
 
+/* kernels/activations.cu:23-26 (silu_derivative), :42-58 (k_swiglu_backward): the products are taken left to right,
+ * grad_gate = bf16((grad * up) * silu'(gate)), grad_up = bf16(grad * silu(gate)). */
+void orc_swiglu_backward(const uint16_t* grad_out, const uint16_t* gate, const uint16_t* up,
+                         uint16_t* grad_gate, uint16_t* grad_up, int n) {
+    for (int i = 0; i < n; ++i) {
+        const float g = orc_bf16_to_f32(gate[i]);
+        const float u = orc_bf16_to_f32(up[i]);
+        const float d = orc_bf16_to_f32(grad_out[i]);
+        const float sg = stable_sigmoid(g);
+        const float dsilu = sg * (1.0f + g * (1.0f - sg));
+        const float silu = g * sg;
+        grad_gate[i] = orc_bf16_from_f32((d * u) * dsilu);
+        grad_up[i] = orc_bf16_from_f32(d * silu);
+    }
+}
+
+/* kernels/moe.cu:335-348 (k_col_sum_strided_bf16): one fp32 running sum per column over the rows in ascending
+ * order, started at zero and then added to what the accumulator holds. */
+void orc_col_sum_strided_bf16(const uint16_t* in, float* out_accum, int rows, int cols, int row_stride, int base) {
+    for (int c = 0; c < cols; ++c) {
+        float acc = 0.0f;
+        for (int r = 0; r < rows; ++r) acc += orc_bf16_to_f32(in[(size_t)r * row_stride + base + c]);
+        out_accum[c] += acc;
+    }
+}
+
 /* kernels/moe.cu:325-334 */
 void orc_bias_add_strided_bf16(uint16_t* inout, const uint16_t* bias,
                                int rows, int cols, int row_stride, int base) {

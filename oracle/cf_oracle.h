@@ -127,6 +127,13 @@ void orc_quantize_block_128x128(const uint16_t* x, int rows, int K,
 void orc_swiglu_forward(const uint16_t* gate, const uint16_t* up, uint16_t* out, int n);
 void orc_bias_add_strided_bf16(uint16_t* inout, const uint16_t* bias,
                                int rows, int cols, int row_stride, int base);
+/* swiglu_backward (kernels/activations.cu:42-58, 89-106) and the bias gradient col_sum_strided_bf16
+ * (kernels/moe.cu:335-348, 357-364).  Pins: grad_up equals the forward applied to (gate, grad_out) bit for bit
+ * (one commutative product), grad_gate against the closed form in double to half a bf16 ulp; the column sum
+ * against numpy on exactly summable integers and on a column whose sequential sum differs from every tree. */
+void orc_swiglu_backward(const uint16_t* grad_out, const uint16_t* gate, const uint16_t* up,
+                         uint16_t* grad_gate, uint16_t* grad_up, int n);
+void orc_col_sum_strided_bf16(const uint16_t* in, float* out_accum, int rows, int cols, int row_stride, int base);
 
 /* ---- producers of the quantizer's input (cf_oracle_norm.c) ----------------
  * RMSNorm forward (kernels/rmsnorm.cu:13-54,101-108) and the absolute-ceiling

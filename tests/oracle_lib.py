@@ -307,6 +307,23 @@ def bias_add_strided(inout, bias, rows, cols, row_stride, base):
     return inout
 
 
+def swiglu_backward(grad_out, gate, up):
+    grad_out = np.ascontiguousarray(grad_out, dtype=np.uint16)
+    gate = np.ascontiguousarray(gate, dtype=np.uint16)
+    up = np.ascontiguousarray(up, dtype=np.uint16)
+    dg = np.empty(gate.shape, np.uint16)
+    du = np.empty(gate.shape, np.uint16)
+    _call("orc_swiglu_backward", grad_out, gate, up, dg, du, c_i(gate.size))
+    return dg, du
+
+
+def col_sum_strided(x, out_accum, rows, cols, row_stride, base):
+    x = np.ascontiguousarray(x, dtype=np.uint16)
+    out = np.ascontiguousarray(out_accum, dtype=np.float32).copy()
+    _call("orc_col_sum_strided_bf16", x, out, c_i(rows), c_i(cols), c_i(row_stride), c_i(base))
+    return out
+
+
 # ---- producers of the quantizer's input ----------------------------------------------
 def rmsnorm_forward(x, weight, eps=1e-6):
     x = np.ascontiguousarray(x, dtype=np.uint16)

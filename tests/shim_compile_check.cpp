@@ -18,6 +18,9 @@ int main() {
     void (*f9)(int, int, int, const void*, int, bool, const float*, const void*, const float*, bf16*, int, hipStream_t) = &lt_gemm_fp8_nt;
     void (*f10)(int, int, int, const void*, const float*, const void*, const float*, float*, int, hipStream_t) = &lt_gemm_fp8_tn_accum_f32;
     void (*f11)(int, int, int, const void*, const float*, const void*, const float*, bf16*, int, hipStream_t) = &lt_gemm_fp8_tn_accum_f32;
+    void (*f12)(const bf16*, const bf16*, const bf16*, bf16*, bf16*, int, hipStream_t) = &swiglu_backward;
+    void (*f13)(const bf16*, float*, int, int, int, int, hipStream_t) = &col_sum_strided_bf16;
+    if (!f12 || !f13) return 1;
     if (!f1 || !f2 || !f3 || !f4 || !f5 || !f6 || !f7 || !f8 || !f9 || !f10 || !f11) return 1;
     int ok = 0;
     try { swiglu_forward(nullptr, nullptr, nullptr, -1, nullptr); } catch (const std::invalid_argument&) { ++ok; }   // kernels/activations.cu:61-72

@@ -356,6 +356,68 @@ def test_swiglu_on_every_bf16_gate(cf, dev):
     assert bad.size == 0, f"{bad.size} differ; first gate {gate[bad[0]]:#06x} up {up[bad[0]]:#06x} got {got[bad[0]]:#06x} want {want[bad[0]]:#06x}"
 
 
+def test_swiglu_backward(cf, dev):
+    """swiglu_backward against the oracle, bit for bit: ragged and unaligned lengths, then every bf16 gate pattern."""
+    case("swiglu backward")
+    rng = np.random.default_rng(14)
+    for n, off in ((0, 0), (5, 0), (4096, 0), (100003, 0), (100003, 1)):
+        gb = orc.bf16_from_f32(rng.standard_normal(n + off).astype(np.float32) * 4)
+        ub = orc.bf16_from_f32(rng.standard_normal(n + off).astype(np.float32))
+        db = orc.bf16_from_f32(rng.standard_normal(n + off).astype(np.float32) * 1e-2)
+        if n > 10:
+            gb[off:off + 6] = orc.bf16_from_f32(np.array([-100, 100, -20, 20, 0, -0.0], np.float32))
+        dg = torch.empty(n + off, dtype=torch.bfloat16, device=dev)
+        du = torch.empty(n + off, dtype=torch.bfloat16, device=dev)
+        cf.cf_swiglu_backward(dev_bf16(db, dev)[off:], dev_bf16(gb, dev)[off:], dev_bf16(ub, dev)[off:], dg[off:], du[off:], n, stream())
+        torch.cuda.synchronize()
+        wg, wu = orc.swiglu_backward(db[off:], gb[off:], ub[off:])
+        assert np.array_equal(bf16_bits(dg[off:]), wg) and np.array_equal(bf16_bits(du[off:]), wu)
+    gate = np.tile(all_bf16_bits(), 6)
+    ups = orc.bf16_from_f32(np.array([1.0, -0.75, 0.0, 3.0e38, 1e-30, -2.5], np.float32))
+    grads = orc.bf16_from_f32(np.array([1.0, 0.5, -3.0, 1e-30, 3.0e38, 0.0], np.float32))
+    up, grad = np.repeat(ups, 65536), np.repeat(grads, 65536)
+    dg = torch.empty(gate.size, dtype=torch.bfloat16, device=dev)
+    du = torch.empty(gate.size, dtype=torch.bfloat16, device=dev)
+    cf.cf_swiglu_backward(dev_bf16(grad, dev), dev_bf16(gate, dev), dev_bf16(up, dev), dg, du, gate.size, stream())
+    torch.cuda.synchronize()
+    wg, wu = orc.swiglu_backward(grad, gate, up)
+    for got, want in ((bf16_bits(dg), wg), (bf16_bits(du), wu)):
+        # a NaN result must be a NaN; its sign and payload are not defined by the arithmetic
+        nan_w, nan_g = (want & 0x7fff) > 0x7f80, (got & 0x7fff) > 0x7f80
+        assert np.array_equal(nan_w, nan_g)
+        bad = np.nonzero(np.where(nan_g, 0x7fc0, got) != np.where(nan_w, 0x7fc0, want))[0]
+        assert bad.size == 0, f"{bad.size} differ; first gate {gate[bad[0]]:#06x}"
+    assert cf.raw_cf_swiglu_backward(None, None, None, None, None, -1, None) == -1
+    assert cf.raw_cf_swiglu_backward(None, None, None, None, None, 4, None) == -1
+    assert cf.raw_cf_swiglu_backward(None, None, None, None, None, 0, None) == 0
+
+
+@pytest.mark.parametrize("rows,cols,stride,base", [(300, 70, 96, 11), (1, 1, 1, 0), (129, 64, 64, 0), (1000, 200, 256, 8),
+                                                   (4096, 1024, 3072, 2048), (0, 5, 8, 0), (257, 130, 136, 0)])
+def test_col_sum_strided(cf, dev, rows, cols, stride, base):
+    """The bias gradient: fp32 column sums in ascending row order, added to the accumulator; bit for bit against the
+    oracle's sequential loop (16-byte and element-wise fetch paths, ragged row and column tiles)."""
+    case(f"col_sum {rows}x{cols} stride {stride} base {base}")
+    rng = np.random.default_rng(rows + cols)
+    xb = orc.bf16_from_f32((rng.standard_normal((max(rows, 1), stride)) * np.exp(rng.standard_normal((max(rows, 1), 1)))).astype(np.float32))
+    acc0 = rng.standard_normal(cols).astype(np.float32)
+    acc = torch.from_numpy(acc0).to(dev)
+    cf.cf_col_sum_strided_bf16(dev_bf16(xb, dev), acc, rows, cols, stride, base, stream())
+    torch.cuda.synchronize()
+    assert np.array_equal(host(acc), orc.col_sum_strided(xb, acc0, rows, cols, stride, base))
+
+
+def test_col_sum_is_sequential_in_rows(cf, dev):
+    """2^24 followed by ones: added one at a time every 1 is lost (ties to even); any tree keeps some."""
+    case("col_sum order")
+    col = np.array([16777216.0] + [1.0] * 300, np.float32).reshape(-1, 1)
+    x = np.repeat(orc.bf16_from_f32(col), 8, axis=1)
+    acc = torch.zeros(8, device=dev)
+    cf.cf_col_sum_strided_bf16(dev_bf16(x, dev), acc, 301, 8, 8, 0, stream())
+    torch.cuda.synchronize()
+    assert np.all(host(acc) == np.float32(16777216.0))
+
+
 def test_config2_activation_quantize_full_size(cf, dev):
     """M=8192 x K=4096 bf16 ~N(0,1) with 0.1% outliers at +-40 -> E4M3 with per-token scales."""
     case("config 2 activations, full size")

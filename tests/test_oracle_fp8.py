@@ -309,6 +309,58 @@ def test_swiglu_probe_values_and_closed_form():
     assert np.all(np.abs(got - exact) <= 1.01 * orc.bf16_ulp(exact) / 2 + 1e-30 + 3e-7 * np.abs(exact))
 
 
+def test_swiglu_backward_is_the_derivative_of_the_forward():
+    """grad_up = grad * silu(gate) is the forward's product with (gate, grad) -- one commutative multiply, so the
+    bits must equal swiglu_forward(gate, grad).  grad_gate against the closed form d/dg [g sigmoid(g)] u grad in double,
+    and against a central difference of the forward's own formula (a dropped `1 +` or a sign error in `1 - sigmoid`
+    misses by tens of percent)."""
+    rng = np.random.default_rng(16)
+    n = 30000
+    gb = orc.bf16_from_f32(rng.standard_normal(n).astype(np.float32) * 4)
+    ub = orc.bf16_from_f32(rng.standard_normal(n).astype(np.float32))
+    db = orc.bf16_from_f32(rng.standard_normal(n).astype(np.float32) * 1e-2)
+    gb[:6] = orc.bf16_from_f32(np.array([-100, 100, -20, 20, 0, -0.0], np.float32))
+    dg, du = orc.swiglu_backward(db, gb, ub)
+    assert np.array_equal(du, orc.swiglu_forward(gb, db))
+    g, u, d = (orc.bf16_to_f32(v).astype(np.float64) for v in (gb, ub, db))
+    sg = 1.0 / (1.0 + np.exp(-g))
+    exact = d * u * sg * (1.0 + g * (1.0 - sg))
+    got = orc.bf16_to_f32(dg).astype(np.float64)
+    assert np.all(np.abs(got - exact) <= 1.01 * orc.bf16_ulp(exact) / 2 + 1e-30 + 6e-7 * np.abs(d * u))
+    silu = lambda x: x / (1.0 + np.exp(-x))
+    h = 1e-4
+    numeric = d * u * (silu(g + h) - silu(g - h)) / (2 * h)
+    assert np.all(np.abs(exact - numeric) <= 1e-6 * np.abs(d * u) + 1e-30)
+    # silu'(0) = 1/2, silu'(large) = 1, silu'(-large) = 0
+    one = orc.bf16_from_f32(np.ones(3, np.float32))
+    dg, _ = orc.swiglu_backward(one, orc.bf16_from_f32(np.array([0.0, 60.0, -60.0], np.float32)), one)
+    assert np.array_equal(orc.bf16_to_f32(dg), np.array([0.5, 1.0, 0.0], np.float32)) or \
+        np.allclose(orc.bf16_to_f32(dg), [0.5, 1.0, 0.0], atol=1e-20)
+
+
+def test_col_sum_strided_order_and_accumulate():
+    rng = np.random.default_rng(17)
+    rows, cols, stride, base = 300, 70, 96, 11
+    xi = rng.integers(-8, 9, (rows, stride)).astype(np.float32)          # every partial sum is exact
+    x = orc.bf16_from_f32(xi)
+    acc0 = rng.integers(-4, 5, cols).astype(np.float32)
+    got = orc.col_sum_strided(x, acc0, rows, cols, stride, base)
+    assert np.array_equal(got, acc0 + xi[:, base:base + cols].sum(0))
+    # a column that separates the sequential order from any tree: 2^24 then ones.  Added one at a time every 1 is
+    # lost to rounding (ties to even); any grouping that first adds two ones together keeps them.
+    col = np.array([16777216.0] + [1.0] * 7, np.float32)
+    x = orc.bf16_from_f32(col.reshape(-1, 1))
+    assert orc.col_sum_strided(x, np.zeros(1, np.float32), 8, 1, 1, 0)[0] == np.float32(16777216.0)
+    # the sum starts from zero and is added to the accumulator once (not accumulated into it term by term)
+    assert orc.col_sum_strided(x[1:], np.array([16777216.0], np.float32), 7, 1, 1, 0)[0] == np.float32(16777224.0)
+    # random data: the float32 chain, restated with numpy scalars
+    xr = orc.bf16_from_f32(rng.standard_normal((257, 5)).astype(np.float32))
+    want = np.zeros(5, np.float32)
+    for r in range(257):
+        want = (want + orc.bf16_to_f32(xr[r])).astype(np.float32)
+    assert np.array_equal(orc.col_sum_strided(xr, np.zeros(5, np.float32), 257, 5, 5, 0), want)
+
+
 def test_bias_add_strided():
     rng = np.random.default_rng(8)
     x = orc.bf16_from_f32(rng.standard_normal((5, 12)).astype(np.float32))

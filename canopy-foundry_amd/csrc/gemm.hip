@@ -1680,6 +1680,63 @@ int cf_fp8_grouped_gemm_nt_bf16_ex(int total_rows, int N, int K, int num_experts
                                     true, 0, stream);
 }
 
+// ---- the grouped GEMM for callers that cannot allocate ---------------------------------------------
+// The tile table lives in a fixed array in the library's device image instead of a caller's workspace.  Each GPU
+// holds its own copy of the array at its own address; host code must not pass the array's name to a kernel (in
+// host code that name is a stand-in, not a device address), so the address is looked up once per device with
+// hipGetSymbolAddress and every use below goes through that pointer.
+constexpr size_t kStaticMapBytes = 64 * 1024;            // 3276 row tiles: e.g. 64 experts and 820,000 selected rows
+static __device__ __align__(256) unsigned char scratch[kStaticMapBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// the address of `scratch` on the current device; looked up on the first call per device
+int static_scratch(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return static_cast<int>(e);
+    if (dev < 0 || dev >= kMaxDevices) return CF_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return static_cast<int>(e);
+        if (!ptr) return CF_ERR_UNSUPPORTED;
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return CF_OK;
+}
+}  // namespace
+
+int cf_fp8_grouped_gemm_static_max_bytes(size_t* bytes) {
+    if (!bytes) return CF_ERR_INVALID_ARG;
+    *bytes = kStaticMapBytes;
+    return CF_OK;
+}
+
+int cf_fp8_grouped_gemm_nt_bf16_static(int total_rows, int N, int K, int num_experts, const int* d_counts,
+                                       const int* d_offsets, const void* A, int a_rows, int lda, const int* d_a_row_index,
+                                       const float* a_descale, const void* B, const float* b_descale, int scale_mode,
+                                       int epilogue, const void* B_up, const float* b_up_descale, uint16_t* C, int ldc,
+                                       cf_stream_t stream) {
+    size_t need = 0;
+    const int rc = cf_fp8_grouped_gemm_workspace_bytes(total_rows, num_experts, &need);
+    if (rc != CF_OK) return rc;
+    if (need > kStaticMapBytes) return CF_ERR_UNSUPPORTED;       // the table of this many row tiles does not fit the fixed array
+    void* ptr = nullptr;
+    const int sc = static_scratch(&ptr);
+    if (sc != CF_OK) return sc;
+    // The table is rebuilt from the counts by every call (k_build_tile_map writes the entry count and every entry the
+    // GEMM reads), so nothing of the previous call's contents is used and nothing needs clearing.
+    return cf::grouped_gemm_nt_bf16(total_rows, N, K, num_experts, d_counts, d_offsets, A, a_rows, lda, d_a_row_index, a_descale, B,
+                                    b_descale, scale_mode, epilogue, B_up, b_up_descale, C, ldc, ptr, kStaticMapBytes,
+                                    true, 0, stream);
+}
+
 }  // extern "C"
 
 // build_map = false: d_workspace already holds the tile table of these counts and offsets (an earlier call of

@@ -352,6 +352,23 @@ int cf_fp8_grouped_gemm_nt_bf16_ex(int total_rows, int N, int K, int num_experts
                                    uint16_t* d_C, int ldc, void* d_workspace,
                                    size_t workspace_bytes, cf_stream_t stream);
 
+/* cf_fp8_grouped_gemm_nt_bf16_ex for callers that cannot allocate device memory or own no workspace: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in
+ * the reference.  Same arguments without the workspace, same kernels, same result bits; the tile table
+ * lives in a fixed 64 KiB array inside the library's device image (one copy per GPU, held until the process
+ * ends), so the call allocates nothing.  A shape whose table needs more than
+ * cf_fp8_grouped_gemm_static_max_bytes() bytes (cf_fp8_grouped_gemm_workspace_bytes tells: more than
+ * 3276 row tiles, total_rows / 256 + num_experts) returns CF_ERR_UNSUPPORTED and launches nothing.  Every
+ * call on a GPU shares that GPU's array: calls that may overlap in time on one GPU (different streams,
+ * different host threads) race on it and must be serialised by the caller; calls on one stream are ordered. */
+int cf_fp8_grouped_gemm_static_max_bytes(size_t* bytes);
+int cf_fp8_grouped_gemm_nt_bf16_static(int total_rows, int N, int K, int num_experts,
+                                       const int* d_counts, const int* d_offsets, const void* d_A,
+                                       int a_rows, int lda, const int* d_a_row_index, const float* d_a_descale,
+                                       const void* d_B, const float* d_b_descale, int scale_mode,
+                                       int epilogue, const void* d_B_up, const float* d_b_up_descale,
+                                       uint16_t* d_C, int ldc, cf_stream_t stream);
+
 /* Row lists of all experts back to back: compact[offsets[e] + s] = row_indices[e, s]
  * (the gather order of moe_gather_rows_u8 over all experts, kernels/moe.cu:594-606). */
 int cf_moe_compact_row_index(const int* d_counts, const int* d_offsets, const int* d_row_indices,

@@ -222,6 +222,11 @@ int grouped_gemm_nt_bf16(int total_rows, int N, int K, int num_experts, const in
                          const float* b_up_descale, uint16_t* C, int ldc, void* d_workspace, size_t workspace_bytes,
                          bool build_map, int a_is_e5m2, cf_stream_t stream);
 
+// The tile table of a grouped GEMM (k_build_tile_map in gemm.hip): tile_map[0] = number of row tiles of 256 rows,
+// then per row tile (expert, its first row, its end row, its first row tile, its row-tile count), experts back to back.
+void build_tile_map(const int* d_counts, const int* d_offsets, int num_experts, int max_row_tiles, int* tile_map,
+                    hipStream_t stream);
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline unsigned ceil_div(size_t a, size_t b) { return static_cast<unsigned>((a + b - 1) / b); }
 

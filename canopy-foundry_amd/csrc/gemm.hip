@@ -1739,6 +1739,11 @@ int cf_fp8_grouped_gemm_nt_bf16_static(int total_rows, int N, int K, int num_exp
 
 }  // extern "C"
 
+void cf::build_tile_map(const int* d_counts, const int* d_offsets, int num_experts, int max_row_tiles, int* tile_map,
+                        hipStream_t stream) {
+    k_build_tile_map<<<1, 64, 0, stream>>>(d_counts, d_offsets, num_experts, max_row_tiles, tile_map);
+}
+
 // build_map = false: d_workspace already holds the tile table of these counts and offsets (an earlier call of
 // the same routing on the same stream built it); a_is_e5m2: the activations are E5M2 (plain epilogue only)
 int cf::grouped_gemm_nt_bf16(int total_rows, int N, int K, int num_experts, const int* d_counts, const int* d_offsets,

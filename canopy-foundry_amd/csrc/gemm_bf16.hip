@@ -1,0 +1,387 @@
+// bf16 GEMMs of the selected-expert MoE backward, dense and grouped per expert.
+//
+// The reference runs four cuBLAS calls per expert behind a host copy of the counts (src/trainer.cu:7727-7740,
+// wrappers :3069-3160): two input gradients  C[n,N] = A[n,K] . B[K,N]  (gemm_bf16, row-major, beta = 0) and two
+// weight gradients  C[M,N] += A[n,M]^T . B[n,N]  (gemm_bf16_tn_f32, beta = 1, the contraction runs over the
+// expert's n rows).  Here one launch covers every expert, with the counts and offsets read on the device.
+//
+// In both forms at least one operand is stored with the contraction index as its SLOW dimension, while an MFMA
+// lane needs eight consecutive k of one row (or column).  Such a tile is parked in LDS as it lies in memory,
+// [k][columns], and read with ds_read_b64_tr_b16: per 16 lanes the instruction takes a 4 (k) x 16 (columns) block,
+// source lane r supplying the address of row r / 4, columns 4 (r % 4) .. +3, and hands lane i the four k values of
+// column i.  Two such reads give a lane its eight k of a 32x32x16 MFMA operand.  An operand that is K-contiguous
+// in memory takes the usual path (128-byte LDS rows, 16-byte chunks xor-swizzled, ds_read_b128).
+//
+// Workgroup tile 256 (M) x 128 (N) x 64 (K), four wavefronts 2 x 2, each 128 x 64 = 4 x 2 tiles of
+// v_mfma_f32_32x32x16_bf16 with fp32 accumulators.  The N-side operand goes to the MFMA "A" side, so a lane
+// ends up with four consecutive output columns of one output row per accumulator quad.  Global loads are
+// register staged two K-tiles ahead (16 bytes per lane), LDS is double buffered, one barrier per K-tile.
+// Rows, columns and k beyond the operands' bounds are read as zeros (buffer loads with the operand's size in their
+// descriptor), so any n_e works.
+#include "common.hpp"
+
+#include <mutex>
+
+namespace cf {
+namespace {
+
+constexpr int TM = 256, TN = 128, TK = 64, kThr = 256;
+constexpr int kPitchKC = TK * 2;               // a K-contiguous tile: 128-byte rows, chunks swizzled
+constexpr int kPitchM = TM * 2 + 64;           // a [k][m] tile of the M side: 576-byte rows
+constexpr int kPitchN = TN * 2 + 64;           // a [k][n] tile of the N side: 320-byte rows
+// the pads put four consecutive k rows into four different quarters of the 256 bytes the banks span
+constexpr int kATile = TK * kPitchM;           // 36,864 bytes: covers both forms of the M-side tile (K-contiguous: 32,768)
+constexpr int kBTile = TK * kPitchN;           // 20,480 bytes
+constexpr int kStage = kATile + kBTile;
+constexpr int kLds = 2 * kStage;               // 114,688 bytes: one workgroup per CU
+
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef __bf16 v4bf __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) v4bf* lds_v4bf_ptr;
+
+enum { OUT_STORE_BF16 = 0, OUT_ACCUM_BF16 = 1, OUT_ACCUM_F32 = 2 };
+
+struct BfArgs {
+    const uint16_t* A; int lda;     // M side.  NN: [M rows][K]; TN: [K rows][M]
+    const uint16_t* B; int ldb;     // N side: [K rows][N]
+    void* C; int ldc;               // [M][N], bf16 or fp32
+    int M, N, K;
+    int tiles_m, tiles_n;
+    int num_experts;
+    // grouped forms
+    const int* counts; const int* offsets;
+    const int* tile_map;            // NN: [0] = row tiles, then (expert, first row, end row, first row tile, row tiles) each
+    long long b_expert_stride;      // NN: elements between the experts' B matrices
+    long long c_expert_stride;      // TN: elements between the experts' C matrices
+};
+
+__device__ __forceinline__ int swz(int row) { return (row ^ ((row >> 3) & 3)) & 7; }
+
+// eight k of one column for every lane: two transposing reads of a [k][columns] tile at `base` (row pitch `pitch`)
+__device__ __forceinline__ v8bf read_ks(const uint8_t* base, int pitch, int krow0, int col0, int lane) {
+    const int b = lane >> 4, r = lane & 15;
+    const uint8_t* p = base + (krow0 + 8 * (b >> 1) + (r >> 2)) * pitch + (col0 + 16 * (b & 1) + 4 * (r & 3)) * 2;
+    const v4bf lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_v4bf_ptr)(p));
+    const v4bf hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_v4bf_ptr)(p + 4 * pitch));
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// A_KS: the M-side operand is stored [K][M] (the weight-gradient form); otherwise [M][K]
+template <bool A_KS, int OUT, bool GROUPED>
+__global__ __launch_bounds__(kThr) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void k_gemm_bf16(const BfArgs p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+
+    // ---- which tile ----
+    // Workgroups go to the 8 XCDs round-robin (launch position % 8), each XCD with its own 4 MiB L2.  Position b is
+    // therefore read as (XCD x = b % 8, that XCD's i-th workgroup), and what an XCD runs at one time is made to share
+    // operands: in the row-major forms XCD x walks the contiguous range [x * per, (x + 1) * per) of the tile order in
+    // patches of 8 row tiles x 4 column tiles; in the grouped weight-gradient form XCD x owns experts x, x + 8, ...
+    // whole, so that all tiles of an expert stream the same rows through one L2.
+    const int x = blockIdx.x % 8, xi = blockIdx.x / 8;
+    int m0, n0, m_end = p.M, k_begin = 0, k_end = p.K;
+    const uint16_t* B = p.B;
+    size_t c_base = 0;
+    if constexpr (GROUPED && A_KS) {
+        const int tiles = p.tiles_m * p.tiles_n;
+        const int e = x + 8 * (xi / tiles), t = xi % tiles;
+        if (e >= p.num_experts) return;
+        m0 = (t % p.tiles_m) * TM;
+        n0 = (t / p.tiles_m) * TN;
+        k_begin = p.offsets[e];
+        k_end = k_begin + p.counts[e];
+        c_base = static_cast<size_t>(e) * p.c_expert_stride;
+    } else {
+        const int row_tiles = (GROUPED ? p.tile_map[0] : p.tiles_m);
+        const int total = row_tiles * p.tiles_n;
+        const int per = (total + 7) / 8;
+        const int t = x * per + xi;
+        if (xi >= per || t >= total) return;
+        constexpr int GM = 8;
+        const int group = t / (GM * p.tiles_n), first = group * GM;
+        const int gm = min(GM, row_tiles - first), in_group = t - group * GM * p.tiles_n;
+        const int tmi = first + in_group % gm;
+        n0 = (in_group / gm) * TN;
+        m0 = tmi * TM;
+        if constexpr (GROUPED) {
+            const int* e = p.tile_map + 1 + 5 * tmi;
+            m0 = e[1] + (tmi - e[3]) * TM;
+            m_end = min(m0 + TM, e[2]);
+            B += static_cast<size_t>(e[0]) * p.b_expert_stride;
+        }
+    }
+    if (k_end <= k_begin) {
+        if constexpr (OUT != OUT_STORE_BF16) return;      // nothing to add
+    }
+    const int nk = (k_end - k_begin + TK - 1) / TK;
+
+    // ---- global -> registers -> LDS: 16-byte chunks through buffer loads ----
+    // A buffer load takes a descriptor with the operand's size in bytes and returns zeros for anything beyond it, so
+    // every load is issued unconditionally (loads under branches would keep the compiler from counting the loads in
+    // flight: it would wait for all of them, the prefetch included, before the first LDS store) and the zero fill of
+    // the ragged ends costs nothing: the descriptor of a [k][columns] operand ends with the last row of the k range,
+    // and a lane whose columns lie outside the operand (or, for the K-contiguous form, whose k chunk lies beyond K)
+    // simply uses an offset beyond every descriptor.  Offsets are 32-bit byte offsets; the launcher keeps operands
+    // below 2 GiB.
+    constexpr uint32_t kOutside = 0x80000000u;
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    auto rsrc = [](const void* base, uint32_t bytes) {
+        return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(bytes), 0x00020000);
+    };
+    auto load16 = [](__amdgpu_buffer_rsrc_t rs, uint32_t off) {
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rs, static_cast<int>(off), 0, 0);
+        return make_uint4(v.x, v.y, v.z, v.w);
+    };
+    // [k][n] operand of the N side; rows below k_end only
+    const __amdgpu_buffer_rsrc_t b_rs = rsrc(B, static_cast<uint32_t>(k_end) * static_cast<uint32_t>(p.ldb) * 2u);
+    const uint32_t b_col = n0 + (tid & 15) * 8 < p.N ? (n0 + (tid & 15) * 8) * 2u : kOutside;
+    // M side: [k][m] rows below k_end, or [m][k] rows below m_end
+    const __amdgpu_buffer_rsrc_t a_rs = rsrc(p.A, static_cast<uint32_t>(A_KS ? k_end : m_end) * static_cast<uint32_t>(p.lda) * 2u);
+    const uint32_t a_col = m0 + (tid & 31) * 8 < p.M ? (m0 + (tid & 31) * 8) * 2u : kOutside;
+    uint32_t arow[8];        // K-contiguous form: byte offsets of this lane's eight rows, fixed for the whole tile
+    if constexpr (!A_KS) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) arow[i] = static_cast<uint32_t>(m0 + (tid >> 3) + 32 * i) * static_cast<uint32_t>(p.lda) * 2u;
+    }
+    auto fetch = [&](int ks, uint4 (&ra)[8], uint4 (&rb)[4]) {
+        const int k0 = k_begin + ks * TK;
+        if constexpr (A_KS) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                ra[i] = load16(a_rs, static_cast<uint32_t>(k0 + (tid >> 5) + 8 * i) * static_cast<uint32_t>(p.lda) * 2u + a_col);
+        } else {
+            const int k = k0 + (tid & 7) * 8;
+            const uint32_t kcol = k < k_end ? k * 2u : kOutside;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ra[i] = load16(a_rs, arow[i] + kcol);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            rb[i] = load16(b_rs, static_cast<uint32_t>(k0 + (tid >> 4) + 16 * i) * static_cast<uint32_t>(p.ldb) * 2u + b_col);
+    };
+    auto stash = [&](int stage, const uint4 (&ra)[8], const uint4 (&rb)[4]) {
+        uint8_t* as = smem + stage * kStage;
+        uint8_t* bs = as + kATile;
+        if constexpr (A_KS) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) *reinterpret_cast<uint4*>(as + ((tid >> 5) + 8 * i) * kPitchM + (tid & 31) * 16) = ra[i];
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int r = (tid >> 3) + 32 * i;
+                *reinterpret_cast<uint4*>(as + r * kPitchKC + (((tid & 7) ^ swz(r)) << 4)) = ra[i];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4*>(bs + ((tid >> 4) + 16 * i) * kPitchN + (tid & 15) * 16) = rb[i];
+    };
+
+    // ---- LDS -> MFMA ----
+    v16f acc[2][4];      // [n tile][m tile]
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[j][i][r] = 0.0f;
+
+    const int frow = lane & 31, khalf = lane >> 5;
+    auto compute = [&](int stage) {
+        const uint8_t* as = smem + stage * kStage;
+        const uint8_t* bs = as + kATile;
+#pragma unroll
+        for (int s = 0; s < TK / 16; ++s) {
+            v8bf nop[2], mop[4];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) nop[j] = read_ks(bs, kPitchN, 16 * s, wn * 64 + 32 * j, lane);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if constexpr (A_KS) {
+                    mop[i] = read_ks(as, kPitchM, 16 * s, wm * 128 + 32 * i, lane);
+                } else {
+                    const int row = wm * 128 + 32 * i + frow;
+                    mop[i] = *reinterpret_cast<const v8bf*>(as + row * kPitchKC + (((2 * s + khalf) ^ swz(row)) << 4));
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(nop[j], mop[i], acc[j][i], 0, 0, 0);
+            // one k-step's operands in registers at a time: the staged global loads of two K-tiles are live across this loop
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    // Tile ks is multiplied from LDS stage ks % 2 while tile ks + 1 waits in (or lands into) one register set and
+    // tile ks + 2 is requested into the other.  The loop body covers two K-tiles and has no exits: a tile past the
+    // end of the k range is fetched as zeros (it lies beyond the descriptors) and adds nothing.
+    uint4 ra0[8], rb0[4], ra1[8], rb1[4];
+    fetch(0, ra0, rb0);
+    fetch(1, ra1, rb1);
+    stash(0, ra0, rb0);
+    __syncthreads();
+    for (int ks = 0; ks < nk; ks += 2) {
+        fetch(ks + 2, ra0, rb0);
+        compute(0);
+        stash(1, ra1, rb1);
+        __syncthreads();
+        fetch(ks + 3, ra1, rb1);
+        compute(1);
+        stash(0, ra0, rb0);
+        __syncthreads();
+    }
+
+    // ---- epilogue: accumulator register r of tile (j, i) is output row m0 + wm*128 + 32 i + lane % 32,
+    //      column n0 + wn*64 + 32 j + 8 (r / 4) + 4 (lane / 32) + r % 4 ----
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = m0 + wm * 128 + 32 * i + frow;
+        if (m >= m_end) continue;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int n = n0 + wn * 64 + 32 * j + 8 * q + 4 * khalf;
+                if (n >= p.N) continue;                      // N % 8 == 0: a quad is inside or outside as a whole
+                const size_t at = c_base + static_cast<size_t>(m) * p.ldc + n;
+                float v[4] = {acc[j][i][4 * q], acc[j][i][4 * q + 1], acc[j][i][4 * q + 2], acc[j][i][4 * q + 3]};
+                if constexpr (OUT == OUT_ACCUM_F32) {
+                    float4* dst = reinterpret_cast<float4*>(static_cast<float*>(p.C) + at);
+                    float4 c = *dst;
+                    c.x += v[0]; c.y += v[1]; c.z += v[2]; c.w += v[3];
+                    *dst = c;
+                } else {
+                    uint2* dst = reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.C) + at);
+                    if constexpr (OUT == OUT_ACCUM_BF16) {
+                        // fp32 sum of the old value and the product, one rounding (cublasGemmEx with a bf16 C, beta = 1)
+                        const uint2 c = *dst;
+                        v[0] += bf16_lo(c.x); v[1] += bf16_hi(c.x); v[2] += bf16_lo(c.y); v[3] += bf16_hi(c.y);
+                    }
+                    *dst = make_uint2(pack_bf16x2_hw(v[0], v[1]), pack_bf16x2_hw(v[2], v[3]));
+                }
+            }
+    }
+}
+
+template <bool A_KS, int OUT, bool GROUPED>
+int launch(const BfArgs& p, dim3 grid, hipStream_t st) {
+    static std::once_flag once;
+    hipError_t attr = hipSuccess;
+    auto kern = k_gemm_bf16<A_KS, OUT, GROUPED>;
+    std::call_once(once, [&] {
+        attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    });
+    if (attr != hipSuccess) return static_cast<int>(attr);
+    kern<<<grid, kThr, kLds, st>>>(p);
+    return launch_status();
+}
+
+bool operands_ok(const void* A, int lda, const void* B, int ldb, const void* C, int ldc, int c_elem_bytes) {
+    return aligned16(A) && aligned16(B) && lda % 8 == 0 && ldb % 8 == 0 && ldc % 4 == 0 &&
+           (reinterpret_cast<uintptr_t>(C) & (4u * c_elem_bytes - 1u)) == 0;
+}
+
+// C[M,N] = A[M,K] . B[K,N]; grouped: per expert over its rows of the compact buffers
+int gemm_nn(int M, int N, int K, int E, const int* counts, const int* offsets, const uint16_t* A, int lda, const uint16_t* B,
+            int ldb, uint16_t* C, int ldc, void* ws, size_t ws_bytes, bool grouped, cf_stream_t stream) {
+    if (M < 0 || N < 0 || K < 0 || E < 0) return CF_ERR_INVALID_ARG;
+    if (M == 0 || N == 0 || (grouped && E == 0)) return CF_OK;
+    if (!A || !B || !C || (grouped && (!counts || !offsets || !ws))) return CF_ERR_INVALID_ARG;
+    if (lda < K || ldb < N || ldc < N) return CF_ERR_INVALID_ARG;
+    if (N % 8 != 0 || K % 8 != 0 || !operands_ok(A, lda, B, ldb, C, ldc, 2)) return CF_ERR_UNSUPPORTED;
+    if (static_cast<size_t>(M) * lda >= (1ull << 30) || static_cast<size_t>(K) * ldb >= (1ull << 30)) return CF_ERR_UNSUPPORTED;
+    hipStream_t st = as_stream(stream);
+    BfArgs p{};
+    p.A = A; p.lda = lda; p.B = B; p.ldb = ldb; p.C = C; p.ldc = ldc;
+    p.M = M; p.N = N; p.K = K;
+    p.tiles_n = (N + TN - 1) / TN;
+    int tiles_m = (M + TM - 1) / TM;
+    auto grid_for = [&](int row_tiles) {      // 8 XCDs x the per-XCD share of the tiles, rounded up
+        const long long total = static_cast<long long>(row_tiles) * p.tiles_n;
+        return dim3(static_cast<unsigned>(8 * ((total + 7) / 8)));
+    };
+    if (grouped) {
+        size_t need = 0;
+        cf_fp8_grouped_gemm_workspace_bytes(M, E, &need);
+        if (ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 3u)) return CF_ERR_INVALID_ARG;
+        tiles_m = M / TM + E;
+        build_tile_map(counts, offsets, E, tiles_m, static_cast<int*>(ws), st);
+        p.counts = counts; p.offsets = offsets;
+        p.tile_map = static_cast<const int*>(ws);
+        p.b_expert_stride = static_cast<long long>(K) * ldb;
+        p.tiles_m = tiles_m;
+        return launch<false, OUT_STORE_BF16, true>(p, grid_for(tiles_m), st);
+    }
+    p.tiles_m = tiles_m;
+    return launch<false, OUT_STORE_BF16, false>(p, grid_for(tiles_m), st);
+}
+
+// C[M,N] += A[K,M]^T . B[K,N]; grouped: per expert, K running over its rows of the compact buffers, C[E,M,N]
+template <int OUT>
+int gemm_tn(int M, int N, int K, int E, const int* counts, const int* offsets, const uint16_t* A, int lda, const uint16_t* B,
+            int ldb, void* C, int ldc, bool grouped, cf_stream_t stream) {
+    if (M < 0 || N < 0 || K < 0 || E < 0) return CF_ERR_INVALID_ARG;
+    if (M == 0 || N == 0 || K == 0 || (grouped && E == 0)) return CF_OK;
+    if (!A || !B || !C || (grouped && (!counts || !offsets))) return CF_ERR_INVALID_ARG;
+    if (lda < M || ldb < N || ldc < N) return CF_ERR_INVALID_ARG;
+    if (N % 8 != 0 || M % 8 != 0 || !operands_ok(A, lda, B, ldb, C, ldc, OUT == OUT_ACCUM_F32 ? 4 : 2)) return CF_ERR_UNSUPPORTED;
+    if (static_cast<size_t>(K) * lda >= (1ull << 30) || static_cast<size_t>(K) * ldb >= (1ull << 30)) return CF_ERR_UNSUPPORTED;
+    hipStream_t st = as_stream(stream);
+    BfArgs p{};
+    p.A = A; p.lda = lda; p.B = B; p.ldb = ldb; p.C = C; p.ldc = ldc;
+    p.M = M; p.N = N; p.K = K;
+    p.tiles_n = (N + TN - 1) / TN;
+    p.tiles_m = (M + TM - 1) / TM;
+    const long long tiles = static_cast<long long>(p.tiles_m) * p.tiles_n;
+    if (grouped) {
+        p.counts = counts; p.offsets = offsets;
+        p.num_experts = E;
+        p.c_expert_stride = static_cast<long long>(M) * ldc;
+        const long long blocks = 8LL * ((E + 7) / 8) * tiles;
+        if (blocks >= (1LL << 31)) return CF_ERR_UNSUPPORTED;
+        return launch<true, OUT, true>(p, dim3(static_cast<unsigned>(blocks)), st);
+    }
+    return launch<true, OUT, false>(p, dim3(static_cast<unsigned>(8 * ((tiles + 7) / 8))), st);
+}
+
+}  // namespace
+}  // namespace cf
+
+using namespace cf;
+
+extern "C" {
+
+int cf_gemm_bf16_nn(int M, int N, int K, const uint16_t* A, int lda, const uint16_t* B, int ldb, uint16_t* C, int ldc,
+                    cf_stream_t stream) {
+    return gemm_nn(M, N, K, 0, nullptr, nullptr, A, lda, B, ldb, C, ldc, nullptr, 0, false, stream);
+}
+int cf_gemm_bf16_tn_accum_f32(int M, int N, int K, const uint16_t* A, int lda, const uint16_t* B, int ldb, float* C, int ldc,
+                              cf_stream_t stream) {
+    return gemm_tn<OUT_ACCUM_F32>(M, N, K, 0, nullptr, nullptr, A, lda, B, ldb, C, ldc, false, stream);
+}
+int cf_gemm_bf16_tn_accum_bf16(int M, int N, int K, const uint16_t* A, int lda, const uint16_t* B, int ldb, uint16_t* C,
+                               int ldc, cf_stream_t stream) {
+    return gemm_tn<OUT_ACCUM_BF16>(M, N, K, 0, nullptr, nullptr, A, lda, B, ldb, C, ldc, false, stream);
+}
+int cf_moe_grouped_gemm_bf16_nn(int total_rows, int N, int K, int num_experts, const int* d_counts, const int* d_offsets,
+                                const uint16_t* A, int lda, const uint16_t* B, uint16_t* C, int ldc, void* d_workspace,
+                                size_t workspace_bytes, cf_stream_t stream) {
+    return gemm_nn(total_rows, N, K, num_experts, d_counts, d_offsets, A, lda, B, N, C, ldc, d_workspace, workspace_bytes, true,
+                   stream);
+}
+int cf_moe_grouped_gemm_bf16_tn_accum_f32(int M, int N, int total_rows, int num_experts, const int* d_counts,
+                                          const int* d_offsets, const uint16_t* A, int lda, const uint16_t* B, int ldb,
+                                          float* C, cf_stream_t stream) {
+    return gemm_tn<OUT_ACCUM_F32>(M, N, total_rows, num_experts, d_counts, d_offsets, A, lda, B, ldb, C, N, true, stream);
+}
+int cf_moe_grouped_gemm_bf16_tn_accum_bf16(int M, int N, int total_rows, int num_experts, const int* d_counts,
+                                           const int* d_offsets, const uint16_t* A, int lda, const uint16_t* B, int ldb,
+                                           uint16_t* C, cf_stream_t stream) {
+    return gemm_tn<OUT_ACCUM_BF16>(M, N, total_rows, num_experts, d_counts, d_offsets, A, lda, B, ldb, C, N, true, stream);
+}
+
+}  // extern "C"

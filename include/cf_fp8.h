@@ -369,6 +369,46 @@ int cf_fp8_grouped_gemm_nt_bf16_static(int total_rows, int N, int K, int num_exp
                                        int epilogue, const void* d_B_up, const float* d_b_up_descale,
                                        uint16_t* d_C, int ldc, cf_stream_t stream);
 
+/* ---- bf16 GEMMs of the selected-expert backward -------------------------------------
+ * The reference's selected-expert backward runs, per expert and behind a host copy of the counts, four
+ * cuBLAS calls on bf16 operands (src/trainer.cu:7727-7740; wrappers gemm_bf16 :3069-3090 and
+ * gemm_bf16_tn_f32 :3116-3160, all with alpha = 1):
+ *   d_act[n,Ie]   = d_expert_out[n,H] . fc_out_w[H,Ie]            gemm_bf16, beta = 0
+ *   g_out[H,Ie]  += d_expert_out[n,H]^T . act[n,Ie]               gemm_bf16_tn_f32, beta = 1
+ *   d_x[n,H]      = d_pre[n,Ie] . fc_in_w[Ie,H]                   gemm_bf16, beta = 0
+ *   g_in[Ie,H]   += d_pre[n,Ie]^T . x[n,H]                        gemm_bf16_tn_f32, beta = 1
+ * The dense forms below take the wrappers' arguments (row-major, row strides in elements); the grouped
+ * forms run every expert in one launch over the forward's saved counts / offsets, the experts' rows
+ * lying back to back in compact buffers (expert e owns rows offsets[e] .. offsets[e] + counts[e]).
+ * fp32 accumulation on the matrix cores, one rounding to bf16.  Needs 16-byte aligned operands, row
+ * strides that are multiples of 8 elements, N % 8 == 0, and K % 8 == 0 (nn) or M % 8 == 0 (tn); the
+ * contraction length of the tn forms (an expert's row count) is arbitrary. */
+
+/* C[M,N] = A[M,K] . B[K,N]   (gemm_bf16 with alpha = 1, beta = 0, src/trainer.cu:3069-3090) */
+int cf_gemm_bf16_nn(int M, int N, int K, const uint16_t* d_A, int lda, const uint16_t* d_B, int ldb,
+                    uint16_t* d_C, int ldc, cf_stream_t stream);
+/* C[M,N] += A[K,M]^T . B[K,N]   (gemm_bf16_tn_f32 with alpha = 1, beta = 1; fp32 C, src/trainer.cu:3116-3137) */
+int cf_gemm_bf16_tn_accum_f32(int M, int N, int K, const uint16_t* d_A, int lda, const uint16_t* d_B, int ldb,
+                              float* d_C, int ldc, cf_stream_t stream);
+/* the same with a bf16 C: bf16(float(C) + product), the overload at src/trainer.cu:3142-3160 */
+int cf_gemm_bf16_tn_accum_bf16(int M, int N, int K, const uint16_t* d_A, int lda, const uint16_t* d_B, int ldb,
+                               uint16_t* d_C, int ldc, cf_stream_t stream);
+/* For each expert e: C[rows of e, :] = A[rows of e, :K] . B[e]  with B [num_experts, K, N] row-major
+ * (the two input-gradient calls, src/trainer.cu:7729, 7738).  total_rows is the host-side bound rows * top_k;
+ * d_workspace holds the tile table: cf_fp8_grouped_gemm_workspace_bytes(total_rows, num_experts) bytes. */
+int cf_moe_grouped_gemm_bf16_nn(int total_rows, int N, int K, int num_experts, const int* d_counts,
+                                const int* d_offsets, const uint16_t* d_A, int lda, const uint16_t* d_B,
+                                uint16_t* d_C, int ldc, void* d_workspace, size_t workspace_bytes,
+                                cf_stream_t stream);
+/* For each expert e: C[e] += A[rows of e, :M]^T . B[rows of e, :N]  with C [num_experts, M, N]
+ * (the two weight-gradient calls, src/trainer.cu:7727, 7736); an expert without rows leaves its C alone. */
+int cf_moe_grouped_gemm_bf16_tn_accum_f32(int M, int N, int total_rows, int num_experts, const int* d_counts,
+                                          const int* d_offsets, const uint16_t* d_A, int lda,
+                                          const uint16_t* d_B, int ldb, float* d_C, cf_stream_t stream);
+int cf_moe_grouped_gemm_bf16_tn_accum_bf16(int M, int N, int total_rows, int num_experts, const int* d_counts,
+                                           const int* d_offsets, const uint16_t* d_A, int lda,
+                                           const uint16_t* d_B, int ldb, uint16_t* d_C, cf_stream_t stream);
+
 /* Row lists of all experts back to back: compact[offsets[e] + s] = row_indices[e, s]
  * (the gather order of moe_gather_rows_u8 over all experts, kernels/moe.cu:594-606). */
 int cf_moe_compact_row_index(const int* d_counts, const int* d_offsets, const int* d_row_indices,

@@ -222,6 +222,25 @@ inline void lt_gemm_fp8_tn_accum_f32(int M, int N, int K, const void* Xt_e4m3, c
     CF_FWD(cf_fp8_gemm_tn_accum_bf16(M, N, K, Xt_e4m3, ds_x, dYt_e5m2, ds_dy, hip_detail::u(dW), ldc_dw, s));
 }
 
+// gemm_bf16 and gemm_bf16_tn_f32, src/trainer.cu:3069-3090 and :3116-3160, as the selected-expert backward calls
+// them (:7727-7740): the cuBLAS handle becomes the stream, alpha is 1, beta is 0 for the input gradients and 1 for the
+// weight gradients; any other pair throws.
+inline void gemm_bf16(hipStream_t s, int M, int N, int K, float alpha, const bf16* A, int lda, const bf16* B, int ldb,
+                      float beta, bf16* C, int ldc) {
+    if (alpha != 1.0f || beta != 0.0f) throw std::invalid_argument("gemm_bf16: only alpha = 1, beta = 0 is built");
+    CF_FWD(cf_gemm_bf16_nn(M, N, K, hip_detail::u(A), lda, hip_detail::u(B), ldb, hip_detail::u(C), ldc, s));
+}
+inline void gemm_bf16_tn_f32(hipStream_t s, int M, int N, int K, float alpha, const bf16* A, int lda, const bf16* B,
+                             int ldb, float beta, float* C, int ldc) {
+    if (alpha != 1.0f || beta != 1.0f) throw std::invalid_argument("gemm_bf16_tn_f32: only alpha = 1, beta = 1 is built");
+    CF_FWD(cf_gemm_bf16_tn_accum_f32(M, N, K, hip_detail::u(A), lda, hip_detail::u(B), ldb, C, ldc, s));
+}
+inline void gemm_bf16_tn_f32(hipStream_t s, int M, int N, int K, float alpha, const bf16* A, int lda, const bf16* B,
+                             int ldb, float beta, bf16* C, int ldc) {
+    if (alpha != 1.0f || beta != 1.0f) throw std::invalid_argument("gemm_bf16_tn_f32: only alpha = 1, beta = 1 is built");
+    CF_FWD(cf_gemm_bf16_tn_accum_bf16(M, N, K, hip_detail::u(A), lda, hip_detail::u(B), ldb, hip_detail::u(C), ldc, s));
+}
+
 #undef CF_FWD
 
 }  // namespace ida_native

@@ -313,6 +313,29 @@ def main():
     hbm("gelu_forward_bf16", f"{total}x{Ie}", 4.0 * total * Ie, lambda: cf.cf_gelu_forward_bf16(pre, gpre, total * Ie, st))
     hbm("gelu_backward_bf16", f"{total}x{Ie}", 6.0 * total * Ie, lambda: cf.cf_gelu_backward_bf16(pre, gpost, gpre, total * Ie, st))
 
+    # the four bf16 GEMMs of the same backward, every expert in one launch (bf16 matrix peak 2.5 PFLOP/s)
+    BF16_PEAK = 2500.0
+
+    def mfma16(name, shape, flop, fn):
+        if args.only not in name:
+            return
+        t = timed(fn)
+        tf = flop / t / 1e12
+        print(f"{name:<64} {shape:<26} {t * 1e6:9.1f} {tf:7.0f} TFLOP/s {100 * tf / BF16_PEAK:7.1f}% (of bf16 peak)", flush=True)
+    wo16 = bf16(E * H, Ie, sigma=0.02); wi16 = bf16(E * Ie, H, sigma=0.02)
+    d_out = bf16(total, H, sigma=0.01); xg = bf16(total, H)
+    d_act = torch.empty((total, Ie), dtype=torch.bfloat16, device=dev); d_x = torch.empty((total, H), dtype=torch.bfloat16, device=dev)
+    g_out = torch.zeros((E * H, Ie), dtype=torch.bfloat16, device=dev); g_in = torch.zeros((E * Ie, H), dtype=torch.bfloat16, device=dev)
+    fl = 2.0 * total * Ie * H
+    mfma16("grouped bf16 dgrad: d_act = d_out . fc_out_w (nn)", f"{total}x{Ie}x{H}", fl,
+           lambda: cf.cf_moe_grouped_gemm_bf16_nn(total, Ie, H, E, counts, offs, d_out, H, wo16, d_act, Ie, ws, sz.value, st))
+    mfma16("grouped bf16 wgrad: g_out += d_out^T . act (tn, bf16 C)", f"{H}x{Ie}x~{total // E} x{E}", fl,
+           lambda: cf.cf_moe_grouped_gemm_bf16_tn_accum_bf16(H, Ie, total, E, counts, offs, d_out, H, pre, Ie, g_out, st))
+    mfma16("grouped bf16 dgrad: d_x = d_pre . fc_in_w (nn)", f"{total}x{H}x{Ie}", fl,
+           lambda: cf.cf_moe_grouped_gemm_bf16_nn(total, H, Ie, E, counts, offs, gpost, Ie, wi16, d_x, H, ws, sz.value, st))
+    mfma16("grouped bf16 wgrad: g_in += d_pre^T . x (tn, bf16 C)", f"{Ie}x{H}x~{total // E} x{E}", fl,
+           lambda: cf.cf_moe_grouped_gemm_bf16_tn_accum_bf16(Ie, H, total, E, counts, offs, gpost, Ie, xg, H, g_in, st))
+
 
 if __name__ == "__main__":
     main()

@@ -380,6 +380,16 @@ def gemm_nt_ref(A, B, a_descale, b_descale, a_e5m2=False, b_e5m2=False, scale_mo
     return ref, absdot
 
 
+def gemm_bf16_nn_ref(A, B):
+    """gemm_bf16 (src/trainer.cu:3069-3090) on bf16 bit patterns, carried in double: A[M,K] . B[K,N]."""
+    return bf16_to_f32(np.asarray(A)).astype(np.float64) @ bf16_to_f32(np.asarray(B)).astype(np.float64)
+
+
+def gemm_bf16_tn_ref(A, B):
+    """gemm_bf16_tn_f32 (src/trainer.cu:3116-3160) without the beta term, in double: A[K,M]^T . B[K,N]."""
+    return bf16_to_f32(np.asarray(A)).astype(np.float64).T @ bf16_to_f32(np.asarray(B)).astype(np.float64)
+
+
 def bf16_ulp(x):
     """Spacing of bf16 at |x| (8 significand bits), floor at the smallest normal."""
     ax = np.maximum(np.abs(np.asarray(x, dtype=np.float64)), 2.0 ** -126)

@@ -20,7 +20,10 @@ int main() {
     void (*f11)(int, int, int, const void*, const float*, const void*, const float*, bf16*, int, hipStream_t) = &lt_gemm_fp8_tn_accum_f32;
     void (*f12)(const bf16*, const bf16*, const bf16*, bf16*, bf16*, int, hipStream_t) = &swiglu_backward;
     void (*f13)(const bf16*, float*, int, int, int, int, hipStream_t) = &col_sum_strided_bf16;
-    if (!f12 || !f13) return 1;
+    void (*f14)(hipStream_t, int, int, int, float, const bf16*, int, const bf16*, int, float, bf16*, int) = &gemm_bf16;
+    void (*f15)(hipStream_t, int, int, int, float, const bf16*, int, const bf16*, int, float, float*, int) = &gemm_bf16_tn_f32;
+    void (*f16)(hipStream_t, int, int, int, float, const bf16*, int, const bf16*, int, float, bf16*, int) = &gemm_bf16_tn_f32;
+    if (!f12 || !f13 || !f14 || !f15 || !f16) return 1;
     if (!f1 || !f2 || !f3 || !f4 || !f5 || !f6 || !f7 || !f8 || !f9 || !f10 || !f11) return 1;
     int ok = 0;
     try { swiglu_forward(nullptr, nullptr, nullptr, -1, nullptr); } catch (const std::invalid_argument&) { ++ok; }   // kernels/activations.cu:61-72

@@ -1,0 +1,222 @@
+"""GPU parity: the bf16 GEMMs of the selected-expert MoE backward (gemm_bf16 / gemm_bf16_tn_f32 of
+src/trainer.cu:3069-3160 as called at :7727-7740), dense and grouped per expert, against the matmul of the
+same bf16 operands carried in double.  The reference's cuBLAS calls accumulate in fp32 in an order that is
+not defined, so the bar is the GEMM bar of the FP8 path: the bf16 results within half a bf16 ulp of the
+double reference plus an fp32 accumulation allowance; exactly summable operands must match to the bit."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import oracle_lib as orc
+from gpu_util import bf16_bits, case, dev_arr, dev_bf16, host, stream
+
+pytestmark = pytest.mark.gpu
+
+ACC = 16.0 * 2.0 ** -24          # fp32 accumulation on the matrix cores, as a multiple of sum |a_k b_k|
+
+
+def rand_bf16(rng, shape, sigma=1.0):
+    return orc.bf16_from_f32((rng.standard_normal(shape) * sigma).astype(np.float32))
+
+
+def absdot(A, B, tn=False):
+    a = np.abs(orc.bf16_to_f32(A).astype(np.float64))
+    b = np.abs(orc.bf16_to_f32(B).astype(np.float64))
+    return (a.T if tn else a) @ b
+
+
+def check_bf16_out(got_bits, ref, ad, what):
+    got = orc.bf16_to_f32(got_bits).astype(np.float64)
+    tol = 0.505 * orc.bf16_ulp(np.maximum(np.abs(ref), np.abs(got))) + ACC * ad
+    bad = np.abs(got - ref) > tol
+    assert not bad.any(), f"{what}: {int(bad.sum())} outside tolerance, worst {float((np.abs(got - ref) / tol).max()):.3f}"
+
+
+def padded(bits, ld):
+    """[r, c] bit patterns -> [r, ld] with NaN padding (a kernel that reads the padding shows up)."""
+    out = np.full((bits.shape[0], ld), 0x7fc0, np.uint16)
+    out[:, :bits.shape[1]] = bits
+    return out
+
+
+@pytest.mark.parametrize("M,N,K,pad", [(256, 128, 64, 0), (300, 200, 136, 8), (1, 8, 8, 0), (513, 264, 1000, 16), (1024, 1408, 2048, 0),
+                                       (40, 136, 72, 0)])
+def test_gemm_bf16_nn(cf, dev, M, N, K, pad):
+    case(f"bf16 nn {M}x{N}x{K} pad {pad}")
+    rng = np.random.default_rng(M + N + K)
+    A, B = rand_bf16(rng, (M, K)), rand_bf16(rng, (K, N), 0.02)
+    lda, ldb, ldc = K + pad, N + pad, N + pad
+    C = torch.full((M, ldc), float("nan"), dtype=torch.bfloat16, device=dev)
+    cf.cf_gemm_bf16_nn(M, N, K, dev_bf16(padded(A, lda), dev), lda, dev_bf16(padded(B, ldb), dev), ldb, C, ldc, stream())
+    torch.cuda.synchronize()
+    got = bf16_bits(C)
+    assert np.all((got[:, N:] & 0x7fff) > 0x7f80)                      # row padding of C left alone
+    check_bf16_out(got[:, :N], orc.gemm_bf16_nn_ref(A, B), absdot(A, B), f"nn {M}x{N}x{K}")
+
+
+def test_gemm_bf16_exact_integers_equal_numpy(cf, dev):
+    """Small integers: every product and partial sum is exact in fp32, so all three forms must match numpy to the
+    bit; the operands are far from symmetric, so a transposed or misindexed operand cannot pass."""
+    case("bf16 GEMMs, exact integers")
+    rng = np.random.default_rng(3)
+    M, N, K = 300, 264, 200
+    a = rng.integers(-4, 5, (M, K)).astype(np.float32)
+    b = rng.integers(-3, 4, (K, N)).astype(np.float32)
+    C = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=dev)
+    cf.cf_gemm_bf16_nn(M, N, K, dev_bf16(orc.bf16_from_f32(a), dev), K, dev_bf16(orc.bf16_from_f32(b), dev), N, C, N, stream())
+    torch.cuda.synchronize()
+    assert np.array_equal(bf16_bits(C), orc.bf16_from_f32((a @ b).astype(np.float32)))
+    # tn: C[M2,N2] += A2[K2,M2]^T . B2[K2,N2]
+    K2, M2, N2 = 333, 264, 136
+    a2 = rng.integers(-4, 5, (K2, M2)).astype(np.float32)
+    b2 = rng.integers(-3, 4, (K2, N2)).astype(np.float32)
+    c0 = rng.integers(-50, 51, (M2, N2)).astype(np.float32)
+    Cf = torch.from_numpy(c0).to(dev)
+    cf.cf_gemm_bf16_tn_accum_f32(M2, N2, K2, dev_bf16(orc.bf16_from_f32(a2), dev), M2, dev_bf16(orc.bf16_from_f32(b2), dev), N2, Cf, N2, stream())
+    Cb = dev_bf16(orc.bf16_from_f32(c0), dev)
+    cf.cf_gemm_bf16_tn_accum_bf16(M2, N2, K2, dev_bf16(orc.bf16_from_f32(a2), dev), M2, dev_bf16(orc.bf16_from_f32(b2), dev), N2, Cb, N2, stream())
+    torch.cuda.synchronize()
+    want = c0 + a2.T @ b2
+    assert np.array_equal(host(Cf), want)
+    assert np.array_equal(bf16_bits(Cb), orc.bf16_from_f32(want))
+    assert not np.array_equal(want[:136, :136], want[:136, :136].T)
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 128, 64), (264, 200, 131), (8, 8, 1), (1408, 512, 777), (520, 136, 2000)])
+def test_gemm_bf16_tn_accumulate(cf, dev, M, N, K):
+    case(f"bf16 tn {M}x{N}x{K}")
+    rng = np.random.default_rng(M * 3 + N + K)
+    A, B = rand_bf16(rng, (K, M), 1e-2), rand_bf16(rng, (K, N))
+    ref, ad = orc.gemm_bf16_tn_ref(A, B), absdot(A, B, tn=True)
+    c0 = (rng.standard_normal((M, N)) * np.abs(ref).mean()).astype(np.float32)
+    Cf = torch.from_numpy(c0).to(dev)
+    cf.cf_gemm_bf16_tn_accum_f32(M, N, K, dev_bf16(A, dev), M, dev_bf16(B, dev), N, Cf, N, stream())
+    c0b = orc.bf16_from_f32(c0)
+    Cb = dev_bf16(c0b, dev)
+    cf.cf_gemm_bf16_tn_accum_bf16(M, N, K, dev_bf16(A, dev), M, dev_bf16(B, dev), N, Cb, N, stream())
+    torch.cuda.synchronize()
+    want = c0.astype(np.float64) + ref
+    assert np.all(np.abs(host(Cf).astype(np.float64) - want) <= ACC * ad + 2.0 ** -22 * (np.abs(want) + np.abs(c0)))
+    check_bf16_out(bf16_bits(Cb), orc.bf16_to_f32(c0b).astype(np.float64) + ref, ad, f"tn bf16 {M}x{N}x{K}")
+
+
+def routing(rng, rows, E, k, zero_expert=None):
+    logits = rng.standard_normal((rows, E)).astype(np.float32)
+    if zero_expert is not None:
+        logits[:, zero_expert] = -50.0
+    rw = orc.moe_topk_route(logits, k)
+    counts, _ = orc.moe_build_expert_row_lists(rw)
+    return counts, orc.moe_expert_offsets(counts)
+
+
+def workspace(cf, dev, total, E):
+    sz = ctypes.c_size_t(0)
+    assert cf.raw_cf_fp8_grouped_gemm_workspace_bytes(total, E, ctypes.byref(sz)) == 0
+    return torch.empty(sz.value, dtype=torch.uint8, device=dev), sz.value
+
+
+@pytest.mark.parametrize("rows,E,k,H,Ie,zero", [(600, 5, 2, 256, 384, None), (300, 4, 2, 264, 136, 2), (1500, 3, 1, 512, 640, None), (40, 8, 3, 128, 72, None)])
+def test_grouped_bf16_backward_gemms(cf, dev, rows, E, k, H, Ie, zero):
+    """The four GEMMs of the selected-expert backward over a ragged routing (src/trainer.cu:7727-7740), each expert
+    against the double reference, and bit for bit against the dense entry point called per expert the way the
+    reference's loop does."""
+    case(f"grouped bf16 backward GEMMs rows={rows} E={E} k={k} H={H} Ie={Ie}")
+    rng = np.random.default_rng(rows + E + H)
+    counts, offsets = routing(rng, rows, E, k, zero)
+    total = rows * k
+    filled = int(counts.sum())
+    d_out = rand_bf16(rng, (total, H), 1e-2)          # d_expert_out, compact
+    act = rand_bf16(rng, (total, Ie))                 # post-GELU activations, compact
+    w_out = rand_bf16(rng, (E, H, Ie), 0.02)          # fc_out_w [E, H, Ie]
+    dc, do = dev_arr(counts, dev), dev_arr(offsets, dev)
+    ws, ws_bytes = workspace(cf, dev, total, E)
+    # input gradient: d_act[n, Ie] = d_out[n, H] . fc_out_w[e]   (K = H, N = Ie)
+    d_act = torch.full((total, Ie), float("nan"), dtype=torch.bfloat16, device=dev)
+    cf.cf_moe_grouped_gemm_bf16_nn(total, Ie, H, E, dc, do, dev_bf16(d_out, dev), H, dev_bf16(w_out, dev), d_act, Ie, ws, ws_bytes, stream())
+    # weight gradient: g_out[e][H, Ie] += d_out[n, H]^T . act[n, Ie]   (M = H, N = Ie, contraction over the expert's rows)
+    g0 = rand_bf16(rng, (E, H, Ie), 1e-2)
+    g_bf = dev_bf16(g0, dev)
+    g_f32 = torch.from_numpy(orc.bf16_to_f32(g0)).to(dev)
+    cf.cf_moe_grouped_gemm_bf16_tn_accum_bf16(H, Ie, total, E, dc, do, dev_bf16(d_out, dev), H, dev_bf16(act, dev), Ie, g_bf, stream())
+    cf.cf_moe_grouped_gemm_bf16_tn_accum_f32(H, Ie, total, E, dc, do, dev_bf16(d_out, dev), H, dev_bf16(act, dev), Ie, g_f32, stream())
+    torch.cuda.synchronize()
+    got_act, got_g, got_gf = bf16_bits(d_act), bf16_bits(g_bf), host(g_f32)
+    assert np.all((got_act[filled:] & 0x7fff) > 0x7f80), "rows past the experts' lists were written"
+    for e in range(E):
+        n, o = int(counts[e]), int(offsets[e])
+        if n == 0:
+            assert np.array_equal(got_g[e], g0[e]) and np.array_equal(got_gf[e], orc.bf16_to_f32(g0[e]))
+            continue
+        check_bf16_out(got_act[o:o + n], orc.gemm_bf16_nn_ref(d_out[o:o + n], w_out[e]), absdot(d_out[o:o + n], w_out[e]), f"d_act expert {e}")
+        ref = orc.gemm_bf16_tn_ref(d_out[o:o + n], act[o:o + n])
+        ad = absdot(d_out[o:o + n], act[o:o + n], tn=True)
+        base = orc.bf16_to_f32(g0[e]).astype(np.float64)
+        check_bf16_out(got_g[e], base + ref, ad, f"g_out expert {e}")
+        assert np.all(np.abs(got_gf[e] - (base + ref)) <= ACC * ad + 2.0 ** -22 * (np.abs(base + ref) + np.abs(base)))
+        # the reference's loop: one dense call per expert on that expert's slice
+        one = torch.full((n, Ie), float("nan"), dtype=torch.bfloat16, device=dev)
+        cf.cf_gemm_bf16_nn(n, Ie, H, dev_bf16(d_out[o:o + n], dev), H, dev_bf16(w_out[e], dev), Ie, one, Ie, stream())
+        ge = dev_bf16(g0[e], dev)
+        cf.cf_gemm_bf16_tn_accum_bf16(H, Ie, n, dev_bf16(d_out[o:o + n], dev), H, dev_bf16(act[o:o + n], dev), Ie, ge, Ie, stream())
+        torch.cuda.synchronize()
+        assert np.array_equal(bf16_bits(one), got_act[o:o + n]) and np.array_equal(bf16_bits(ge), got_g[e])
+
+
+def test_grouped_bf16_backward_gemms_config5_size(cf, dev):
+    """16384 tokens, 64 experts, top-6, H = 2048, Ie = 1408: the four GEMMs at full size, sampled against the
+    double reference (every expert, a few rows or weight-gradient rows each)."""
+    case("grouped bf16 backward GEMMs, config 5 size")
+    rows, E, k, H, Ie = 16384, 64, 6, 2048, 1408
+    rng = np.random.default_rng(55)
+    counts, offsets = routing(rng, rows, E, k)
+    total = rows * k
+    g = torch.Generator(device=dev).manual_seed(5)
+    d_out = (torch.randn((total, H), generator=g, device=dev) * 1e-2).to(torch.bfloat16)
+    d_pre = (torch.randn((total, Ie), generator=g, device=dev) * 1e-2).to(torch.bfloat16)
+    x = torch.randn((total, H), generator=g, device=dev).to(torch.bfloat16)
+    w_out = (torch.randn((E, H, Ie), generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    w_in = (torch.randn((E, Ie, H), generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    dc, do = dev_arr(counts, dev), dev_arr(offsets, dev)
+    ws, ws_bytes = workspace(cf, dev, total, E)
+    d_act = torch.empty((total, Ie), dtype=torch.bfloat16, device=dev)
+    d_x = torch.empty((total, H), dtype=torch.bfloat16, device=dev)
+    g_out = torch.zeros((E, H, Ie), dtype=torch.bfloat16, device=dev)
+    g_in = torch.zeros((E, Ie, H), dtype=torch.bfloat16, device=dev)
+    cf.cf_moe_grouped_gemm_bf16_nn(total, Ie, H, E, dc, do, d_out, H, w_out, d_act, Ie, ws, ws_bytes, stream())
+    cf.cf_moe_grouped_gemm_bf16_tn_accum_bf16(H, Ie, total, E, dc, do, d_out, H, d_pre, Ie, g_out, stream())
+    cf.cf_moe_grouped_gemm_bf16_nn(total, H, Ie, E, dc, do, d_pre, Ie, w_in, d_x, H, ws, ws_bytes, stream())
+    cf.cf_moe_grouped_gemm_bf16_tn_accum_bf16(Ie, H, total, E, dc, do, d_pre, Ie, x, H, g_in, stream())
+    torch.cuda.synchronize()
+    for e in range(0, E, 7):
+        n, o = int(counts[e]), int(offsets[e])
+        sel = np.sort(np.random.default_rng(e).choice(n, 6, replace=False)) + o
+        sidx = torch.from_numpy(sel).to(dev)
+        A = bf16_bits(d_out[sidx]); W = bf16_bits(w_out[e])
+        check_bf16_out(bf16_bits(d_act[sidx]), orc.gemm_bf16_nn_ref(A, W), absdot(A, W), f"d_act expert {e}")
+        A = bf16_bits(d_pre[sidx]); W = bf16_bits(w_in[e])
+        check_bf16_out(bf16_bits(d_x[sidx]), orc.gemm_bf16_nn_ref(A, W), absdot(A, W), f"d_x expert {e}")
+        # weight gradients: a few output rows (columns of the M-side operand), the whole contraction
+        mrows = np.sort(np.random.default_rng(100 + e).choice(Ie, 5, replace=False))
+        midx = torch.from_numpy(mrows).to(dev)
+        A = bf16_bits(d_out[o:o + n][:, midx]); Bm = bf16_bits(d_pre[o:o + n])
+        check_bf16_out(bf16_bits(g_out[e][midx]), orc.gemm_bf16_tn_ref(A, Bm), absdot(A, Bm, tn=True), f"g_out expert {e}")
+        A = bf16_bits(d_pre[o:o + n][:, midx]); Bm = bf16_bits(x[o:o + n])
+        check_bf16_out(bf16_bits(g_in[e][midx]), orc.gemm_bf16_tn_ref(A, Bm), absdot(A, Bm, tn=True), f"g_in expert {e}")
+
+
+def test_gemm_bf16_argument_errors(cf, dev):
+    a = torch.zeros(64 * 64, dtype=torch.bfloat16, device=dev)
+    c = torch.zeros(64 * 64, dtype=torch.bfloat16, device=dev)
+    p = lambda t: t.data_ptr()
+    assert cf.raw_cf_gemm_bf16_nn(-1, 8, 8, p(a), 8, p(a), 8, p(c), 8, None) == -1
+    assert cf.raw_cf_gemm_bf16_nn(8, 8, 8, None, 8, p(a), 8, p(c), 8, None) == -1
+    assert cf.raw_cf_gemm_bf16_nn(8, 8, 16, p(a), 8, p(a), 8, p(c), 8, None) == -1          # lda < K
+    assert cf.raw_cf_gemm_bf16_nn(8, 12, 8, p(a), 8, p(a), 16, p(c), 16, None) == -2        # N % 8
+    assert cf.raw_cf_gemm_bf16_nn(8, 8, 8, p(a) + 2, 8, p(a), 8, p(c), 8, None) == -2       # unaligned operand
+    assert cf.raw_cf_gemm_bf16_nn(0, 8, 8, p(a), 8, p(a), 8, p(c), 8, None) == 0
+    assert cf.raw_cf_gemm_bf16_tn_accum_bf16(12, 8, 8, p(a), 16, p(a), 8, p(c), 8, None) == -2   # M % 8
+    assert cf.raw_cf_gemm_bf16_tn_accum_bf16(8, 8, 0, p(a), 8, p(a), 8, p(c), 8, None) == 0
+    torch.cuda.synchronize()
+    assert torch.all(c == 0)

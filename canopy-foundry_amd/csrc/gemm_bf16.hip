@@ -12,7 +12,7 @@
 // column i.  Two such reads give a lane its eight k of a 32x32x16 MFMA operand.  An operand that is K-contiguous
 // in memory takes the usual path (128-byte LDS rows, 16-byte chunks xor-swizzled, ds_read_b128).
 //
-// Workgroup tile 256 (M) x 128 (N) x 64 (K), four wavefronts 2 x 2, each 128 x 64 = 4 x 2 tiles of
+// Workgroup tile 256 (M) x 256 (N) x 64 (K), four wavefronts 2 x 2, each 128 x 128 = 4 x 4 tiles of
 // v_mfma_f32_32x32x16_bf16 with fp32 accumulators.  The N-side operand goes to the MFMA "A" side, so a lane
 // ends up with four consecutive output columns of one output row per accumulator quad.  Global loads are
 // register staged two K-tiles ahead (16 bytes per lane), LDS is double buffered, one barrier per K-tile.
@@ -21,19 +21,21 @@
 #include "common.hpp"
 
 #include <mutex>
+#include <type_traits>
 
 namespace cf {
 namespace {
 
-constexpr int TM = 256, TN = 128, TK = 64, kThr = 256;
-constexpr int kPitchKC = TK * 2;               // a K-contiguous tile: 128-byte rows, chunks swizzled
+constexpr int TM = 256, TN = 256, kThr = 256;
+constexpr int kMaxTK = 64;
+constexpr int kPitchKC = kMaxTK * 2;           // a K-contiguous tile: 128-byte rows, chunks swizzled
 constexpr int kPitchM = TM * 2 + 64;           // a [k][m] tile of the M side: 576-byte rows
-constexpr int kPitchN = TN * 2 + 64;           // a [k][n] tile of the N side: 320-byte rows
+constexpr int kPitchN = TN * 2 + 64;           // a [k][n] tile of the N side: 576-byte rows
 // the pads put four consecutive k rows into four different quarters of the 256 bytes the banks span
-constexpr int kATile = TK * kPitchM;           // 36,864 bytes: covers both forms of the M-side tile (K-contiguous: 32,768)
-constexpr int kBTile = TK * kPitchN;           // 20,480 bytes
+constexpr int kATile = kMaxTK * kPitchM;           // 36,864 bytes: covers both forms of the M-side tile (K-contiguous: 32,768)
+constexpr int kBTile = kMaxTK * kPitchN;           // 36,864 bytes
 constexpr int kStage = kATile + kBTile;
-constexpr int kLds = 2 * kStage;               // 114,688 bytes: one workgroup per CU
+constexpr int kLds = 2 * kStage;               // 147,456 bytes: one workgroup per CU
 
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef __bf16 v4bf __attribute__((ext_vector_type(4)));
@@ -55,14 +57,28 @@ struct BfArgs {
     long long c_expert_stride;      // TN: elements between the experts' C matrices
 };
 
+// An accumulator element as a vector-ALU operand.  The explicit read keeps the register allocator from moving whole
+// accumulator tiles into ordinary registers around the epilogue.
+__device__ __forceinline__ float acc_read(float a) {
+    float v;
+    asm("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
+    return v;
+}
+
 __device__ __forceinline__ int swz(int row) { return (row ^ ((row >> 3) & 3)) & 7; }
 
-// eight k of one column for every lane: two transposing reads of a [k][columns] tile at `base` (row pitch `pitch`)
-__device__ __forceinline__ v8bf read_ks(const uint8_t* base, int pitch, int krow0, int col0, int lane) {
+// Eight k of one column for every lane: two transposing reads of a [k][columns] tile.  `lane_ptr` is the tile's base
+// plus this lane's share of the address (ks_lane_offset); the k-step and the column block are compile-time
+// constants, so they end up in the instructions' immediate offsets and no address register is spent on them.
+__device__ __forceinline__ int ks_lane_offset(int pitch, int lane) {
     const int b = lane >> 4, r = lane & 15;
-    const uint8_t* p = base + (krow0 + 8 * (b >> 1) + (r >> 2)) * pitch + (col0 + 16 * (b & 1) + 4 * (r & 3)) * 2;
+    return (8 * (b >> 1) + (r >> 2)) * pitch + (16 * (b & 1) + 4 * (r & 3)) * 2;
+}
+template <int PITCH>
+__device__ __forceinline__ v8bf read_ks(const uint8_t* lane_ptr, int krow0, int col0) {
+    const uint8_t* p = lane_ptr + krow0 * PITCH + col0 * 2;
     const v4bf lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_v4bf_ptr)(p));
-    const v4bf hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_v4bf_ptr)(p + 4 * pitch));
+    const v4bf hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_v4bf_ptr)(p + 4 * PITCH));
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
@@ -91,11 +107,12 @@ void k_gemm_bf16(const BfArgs p) {
         if (e >= p.num_experts) return;
         m0 = (t % p.tiles_m) * TM;
         n0 = (t / p.tiles_m) * TN;
-        k_begin = p.offsets[e];
-        k_end = k_begin + p.counts[e];
+        // uniform values, but loaded through the vector path: moved to scalar registers, where the descriptors need them
+        k_begin = __builtin_amdgcn_readfirstlane(p.offsets[e]);
+        k_end = k_begin + __builtin_amdgcn_readfirstlane(p.counts[e]);
         c_base = static_cast<size_t>(e) * p.c_expert_stride;
     } else {
-        const int row_tiles = (GROUPED ? p.tile_map[0] : p.tiles_m);
+        const int row_tiles = GROUPED ? __builtin_amdgcn_readfirstlane(p.tile_map[0]) : p.tiles_m;
         const int total = row_tiles * p.tiles_n;
         const int per = (total + 7) / 8;
         const int t = x * per + xi;
@@ -108,66 +125,65 @@ void k_gemm_bf16(const BfArgs p) {
         m0 = tmi * TM;
         if constexpr (GROUPED) {
             const int* e = p.tile_map + 1 + 5 * tmi;
-            m0 = e[1] + (tmi - e[3]) * TM;
-            m_end = min(m0 + TM, e[2]);
-            B += static_cast<size_t>(e[0]) * p.b_expert_stride;
+            const int expert = __builtin_amdgcn_readfirstlane(e[0]), first_row = __builtin_amdgcn_readfirstlane(e[1]);
+            const int end_row = __builtin_amdgcn_readfirstlane(e[2]), first_tile = __builtin_amdgcn_readfirstlane(e[3]);
+            m0 = first_row + (tmi - first_tile) * TM;
+            m_end = min(m0 + TM, end_row);
+            B += static_cast<size_t>(expert) * p.b_expert_stride;
         }
     }
     if (k_end <= k_begin) {
         if constexpr (OUT != OUT_STORE_BF16) return;      // nothing to add
     }
+    constexpr int TK = 64;
+    constexpr int NA = A_KS ? TK / 8 : 8, NB = TK / 8;       // 16-byte chunks per lane and K-tile
     const int nk = (k_end - k_begin + TK - 1) / TK;
 
     // ---- global -> registers -> LDS: 16-byte chunks through buffer loads ----
-    // A buffer load takes a descriptor with the operand's size in bytes and returns zeros for anything beyond it, so
-    // every load is issued unconditionally (loads under branches would keep the compiler from counting the loads in
-    // flight: it would wait for all of them, the prefetch included, before the first LDS store) and the zero fill of
-    // the ragged ends costs nothing: the descriptor of a [k][columns] operand ends with the last row of the k range,
-    // and a lane whose columns lie outside the operand (or, for the K-contiguous form, whose k chunk lies beyond K)
-    // simply uses an offset beyond every descriptor.  Offsets are 32-bit byte offsets; the launcher keeps operands
+    // A buffer load takes a descriptor with a base and a size in bytes and returns zeros for a lane whose offset lies
+    // beyond the size, so every load is issued unconditionally (loads under branches would keep the compiler from
+    // counting the loads in flight: it would wait for all of them, the prefetch included, before the first LDS store)
+    // and the zero fill of the ragged ends costs nothing.  Each load gets a descriptor of its own, built with scalar
+    // instructions: the base is the first of the eight-row (32-row) group it fetches, the size what is left of the
+    // operand from there (nothing, past the end of the k range), so the lane's offset is one constant per operand: its
+    // row within the group and its 16-byte column; a lane whose columns lie outside the operand (or, for the
+    // K-contiguous form, whose k chunk lies beyond K) uses an offset beyond every size.  The launcher keeps operands
     // below 2 GiB.
     constexpr uint32_t kOutside = 0x80000000u;
     typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-    auto rsrc = [](const void* base, uint32_t bytes) {
-        return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(bytes), 0x00020000);
-    };
-    auto load16 = [](__amdgpu_buffer_rsrc_t rs, uint32_t off) {
-        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rs, static_cast<int>(off), 0, 0);
+    // rows [row0, row_end) of a row-major operand with `ld` elements per row, seen from element `col0` of row row0
+    auto load_rows = [](const uint16_t* base, int ld, int row0, int row_end, int col0, uint32_t lane_off) {
+        const int rows_left = max(row_end - row0, 0);
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<uint16_t*>(base + static_cast<size_t>(row0) * ld + col0), 0,
+            static_cast<int>(static_cast<uint32_t>(rows_left) * static_cast<uint32_t>(ld) * 2u), 0x00020000);
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rs, static_cast<int>(lane_off), 0, 0);
         return make_uint4(v.x, v.y, v.z, v.w);
     };
-    // [k][n] operand of the N side; rows below k_end only
-    const __amdgpu_buffer_rsrc_t b_rs = rsrc(B, static_cast<uint32_t>(k_end) * static_cast<uint32_t>(p.ldb) * 2u);
-    const uint32_t b_col = n0 + (tid & 15) * 8 < p.N ? (n0 + (tid & 15) * 8) * 2u : kOutside;
-    // M side: [k][m] rows below k_end, or [m][k] rows below m_end
-    const __amdgpu_buffer_rsrc_t a_rs = rsrc(p.A, static_cast<uint32_t>(A_KS ? k_end : m_end) * static_cast<uint32_t>(p.lda) * 2u);
-    const uint32_t a_col = m0 + (tid & 31) * 8 < p.M ? (m0 + (tid & 31) * 8) * 2u : kOutside;
-    uint32_t arow[8];        // K-contiguous form: byte offsets of this lane's eight rows, fixed for the whole tile
-    if constexpr (!A_KS) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) arow[i] = static_cast<uint32_t>(m0 + (tid >> 3) + 32 * i) * static_cast<uint32_t>(p.lda) * 2u;
-    }
-    auto fetch = [&](int ks, uint4 (&ra)[8], uint4 (&rb)[4]) {
+    // [k][columns] operands: this lane's row within a group of eight k rows and its 16-byte column
+    const uint32_t b_lane = n0 + (tid & 31) * 8 < p.N ? (tid >> 5) * static_cast<uint32_t>(p.ldb) * 2u + (tid & 31) * 16u : kOutside;
+    const uint32_t a_lane_ks = m0 + (tid & 31) * 8 < p.M ? (tid >> 5) * static_cast<uint32_t>(p.lda) * 2u + (tid & 31) * 16u : kOutside;
+    // [m][k] operand: this lane's row within a group of 32 rows and its 16-byte k chunk
+    const uint32_t a_lane_kc = (tid >> 3) * static_cast<uint32_t>(p.lda) * 2u + (tid & 7) * 16u;
+    auto fetch = [&](int ks, uint4 (&ra)[NA], uint4 (&rb)[NB]) {
         const int k0 = k_begin + ks * TK;
         if constexpr (A_KS) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i)
-                ra[i] = load16(a_rs, static_cast<uint32_t>(k0 + (tid >> 5) + 8 * i) * static_cast<uint32_t>(p.lda) * 2u + a_col);
+            for (int i = 0; i < NA; ++i) ra[i] = load_rows(p.A, p.lda, k0 + 8 * i, k_end, m0, a_lane_ks);
         } else {
-            const int k = k0 + (tid & 7) * 8;
-            const uint32_t kcol = k < k_end ? k * 2u : kOutside;
+            const uint32_t off = k0 + (tid & 7) * 8 < k_end ? a_lane_kc : kOutside;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) ra[i] = load16(a_rs, arow[i] + kcol);
+            for (int i = 0; i < 8; ++i) ra[i] = load_rows(p.A, p.lda, m0 + 32 * i, m_end, k0, off);
         }
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            rb[i] = load16(b_rs, static_cast<uint32_t>(k0 + (tid >> 4) + 16 * i) * static_cast<uint32_t>(p.ldb) * 2u + b_col);
+        for (int i = 0; i < NB; ++i) rb[i] = load_rows(B, p.ldb, k0 + 8 * i, k_end, n0, b_lane);
     };
-    auto stash = [&](int stage, const uint4 (&ra)[8], const uint4 (&rb)[4]) {
+    auto stash = [&](int stage, const uint4 (&ra)[NA], const uint4 (&rb)[NB]) {
         uint8_t* as = smem + stage * kStage;
         uint8_t* bs = as + kATile;
         if constexpr (A_KS) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) *reinterpret_cast<uint4*>(as + ((tid >> 5) + 8 * i) * kPitchM + (tid & 31) * 16) = ra[i];
+            for (int i = 0; i < NA; ++i) *reinterpret_cast<uint4*>(as + ((tid >> 5) + 8 * i) * kPitchM + (tid & 31) * 16) = ra[i];
         } else {
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
@@ -176,42 +192,50 @@ void k_gemm_bf16(const BfArgs p) {
             }
         }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4*>(bs + ((tid >> 4) + 16 * i) * kPitchN + (tid & 15) * 16) = rb[i];
+        for (int i = 0; i < NB; ++i) *reinterpret_cast<uint4*>(bs + ((tid >> 5) + 8 * i) * kPitchN + (tid & 31) * 16) = rb[i];
     };
 
     // ---- LDS -> MFMA ----
-    v16f acc[2][4];      // [n tile][m tile]
+    v16f acc[4][4];      // [n tile][m tile]
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < 4; ++j)
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[j][i][r] = 0.0f;
 
     const int frow = lane & 31, khalf = lane >> 5;
-    auto compute = [&](int stage) {
+    const int ks_n = ks_lane_offset(kPitchN, lane) + wn * 128 * 2, ks_m = ks_lane_offset(kPitchM, lane) + wm * 128 * 2;
+    // The fragments of k-step s + 1 are read while the MFMAs of k-step s run (one wavefront per SIMD: nobody else
+    // would fill the matrix cores during an LDS round trip), two fragment sets in turn.
+    auto compute = [&](auto stage_c) {
+        constexpr int stage = decltype(stage_c)::value;
         const uint8_t* as = smem + stage * kStage;
         const uint8_t* bs = as + kATile;
+        v8bf nop[2][4], mop[2][4];
+        auto read_frags = [&](int s, v8bf (&nf)[4], v8bf (&mf)[4]) {
 #pragma unroll
-        for (int s = 0; s < TK / 16; ++s) {
-            v8bf nop[2], mop[4];
-#pragma unroll
-            for (int j = 0; j < 2; ++j) nop[j] = read_ks(bs, kPitchN, 16 * s, wn * 64 + 32 * j, lane);
+            for (int j = 0; j < 4; ++j) nf[j] = read_ks<kPitchN>(bs + ks_n, 16 * s, 32 * j);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 if constexpr (A_KS) {
-                    mop[i] = read_ks(as, kPitchM, 16 * s, wm * 128 + 32 * i, lane);
+                    mf[i] = read_ks<kPitchM>(as + ks_m, 16 * s, 32 * i);
                 } else {
                     const int row = wm * 128 + 32 * i + frow;
-                    mop[i] = *reinterpret_cast<const v8bf*>(as + row * kPitchKC + (((2 * s + khalf) ^ swz(row)) << 4));
+                    mf[i] = *reinterpret_cast<const v8bf*>(as + row * kPitchKC + (((2 * s + khalf) ^ swz(row)) << 4));
                 }
             }
+        };
+        read_frags(0, nop[0], mop[0]);
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
+        for (int s = 0; s < TK / 16; ++s) {
+            if (s + 1 < TK / 16) read_frags(s + 1, nop[(s + 1) & 1], mop[(s + 1) & 1]);
+            __builtin_amdgcn_sched_barrier(0);        // the next fragments are requested before this k-step's MFMAs
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(nop[j], mop[i], acc[j][i], 0, 0, 0);
-            // one k-step's operands in registers at a time: the staged global loads of two K-tiles are live across this loop
+                    acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(nop[s & 1][j], mop[s & 1][i], acc[j][i], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -219,36 +243,37 @@ void k_gemm_bf16(const BfArgs p) {
     // Tile ks is multiplied from LDS stage ks % 2 while tile ks + 1 waits in (or lands into) one register set and
     // tile ks + 2 is requested into the other.  The loop body covers two K-tiles and has no exits: a tile past the
     // end of the k range is fetched as zeros (it lies beyond the descriptors) and adds nothing.
-    uint4 ra0[8], rb0[4], ra1[8], rb1[4];
+    uint4 ra0[NA], rb0[NB], ra1[NA], rb1[NB];
     fetch(0, ra0, rb0);
     fetch(1, ra1, rb1);
     stash(0, ra0, rb0);
     __syncthreads();
     for (int ks = 0; ks < nk; ks += 2) {
         fetch(ks + 2, ra0, rb0);
-        compute(0);
+        compute(std::integral_constant<int, 0>{});
         stash(1, ra1, rb1);
         __syncthreads();
         fetch(ks + 3, ra1, rb1);
-        compute(1);
+        compute(std::integral_constant<int, 1>{});
         stash(0, ra0, rb0);
         __syncthreads();
     }
 
     // ---- epilogue: accumulator register r of tile (j, i) is output row m0 + wm*128 + 32 i + lane % 32,
-    //      column n0 + wn*64 + 32 j + 8 (r / 4) + 4 (lane / 32) + r % 4 ----
+    //      column n0 + wn*128 + 32 j + 8 (r / 4) + 4 (lane / 32) + r % 4 ----
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int m = m0 + wm * 128 + 32 * i + frow;
         if (m >= m_end) continue;
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < 4; ++j)
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const int n = n0 + wn * 64 + 32 * j + 8 * q + 4 * khalf;
+                const int n = n0 + wn * 128 + 32 * j + 8 * q + 4 * khalf;
                 if (n >= p.N) continue;                      // N % 8 == 0: a quad is inside or outside as a whole
                 const size_t at = c_base + static_cast<size_t>(m) * p.ldc + n;
-                float v[4] = {acc[j][i][4 * q], acc[j][i][4 * q + 1], acc[j][i][4 * q + 2], acc[j][i][4 * q + 3]};
+                float v[4] = {acc_read(acc[j][i][4 * q]), acc_read(acc[j][i][4 * q + 1]), acc_read(acc[j][i][4 * q + 2]),
+                              acc_read(acc[j][i][4 * q + 3])};
                 if constexpr (OUT == OUT_ACCUM_F32) {
                     float4* dst = reinterpret_cast<float4*>(static_cast<float*>(p.C) + at);
                     float4 c = *dst;
@@ -263,6 +288,9 @@ void k_gemm_bf16(const BfArgs p) {
                     }
                     *dst = make_uint2(pack_bf16x2_hw(v[0], v[1]), pack_bf16x2_hw(v[2], v[3]));
                 }
+                // one quad's loads and stores at a time: pulling the whole tile's reads of C to the front would need
+                // more registers than the main loop leaves
+                if constexpr (OUT != OUT_STORE_BF16) __builtin_amdgcn_sched_barrier(0);
             }
     }
 }

@@ -93,7 +93,18 @@ class PowerSampler:
         self._stop = True
         self._t.join()
 
-    def report(self):
+    def cap_watts(self):
+        try:
+            return int(open(self.power.replace("power1_input", "power1_cap")).read()) / 1e6 if self.power else None
+        except (OSError, ValueError):
+            return None
+
+    def report(self, skip_fraction=0.0):
+        """Averages over the samples after the first `skip_fraction` of them (the power reading is a moving average
+        that lags the load by a few hundred milliseconds)."""
+        k = int(len(self.watts) * skip_fraction)
+        self.watts = self.watts[k:]
+        self.mhz = self.mhz[int(len(self.mhz) * skip_fraction):]
         out = {}
         if self.watts:
             out["socket_power_w_avg"] = round(sum(self.watts) / len(self.watts), 1)
@@ -290,6 +301,23 @@ def main():
             ts.append(a.elapsed_time(b) / launches)
         return sorted(ts)[len(ts) // 2]
 
+    # The power reading behind "power-limited": the same step, eager, for 1.5 s (the hwmon figure is a moving average;
+    # the 50 timed steps are over before it has risen), averaged over the second half of the samples.
+    sustained = None
+    with PowerSampler(period_s=0.01) as long_sampler:
+        s0 = time.perf_counter()
+        n_sus = 0
+        while time.perf_counter() - s0 < 1.5:
+            for _ in range(25):
+                step(0)
+            torch.cuda.synchronize()
+            n_sus += 25
+        s1 = time.perf_counter()
+    sustained = long_sampler.report(skip_fraction=0.5)
+    sustained.update({"seconds": round(s1 - s0, 2), "steps": n_sus, "ms_per_step": round((s1 - s0) * 1e3 / n_sus, 4),
+                      "socket_power_cap_w": long_sampler.cap_watts(),
+                      "note": "the same eager step for 1.5 s; power and clock averaged over the second half of the samples"})
+
     # The same four launches recorded once into a HIP graph and replayed: what the step costs without the per-launch
     # host work and without the event brackets.  Captured on a side stream (the library launches on the stream it is
     # given), replayed `steps` times between two synchronisations.
@@ -407,6 +435,7 @@ def main():
                          "tflops": None if graph_ms is None else round(total_flop / (graph_ms * 1e-3) / 1e12, 2),
                          "note": graph_note},
         "timed_region_power": sampler.report(),
+        "sustained_power": sustained,
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()

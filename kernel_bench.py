@@ -153,7 +153,13 @@ def main():
     gate = bf16(M, N); up = bf16(M, N); out = torch.empty_like(gate)
     hbm("swiglu_forward (stand-alone)", f"{M}x{N}", 6.0 * gate.numel(),
         lambda: cf.cf_swiglu_forward(gate, up, out, gate.numel(), st))
-    del gate, up, out, h, hq, hq2, w, wt, w8
+    dout = bf16(M, N, sigma=0.01); dgate = torch.empty_like(gate); dup = torch.empty_like(gate)
+    hbm("swiglu_backward (stand-alone)", f"{M}x{N}", 10.0 * gate.numel(),
+        lambda: cf.cf_swiglu_backward(dout, gate, up, dgate, dup, gate.numel(), st))
+    acc32 = torch.zeros(N, device=dev)
+    hbm("col_sum_strided_bf16 (bias gradient, sequential rows)", f"{M}x{N}", 2.0 * gate.numel(),
+        lambda: cf.cf_col_sum_strided_bf16(gate, acc32, M, N, N, 0, st))
+    del gate, up, out, h, hq, hq2, w, wt, w8, dout, dgate, dup
 
     # ---- config 3: block-scaled ---------------------------------------------------------------------
     M3, N3, K3 = 4096, 7168, 7168

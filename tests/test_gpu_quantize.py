@@ -320,7 +320,7 @@ def test_clip_probes_and_calibration_minmax(cf, dev):
 def test_swiglu_and_bias_add(cf, dev):
     case("swiglu / bias")
     rng = np.random.default_rng(13)
-    for n, off in ((0, 0), (5, 0), (4096, 0), (100003, 0), (100003, 1)):
+    for n, off in ((0, 0), (5, 0), (4096, 0), (100003, 0), (100003, 1), (300007, 0)):     # the last one: table path + tail
         gb = orc.bf16_from_f32(rng.standard_normal(n + off).astype(np.float32) * 4)
         ub = orc.bf16_from_f32(rng.standard_normal(n + off).astype(np.float32))
         if n > 10:
@@ -360,7 +360,7 @@ def test_swiglu_backward(cf, dev):
     """swiglu_backward against the oracle, bit for bit: ragged and unaligned lengths, then every bf16 gate pattern."""
     case("swiglu backward")
     rng = np.random.default_rng(14)
-    for n, off in ((0, 0), (5, 0), (4096, 0), (100003, 0), (100003, 1)):
+    for n, off in ((0, 0), (5, 0), (4096, 0), (100003, 0), (100003, 1), (300007, 0)):     # the last one: table path + tail
         gb = orc.bf16_from_f32(rng.standard_normal(n + off).astype(np.float32) * 4)
         ub = orc.bf16_from_f32(rng.standard_normal(n + off).astype(np.float32))
         db = orc.bf16_from_f32(rng.standard_normal(n + off).astype(np.float32) * 1e-2)

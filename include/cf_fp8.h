@@ -409,6 +409,41 @@ int cf_moe_grouped_gemm_bf16_tn_accum_bf16(int M, int N, int total_rows, int num
                                            const int* d_offsets, const uint16_t* d_A, int lda,
                                            const uint16_t* d_B, int ldb, uint16_t* d_C, cf_stream_t stream);
 
+/* The selected-expert backward of the GELU expert bank (src/trainer.cu:7669-7741: per expert and behind the
+ * host copy of the counts, the FP8 recompute of the forward, moe_row_dot_selected_bf16,
+ * moe_gather_scale_rows_bf16, two gemm_bf16_tn_f32, two gemm_bf16, gelu_backward, moe_gather_rows_bf16 and
+ * moe_scatter_add_rows_bf16) for every expert in one call with no host round trip, over the forward's saved
+ * counts / offsets / row_indices.  Inputs: d_grad_mixed [rows,H] bf16; the FP8 hidden states [rows,H] with
+ * their per-tensor descale and the bf16 hidden states [rows,H] (moe_hidden_gated); the dense route weights
+ * [rows,E]; the expert weights as FP8 [E,Ie,H] / [E,H,Ie] with per-tensor descales (recompute) and as bf16
+ * (gradients).  Outputs: d_grad_route_weights [rows,E] fp32 (cleared, then one entry per selected pair),
+ * d_grad_fc_in [E,Ie,H] and d_grad_fc_out [E,H,Ie] bf16 (accumulated into), d_grad_hidden [rows,H] bf16
+ * (accumulated into, experts in ascending order).  As in cf_moe_grouped_gelu_forward_fp8 the recomputed
+ * activation is quantized with one scale per token row (the loop's per-expert delayed scale is host-side slot
+ * state).  H and Ie multiples of 128 and at least 256; total_selected_rows the sum of the counts; d_workspace
+ * 256-byte aligned.  cf_moe_grouped_gelu_backward_workspace gives the workspace size and, when `offsets` is
+ * not null, the byte offsets of the intermediates inside it (CF_MOE_BWD_WS_* order), which stay valid after
+ * the call: pre / post / postq / d_out / d_post / d_pre / x / d_x, experts back to back. */
+enum {
+    CF_MOE_BWD_WS_TILE_MAP = 0, CF_MOE_BWD_WS_INDEX, CF_MOE_BWD_WS_HIDDEN_DESCALE, CF_MOE_BWD_WS_IN_DESCALE,
+    CF_MOE_BWD_WS_OUT_DESCALE, CF_MOE_BWD_WS_PRE, CF_MOE_BWD_WS_POST, CF_MOE_BWD_WS_POSTQ, CF_MOE_BWD_WS_POST_SCALE,
+    CF_MOE_BWD_WS_POST_DESCALE, CF_MOE_BWD_WS_D_OUT, CF_MOE_BWD_WS_D_POST, CF_MOE_BWD_WS_D_PRE, CF_MOE_BWD_WS_X,
+    CF_MOE_BWD_WS_D_X, CF_MOE_BWD_WS_COUNT
+};
+int cf_moe_grouped_gelu_backward_workspace(int rows, int total_selected_rows, int num_experts, int H, int Ie,
+                                           size_t* offsets, size_t* bytes);
+int cf_moe_grouped_gelu_backward_fp8(const uint16_t* d_grad_mixed, const void* d_hidden_fp8,
+                                     const float* d_fcin_descale, int fcin_is_e5m2,
+                                     const uint16_t* d_hidden_bf16, const float* d_route_weights,
+                                     const int* d_counts, const int* d_offsets, const int* d_row_indices,
+                                     const void* d_fc_in_w8, const float* d_fc_in_descale,
+                                     const void* d_fc_out_w8, const float* d_fc_out_descale,
+                                     const uint16_t* d_fc_in_w, const uint16_t* d_fc_out_w,
+                                     float* d_grad_route_weights, uint16_t* d_grad_fc_in,
+                                     uint16_t* d_grad_fc_out, uint16_t* d_grad_hidden, int rows, int H, int Ie,
+                                     int num_experts, int total_selected_rows, void* d_workspace,
+                                     size_t workspace_bytes, cf_stream_t stream);
+
 /* Row lists of all experts back to back: compact[offsets[e] + s] = row_indices[e, s]
  * (the gather order of moe_gather_rows_u8 over all experts, kernels/moe.cu:594-606). */
 int cf_moe_compact_row_index(const int* d_counts, const int* d_offsets, const int* d_row_indices,

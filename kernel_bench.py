@@ -342,6 +342,20 @@ def main():
     mfma16("grouped bf16 wgrad: g_in += d_pre^T . x (tn, bf16 C)", f"{Ie}x{H}x~{total // E} x{E}", fl,
            lambda: cf.cf_moe_grouped_gemm_bf16_tn_accum_bf16(Ie, H, total, E, counts, offs, gpost, Ie, xg, H, g_in, st))
 
+    # the whole selected-expert backward of the GELU bank in one call: FP8 recompute, route gradient, four bf16 GEMMs,
+    # gelu_backward, scatter-add (16 launches per expert in the reference's host loop)
+    szb = ctypes.c_size_t(0)
+    cf.raw_cf_moe_grouped_gelu_backward_workspace(T, total, E, H, Ie, None, ctypes.byref(szb))
+    wsb = u8(szb.value + 256)
+    wsb_ptr = wsb.data_ptr() + (-wsb.data_ptr()) % 256
+    hid16 = bf16(T, H); d_rw = torch.empty((T, E), dtype=torch.float32, device=dev)
+    if args.only in "grouped GELU expert bank backward, whole pipeline":
+        t = timed(lambda: cf.cf_moe_grouped_gelu_backward_fp8(dmixed, hq, one, 0, hid16, rw, counts, offs, idx, wg, one, wd, one, wi16, wo16,
+                                                                d_rw, g_in, g_out, dhid, T, H, Ie, E, total, wsb_ptr, szb.value, st))
+        fl8, fl16 = 4.0 * total * Ie * H, 8.0 * total * Ie * H
+        print(f"{'grouped GELU expert bank backward, whole pipeline':<64} {f'T={T} E={E} k={k}':<26} {t * 1e6:9.1f} "
+              f"{(fl8 + fl16) / t / 1e12:7.0f} TFLOP/s (FP8 recompute {fl8 / 1e12:.2f} + bf16 {fl16 / 1e12:.2f} TFLOP)", flush=True)
+
 
 if __name__ == "__main__":
     main()

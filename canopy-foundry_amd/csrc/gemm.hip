@@ -1712,10 +1712,13 @@ int static_scratch(void** out) {
 }
 }  // namespace
 
+// Also the set-up call: it looks up the array's address on the current device, so that a later call of the entry point
+// (under graph capture, say) finds it ready and makes no runtime query of its own.
 int cf_fp8_grouped_gemm_static_max_bytes(size_t* bytes) {
     if (!bytes) return CF_ERR_INVALID_ARG;
     *bytes = kStaticMapBytes;
-    return CF_OK;
+    void* ptr = nullptr;
+    return static_scratch(&ptr);
 }
 
 int cf_fp8_grouped_gemm_nt_bf16_static(int total_rows, int N, int K, int num_experts, const int* d_counts,

@@ -360,7 +360,10 @@ int cf_fp8_grouped_gemm_nt_bf16_ex(int total_rows, int N, int K, int num_experts
  * cf_fp8_grouped_gemm_static_max_bytes() bytes (cf_fp8_grouped_gemm_workspace_bytes tells: more than
  * 3276 row tiles, total_rows / 256 + num_experts) returns CF_ERR_UNSUPPORTED and launches nothing.  Every
  * call on a GPU shares that GPU's array: calls that may overlap in time on one GPU (different streams,
- * different host threads) race on it and must be serialised by the caller; calls on one stream are ordered. */
+ * different host threads) race on it and must be serialised by the caller; calls on one stream are ordered.
+ * cf_fp8_grouped_gemm_static_max_bytes is also the set-up call: it looks up the array's address on the
+ * current device, so a caller that will record the entry point into a graph calls it once per device first
+ * (without it the first call of the entry point on a device does the lookup). */
 int cf_fp8_grouped_gemm_static_max_bytes(size_t* bytes);
 int cf_fp8_grouped_gemm_nt_bf16_static(int total_rows, int N, int K, int num_experts,
                                        const int* d_counts, const int* d_offsets, const void* d_A,

@@ -48,6 +48,19 @@
  *                                 with the reference's summation tree, closed
  *                                 forms; libm erff / expf stand in for CUDA's in
  *                                 the GELU pair: parity unpinned beyond 1 bf16 ulp).
+ *   swiglu backward               grad_up must equal the forward applied to
+ *                                 (gate, grad_out) bit for bit (one commutative
+ *                                 product); grad_gate against the closed form in
+ *                                 double and a central difference; orc_expf
+ *                                 stands in for CUDA's expf, as in the forward:
+ *                                 parity unpinned beyond 1 bf16 ulp.
+ *   column sum (bias gradient)    exactly summable integers against numpy; a
+ *                                 column (2^24, then ones) whose sequential sum
+ *                                 differs from every tree.
+ *   bf16 GEMMs of the MoE backward (tests/oracle_lib.py: gemm_bf16_*_ref) double
+ *                                 matmul of the same bf16 operands; exact-integer
+ *                                 cases bit for bit.  cuBLAS's accumulation order:
+ *                                 parity unpinned.
  *   GEMM references               definition from the task statement: matmul
  *                                 of the dequantised operands; special cases
  *                                 reduce to numpy matmul.  cuBLASLt's own

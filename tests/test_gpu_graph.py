@@ -153,3 +153,70 @@ def test_moe_layer_replays_from_a_graph(cf, dev):
         assert torch.equal(out_swiglu.view(torch.int16), want[0].view(torch.int16)), f"replay {i}"
         assert torch.equal(out_gelu.view(torch.int16), want[1].view(torch.int16)), f"replay {i}"
         assert float(scratch) == float(scratch)
+
+
+def test_moe_backward_and_static_grouped_gemm_replay_from_a_graph(cf, dev):
+    """The one-call selected-expert backward (its route-weight gradient is cleared by a kernel, not a memset node) and
+    the grouped GEMM whose tile table lives in the library's own device array (set up before the capture) in one
+    captured graph; replays on new gradients must reproduce the eager run bit for bit."""
+    import ctypes
+    import numpy as np
+    import oracle_lib as orc
+    from gpu_util import dev_arr
+    case("graph capture: GELU bank backward + static grouped GEMM")
+    T, E, k, H, Ie = 512, 4, 2, 256, 256
+    g = torch.Generator(device=dev); g.manual_seed(31)
+    rng = np.random.default_rng(31)
+    rw_h = orc.moe_topk_route(rng.standard_normal((T, E)).astype(np.float32), k)
+    counts_h, idx_h = orc.moe_build_expert_row_lists(rw_h)
+    offs_h = orc.moe_expert_offsets(counts_h)
+    total = int(counts_h.sum())
+    rw, counts, offs, idx = dev_arr(rw_h, dev), dev_arr(counts_h, dev), dev_arr(offs_h, dev), dev_arr(idx_h, dev)
+    w_in8, w_in_d = fp8_weights(E * Ie, H, dev, g); w_out8, w_out_d = fp8_weights(E * H, Ie, dev, g)
+    one = torch.full((1,), 0.02, device=dev)
+    w_in = (torch.randn(E * Ie, H, device=dev, generator=g) * 0.05).to(torch.bfloat16)
+    w_out = (torch.randn(E * H, Ie, device=dev, generator=g) * 0.05).to(torch.bfloat16)
+    hidden = torch.randn(T, H, device=dev, generator=g).to(torch.bfloat16)
+    hq = (hidden.float() * (448.0 / hidden.float().abs().max())).to(torch.float8_e4m3fn).view(torch.uint8)
+    hd = (hidden.float().abs().max() / 448.0).reshape(1)
+    hrow_d = hd.expand(T).contiguous()
+    d_mixed = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+    d_rw = torch.empty((T, E), device=dev)
+    g_in = torch.zeros((E * Ie, H), dtype=torch.bfloat16, device=dev); g_out = torch.zeros((E * H, Ie), dtype=torch.bfloat16, device=dev)
+    d_hidden = torch.zeros((T, H), dtype=torch.bfloat16, device=dev)
+    cidx = torch.empty(total, dtype=torch.int32, device=dev)
+    static_out = torch.empty((total, Ie), dtype=torch.bfloat16, device=dev)
+    size = ctypes.c_size_t(0)
+    assert cf.raw_cf_moe_grouped_gelu_backward_workspace(T, total, E, H, Ie, None, ctypes.byref(size)) == 0
+    ws = torch.empty(size.value + 256, dtype=torch.uint8, device=dev); wp = ws.data_ptr() + (-ws.data_ptr()) % 256
+    mx = ctypes.c_size_t(0)
+    assert cf.raw_cf_fp8_grouped_gemm_static_max_bytes(ctypes.byref(mx)) == 0          # set-up: before any capture
+
+    def step():
+        s = stream()
+        g_in.zero_(); g_out.zero_(); d_hidden.zero_()
+        cf.cf_moe_grouped_gelu_backward_fp8(d_mixed, hq, hd, 0, hidden, rw, counts, offs, idx, w_in8, one, w_out8, one, w_in, w_out,
+                                            d_rw, g_in, g_out, d_hidden, T, H, Ie, E, total, wp, size.value, s)
+        cf.cf_moe_compact_row_index(counts, offs, idx, T, E, cidx, s)
+        cf.cf_fp8_grouped_gemm_nt_bf16_static(total, Ie, H, E, counts, offs, hq, T, H, cidx, hrow_d, w_in8, w_in_d, 1, 0, None, None,
+                                              static_out, Ie, s)
+
+    d_mixed.copy_((torch.randn(T, H, device=dev, generator=g) * 1e-2).to(torch.bfloat16)); step(); torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for i in range(3):
+        d_mixed.copy_((torch.randn(T, H, device=dev, generator=g) * 1e-2 * (1 + i)).to(torch.bfloat16))
+        step()
+        torch.cuda.synchronize()
+        want = [t.clone() for t in (d_rw, g_in, g_out, d_hidden, static_out)]
+        for t in (d_rw, g_in, g_out, d_hidden, static_out):
+            t.fill_(3.0)
+        scratch = torch.randn(1 << 20, device=dev).sum()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, a, b in zip(("d_rw", "g_in", "g_out", "d_hidden", "static_out"), (d_rw, g_in, g_out, d_hidden, static_out), want):
+            assert torch.equal(a.view(torch.int32 if a.dtype == torch.float32 else torch.int16),
+                               b.view(torch.int32 if b.dtype == torch.float32 else torch.int16)), f"replay {i}: {name}"
+        assert float(scratch) == float(scratch)

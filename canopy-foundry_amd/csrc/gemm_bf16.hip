@@ -57,6 +57,14 @@ struct BfArgs {
     long long c_expert_stride;      // TN: elements between the experts' C matrices
 };
 
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
 // An accumulator element as a vector-ALU operand.  The explicit read keeps the register allocator from moving whole
 // accumulator tiles into ordinary registers around the epilogue.
 __device__ __forceinline__ float acc_read(float a) {
@@ -165,34 +173,35 @@ void k_gemm_bf16(const BfArgs p) {
     const uint32_t a_lane_ks = m0 + (tid & 31) * 8 < p.M ? (tid >> 5) * static_cast<uint32_t>(p.lda) * 2u + (tid & 31) * 16u : kOutside;
     // [m][k] operand: this lane's row within a group of 32 rows and its 16-byte k chunk
     const uint32_t a_lane_kc = (tid >> 3) * static_cast<uint32_t>(p.lda) * 2u + (tid & 7) * 16u;
-    auto fetch = [&](int ks, uint4 (&ra)[NA], uint4 (&rb)[NB]) {
+    // chunk c (0 .. NA-1: M side, NA .. NA+NB-1: N side) of K-tile ks into its staging register
+    auto load_one = [&](int ks, auto cc, uint4 (&ra)[NA], uint4 (&rb)[NB]) {
+        constexpr int c = decltype(cc)::value;
         const int k0 = k_begin + ks * TK;
-        if constexpr (A_KS) {
-#pragma unroll
-            for (int i = 0; i < NA; ++i) ra[i] = load_rows(p.A, p.lda, k0 + 8 * i, k_end, m0, a_lane_ks);
-        } else {
-            const uint32_t off = k0 + (tid & 7) * 8 < k_end ? a_lane_kc : kOutside;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) ra[i] = load_rows(p.A, p.lda, m0 + 32 * i, m_end, k0, off);
-        }
-#pragma unroll
-        for (int i = 0; i < NB; ++i) rb[i] = load_rows(B, p.ldb, k0 + 8 * i, k_end, n0, b_lane);
-    };
-    auto stash = [&](int stage, const uint4 (&ra)[NA], const uint4 (&rb)[NB]) {
-        uint8_t* as = smem + stage * kStage;
-        uint8_t* bs = as + kATile;
-        if constexpr (A_KS) {
-#pragma unroll
-            for (int i = 0; i < NA; ++i) *reinterpret_cast<uint4*>(as + ((tid >> 5) + 8 * i) * kPitchM + (tid & 31) * 16) = ra[i];
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const int r = (tid >> 3) + 32 * i;
-                *reinterpret_cast<uint4*>(as + r * kPitchKC + (((tid & 7) ^ swz(r)) << 4)) = ra[i];
+        if constexpr (c < NA) {
+            if constexpr (A_KS) {
+                ra[c] = load_rows(p.A, p.lda, k0 + 8 * c, k_end, m0, a_lane_ks);
+            } else {
+                const uint32_t off = k0 + (tid & 7) * 8 < k_end ? a_lane_kc : kOutside;
+                ra[c] = load_rows(p.A, p.lda, m0 + 32 * c, m_end, k0, off);
             }
+        } else {
+            rb[c - NA] = load_rows(B, p.ldb, k0 + 8 * (c - NA), k_end, n0, b_lane);
         }
-#pragma unroll
-        for (int i = 0; i < NB; ++i) *reinterpret_cast<uint4*>(bs + ((tid >> 5) + 8 * i) * kPitchN + (tid & 31) * 16) = rb[i];
+    };
+    // the same chunk from its staging register into LDS stage `stage`
+    auto park_one = [&](int stage, auto cc, const uint4 (&ra)[NA], const uint4 (&rb)[NB]) {
+        constexpr int c = decltype(cc)::value;
+        uint8_t* as = smem + stage * kStage;
+        if constexpr (c < NA) {
+            if constexpr (A_KS) {
+                *reinterpret_cast<uint4*>(as + ((tid >> 5) + 8 * c) * kPitchM + (tid & 31) * 16) = ra[c];
+            } else {
+                const int r = (tid >> 3) + 32 * c;
+                *reinterpret_cast<uint4*>(as + r * kPitchKC + (((tid & 7) ^ swz(r)) << 4)) = ra[c];
+            }
+        } else {
+            *reinterpret_cast<uint4*>(as + kATile + ((tid >> 5) + 8 * (c - NA)) * kPitchN + (tid & 31) * 16) = rb[c - NA];
+        }
     };
 
     // ---- LDS -> MFMA ----
@@ -206,57 +215,56 @@ void k_gemm_bf16(const BfArgs p) {
 
     const int frow = lane & 31, khalf = lane >> 5;
     const int ks_n = ks_lane_offset(kPitchN, lane) + wn * 128 * 2, ks_m = ks_lane_offset(kPitchM, lane) + wm * 128 * 2;
-    // The fragments of k-step s + 1 are read while the MFMAs of k-step s run (one wavefront per SIMD: nobody else
-    // would fill the matrix cores during an LDS round trip), two fragment sets in turn.
-    auto compute = [&](auto stage_c) {
-        constexpr int stage = decltype(stage_c)::value;
+    // operand fragments, two sets: k-step s of any K-tile lives in set s % 2
+    v8bf nop[2][4], mop[2][4];
+    // fragment u (0..3: N side, 4..7: M side) of k-step s of the K-tile in LDS stage `stage`
+    auto read_unit = [&](int stage, auto sc, auto uc) {
+        constexpr int ks16 = decltype(sc)::value, u = decltype(uc)::value;
         const uint8_t* as = smem + stage * kStage;
-        const uint8_t* bs = as + kATile;
-        v8bf nop[2][4], mop[2][4];
-        auto read_frags = [&](int s, v8bf (&nf)[4], v8bf (&mf)[4]) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) nf[j] = read_ks<kPitchN>(bs + ks_n, 16 * s, 32 * j);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                if constexpr (A_KS) {
-                    mf[i] = read_ks<kPitchM>(as + ks_m, 16 * s, 32 * i);
-                } else {
-                    const int row = wm * 128 + 32 * i + frow;
-                    mf[i] = *reinterpret_cast<const v8bf*>(as + row * kPitchKC + (((2 * s + khalf) ^ swz(row)) << 4));
-                }
-            }
-        };
-        read_frags(0, nop[0], mop[0]);
-#pragma unroll
-        for (int s = 0; s < TK / 16; ++s) {
-            if (s + 1 < TK / 16) read_frags(s + 1, nop[(s + 1) & 1], mop[(s + 1) & 1]);
-            __builtin_amdgcn_sched_barrier(0);        // the next fragments are requested before this k-step's MFMAs
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(nop[s & 1][j], mop[s & 1][i], acc[j][i], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
+        if constexpr (u < 4) {
+            nop[ks16 & 1][u] = read_ks<kPitchN>(as + kATile + ks_n, 16 * ks16, 32 * u);
+        } else if constexpr (A_KS) {
+            mop[ks16 & 1][u - 4] = read_ks<kPitchM>(as + ks_m, 16 * ks16, 32 * (u - 4));
+        } else {
+            const int row = wm * 128 + 32 * (u - 4) + frow;
+            mop[ks16 & 1][u - 4] = *reinterpret_cast<const v8bf*>(as + row * kPitchKC + (((2 * ks16 + khalf) ^ swz(row)) << 4));
         }
     };
 
-    // Tile ks is multiplied from LDS stage ks % 2 while tile ks + 1 waits in (or lands into) one register set and
-    // tile ks + 2 is requested into the other.  The loop body covers two K-tiles and has no exits: a tile past the
-    // end of the k range is fetched as zeros (it lies beyond the descriptors) and adds nothing.
+    // One K-tile (64 MFMAs per wavefront) with everything else woven between them, one item per MFMA at most (one
+    // wavefront per SIMD: whatever waits, the matrix cores wait with it).  While tile ks is multiplied from `stage`:
+    //   - the fragments of k-step s + 1 are read during k-step s;
+    //   - the 16 loads of tile ks + 2 go out one every fourth MFMA, into the register set tile ks just left;
+    //   - tile ks + 1 (requested one tile ago) is parked in the other stage one chunk every third MFMA, done by MFMA 47;
+    //   - the barrier follows, and the first fragments of tile ks + 1 are read under the last 16 MFMAs.
+    // A tile past the end of the k range is fetched as zeros (it lies beyond the descriptors) and adds nothing, so the
+    // loop needs no tail.
+    auto ktile = [&](auto stage_c, int ks, uint4 (&ra_new)[NA], uint4 (&rb_new)[NB], const uint4 (&ra_next)[NA], const uint4 (&rb_next)[NB]) {
+        constexpr int stage = decltype(stage_c)::value;
+        static_for<0, 64>([&](auto mc) {
+            constexpr int m = decltype(mc)::value, ks16 = m / 16, q = m % 16;
+            acc[q >> 2][q & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(nop[ks16 & 1][q >> 2], mop[ks16 & 1][q & 3], acc[q >> 2][q & 3], 0, 0, 0);
+            if constexpr (q < 8) {
+                if constexpr (ks16 < 3) read_unit(stage, std::integral_constant<int, (ks16 + 1) % 4>{}, std::integral_constant<int, q % 8>{});
+                else                    read_unit(stage ^ 1, std::integral_constant<int, 0>{}, std::integral_constant<int, q % 8>{});
+            }
+            if constexpr (m % 4 == 1) load_one(ks + 2, std::integral_constant<int, m / 4>{}, ra_new, rb_new);
+            if constexpr (m < 48 && m % 3 == 2) park_one(stage ^ 1, std::integral_constant<int, (m / 3) % 16>{}, ra_next, rb_next);
+            if constexpr (m == 47) __syncthreads();
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+
+    static_assert(NA + NB == 16, "the weave above places 16 loads and 16 LDS stores per K-tile");
     uint4 ra0[NA], rb0[NB], ra1[NA], rb1[NB];
-    fetch(0, ra0, rb0);
-    fetch(1, ra1, rb1);
-    stash(0, ra0, rb0);
+    static_for<0, 16>([&](auto c) { load_one(0, c, ra0, rb0); });
+    static_for<0, 16>([&](auto c) { load_one(1, c, ra1, rb1); });
+    static_for<0, 16>([&](auto c) { park_one(0, c, ra0, rb0); });
     __syncthreads();
+    static_for<0, 8>([&](auto u) { read_unit(0, std::integral_constant<int, 0>{}, u); });
     for (int ks = 0; ks < nk; ks += 2) {
-        fetch(ks + 2, ra0, rb0);
-        compute(std::integral_constant<int, 0>{});
-        stash(1, ra1, rb1);
-        __syncthreads();
-        fetch(ks + 3, ra1, rb1);
-        compute(std::integral_constant<int, 1>{});
-        stash(0, ra0, rb0);
-        __syncthreads();
+        ktile(std::integral_constant<int, 0>{}, ks, ra0, rb0, ra1, rb1);
+        ktile(std::integral_constant<int, 1>{}, ks + 1, ra1, rb1, ra0, rb0);
     }
 
     // ---- epilogue: accumulator register r of tile (j, i) is output row m0 + wm*128 + 32 i + lane % 32,

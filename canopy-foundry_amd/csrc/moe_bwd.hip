@@ -188,10 +188,45 @@ __global__ __launch_bounds__(kLutThreads) void k_gelu_lut(const uint4* __restric
     }
 }
 
+// The backward for large tensors: the derivative in fp32 depends on the 16 bits of the pre-activation only; erff and
+// expf are what the plain kernel waits for.  A workgroup that stays on its CU builds the table of the derivative for
+// every bf16 pre-activation with 2^-25 <= |x| < 128 (4096 magnitudes x 2 signs, 32 KiB) with the same expression; the
+// few values outside (zeros, tiny, huge, non-finite) are evaluated directly.  Same bits either way.
+constexpr uint32_t kDerivLo = 0x3300u, kDerivSpan = 0x1000u;
+__global__ __launch_bounds__(kLutThreads) void k_gelu_bwd_lut(const uint4* __restrict__ x, const uint4* __restrict__ g,
+                                                              uint4* __restrict__ out, size_t nvec) {
+    __shared__ float lut[2 * kDerivSpan];
+    for (uint32_t i = threadIdx.x; i < 2 * kDerivSpan; i += kLutThreads)
+        lut[i] = gelu_deriv(bf16_to_f32(static_cast<uint16_t>((i >= kDerivSpan ? 0x8000u : 0u) | (kDerivLo + (i & (kDerivSpan - 1))))));
+    __syncthreads();
+    auto deriv = [&](uint32_t b16) {
+        const uint32_t slot = (b16 & 0x7fffu) - kDerivLo;
+        return slot < kDerivSpan ? lut[slot + (b16 >> 15) * kDerivSpan] : gelu_deriv(bf16_to_f32(static_cast<uint16_t>(b16)));
+    };
+    auto one = [&](uint32_t pre, uint32_t gr) { return pack_bf16x2(bf16_lo(gr) * deriv(pre & 0xffffu), bf16_hi(gr) * deriv(pre >> 16)); };
+    for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec; i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+        const uint4 v = x[i], u = g[i];
+        store_stream16(out + i, make_uint4(one(v.x, u.x), one(v.y, u.y), one(v.z, u.z), one(v.w, u.w)));
+    }
+}
+
 template <bool BWD>
 int launch_gelu(const uint16_t* x, const uint16_t* g, uint16_t* out, size_t n, hipStream_t st) {
     const bool vec = aligned16(x) && aligned16(out) && (!BWD || aligned16(g));
     const size_t nvec = vec ? n / 8 : 0;
+    if constexpr (BWD) {
+        if (nvec >= (1u << 17)) {        // 1 Mi elements: from here on 256 small tables pay for themselves
+            static int cus = [] {
+                int dev = 0, c = 0;
+                return (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&c, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && c > 0) ? c : 256;
+            }();
+            k_gelu_bwd_lut<<<cus, kLutThreads, 0, st>>>(reinterpret_cast<const uint4*>(x), reinterpret_cast<const uint4*>(g),
+                                                       reinterpret_cast<uint4*>(out), nvec);
+            if (nvec * 8 < n)
+                k_gelu_scalar<BWD><<<static_cast<unsigned>(min(ceil_div(n - nvec * 8, kThreads), 65536u)), kThreads, 0, st>>>(x, g, out, nvec * 8, n);
+            return launch_status();
+        }
+    }
     if constexpr (!BWD) {
         if (nvec >= (8u << 20)) {        // 64 Mi elements: enough to pay for one table per CU
             static std::once_flag once;

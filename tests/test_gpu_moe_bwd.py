@@ -281,3 +281,24 @@ def test_gelu_forward_table_form_matches_the_plain_kernel(cf, dev):
         cf.cf_gelu_forward_bf16(x[a:a + m], want[a:a + m], m, stream())
     torch.cuda.synchronize()
     assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+
+
+def test_gelu_backward_table_form_matches_the_plain_kernel(cf, dev):
+    """Tensors of 1 Mi elements and more take the form that looks the derivative up in a per-workgroup table; it must
+    give the bits of the plain kernel (run here on the same data in pieces below that size), every bf16 pre-activation
+    and an unaligned tail included."""
+    case("gelu backward, table form")
+    n = (2 << 20) + 8 * 100 + 5
+    g = torch.Generator(device=dev); g.manual_seed(6)
+    pre = (torch.randn(n, device=dev, generator=g) * 3.0).to(torch.bfloat16)
+    pre[:65536] = torch.arange(65536, device=dev, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    grad = (torch.randn(n, device=dev, generator=g) * 1e-2).to(torch.bfloat16)
+    out = torch.empty_like(pre)
+    cf.cf_gelu_backward_bf16(pre, grad, out, n, stream())
+    want = torch.empty_like(pre)
+    piece = 1 << 19
+    for a in range(0, n, piece):
+        m = min(piece, n - a)
+        cf.cf_gelu_backward_bf16(pre[a:a + m], grad[a:a + m], want[a:a + m], m, stream())
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16))

@@ -222,6 +222,15 @@ int grouped_gemm_nt_bf16(int total_rows, int N, int K, int num_experts, const in
                          const float* b_up_descale, uint16_t* C, int ldc, void* d_workspace, size_t workspace_bytes,
                          bool build_map, int a_is_e5m2, cf_stream_t stream);
 
+// Two forms that exist on the ring kernel only and take a tile table already built (gemm.hip): fp32 store with
+// per-tensor descales and a row gather; the term-split form (activation rows = several E4M3 terms side by side,
+// term t weighted 2^(-4 t) inside the matrix cores).
+int grouped_gemm_nt_store_f32(int total_rows, int N, int K, int num_experts, const void* A, int a_rows, int lda,
+                              const int* d_a_row_index, const float* a_descale, const void* B, const float* b_descale,
+                              float* C, int ldc, const int* d_tile_map, int a_is_e5m2, cf_stream_t stream);
+int grouped_gemm_nt_bf16_terms(int total_rows, int N, int Kb, int terms, int num_experts, const void* A, int lda,
+                               const float* a_descale, const void* B, const float* b_descale, uint16_t* C, int ldc,
+                               const int* d_tile_map, cf_stream_t stream);
 // The tile table of a grouped GEMM (k_build_tile_map in gemm.hip): tile_map[0] = number of row tiles of 256 rows,
 // then per row tile (expert, its first row, its end row, its first row tile, its row-tile count), experts back to back.
 void build_tile_map(const int* d_counts, const int* d_offsets, int num_experts, int max_row_tiles, int* tile_map,

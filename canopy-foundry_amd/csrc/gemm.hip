@@ -38,8 +38,8 @@ constexpr int kStageBytes = 2 * kTileBytes;       // X tile + W tile
 constexpr int kLdsBytes = 2 * kStageBytes;        // double buffered: 128 KiB
 constexpr int kXcds = 8;
 
-enum { EPI_NONE = 0, EPI_BIAS = 1, EPI_SILU_GATE = 2, EPI_ACCUM_F32 = 3, EPI_ACCUM_BF16 = 4 };
-enum { SCALE_TENSOR = 0, SCALE_ROWCOL = 1, SCALE_BLOCK = 2 };
+enum { EPI_NONE = 0, EPI_BIAS = 1, EPI_SILU_GATE = 2, EPI_ACCUM_F32 = 3, EPI_ACCUM_BF16 = 4, EPI_STORE_F32 = 5 };
+enum { SCALE_TENSOR = 0, SCALE_ROWCOL = 1, SCALE_BLOCK = 2, SCALE_ROW = 3 };   // SCALE_ROW: sa per row, sb one scalar (ring kernel)
 
 struct GemmArgs {
     int M, N, K;                 // N = output columns
@@ -60,6 +60,10 @@ struct GemmArgs {
     int a_rows;                  // rows of the A buffer (= M without a row index)
     long long b_expert_stride;   // bytes between the weight matrices of consecutive experts
     int sb_expert_stride;        // elements between the channel descales of consecutive experts
+    // term-split form (ring kernel, MX instantiation only): A's K axis is `K / b_k_period` terms laid side by side,
+    // term t = the residual of the terms before it scaled by 16^t; every term multiplies the same b_k_period
+    // columns of B, and the matrix cores scale its products by 2^(-4 t)
+    int b_k_period;
 };
 
 // where a workgroup's tile lives: rows [m0, m_end) of the output, columns from n0, weights of `expert`
@@ -538,7 +542,7 @@ struct TileScales {
 
 template <int EPI, int SCALE>
 __device__ __forceinline__ void load_row_scales(TileScales<EPI>& s, const GemmArgs& p, const TilePos& t, int wm, int lane) {
-    if constexpr (SCALE == SCALE_ROWCOL) {
+    if constexpr (SCALE == SCALE_ROWCOL || SCALE == SCALE_ROW) {
         // Two complete paths: these loads are issued among the copies of the tile's last K-tile, and a wait between
         // a row-index load and the scale load that depends on it also waits for every copy in flight.  Without a
         // row index nothing waits; with one, the four index loads share a single wait.
@@ -650,7 +654,7 @@ __device__ __forceinline__ void drain_tile(v16f (&acc)[4][4], TileScales<EPI>& s
 #pragma unroll
             for (int bb = 0; bb < 2; ++bb) {
                 const int b = half * 2 + bb;
-                const float sa = SCALE == SCALE_ROWCOL ? s.sa[b] : 1.0f;
+                const float sa = (SCALE == SCALE_ROWCOL || SCALE == SCALE_ROW) ? s.sa[b] : 1.0f;
 #pragma unroll
                 for (int uu = 0; uu < 2; ++uu) {
                     const int unit = pair * 2 + uu;
@@ -718,7 +722,9 @@ __device__ __forceinline__ void drain_tile(v16f (&acc)[4][4], TileScales<EPI>& s
 // xor-swizzled by row), read back 16 bytes per lane, sixteen lanes per row, added to what C holds (fetched while
 // the block is being scaled) and stored: whole lines in both directions (128 bytes of fp32, 64 of bf16 per
 // sixteen lanes), non-temporal both ways.
-template <bool RAGGED, bool OUT_BF16, class Landed>
+// STORE: C = product (nothing is fetched).  RAGGED also covers a last column tile that N cuts short (N % 4 == 0: a
+// lane's four columns are in or out as a whole).
+template <bool RAGGED, bool OUT_BF16, bool STORE, class Landed>
 __device__ __forceinline__ void drain_tile_accum(v16f (&acc)[4][4], float s1, const GemmArgs& p, const TilePos& t,
                                                  int wm, int wn, int lane, uint8_t* stage, Landed&& landed) {
     const int row = lane & 31, khalf = lane >> 5;
@@ -726,6 +732,7 @@ __device__ __forceinline__ void drain_tile_accum(v16f (&acc)[4][4], float s1, co
     const int wswz = row & 15;
     const int rr = lane >> 4, rc = lane & 15;
     const int mrow0 = t.m0 + wm * 128 + rr;
+    const int ncol0 = t.n0 + wn * 128 + rc * 4;                 // + 64 per pair
     constexpr uint32_t ES = OUT_BF16 ? 2u : 4u;                 // bytes per element of C
     const size_t c_first = static_cast<size_t>(t.m0 + wm * 128) * p.ldc + t.n0 + wn * 128;
     uint8_t* cu = OUT_BF16 ? reinterpret_cast<uint8_t*>(p.C + c_first) : reinterpret_cast<uint8_t*>(p.Cf + c_first);
@@ -746,11 +753,11 @@ __device__ __forceinline__ void drain_tile_accum(v16f (&acc)[4][4], float s1, co
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             old[k % DEPTH][i] = Raw{};
-            if (!RAGGED || mrow0 + b * 32 + i * 4 < t.m_end)
+            if (!STORE && (!RAGGED || (mrow0 + b * 32 + i * 4 < t.m_end && ncol0 + pair * 64 < p.N)))
                 old[k % DEPTH][i] = __builtin_nontemporal_load(reinterpret_cast<const Raw*>(cu + ((b * 8 + i) * cstep + pair * pair_bytes) + coff));
         }
     };
-    static_for<0, DEPTH>([&](auto kc) { fetch_old(kc); });
+    if constexpr (!STORE) static_for<0, DEPTH>([&](auto kc) { fetch_old(kc); });
 
     static_for<0, 8>([&](auto kc) {
         constexpr int k = decltype(kc)::value, pair = k >> 2, b = k & 3;
@@ -778,9 +785,10 @@ __device__ __forceinline__ void drain_tile_accum(v16f (&acc)[4][4], float s1, co
         for (int i = 0; i < 8; ++i) {
             const int r = i * 4 + rr;
             const float4 v = *reinterpret_cast<const float4*>(stage + r * 256 + ((rc ^ (r & 15)) << 4));
-            if (!RAGGED || mrow0 + b * 32 + i * 4 < t.m_end) {
+            if (!RAGGED || (mrow0 + b * 32 + i * 4 < t.m_end && ncol0 + pair * 64 < p.N)) {
                 uint8_t* dst = cu + ((b * 8 + i) * cstep + pair * pair_bytes) + coff;
-                const Raw c = old[k % DEPTH][i];
+                Raw c{};
+                if constexpr (!STORE) c = old[k % DEPTH][i];
                 if constexpr (OUT_BF16) {
                     const u32x2 o = {pack_bf16x2_hw(v.x + bf16_lo(c[0]), v.y + bf16_hi(c[0])),
                                      pack_bf16x2_hw(v.z + bf16_lo(c[1]), v.w + bf16_hi(c[1]))};
@@ -792,7 +800,7 @@ __device__ __forceinline__ void drain_tile_accum(v16f (&acc)[4][4], float s1, co
             }
         }
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (k + DEPTH < 8) {
+        if constexpr (!STORE && k + DEPTH < 8) {
             fetch_old(std::integral_constant<int, (k + DEPTH < 8) ? k + DEPTH : 0>{});
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -804,7 +812,12 @@ __device__ __forceinline__ void drain_tile_accum(v16f (&acc)[4][4], float s1, co
 // K-tiles pay memory latency.  A tile's first MFMAs take a zero C operand (no accumulator clearing),
 // its scale factors are fetched under its last MFMAs, and its drain runs while the next tile's first
 // two K-tiles land.
-template <int FMT, int EPI, int SCALE>
+// MX: the term-split form of GemmArgs::b_k_period.  The copy stream's position in B wraps at the period, and each
+// K-tile's MFMAs take a power-of-two scale 2^(-4 term) on the activation side (E8M0 byte 127 - 4 term in
+// v_mfma_scale_f32_32x32x64_f8f6f4; 127 = 2^0 on the weight side), so the terms add up in the accumulator with
+// their weights and nothing else changes.  b_k_period is a multiple of BK.  This form takes no row index (the
+// rows of a tile follow from its position), which frees the registers the scale needs.
+template <int FMT, int EPI, int SCALE, int MX = 0>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void k_gemm_nt_ring(const GemmArgs p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -813,7 +826,7 @@ void k_gemm_nt_ring(const GemmArgs p) {
     constexpr int OUT_BN = GATE ? BN / 2 : BN;
     // the LDS-staged drain covers these epilogues; the launcher sends such a call here only when N is a multiple
     // of the tile's output width and C and the channel descales allow 16-byte accesses
-    constexpr bool ACCUM = EPI == EPI_ACCUM_F32 || EPI == EPI_ACCUM_BF16;
+    constexpr bool ACCUM = EPI == EPI_ACCUM_F32 || EPI == EPI_ACCUM_BF16 || EPI == EPI_STORE_F32;
     constexpr bool DRAIN = EPI == EPI_NONE || EPI == EPI_BIAS || EPI == EPI_SILU_GATE || ACCUM;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -837,12 +850,22 @@ void k_gemm_nt_ring(const GemmArgs p) {
     }
     if (my_tiles <= 0) return;        // grouped launches size the grid by an upper bound of the tile count
     const int ktiles = p.K / BK;      // >= 2, checked by the launcher
+    const int term_ktiles = MX ? p.b_k_period / BK : ktiles;      // K-tiles per term
+    // one register for both scale operands: byte 0 = 127 (2^0, the weight side), byte 1 = 127 - 4 term (the activation side)
+    constexpr int kMxOne = 0x7f7f, kMxStep = 0x0400;
+    int mx_scale = kMxOne, mx_left = term_ktiles;                  // scale of the K-tile being computed
+    auto mx_next = [&]() {                                         // ... moves on to the next K-tile of the tile
+        if constexpr (MX) {
+            if (--mx_left == 0) { mx_left = term_ktiles; mx_scale -= kMxStep; }
+        }
+    };
 
     float s1 = 0.0f, s2 = 0.0f;
     if constexpr (SCALE == SCALE_TENSOR && DRAIN) {
         s1 = p.sa[0] * p.sb[0];
         if constexpr (GATE) s2 = p.sa[0] * p.sb2[0];
     }
+    if constexpr (SCALE == SCALE_ROW) s1 = p.sb[0];
 
     // ---- global -> LDS: wave w copies rows [64w, 64w+64) of an operand tile, 8 rows per instruction ----
     const int lrow = lane >> 3, lslot = lane & 7;
@@ -855,6 +878,7 @@ void k_gemm_nt_ring(const GemmArgs p) {
     // after that tile's drain has waited for all memory traffic), the rows inside that drain.
     auto fetch_pos = [&](int seq, TilePos& t) { t = locate_tile<OUT_BN>(p, lin0 + seq * lstep); };
     auto fetch_rows = [&](const TilePos& t, int (&rows)[8]) {
+        if constexpr (MX) return;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int arow = min(t.m0 + wave * 64 + j * 8 + lrow, t.m_end - 1);
@@ -872,7 +896,8 @@ void k_gemm_nt_ring(const GemmArgs p) {
         for (int j = 0; j < 8; ++j) {
             const int row = wave * 64 + j * 8 + lrow;
             const uint32_t gchunk = (lslot ^ swz(row)) * 16;
-            xoff[j] = static_cast<uint32_t>(rows[j]) * static_cast<uint32_t>(p.lda) + gchunk;
+            const int arow = MX ? min(t.m0 + row, t.m_end - 1) : rows[j];
+            xoff[j] = static_cast<uint32_t>(arow) * static_cast<uint32_t>(p.lda) + gchunk;
             int n = t.n0 + row;
             if constexpr (GATE) {
                 // LDS weight rows of a wave: [gate 32 | up 32 | gate 32 | up 32] over the same 64 output columns;
@@ -933,7 +958,10 @@ void k_gemm_nt_ring(const GemmArgs p) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) c[r] = 0.0f;
         }
-        acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wq[H][a], xq[H][b], c, (FMT >> 1) & 1, FMT & 1, 0, 0, 0, 0);
+        if constexpr (MX)
+            acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wq[H][a], xq[H][b], c, (FMT >> 1) & 1, FMT & 1, 0, mx_scale, 1, mx_scale);
+        else
+            acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wq[H][a], xq[H][b], c, (FMT >> 1) & 1, FMT & 1, 0, 0, 0, 0);
     };
     using C0 = std::integral_constant<int, 0>;
     using C1 = std::integral_constant<int, 1>;
@@ -954,7 +982,7 @@ void k_gemm_nt_ring(const GemmArgs p) {
     int nrows[8];
     int fetch_seq = 0;                                 // the tile END fetches next (into t2 / nrows)
 
-    auto ktile = [&](auto first_c, auto end_c, int dk0, const TilePos& t, bool wait) {
+    auto ktile = [&](auto first_c, auto end_c, int dk0, int dkw, const TilePos& t, bool wait) {
         constexpr bool END = decltype(end_c)::value != 0;
         // step (g,0)
         static_for<0, 16>([&](auto ic) {
@@ -978,7 +1006,7 @@ void k_gemm_nt_ring(const GemmArgs p) {
                 read_one(a2, a3, C0{}, std::integral_constant<int, i - 2>{});
                 if constexpr (i >= 14) read_one(a2, a3, C0{}, ic);       // reads 14 and 15 ride with the last two MFMAs
             }
-            if constexpr (i >= 2 && i < 10) dma_w(a0, dk0, std::integral_constant<int, (i >= 2 && i < 10) ? i - 2 : 0>{});
+            if constexpr (i >= 2 && i < 10) dma_w(a0, dkw, std::integral_constant<int, (i >= 2 && i < 10) ? i - 2 : 0>{});
             if constexpr (END && i == 11) {
                 if (fetch_seq < my_tiles) fetch_pos(fetch_seq, t2);
             }
@@ -998,6 +1026,7 @@ void k_gemm_nt_ring(const GemmArgs p) {
     // Past the workgroup's last tile the stream simply re-reads that tile: the last two K-tiles then run
     // the same code as every other one, and what they copy is never used.
     int dkt = 2 % ktiles, dseq = 2 / ktiles;
+    int dkw = (dkt % term_ktiles) * BK;        // the stream's position in B (bytes along K): wraps at the term length
     // With three or more K-tiles per tile the stream turns to tile s+1 while tile s is being computed, and
     // (t1, nrows) were fetched under the last K-tile of tile s-1.  With two K-tiles per tile the stream is a
     // whole tile ahead; that shape simply fetches at the turn and waits.
@@ -1007,7 +1036,7 @@ void k_gemm_nt_ring(const GemmArgs p) {
     // first copy is issued (the copy pipeline must never wait on them); then K-tiles 0 and 1 of the stream
     // in flight, K-tile 0 landed and visible, operands (0,0) in set 0
     {
-        int rows0[8];
+        int rows0[8] = {};
         fetch_tile(0, t0, rows0);
         aim(t0, rows0);
         t1 = t0; t2 = t0;
@@ -1018,7 +1047,7 @@ void k_gemm_nt_ring(const GemmArgs p) {
         static_for<0, 8>([&](auto jc) { dma_x(a0, 0, jc); });
         static_for<0, 8>([&](auto jc) { dma_w(a1, 0, jc); });
         static_for<0, 8>([&](auto jc) { dma_x(a2, BK, jc); });
-        static_for<0, 8>([&](auto jc) { dma_w(a3, BK, jc); });
+        static_for<0, 8>([&](auto jc) { dma_w(a3, (1 % term_ktiles) * BK, jc); });
         if (!ahead && my_tiles > 1) {
             fetch_tile(1, t1, rows0);
             aim(t1, rows0);
@@ -1029,14 +1058,17 @@ void k_gemm_nt_ring(const GemmArgs p) {
     static_for<0, 16>([&](auto ic) { read_one(a0, a1, C0{}, ic); });
 
     auto advance_copy = [&]() {
+        dkw += BK;
+        if (MX && dkw == p.b_k_period) dkw = 0;
         if (++dkt == ktiles) {                   // the stream moves on to the next tile
             dkt = 0;
+            dkw = 0;
             if (++dseq < my_tiles) {
                 if (ahead) {
                     aim(t1, nrows);
                 } else {
                     TilePos tt;
-                    int rr[8];
+                    int rr[8] = {};
                     fetch_tile(dseq, tt, rr);
                     aim(tt, rr);
                 }
@@ -1048,14 +1080,15 @@ void k_gemm_nt_ring(const GemmArgs p) {
         if (!ahead) fetch_pos(seq, t0);
         const TilePos t = t0;
         // after a drain the first K-tile's successor has been waited for already
-        ktile(C1{}, C0{}, dkt * BK, t, !(DRAIN && seq > 0));
-        rotate(); advance_copy();
+        if constexpr (MX) { mx_scale = kMxOne; mx_left = term_ktiles; }
+        ktile(C1{}, C0{}, dkt * BK, dkw, t, !(DRAIN && seq > 0));
+        rotate(); advance_copy(); mx_next();
         for (int kt = 1; kt + 1 < ktiles; ++kt) {
-            ktile(C0{}, C0{}, dkt * BK, t, true);
-            rotate(); advance_copy();
+            ktile(C0{}, C0{}, dkt * BK, dkw, t, true);
+            rotate(); advance_copy(); mx_next();
         }
         fetch_seq = ahead ? seq + 2 : my_tiles;       // what the last K-tile fetches into (t2, nrows)
-        ktile(C0{}, C1{}, dkt * BK, t, true);
+        ktile(C0{}, C1{}, dkt * BK, dkw, t, true);
         rotate(); advance_copy();
         // After the rotation a4 is the slot that held W of the K-tile just finished.  Every wavefront has
         // finished reading it (barrier of the last step) and only X of the stream's third K-tile from here
@@ -1066,9 +1099,9 @@ void k_gemm_nt_ring(const GemmArgs p) {
         if constexpr (DRAIN) {
             uint8_t* stage = smem + a4 + wave * (64 * BK);
             if constexpr (ACCUM) {
-                constexpr bool BF = EPI == EPI_ACCUM_BF16;
-                if (t.m0 + BM <= t.m_end) drain_tile_accum<false, BF>(acc, s1, p, t, wm, wn, lane, stage, landed);
-                else                      drain_tile_accum<true, BF>(acc, s1, p, t, wm, wn, lane, stage, landed);
+                constexpr bool BF = EPI == EPI_ACCUM_BF16, ST = EPI == EPI_STORE_F32;
+                if (t.m0 + BM <= t.m_end && t.n0 + BN <= p.N) drain_tile_accum<false, BF, ST>(acc, s1, p, t, wm, wn, lane, stage, landed);
+                else                      drain_tile_accum<true, BF, ST>(acc, s1, p, t, wm, wn, lane, stage, landed);
             } else {
                 constexpr int out_bn = EPI == EPI_SILU_GATE ? BN / 2 : BN;
                 if (t.m0 + BM <= t.m_end && t.n0 + out_bn <= p.N) drain_tile<EPI, SCALE, false>(acc, sc, s1, s2, p, t, wm, wn, lane, stage, landed);
@@ -1080,7 +1113,7 @@ void k_gemm_nt_ring(const GemmArgs p) {
             q.M = t.m_end;
             epilogue<EPI, SCALE>(acc, q, t.m0, t.n0, wm, wn, lane);
         }
-        if (more) {
+        if (more && !MX) {
             // the row loads are older than the drain's last stores: requiring them here waits for nothing else
 #pragma unroll
             for (int j = 0; j < 8; ++j) asm volatile("" :: "v"(nrows[j]));
@@ -1797,6 +1830,83 @@ int cf::grouped_gemm_nt_bf16(int total_rows, int N, int K, int num_experts, cons
     return epilogue == EPI_SILU_GATE ? launch_tiled<0, EPI_SILU_GATE, SCALE_ROWCOL>(p, st)
                                      : launch_tiled<0, EPI_NONE, SCALE_ROWCOL>(p, st);
 }
+
+namespace cf {
+namespace {
+// the ring kernel and nothing else: for the forms that exist only there
+template <int FMT, int EPI, int SCALE, int MX>
+int launch_ring_only(const GemmArgs& p, hipStream_t st) {
+    static std::once_flag once;
+    static hipError_t err = hipSuccess;
+    std::call_once(once, [] {
+        err = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_nt_ring<FMT, EPI, SCALE, MX>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, kRingLds);
+    });
+    if (err != hipSuccess) return static_cast<int>(err);
+    const int total = p.tiles_m * p.tiles_n;
+    int grid = total < num_cus() ? total : num_cus();
+    if (grid >= kXcds) grid -= grid % kXcds;
+    k_gemm_nt_ring<FMT, EPI, SCALE, MX><<<grid, kThreads, kRingLds, st>>>(p);
+    return launch_status();
+}
+}  // namespace
+
+// C[r, :] = (A[index[r], :] . B[expert(r)]^T) * (a_descale[0] * b_descale[0]) in fp32, rows grouped by expert as in
+// grouped_gemm_nt_bf16; d_tile_map is the table build_tile_map made for these counts.  N % 4 == 0.
+int grouped_gemm_nt_store_f32(int total_rows, int N, int K, int num_experts, const void* A, int a_rows, int lda,
+                              const int* d_a_row_index, const float* a_descale, const void* B, const float* b_descale,
+                              float* C, int ldc, const int* d_tile_map, int a_is_e5m2, cf_stream_t stream) {
+    if (total_rows <= 0 || N <= 0 || num_experts <= 0) return CF_OK;
+    if (!A || !B || !C || !a_descale || !b_descale || !d_tile_map) return CF_ERR_INVALID_ARG;
+    if (K % BK != 0 || K < 2 * BK || lda % 16 != 0 || lda < K || !aligned16(A) || !aligned16(B) || N % 4 != 0 || ldc % 4 != 0 ||
+        ldc < N || !aligned16(C) || static_cast<size_t>(a_rows) * lda >= (1ull << 32) || static_cast<size_t>(N) * K >= (1ull << 32))
+        return CF_ERR_UNSUPPORTED;
+    GemmArgs p{};
+    p.M = total_rows; p.N = N; p.K = K;
+    p.A = static_cast<const uint8_t*>(A); p.lda = lda;
+    p.B = static_cast<const uint8_t*>(B); p.ldb = K;
+    p.sa = a_descale; p.sb = b_descale;
+    p.Cf = C; p.ldc = ldc;
+    p.tile_map = d_tile_map;
+    p.a_row_index = d_a_row_index;
+    p.a_rows = a_rows;
+    p.b_expert_stride = static_cast<long long>(N) * K;
+    p.tiles_m = total_rows / BM + num_experts;
+    p.tiles_n = (N + BN - 1) / BN;
+    hipStream_t st = as_stream(stream);
+    return a_is_e5m2 ? launch_ring_only<1, EPI_STORE_F32, SCALE_TENSOR, 0>(p, st)
+                     : launch_ring_only<0, EPI_STORE_F32, SCALE_TENSOR, 0>(p, st);
+}
+
+// C[r, :] = bf16( a_descale[r] * b_descale[:] * sum_t 2^(-4 t) A[r, t*Kb : (t+1)*Kb] . B[expert(r)]^T ): the activation
+// rows are `terms` E4M3 terms side by side (lda >= terms * Kb), B is [num_experts, N, Kb] E4M3, b_descale one scalar
+// for all experts.  Kb % 128 == 0; terms * Kb >= 256.
+int grouped_gemm_nt_bf16_terms(int total_rows, int N, int Kb, int terms, int num_experts, const void* A, int lda,
+                               const float* a_descale, const void* B, const float* b_descale, uint16_t* C, int ldc,
+                               const int* d_tile_map, cf_stream_t stream) {
+    if (total_rows <= 0 || N <= 0 || num_experts <= 0) return CF_OK;
+    if (!A || !B || !C || !a_descale || !b_descale || !d_tile_map || terms < 1 || terms > 8) return CF_ERR_INVALID_ARG;
+    const long long K = static_cast<long long>(terms) * Kb;
+    if (Kb % BK != 0 || Kb < BK || K < 2 * BK || lda % 16 != 0 || lda < K || !aligned16(A) || !aligned16(B) || N % 8 != 0 || N < 8 ||
+        ldc % 8 != 0 || ldc < N || !aligned16(C) ||
+        static_cast<size_t>(total_rows) * lda >= (1ull << 32) || static_cast<size_t>(N) * Kb >= (1ull << 32))
+        return CF_ERR_UNSUPPORTED;
+    GemmArgs p{};
+    p.M = total_rows; p.N = N; p.K = static_cast<int>(K);
+    p.A = static_cast<const uint8_t*>(A); p.lda = lda;
+    p.B = static_cast<const uint8_t*>(B); p.ldb = Kb;
+    p.sa = a_descale; p.sb = b_descale;
+    p.C = C; p.ldc = ldc;
+    p.tile_map = d_tile_map;
+    p.a_rows = total_rows;
+    p.b_expert_stride = static_cast<long long>(N) * Kb;
+    p.sb_expert_stride = 0;
+    p.b_k_period = Kb;
+    p.tiles_m = total_rows / BM + num_experts;
+    p.tiles_n = (N + BN - 1) / BN;
+    return launch_ring_only<0, EPI_NONE, SCALE_ROW, 1>(p, as_stream(stream));
+}
+}  // namespace cf
 
 extern "C" {
 

@@ -555,6 +555,37 @@ int cf_moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_fcin_
                                       int H, int Ie, int num_experts, int total_selected_rows,
                                       cf_stream_t stream);
 
+/* moe_grouped_expert_forward_fp8 (kernels.hpp:400-423, kernels/moe.cu:950-1127) with a workspace: the same
+ * arguments and contract as cf_moe_grouped_expert_forward_fp8, run as whole-matrix launches when H % 128 == 0,
+ * H >= 256, Ie % 128 == 0, Ie <= 4096 and hidden, weights and d_mixed are 16-byte aligned (other shapes are
+ * passed on to that function and need no workspace).  fc_in is one grouped FP8 GEMM over the gathered token
+ * rows with fp32 output; the GELU is taken in fp32 (erf to 1.5e-7 absolute) and each row is written as three
+ * E4M3 terms under one per-row scale (value * scale = q0 + q1 / 16 + q2 / 256 to 2^-13: 12 to 13 significand
+ * bits, not re-quantized to a single fp8 value); fc_out is one grouped FP8 GEMM over K = 3 Ie in which the
+ * matrix cores weight term t by 2^(-4 t) (E8M0 scales of the MX form of the FP8 MFMA), so the three partial
+ * products add in one fp32 accumulator; w * y is then added into d_mixed per token row over its experts in
+ * ascending order, one bf16 rounding per expert.  Differences from the reference kernel: y is rounded to bf16
+ * before it is weighted and added (one more bf16 rounding per (row, expert)), and the order of the adds is
+ * fixed.  total_selected_rows must be the sum of d_counts; d_offsets may be null (the offsets are recomputed).
+ * d_workspace 256-byte aligned; cf_moe_grouped_expert_forward_fp8_workspace gives its size and, when
+ * `offsets` is not null, the byte offsets of the intermediates (CF_MOE_FWD_WS_* order), which stay valid
+ * after the call: pre [total, Ie] fp32, split [total, 3 Ie] E4M3, split_descale [total] fp32, y [total, H] bf16,
+ * experts back to back. */
+enum {
+    CF_MOE_FWD_WS_TILE_MAP = 0, CF_MOE_FWD_WS_OFFSETS, CF_MOE_FWD_WS_INDEX, CF_MOE_FWD_WS_SLOT, CF_MOE_FWD_WS_PRE,
+    CF_MOE_FWD_WS_SPLIT, CF_MOE_FWD_WS_SPLIT_DESCALE, CF_MOE_FWD_WS_Y, CF_MOE_FWD_WS_COUNT
+};
+int cf_moe_grouped_expert_forward_fp8_workspace(int rows, int total_selected_rows, int num_experts, int H,
+                                                int Ie, size_t* offsets, size_t* bytes);
+int cf_moe_grouped_expert_forward_fp8_ws(const void* d_hidden, const float* d_fcin_descale,
+                                         int fcin_is_e5m2, const float* d_route_weights,
+                                         const int* d_counts, const int* d_offsets,
+                                         const int* d_row_indices, const void* d_fc_in_w,
+                                         const float* d_fc_in_descale, const void* d_fc_out_w,
+                                         const float* d_fc_out_descale, uint16_t* d_mixed, int rows,
+                                         int H, int Ie, int num_experts, int total_selected_rows,
+                                         void* d_workspace, size_t workspace_bytes, cf_stream_t stream);
+
 /* moe_grouped_expert_forward_bf16, kernels.hpp:400-407: the same device-scheduled expert bank on
  * bf16 hidden states and bf16 weights (fc_in_w [E,Ie,H], fc_out_w [E,H,Ie]), no descales; fp32
  * accumulation, exact-erf GELU kept in fp32, compare-and-swap accumulation into d_mixed.  The

@@ -283,6 +283,14 @@ def main():
     mfma("grouped GELU expert bank, whole pipeline (re-quantizing)", f"T={T} E={E} k={k}", 4.0 * total * Ie * H,
          lambda: cf.cf_moe_grouped_gelu_forward_fp8(hq, one, 0, rw, counts, offs, idx, wg, one, wd, one, mixed, T, H, Ie, E, total,
                                                     ws3, sz3.value, st))
+    sz4 = ctypes.c_size_t(0)
+    cf.raw_cf_moe_grouped_expert_forward_fp8_workspace(T, total, E, H, Ie, None, ctypes.byref(sz4))
+    ws4 = u8(sz4.value)
+    mfma("moe_grouped_expert_forward_fp8 with a workspace (fp32 fc_in, 3-term E4M3 GELU, FP8 fc_out)", f"T={T} E={E} k={k}",
+         4.0 * total * Ie * H,
+         lambda: cf.cf_moe_grouped_expert_forward_fp8_ws(hq, one, 0, rw, counts, None, idx, wg, one, wd, one, mixed, T, H, Ie, E, total,
+                                                         ws4, sz4.value, st))
+    del ws4
     iters, args.iters = args.iters, 5
     mfma("moe_grouped_expert_forward_fp8 form (fp32 GELU kept, MFMA)", f"T={T} E={E} k={k}", 4.0 * total * Ie * H,
          lambda: cf.cf_moe_grouped_expert_forward_fp8(hq, one, 0, rw, counts, offs, idx, wg, one, wd, one, mixed, T, H, Ie, E, total, st))

@@ -1,0 +1,205 @@
+"""GPU parity: moe_grouped_expert_forward_fp8 (/root/reference/kernels/moe.cu:950-1127) as whole-matrix launches with
+a workspace (cf_moe_grouped_expert_forward_fp8_ws).
+
+Every stage is checked on the intermediates the call leaves in its workspace, given that stage's own (GPU) inputs:
+the fp32 projections against the double product of the dequantized operands; the three-term E4M3 split of the GELU
+against the exact-erf GELU of those projections (12 bits and better, and the row maximum lands on 448); the fc_out
+GEMM, whose matrix-core scales weight term t by 16^-t, against the double product of the recombined terms to one bf16
+rounding; the result against the oracle of the reference kernel at the bars of the one-kernel form's test."""
+import ctypes
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import oracle_lib as orc
+from gpu_util import bf16_bits, case, dev_arr, dev_bf16, host, stream
+
+pytestmark = pytest.mark.gpu
+
+NAMES = ["TILE_MAP", "OFFSETS", "INDEX", "SLOT", "PRE", "SPLIT", "SPLIT_DESCALE", "Y"]
+erf = np.vectorize(math.erf, otypes=[np.float64])
+
+
+def gelu64(x):
+    return 0.5 * x * (1.0 + erf(x * 0.70710678118654752440))
+
+
+class Bank:
+    def __init__(self, dev, rows, E, k, H, Ie, e5m2, seed, zero_expert=None):
+        rng = np.random.default_rng(seed)
+        self.rows, self.E, self.k, self.H, self.Ie, self.e5m2, self.dev = rows, E, k, H, Ie, e5m2, dev
+        x = rng.standard_normal((rows, H)).astype(np.float32)
+        fmax = 57344.0 if e5m2 else 448.0
+        sx = np.float32(fmax) / np.abs(x).max()
+        self.hq = (orc.e5m2_satfinite if e5m2 else orc.e4m3_satfinite)(x * sx)
+        win = (0.05 * rng.standard_normal((E, Ie, H))).astype(np.float32)
+        wout = (0.05 * rng.standard_normal((E, H, Ie))).astype(np.float32)
+        s_in, s_out = np.float32(448.0) / np.abs(win).max(), np.float32(448.0) / np.abs(wout).max()
+        self.winq, self.woutq = orc.e4m3_satfinite(win * s_in), orc.e4m3_satfinite(wout * s_out)
+        self.d_h, self.d_in, self.d_out = np.float32(1) / sx, np.float32(1) / s_in, np.float32(1) / s_out
+        logits = rng.standard_normal((rows, E)).astype(np.float32)
+        if zero_expert is not None:
+            logits[:, zero_expert] = -50.0
+        self.rw = orc.moe_topk_route(logits, k)
+        self.counts, self.idx = orc.moe_build_expert_row_lists(self.rw)
+        self.total = int(self.counts.sum())
+        self.mixed0 = orc.bf16_from_f32(rng.standard_normal((rows, H)).astype(np.float32))
+
+    def compact_index(self):
+        return np.concatenate([self.idx[e, : self.counts[e]] for e in range(self.E)])
+
+    def expert_of_compact(self):
+        return np.repeat(np.arange(self.E), self.counts)
+
+
+def workspace(cf, b):
+    offs = (ctypes.c_size_t * len(NAMES))()
+    nbytes = ctypes.c_size_t()
+    cf.cf_moe_grouped_expert_forward_fp8_workspace(b.rows, b.total, b.E, b.H, b.Ie, offs, ctypes.byref(nbytes))
+    return {n: int(offs[i]) for i, n in enumerate(NAMES)}, int(nbytes.value)
+
+
+def run(cf, b, pass_offsets=False):
+    dev = b.dev
+    off, nbytes = workspace(cf, b)
+    ws = torch.empty(max(nbytes, 256) + 256, dtype=torch.uint8, device=dev)
+    ws.fill_(0xCD)
+    shift = (-ws.data_ptr()) % 256
+    ws = ws[shift:shift + max(nbytes, 256)]
+    mixed = dev_bf16(b.mixed0, dev)
+    sc = lambda v: torch.tensor([v], dtype=torch.float32, device=dev)
+    offsets = dev_arr(orc.moe_expert_offsets(b.counts), dev) if pass_offsets else None
+    cf.cf_moe_grouped_expert_forward_fp8_ws(dev_arr(b.hq, dev), sc(b.d_h), int(b.e5m2), dev_arr(b.rw, dev), dev_arr(b.counts, dev), offsets,
+                                            dev_arr(b.idx, dev), dev_arr(b.winq, dev), sc(b.d_in), dev_arr(b.woutq, dev), sc(b.d_out),
+                                            mixed, b.rows, b.H, b.Ie, b.E, b.total, ws if nbytes else None, nbytes, stream())
+    torch.cuda.synchronize()
+    return mixed, ws, off, nbytes
+
+
+def check_result(b, mixed):
+    start = orc.bf16_to_f32(b.mixed0).astype(np.float64)
+    ref = orc.moe_grouped_expert_forward_fp8_ref(b.hq, b.d_h, b.e5m2, b.rw, b.counts, b.idx, b.winq, b.d_in, b.woutq, b.d_out, start)
+    got = orc.bf16_to_f32(bf16_bits(mixed)).astype(np.float64)
+    rel = np.sqrt(((got - ref) ** 2).sum() / (ref ** 2).sum())
+    assert rel <= 4e-3, rel
+    # every one of the k accumulations rounds the running value to bf16, y is rounded once before it: bound as in the
+    # test of the one-kernel form, with one more rounding per expert
+    typical = np.sqrt(((ref - start) ** 2).mean())
+    bound = (2 * b.k + 1) * 2.0 ** -8 * (np.abs(start) + np.abs(ref) + 2.0 * typical)
+    assert np.all(np.abs(got - ref) <= bound)
+    untouched = ~(b.rw > 0).any(axis=1)
+    assert np.array_equal(bf16_bits(mixed)[untouched], b.mixed0[untouched])
+    return rel
+
+
+@pytest.mark.parametrize("rows,E,k,H,Ie,e5m2,zero", [
+    (70, 3, 3, 2048, 1408, False, None),       # config 5's widths: 11 K-tiles per term
+    (40, 3, 2, 2304, 128, False, None),        # one K-tile per term: the weight columns wrap at every K-tile
+    (300, 6, 3, 256, 384, True, None),         # E5M2 hidden states, two K-tiles of fc_in
+    (1000, 5, 2, 384, 256, False, 2),          # several row tiles per expert, ragged last ones, an expert with no rows
+    (64, 2, 1, 256, 4096, False, None),        # the widest row the split keeps in registers
+])
+def test_staged_bank_stage_by_stage(cf, dev, rows, E, k, H, Ie, e5m2, zero):
+    case(f"staged gelu bank rows={rows} E={E} k={k} H={H} Ie={Ie} e5m2={e5m2} zero_expert={zero}")
+    b = Bank(dev, rows, E, k, H, Ie, e5m2, seed=rows + Ie, zero_expert=zero)
+    mixed, ws, off, nbytes = run(cf, b)
+    assert nbytes > 0
+    T = b.total
+    raw = host(ws)
+    take = lambda name, dtype, count: raw[off[name]: off[name] + count * np.dtype(dtype).itemsize].view(dtype)
+    index = take("INDEX", np.int32, T)
+    assert np.array_equal(index, b.compact_index())
+    assert np.array_equal(take("OFFSETS", np.int32, E), orc.moe_expert_offsets(b.counts))
+    expert = b.expert_of_compact()
+
+    # fc_in: fp32 projections of the gathered rows
+    hx = (orc.e5m2_unpack if e5m2 else orc.e4m3_unpack)(b.hq).astype(np.float64)
+    win = orc.e4m3_unpack(b.winq).astype(np.float64)
+    wout = orc.e4m3_unpack(b.woutq).astype(np.float64)
+    pre = take("PRE", np.float32, T * Ie).reshape(T, Ie).astype(np.float64)
+    s_in = float(np.float32(b.d_h) * np.float32(b.d_in))
+    for e in range(E):
+        sel = expert == e
+        if not sel.any():
+            continue
+        want = (hx[index[sel]] @ win[e].T) * s_in
+        ad = (np.abs(hx[index[sel]]) @ np.abs(win[e]).T) * s_in
+        assert np.all(np.abs(pre[sel] - want) <= 2.0 ** -22 * np.abs(want) + orc.ACC_MFMA * ad), f"fc_in expert {e}"
+
+    # split: three terms recombine to the exact-erf GELU of the GPU's projections
+    q = take("SPLIT", np.uint8, T * 3 * Ie).reshape(T, 3, Ie)
+    d = take("SPLIT_DESCALE", np.float32, T).astype(np.float64)
+    terms = orc.e4m3_unpack(q).astype(np.float64)
+    recon = (terms[:, 0] + terms[:, 1] / 16.0 + terms[:, 2] / 256.0) * d[:, None]
+    g = gelu64(pre)
+    amax = np.abs(g).max(axis=1)
+    assert np.allclose(d, amax / 448.0, rtol=1e-5), "row descale is amax / 448"
+    assert np.all(np.abs(terms[:, 0]).max(axis=1) == 448.0), "the row maximum lands on the largest E4M3 value"
+    tol = 2.0 ** -12 * np.abs(g) + (amax * 2.0 ** -17 / 448.0)[:, None] + 4e-7 * (np.abs(pre) + 1e-3)
+    worst = np.abs(recon - g) / tol
+    assert worst.max() <= 1.0, f"split worst {worst.max():.3f}"
+    # ... and carries more than bf16 would: compare the two errors over the elements that matter
+    big = np.abs(g) >= amax[:, None] * 2.0 ** -6
+    bf = orc.bf16_to_f32(orc.bf16_from_f32(g.astype(np.float32))).astype(np.float64)
+    assert np.abs(recon - g)[big].max() / np.abs(g)[big].max() < 2.0 ** -12
+    assert np.sqrt(((recon - g)[big] ** 2).mean()) < 0.125 * np.sqrt(((bf - g)[big] ** 2).mean())
+
+    # fc_out: the matrix cores weight the terms; one bf16 rounding of the fp32 sum
+    y = orc.bf16_to_f32(take("Y", np.uint16, T * H).reshape(T, H)).astype(np.float64)
+    act = terms[:, 0] + terms[:, 1] / 16.0 + terms[:, 2] / 256.0
+    act_abs = np.abs(terms[:, 0]) + np.abs(terms[:, 1]) / 16.0 + np.abs(terms[:, 2]) / 256.0
+    for e in range(E):
+        sel = expert == e
+        if not sel.any():
+            continue
+        rowscale = d[sel][:, None] * float(b.d_out)
+        want = (act[sel] @ wout[e].T) * rowscale
+        ad = (act_abs[sel] @ np.abs(wout[e]).T) * rowscale
+        tol = 0.505 * orc.bf16_ulp(np.maximum(np.abs(want), np.abs(y[sel]))) + orc.ACC_MFMA * ad
+        worst = np.abs(y[sel] - want) / tol
+        assert worst.max() <= 1.0, f"fc_out expert {e}: worst {worst.max():.3f}"
+
+    check_result(b, mixed)
+
+
+def test_staged_bank_takes_offsets_and_repeats(cf, dev):
+    """Offsets handed in or recomputed, and a second call on a dirty workspace: the same bits."""
+    case("staged gelu bank, offsets given / recomputed, repeated")
+    b = Bank(dev, 500, 8, 2, 512, 256, False, seed=5)
+    m1, ws, off, nbytes = run(cf, b)
+    m2, _, _, _ = run(cf, b, pass_offsets=True)
+    assert np.array_equal(bf16_bits(m1), bf16_bits(m2))
+    check_result(b, m1)
+
+
+def test_other_shapes_pass_through_without_a_workspace(cf, dev):
+    case("staged gelu bank entry on a shape of the one-kernel forms")
+    b = Bank(dev, 200, 4, 2, 128, 64, False, seed=9)
+    mixed, _, _, nbytes = run(cf, b)
+    assert nbytes == 0
+    start = orc.bf16_to_f32(b.mixed0).astype(np.float64)
+    ref = orc.moe_grouped_expert_forward_fp8_ref(b.hq, b.d_h, False, b.rw, b.counts, b.idx, b.winq, b.d_in, b.woutq, b.d_out, start)
+    got = orc.bf16_to_f32(bf16_bits(mixed)).astype(np.float64)
+    assert np.sqrt(((got - ref) ** 2).sum() / (ref ** 2).sum()) <= 4e-3
+
+
+def cf_conv(v):
+    return v.data_ptr() if hasattr(v, "data_ptr") else v
+
+
+def test_staged_bank_rejects_a_short_workspace(cf, dev):
+    case("staged gelu bank, short or missing workspace")
+    b = Bank(dev, 64, 2, 1, 256, 128, False, seed=3)
+    off, nbytes = workspace(cf, b)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    mixed = dev_bf16(b.mixed0, dev)
+    sc = lambda v: torch.tensor([v], dtype=torch.float32, device=dev)
+    args = lambda w, n: (dev_arr(b.hq, dev), sc(b.d_h), 0, dev_arr(b.rw, dev), dev_arr(b.counts, dev), None, dev_arr(b.idx, dev),
+                         dev_arr(b.winq, dev), sc(b.d_in), dev_arr(b.woutq, dev), sc(b.d_out), mixed, b.rows, b.H, b.Ie, b.E, b.total,
+                         w, n, stream())
+    assert cf.raw_cf_moe_grouped_expert_forward_fp8_ws(*[cf_conv(a) for a in args(ws, nbytes - 1)]) == -1
+    assert cf.raw_cf_moe_grouped_expert_forward_fp8_ws(*[cf_conv(a) for a in args(None, nbytes)]) == -1
+    torch.cuda.synchronize()
+    assert np.array_equal(bf16_bits(mixed), b.mixed0)

@@ -23,7 +23,12 @@ int main() {
     void (*f14)(hipStream_t, int, int, int, float, const bf16*, int, const bf16*, int, float, bf16*, int) = &gemm_bf16;
     void (*f15)(hipStream_t, int, int, int, float, const bf16*, int, const bf16*, int, float, float*, int) = &gemm_bf16_tn_f32;
     void (*f16)(hipStream_t, int, int, int, float, const bf16*, int, const bf16*, int, float, bf16*, int) = &gemm_bf16_tn_f32;
-    if (!f12 || !f13 || !f14 || !f15 || !f16) return 1;
+    void (*f17)(const void*, const float*, int, const float*, const int*, const int*, const int*, const void*, const float*, const void*,
+                const float*, bf16*, int, int, int, int, int, hipStream_t) = &moe_grouped_expert_forward_fp8;
+    void (*f18)(const void*, const float*, int, const float*, const int*, const int*, const int*, const void*, const float*, const void*,
+                const float*, bf16*, int, int, int, int, int, void*, std::size_t, hipStream_t) = &moe_grouped_expert_forward_fp8;
+    std::size_t (*f19)(int, int, int, int, int) = &moe_grouped_expert_forward_fp8_workspace_bytes;
+    if (!f12 || !f13 || !f14 || !f15 || !f16 || !f17 || !f18 || !f19) return 1;
     if (!f1 || !f2 || !f3 || !f4 || !f5 || !f6 || !f7 || !f8 || !f9 || !f10 || !f11) return 1;
     int ok = 0;
     try { swiglu_forward(nullptr, nullptr, nullptr, -1, nullptr); } catch (const std::invalid_argument&) { ++ok; }   // kernels/activations.cu:61-72

@@ -231,6 +231,10 @@ int grouped_gemm_nt_store_f32(int total_rows, int N, int K, int num_experts, con
 int grouped_gemm_nt_bf16_terms(int total_rows, int N, int Kb, int terms, int num_experts, const void* A, int lda,
                                const float* a_descale, const void* B, const float* b_descale, uint16_t* C, int ldc,
                                const int* d_tile_map, cf_stream_t stream);
+// The forward-pass form of the grouped bf16 GEMM (gemm_bf16.hip): C[r, :] = sum_t A[r, t*Kb:(t+1)*Kb] . B[expert(r)]^T,
+// B [num_experts, N, Kb], C bf16 or fp32, tile table already built.
+int grouped_gemm_bf16_nt(int total_rows, int N, int Kb, int terms, int num_experts, const uint16_t* A, int lda,
+                         const uint16_t* B, void* C, int ldc, bool c_is_f32, const int* d_tile_map, cf_stream_t stream);
 // The tile table of a grouped GEMM (k_build_tile_map in gemm.hip): tile_map[0] = number of row tiles of 256 rows,
 // then per row tile (expert, its first row, its end row, its first row tile, its row-tile count), experts back to back.
 void build_tile_map(const int* d_counts, const int* d_offsets, int num_experts, int max_row_tiles, int* tile_map,

@@ -41,11 +41,11 @@ typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef __bf16 v4bf __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) v4bf* lds_v4bf_ptr;
 
-enum { OUT_STORE_BF16 = 0, OUT_ACCUM_BF16 = 1, OUT_ACCUM_F32 = 2 };
+enum { OUT_STORE_BF16 = 0, OUT_ACCUM_BF16 = 1, OUT_ACCUM_F32 = 2, OUT_STORE_F32 = 3 };
 
 struct BfArgs {
     const uint16_t* A; int lda;     // M side.  NN: [M rows][K]; TN: [K rows][M]
-    const uint16_t* B; int ldb;     // N side: [K rows][N]
+    const uint16_t* B; int ldb;     // N side: [K rows][N]; NT (B_KC): [N rows][K]
     void* C; int ldc;               // [M][N], bf16 or fp32
     int M, N, K;
     int tiles_m, tiles_n;
@@ -55,6 +55,8 @@ struct BfArgs {
     const int* tile_map;            // NN: [0] = row tiles, then (expert, first row, end row, first row tile, row tiles) each
     long long b_expert_stride;      // NN: elements between the experts' B matrices
     long long c_expert_stride;      // TN: elements between the experts' C matrices
+    int b_k_period;                 // NT: B has this many columns and k runs over them again and again (K a multiple:
+                                    // A's rows are several terms side by side against the same B); 0 = B has K columns
 };
 
 template <int I, int N, class F>
@@ -90,8 +92,9 @@ __device__ __forceinline__ v8bf read_ks(const uint8_t* lane_ptr, int krow0, int 
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
-// A_KS: the M-side operand is stored [K][M] (the weight-gradient form); otherwise [M][K]
-template <bool A_KS, int OUT, bool GROUPED>
+// A_KS: the M-side operand is stored [K][M] (the weight-gradient form); otherwise [M][K].
+// B_KC: the N-side operand is stored [N][K] (a weight matrix as the forward pass holds it); otherwise [K][N].
+template <bool A_KS, int OUT, bool GROUPED, bool B_KC = false>
 __global__ __launch_bounds__(kThr) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void k_gemm_bf16(const BfArgs p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -141,7 +144,7 @@ void k_gemm_bf16(const BfArgs p) {
         }
     }
     if (k_end <= k_begin) {
-        if constexpr (OUT != OUT_STORE_BF16) return;      // nothing to add
+        if constexpr (OUT == OUT_ACCUM_BF16 || OUT == OUT_ACCUM_F32) return;      // nothing to add
     }
     constexpr int TK = 64;
     constexpr int NA = A_KS ? TK / 8 : 8, NB = TK / 8;       // 16-byte chunks per lane and K-tile
@@ -173,6 +176,10 @@ void k_gemm_bf16(const BfArgs p) {
     const uint32_t a_lane_ks = m0 + (tid & 31) * 8 < p.M ? (tid >> 5) * static_cast<uint32_t>(p.lda) * 2u + (tid & 31) * 16u : kOutside;
     // [m][k] operand: this lane's row within a group of 32 rows and its 16-byte k chunk
     const uint32_t a_lane_kc = (tid >> 3) * static_cast<uint32_t>(p.lda) * 2u + (tid & 7) * 16u;
+    const uint32_t b_lane_kc = (tid >> 3) * static_cast<uint32_t>(p.ldb) * 2u + (tid & 7) * 16u;
+    // NT with a period: where tile ks of the k range starts in B's columns
+    const int b_period = B_KC && p.b_k_period ? p.b_k_period : 0x7fffffff;
+    int kb_load = 0;              // ... for the tile the next load_one calls fetch (set by the callers)
     // chunk c (0 .. NA-1: M side, NA .. NA+NB-1: N side) of K-tile ks into its staging register
     auto load_one = [&](int ks, auto cc, uint4 (&ra)[NA], uint4 (&rb)[NB]) {
         constexpr int c = decltype(cc)::value;
@@ -184,6 +191,9 @@ void k_gemm_bf16(const BfArgs p) {
                 const uint32_t off = k0 + (tid & 7) * 8 < k_end ? a_lane_kc : kOutside;
                 ra[c] = load_rows(p.A, p.lda, m0 + 32 * c, m_end, k0, off);
             }
+        } else if constexpr (B_KC) {
+            const uint32_t off = k0 + (tid & 7) * 8 < k_end ? b_lane_kc : kOutside;
+            rb[c - NA] = load_rows(B, p.ldb, n0 + 32 * (c - NA), p.N, kb_load, off);
         } else {
             rb[c - NA] = load_rows(B, p.ldb, k0 + 8 * (c - NA), k_end, n0, b_lane);
         }
@@ -199,6 +209,9 @@ void k_gemm_bf16(const BfArgs p) {
                 const int r = (tid >> 3) + 32 * c;
                 *reinterpret_cast<uint4*>(as + r * kPitchKC + (((tid & 7) ^ swz(r)) << 4)) = ra[c];
             }
+        } else if constexpr (B_KC) {
+            const int r = (tid >> 3) + 32 * (c - NA);
+            *reinterpret_cast<uint4*>(as + kATile + r * kPitchKC + (((tid & 7) ^ swz(r)) << 4)) = rb[c - NA];
         } else {
             *reinterpret_cast<uint4*>(as + kATile + ((tid >> 5) + 8 * (c - NA)) * kPitchN + (tid & 31) * 16) = rb[c - NA];
         }
@@ -221,7 +234,10 @@ void k_gemm_bf16(const BfArgs p) {
     auto read_unit = [&](int stage, auto sc, auto uc) {
         constexpr int ks16 = decltype(sc)::value, u = decltype(uc)::value;
         const uint8_t* as = smem + stage * kStage;
-        if constexpr (u < 4) {
+        if constexpr (u < 4 && B_KC) {
+            const int row = wn * 128 + 32 * u + frow;
+            nop[ks16 & 1][u] = *reinterpret_cast<const v8bf*>(as + kATile + row * kPitchKC + (((2 * ks16 + khalf) ^ swz(row)) << 4));
+        } else if constexpr (u < 4) {
             nop[ks16 & 1][u] = read_ks<kPitchN>(as + kATile + ks_n, 16 * ks16, 32 * u);
         } else if constexpr (A_KS) {
             mop[ks16 & 1][u - 4] = read_ks<kPitchM>(as + ks_m, 16 * ks16, 32 * (u - 4));
@@ -253,12 +269,18 @@ void k_gemm_bf16(const BfArgs p) {
             if constexpr (m == 47) __syncthreads();
             __builtin_amdgcn_sched_barrier(0);
         });
+        if constexpr (B_KC) {          // the next K-tile's loads are one tile further
+            kb_load += TK;
+            if (kb_load >= b_period) kb_load -= b_period;
+        }
     };
 
     static_assert(NA + NB == 16, "the weave above places 16 loads and 16 LDS stores per K-tile");
     uint4 ra0[NA], rb0[NB], ra1[NA], rb1[NB];
     static_for<0, 16>([&](auto c) { load_one(0, c, ra0, rb0); });
+    if constexpr (B_KC) kb_load = TK % b_period;
     static_for<0, 16>([&](auto c) { load_one(1, c, ra1, rb1); });
+    if constexpr (B_KC) kb_load = (2 * TK) % b_period;
     static_for<0, 16>([&](auto c) { park_one(0, c, ra0, rb0); });
     __syncthreads();
     static_for<0, 8>([&](auto u) { read_unit(0, std::integral_constant<int, 0>{}, u); });
@@ -282,7 +304,9 @@ void k_gemm_bf16(const BfArgs p) {
                 const size_t at = c_base + static_cast<size_t>(m) * p.ldc + n;
                 float v[4] = {acc_read(acc[j][i][4 * q]), acc_read(acc[j][i][4 * q + 1]), acc_read(acc[j][i][4 * q + 2]),
                               acc_read(acc[j][i][4 * q + 3])};
-                if constexpr (OUT == OUT_ACCUM_F32) {
+                if constexpr (OUT == OUT_STORE_F32) {
+                    *reinterpret_cast<float4*>(static_cast<float*>(p.C) + at) = make_float4(v[0], v[1], v[2], v[3]);
+                } else if constexpr (OUT == OUT_ACCUM_F32) {
                     float4* dst = reinterpret_cast<float4*>(static_cast<float*>(p.C) + at);
                     float4 c = *dst;
                     c.x += v[0]; c.y += v[1]; c.z += v[2]; c.w += v[3];
@@ -298,16 +322,16 @@ void k_gemm_bf16(const BfArgs p) {
                 }
                 // one quad's loads and stores at a time: pulling the whole tile's reads of C to the front would need
                 // more registers than the main loop leaves
-                if constexpr (OUT != OUT_STORE_BF16) __builtin_amdgcn_sched_barrier(0);
+                if constexpr (OUT == OUT_ACCUM_BF16 || OUT == OUT_ACCUM_F32) __builtin_amdgcn_sched_barrier(0);
             }
     }
 }
 
-template <bool A_KS, int OUT, bool GROUPED>
+template <bool A_KS, int OUT, bool GROUPED, bool B_KC = false>
 int launch(const BfArgs& p, dim3 grid, hipStream_t st) {
     static std::once_flag once;
     hipError_t attr = hipSuccess;
-    auto kern = k_gemm_bf16<A_KS, OUT, GROUPED>;
+    auto kern = k_gemm_bf16<A_KS, OUT, GROUPED, B_KC>;
     std::call_once(once, [&] {
         attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
     });
@@ -385,6 +409,31 @@ int gemm_tn(int M, int N, int K, int E, const int* counts, const int* offsets, c
 }
 
 }  // namespace
+
+// C[r, :] = sum over terms t of A[r, t*Kb : (t+1)*Kb] . B[expert(r)]^T: the forward-pass form, A [total_rows, terms*Kb]
+// with its rows grouped by expert, B [num_experts, N, Kb] as a weight matrix lies in memory, C bf16 or fp32 [total, N];
+// d_tile_map is the table build_tile_map made for these counts.  Kb % 8 == 0 (% 64 with several terms), N % 8 == 0.
+int grouped_gemm_bf16_nt(int total_rows, int N, int Kb, int terms, int num_experts, const uint16_t* A, int lda,
+                         const uint16_t* B, void* C, int ldc, bool c_is_f32, const int* d_tile_map, cf_stream_t stream) {
+    if (total_rows <= 0 || N <= 0 || num_experts <= 0) return CF_OK;
+    if (!A || !B || !C || !d_tile_map || terms < 1) return CF_ERR_INVALID_ARG;
+    const long long K = static_cast<long long>(terms) * Kb;
+    if ((terms > 1 ? Kb % kMaxTK : Kb % 8) != 0 || Kb <= 0 || lda < K || ldc < N || N % 8 != 0 || !operands_ok(A, lda, B, Kb, C, ldc, c_is_f32 ? 4 : 2) ||
+        static_cast<size_t>(total_rows) * lda >= (1ull << 30) || static_cast<size_t>(N) * Kb >= (1ull << 30))
+        return CF_ERR_UNSUPPORTED;
+    BfArgs p{};
+    p.A = A; p.lda = lda; p.B = B; p.ldb = Kb; p.C = C; p.ldc = ldc;
+    p.M = total_rows; p.N = N; p.K = static_cast<int>(K);
+    p.tiles_n = (N + TN - 1) / TN;
+    p.tiles_m = total_rows / TM + num_experts;
+    p.tile_map = d_tile_map;
+    p.b_expert_stride = static_cast<long long>(N) * Kb;
+    p.b_k_period = terms > 1 ? Kb : 0;
+    const long long total = static_cast<long long>(p.tiles_m) * p.tiles_n;
+    const dim3 grid(static_cast<unsigned>(8 * ((total + 7) / 8)));
+    hipStream_t st = as_stream(stream);
+    return c_is_f32 ? launch<false, OUT_STORE_F32, true, true>(p, grid, st) : launch<false, OUT_STORE_BF16, true, true>(p, grid, st);
+}
 }  // namespace cf
 
 using namespace cf;

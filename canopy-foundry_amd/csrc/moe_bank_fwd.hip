@@ -98,7 +98,7 @@ __global__ __launch_bounds__(kSplitThreads) void k_gelu_split3(const float* __re
 }
 
 struct FwdWs { size_t off[CF_MOE_FWD_WS_COUNT]; size_t slot_bytes, total; };
-FwdWs fwd_layout(int rows, int total_rows, int num_experts, int H, int Ie) {
+FwdWs fwd_layout(int rows, int total_rows, int num_experts, int H, int Ie, bool bf16_form = false) {
     auto up = [](size_t v) { return (v + 255) & ~static_cast<size_t>(255); };
     FwdWs w{};
     size_t map_bytes = 0;
@@ -113,15 +113,46 @@ FwdWs fwd_layout(int rows, int total_rows, int num_experts, int H, int Ie) {
     if (w.slot_bytes > (64u << 20)) w.slot_bytes = 0;
     w.off[CF_MOE_FWD_WS_SLOT] = off; off = up(off + w.slot_bytes);
     w.off[CF_MOE_FWD_WS_PRE] = off; off = up(off + sizeof(float) * T * Ie);
-    w.off[CF_MOE_FWD_WS_SPLIT] = off; off = up(off + kTerms * T * Ie);
-    w.off[CF_MOE_FWD_WS_SPLIT_DESCALE] = off; off = up(off + sizeof(float) * T);
-    w.off[CF_MOE_FWD_WS_Y] = off; off = up(off + 2 * T * H);
+    if (bf16_form) {
+        // two bf16 terms per value, no scales; the gathered token rows
+        w.off[CF_MOE_FWD_WS_SPLIT] = off; off = up(off + 2 * 2 * T * Ie);
+        w.off[CF_MOE_FWD_WS_SPLIT_DESCALE] = off;
+        w.off[CF_MOE_FWD_WS_Y] = off; off = up(off + 2 * T * H);
+        w.off[CF_MOE_FWD_WS_X] = off; off = up(off + 2 * T * H);
+    } else {
+        w.off[CF_MOE_FWD_WS_SPLIT] = off; off = up(off + kTerms * T * Ie);
+        w.off[CF_MOE_FWD_WS_SPLIT_DESCALE] = off; off = up(off + sizeof(float) * T);
+        w.off[CF_MOE_FWD_WS_Y] = off; off = up(off + 2 * T * H);
+        w.off[CF_MOE_FWD_WS_X] = off;
+    }
     w.total = off;
     return w;
 }
 
 // the shapes the pipeline takes; everything else stays with the one-kernel forms
 bool staged_shape(int H, int Ie) { return H % 128 == 0 && H >= 256 && Ie % 128 == 0 && Ie >= 128 && Ie <= 4096; }
+bool staged_shape_bf16(int H, int Ie) { return H % 8 == 0 && Ie % 64 == 0; }
+
+// GELU of the fp32 projections as two bf16 terms side by side: out[r, 0:K] = bf16(g), out[r, K:2K] = bf16(g - bf16(g)),
+// 16 significand bits between them.  K % 4 == 0.
+__global__ __launch_bounds__(kSplitThreads) void k_gelu_split2_bf16(const float* __restrict__ pre, size_t rows, int K,
+                                                                    uint16_t* __restrict__ out) {
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    const int kv = K / 4;
+    const size_t n = rows * kv;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * kSplitThreads + threadIdx.x; i < n; i += static_cast<size_t>(gridDim.x) * kSplitThreads) {
+        const size_t r = i / kv;
+        const int c = static_cast<int>(i - r * kv) * 4;
+        const f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(pre + r * K + c));
+        const float g[4] = {gelu_tail_form(v[0]), gelu_tail_form(v[1]), gelu_tail_form(v[2]), gelu_tail_form(v[3])};
+        const uint32_t h01 = pack_bf16x2_hw(g[0], g[1]), h23 = pack_bf16x2_hw(g[2], g[3]);
+        const uint32_t r01 = pack_bf16x2_hw(g[0] - bf16_lo(h01), g[1] - bf16_hi(h01));
+        const uint32_t r23 = pack_bf16x2_hw(g[2] - bf16_lo(h23), g[3] - bf16_hi(h23));
+        uint16_t* o = out + r * (2 * static_cast<size_t>(K)) + c;
+        store_stream8(o, make_uint2(h01, h23));
+        store_stream8(o + K, make_uint2(r01, r23));
+    }
+}
 
 }  // namespace
 }  // namespace cf
@@ -205,6 +236,82 @@ int cf_moe_grouped_expert_forward_fp8_ws(const void* d_hidden, const float* d_fc
     }
     rc = grouped_gemm_nt_bf16_terms(total_selected_rows, H, Ie, kTerms, num_experts, split, kTerms * Ie, split_descale, d_fc_out_w,
                                     d_fc_out_descale, y, H, tile_map, stream);
+    if (rc) return rc;
+    if (slot) return cf_moe_unpermute_indexed_bf16(d_mixed, y, d_route_weights, slot, rows, num_experts, H, 0, stream);
+    return cf_moe_unpermute_weighted_bf16(d_mixed, y, d_route_weights, d_counts, offsets, d_row_indices, rows, num_experts, H,
+                                          stream);
+}
+
+// moe_grouped_expert_forward_bf16 (kernels.hpp:400-407) with a workspace: the same pipeline on bf16 operands.  The
+// token rows are gathered, fc_in is one grouped bf16 GEMM with fp32 output, the GELU output goes to fc_out as two bf16
+// terms side by side (value = head + remainder to 2^-17) against the same weight columns, K = 2 Ie, so both terms add
+// in the fp32 accumulator.
+int cf_moe_grouped_expert_forward_bf16_workspace(int rows, int total_selected_rows, int num_experts, int H, int Ie,
+                                                 size_t* offsets, size_t* bytes) {
+    if (rows < 0 || total_selected_rows < 0 || num_experts < 0 || H < 0 || Ie < 0 || !bytes) return CF_ERR_INVALID_ARG;
+    if (!staged_shape_bf16(H, Ie)) {
+        *bytes = 0;
+        if (offsets)
+            for (int i = 0; i < CF_MOE_FWD_WS_COUNT; ++i) offsets[i] = 0;
+        return CF_OK;
+    }
+    const FwdWs w = fwd_layout(rows, total_selected_rows, num_experts, H, Ie, true);
+    *bytes = w.total;
+    if (offsets)
+        for (int i = 0; i < CF_MOE_FWD_WS_COUNT; ++i) offsets[i] = w.off[i];
+    return CF_OK;
+}
+
+int cf_moe_grouped_expert_forward_bf16_ws(const uint16_t* d_hidden, const float* d_route_weights, const int* d_counts,
+                                          const int* d_offsets, const int* d_row_indices, const uint16_t* d_fc_in_w,
+                                          const uint16_t* d_fc_out_w, uint16_t* d_mixed, int rows, int H, int Ie,
+                                          int num_experts, int total_selected_rows, void* d_workspace, size_t workspace_bytes,
+                                          cf_stream_t stream) {
+    if (rows < 0 || H < 0 || Ie < 0 || num_experts < 0 || total_selected_rows < 0) return CF_ERR_INVALID_ARG;
+    if (rows == 0 || num_experts == 0 || H == 0 || Ie == 0 || total_selected_rows == 0) return CF_OK;
+    if (!d_hidden || !d_route_weights || !d_counts || !d_row_indices || !d_fc_in_w || !d_fc_out_w || !d_mixed) return CF_ERR_INVALID_ARG;
+    const bool staged = staged_shape_bf16(H, Ie) && aligned16(d_hidden) && aligned16(d_fc_in_w) && aligned16(d_fc_out_w) &&
+                        aligned16(d_mixed) && static_cast<size_t>(total_selected_rows) * H < (1ull << 30) &&
+                        static_cast<size_t>(total_selected_rows) * 2 * Ie < (1ull << 30) && static_cast<size_t>(H) * Ie < (1ull << 30);
+    if (!staged)
+        return cf_moe_grouped_expert_forward_bf16(d_hidden, d_route_weights, d_counts, d_offsets, d_row_indices, d_fc_in_w, d_fc_out_w,
+                                                  d_mixed, rows, H, Ie, num_experts, total_selected_rows, stream);
+    const FwdWs w = fwd_layout(rows, total_selected_rows, num_experts, H, Ie, true);
+    if (!d_workspace || workspace_bytes < w.total || (reinterpret_cast<uintptr_t>(d_workspace) & 255u)) return CF_ERR_INVALID_ARG;
+    auto* base = static_cast<uint8_t*>(d_workspace);
+    int* tile_map = reinterpret_cast<int*>(base + w.off[CF_MOE_FWD_WS_TILE_MAP]);
+    int* offsets = reinterpret_cast<int*>(base + w.off[CF_MOE_FWD_WS_OFFSETS]);
+    int* index = reinterpret_cast<int*>(base + w.off[CF_MOE_FWD_WS_INDEX]);
+    int* slot = w.slot_bytes ? reinterpret_cast<int*>(base + w.off[CF_MOE_FWD_WS_SLOT]) : nullptr;
+    float* pre = reinterpret_cast<float*>(base + w.off[CF_MOE_FWD_WS_PRE]);
+    uint16_t* split = reinterpret_cast<uint16_t*>(base + w.off[CF_MOE_FWD_WS_SPLIT]);
+    uint16_t* y = reinterpret_cast<uint16_t*>(base + w.off[CF_MOE_FWD_WS_Y]);
+    uint16_t* xg = reinterpret_cast<uint16_t*>(base + w.off[CF_MOE_FWD_WS_X]);
+    hipStream_t st = as_stream(stream);
+
+    int rc = cf_moe_expert_offsets_from_counts(d_counts, offsets, num_experts, stream);
+    if (rc) return rc;
+    rc = cf_moe_compact_row_index(d_counts, offsets, d_row_indices, rows, num_experts, index, stream);
+    if (rc) return rc;
+    if (slot) {
+        rc = cf_moe_build_slot_index(d_counts, offsets, d_row_indices, rows, num_experts, slot, stream);
+        if (rc) return rc;
+    }
+    build_tile_map(d_counts, offsets, num_experts, total_selected_rows / 256 + num_experts, tile_map, st);
+    rc = launch_status();
+    if (rc) return rc;
+    rc = cf_moe_gather_rows_bf16(d_hidden, xg, index, total_selected_rows, H, stream);
+    if (rc) return rc;
+    rc = grouped_gemm_bf16_nt(total_selected_rows, Ie, H, 1, num_experts, xg, H, d_fc_in_w, pre, Ie, true, tile_map, stream);
+    if (rc) return rc;
+    {
+        const size_t n = static_cast<size_t>(total_selected_rows) * (Ie / 4);
+        const unsigned want = ceil_div(n, kSplitThreads);
+        k_gelu_split2_bf16<<<want < 16384u ? want : 16384u, kSplitThreads, 0, st>>>(pre, static_cast<size_t>(total_selected_rows), Ie, split);
+        rc = launch_status();
+        if (rc) return rc;
+    }
+    rc = grouped_gemm_bf16_nt(total_selected_rows, H, Ie, 2, num_experts, split, 2 * Ie, d_fc_out_w, y, H, false, tile_map, stream);
     if (rc) return rc;
     if (slot) return cf_moe_unpermute_indexed_bf16(d_mixed, y, d_route_weights, slot, rows, num_experts, H, 0, stream);
     return cf_moe_unpermute_weighted_bf16(d_mixed, y, d_route_weights, d_counts, offsets, d_row_indices, rows, num_experts, H,

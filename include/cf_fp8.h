@@ -570,10 +570,10 @@ int cf_moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_fcin_
  * d_workspace 256-byte aligned; cf_moe_grouped_expert_forward_fp8_workspace gives its size and, when
  * `offsets` is not null, the byte offsets of the intermediates (CF_MOE_FWD_WS_* order), which stay valid
  * after the call: pre [total, Ie] fp32, split [total, 3 Ie] E4M3, split_descale [total] fp32, y [total, H] bf16,
- * experts back to back. */
+ * experts back to back (CF_MOE_FWD_WS_X is used by the bf16 form only). */
 enum {
     CF_MOE_FWD_WS_TILE_MAP = 0, CF_MOE_FWD_WS_OFFSETS, CF_MOE_FWD_WS_INDEX, CF_MOE_FWD_WS_SLOT, CF_MOE_FWD_WS_PRE,
-    CF_MOE_FWD_WS_SPLIT, CF_MOE_FWD_WS_SPLIT_DESCALE, CF_MOE_FWD_WS_Y, CF_MOE_FWD_WS_COUNT
+    CF_MOE_FWD_WS_SPLIT, CF_MOE_FWD_WS_SPLIT_DESCALE, CF_MOE_FWD_WS_Y, CF_MOE_FWD_WS_X, CF_MOE_FWD_WS_COUNT
 };
 int cf_moe_grouped_expert_forward_fp8_workspace(int rows, int total_selected_rows, int num_experts, int H,
                                                 int Ie, size_t* offsets, size_t* bytes);
@@ -585,6 +585,23 @@ int cf_moe_grouped_expert_forward_fp8_ws(const void* d_hidden, const float* d_fc
                                          const float* d_fc_out_descale, uint16_t* d_mixed, int rows,
                                          int H, int Ie, int num_experts, int total_selected_rows,
                                          void* d_workspace, size_t workspace_bytes, cf_stream_t stream);
+
+/* moe_grouped_expert_forward_bf16 (kernels.hpp:400-407) with a workspace: the same arguments and contract as
+ * cf_moe_grouped_expert_forward_bf16, run as whole-matrix launches when H % 8 == 0, Ie % 64 == 0 and the
+ * operands are 16-byte aligned (other shapes are passed on to that function).  The selected token rows are
+ * gathered (x, CF_MOE_FWD_WS_X), fc_in is one grouped bf16 GEMM with fp32 output (pre), the GELU (fp32, erf to
+ * 1.5e-7 absolute) is written as two bf16 terms side by side (split [total, 2 Ie]: bf16(g) and bf16(g - bf16(g)),
+ * 16 significand bits), fc_out is one grouped bf16 GEMM over K = 2 Ie against the same weight columns, bf16
+ * out (y), then the ordered add into d_mixed as in cf_moe_grouped_expert_forward_fp8_ws, with the same two
+ * differences from the reference kernel.  Workspace rules as there; CF_MOE_FWD_WS_SPLIT_DESCALE is unused. */
+int cf_moe_grouped_expert_forward_bf16_workspace(int rows, int total_selected_rows, int num_experts, int H,
+                                                 int Ie, size_t* offsets, size_t* bytes);
+int cf_moe_grouped_expert_forward_bf16_ws(const uint16_t* d_hidden, const float* d_route_weights,
+                                          const int* d_counts, const int* d_offsets,
+                                          const int* d_row_indices, const uint16_t* d_fc_in_w,
+                                          const uint16_t* d_fc_out_w, uint16_t* d_mixed, int rows, int H,
+                                          int Ie, int num_experts, int total_selected_rows,
+                                          void* d_workspace, size_t workspace_bytes, cf_stream_t stream);
 
 /* moe_grouped_expert_forward_bf16, kernels.hpp:400-407: the same device-scheduled expert bank on
  * bf16 hidden states and bf16 weights (fc_in_w [E,Ie,H], fc_out_w [E,H,Ie]), no descales; fp32

@@ -201,6 +201,21 @@ inline void moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_
                                              d_row_indices, d_fc_in_w, d_fc_in_descale, d_fc_out_w, d_fc_out_descale,
                                              hip_detail::u(d_mixed), rows, H, Ie, num_experts, total_selected_rows, stream));
 }
+// The bf16 bank with a workspace slice: both projections as whole-matrix grouped bf16 GEMMs where the shape allows.
+inline size_t moe_grouped_expert_forward_bf16_workspace_bytes(int rows, int H, int Ie, int num_experts, int total_selected_rows) {
+    size_t bytes = 0;
+    CF_FWD(cf_moe_grouped_expert_forward_bf16_workspace(rows, total_selected_rows, num_experts, H, Ie, nullptr, &bytes));
+    return bytes;
+}
+inline void moe_grouped_expert_forward_bf16(const bf16* d_hidden, const float* d_route_weights, const int* d_counts,
+                                            const int* d_offsets, const int* d_row_indices, const bf16* d_fc_in_w,
+                                            const bf16* d_fc_out_w, bf16* d_mixed, int rows, int H, int Ie, int num_experts,
+                                            int total_selected_rows, void* d_workspace, size_t workspace_bytes,
+                                            hipStream_t stream) {
+    CF_FWD(cf_moe_grouped_expert_forward_bf16_ws(hip_detail::u(d_hidden), d_route_weights, d_counts, d_offsets, d_row_indices,
+                                                 hip_detail::u(d_fc_in_w), hip_detail::u(d_fc_out_w), hip_detail::u(d_mixed), rows,
+                                                 H, Ie, num_experts, total_selected_rows, d_workspace, workspace_bytes, stream));
+}
 // The same call with a workspace slice (the trainer's arena can supply one): both projections then run as whole-matrix
 // FP8 GEMMs where the shape allows.  moe_grouped_expert_forward_fp8_workspace_bytes gives the size (0: not needed).
 inline size_t moe_grouped_expert_forward_fp8_workspace_bytes(int rows, int H, int Ie, int num_experts, int total_selected_rows) {

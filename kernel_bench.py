@@ -76,6 +76,15 @@ def main():
         gbps = nbytes / t / 1e9
         print(f"{name:<64} {shape:<26} {t * 1e6:9.1f} {gbps:9.0f} GB/s {100 * gbps / HBM_PEAK:7.1f}%", flush=True)
 
+    BF16_PEAK = 2500.0          # dense bf16 matrix peak, TFLOP/s
+
+    def mfma16(name, shape, flop, fn):
+        if args.only not in name:
+            return
+        t = timed(fn)
+        tf = flop / t / 1e12
+        print(f"{name:<64} {shape:<26} {t * 1e6:9.1f} {tf:7.0f} TFLOP/s {100 * tf / BF16_PEAK:7.1f}% (of bf16 peak)", flush=True)
+
     def mfma(name, shape, flop, fn):
         if args.only not in name:
             fn()                         # later rows use what this one leaves behind
@@ -295,6 +304,14 @@ def main():
     mfma("moe_grouped_expert_forward_fp8 form (fp32 GELU kept, MFMA)", f"T={T} E={E} k={k}", 4.0 * total * Ie * H,
          lambda: cf.cf_moe_grouped_expert_forward_fp8(hq, one, 0, rw, counts, offs, idx, wg, one, wd, one, mixed, T, H, Ie, E, total, st))
     hb16 = bf16(T, H); wi16 = bf16(E * Ie, H, sigma=0.02); wo16 = bf16(E * H, Ie, sigma=0.02)
+    sz5 = ctypes.c_size_t(0)
+    cf.raw_cf_moe_grouped_expert_forward_bf16_workspace(T, total, E, H, Ie, None, ctypes.byref(sz5))
+    ws5 = u8(sz5.value)
+    mfma16("moe_grouped_expert_forward_bf16 with a workspace (grouped bf16 GEMMs, two-term GELU)", f"T={T} E={E} k={k}",
+           4.0 * total * Ie * H,
+           lambda: cf.cf_moe_grouped_expert_forward_bf16_ws(hb16, rw, counts, None, idx, wi16, wo16, mixed, T, H, Ie, E, total,
+                                                            ws5, sz5.value, st))
+    del ws5
     mfma("moe_grouped_expert_forward_bf16 (the bf16 sibling, MFMA)", f"T={T} E={E} k={k}", 4.0 * total * Ie * H,
          lambda: cf.cf_moe_grouped_expert_forward_bf16(hb16, rw, counts, offs, idx, wi16, wo16, mixed, T, H, Ie, E, total, st))
     args.iters = iters
@@ -328,14 +345,6 @@ def main():
     hbm("gelu_backward_bf16", f"{total}x{Ie}", 6.0 * total * Ie, lambda: cf.cf_gelu_backward_bf16(pre, gpost, gpre, total * Ie, st))
 
     # the four bf16 GEMMs of the same backward, every expert in one launch (bf16 matrix peak 2.5 PFLOP/s)
-    BF16_PEAK = 2500.0
-
-    def mfma16(name, shape, flop, fn):
-        if args.only not in name:
-            return
-        t = timed(fn)
-        tf = flop / t / 1e12
-        print(f"{name:<64} {shape:<26} {t * 1e6:9.1f} {tf:7.0f} TFLOP/s {100 * tf / BF16_PEAK:7.1f}% (of bf16 peak)", flush=True)
     wo16 = bf16(E * H, Ie, sigma=0.02); wi16 = bf16(E * Ie, H, sigma=0.02)
     d_out = bf16(total, H, sigma=0.01); xg = bf16(total, H)
     d_act = torch.empty((total, Ie), dtype=torch.bfloat16, device=dev); d_x = torch.empty((total, H), dtype=torch.bfloat16, device=dev)

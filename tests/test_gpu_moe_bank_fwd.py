@@ -1,5 +1,5 @@
 """GPU parity: moe_grouped_expert_forward_fp8 (/root/reference/kernels/moe.cu:950-1127) as whole-matrix launches with
-a workspace (cf_moe_grouped_expert_forward_fp8_ws).
+a workspace (cf_moe_grouped_expert_forward_fp8_ws), and its bf16 sibling (cf_moe_grouped_expert_forward_bf16_ws).
 
 Every stage is checked on the intermediates the call leaves in its workspace, given that stage's own (GPU) inputs:
 the fp32 projections against the double product of the dequantized operands; the three-term E4M3 split of the GELU
@@ -18,7 +18,8 @@ from gpu_util import bf16_bits, case, dev_arr, dev_bf16, host, stream
 
 pytestmark = pytest.mark.gpu
 
-NAMES = ["TILE_MAP", "OFFSETS", "INDEX", "SLOT", "PRE", "SPLIT", "SPLIT_DESCALE", "Y"]
+NAMES = ["TILE_MAP", "OFFSETS", "INDEX", "SLOT", "PRE", "SPLIT", "SPLIT_DESCALE", "Y", "X"]
+ACC_BF16 = 16.0 * 2.0 ** -24          # fp32 accumulation of bf16 products on the matrix cores, per sum |a_k b_k|
 erf = np.vectorize(math.erf, otypes=[np.float64])
 
 
@@ -203,3 +204,110 @@ def test_staged_bank_rejects_a_short_workspace(cf, dev):
     assert cf.raw_cf_moe_grouped_expert_forward_fp8_ws(*[cf_conv(a) for a in args(None, nbytes)]) == -1
     torch.cuda.synchronize()
     assert np.array_equal(bf16_bits(mixed), b.mixed0)
+
+
+# ---- the bf16 sibling --------------------------------------------------------------------------------------------
+
+class Bank16:
+    def __init__(self, dev, rows, E, k, H, Ie, seed, zero_expert=None):
+        rng = np.random.default_rng(seed)
+        self.rows, self.E, self.k, self.H, self.Ie, self.dev = rows, E, k, H, Ie, dev
+        self.hidden = orc.bf16_from_f32(rng.standard_normal((rows, H)).astype(np.float32))
+        self.win = orc.bf16_from_f32((0.05 * rng.standard_normal((E, Ie, H))).astype(np.float32))
+        self.wout = orc.bf16_from_f32((0.05 * rng.standard_normal((E, H, Ie))).astype(np.float32))
+        logits = rng.standard_normal((rows, E)).astype(np.float32)
+        if zero_expert is not None:
+            logits[:, zero_expert] = -50.0
+        self.rw = orc.moe_topk_route(logits, k)
+        self.counts, self.idx = orc.moe_build_expert_row_lists(self.rw)
+        self.total = int(self.counts.sum())
+        self.mixed0 = orc.bf16_from_f32(rng.standard_normal((rows, H)).astype(np.float32))
+
+
+def run16(cf, b):
+    dev = b.dev
+    offs = (ctypes.c_size_t * len(NAMES))()
+    nbytes = ctypes.c_size_t()
+    cf.cf_moe_grouped_expert_forward_bf16_workspace(b.rows, b.total, b.E, b.H, b.Ie, offs, ctypes.byref(nbytes))
+    off, nbytes = {n: int(offs[i]) for i, n in enumerate(NAMES)}, int(nbytes.value)
+    ws = torch.empty(max(nbytes, 256) + 256, dtype=torch.uint8, device=dev)
+    ws.fill_(0xCD)
+    shift = (-ws.data_ptr()) % 256
+    ws = ws[shift:shift + max(nbytes, 256)]
+    mixed = dev_bf16(b.mixed0, dev)
+    cf.cf_moe_grouped_expert_forward_bf16_ws(dev_bf16(b.hidden, dev), dev_arr(b.rw, dev), dev_arr(b.counts, dev), None, dev_arr(b.idx, dev),
+                                             dev_bf16(b.win, dev), dev_bf16(b.wout, dev), mixed, b.rows, b.H, b.Ie, b.E, b.total,
+                                             ws if nbytes else None, nbytes, stream())
+    torch.cuda.synchronize()
+    return mixed, ws, off, nbytes
+
+
+def check_result16(b, mixed):
+    start = orc.bf16_to_f32(b.mixed0).astype(np.float64)
+    ref = orc.moe_grouped_expert_forward_bf16_ref(b.hidden, b.rw, b.counts, b.idx, b.win, b.wout, start)
+    got = orc.bf16_to_f32(bf16_bits(mixed)).astype(np.float64)
+    assert np.sqrt(((got - ref) ** 2).sum() / (ref ** 2).sum()) <= 4e-3
+    typical = np.sqrt(((ref - start) ** 2).mean())
+    assert np.all(np.abs(got - ref) <= (2 * b.k + 1) * 2.0 ** -8 * (np.abs(start) + np.abs(ref) + 2.0 * typical))
+    untouched = ~(b.rw > 0).any(axis=1)
+    assert np.array_equal(bf16_bits(mixed)[untouched], b.mixed0[untouched])
+
+
+@pytest.mark.parametrize("rows,E,k,H,Ie,zero", [
+    (70, 3, 3, 2048, 1408, None),        # config 5's widths
+    (300, 6, 3, 256, 320, None),         # Ie = 5 K-tiles: the second term starts at an odd K-tile
+    (200, 4, 2, 64, 64, None),           # one K-tile per term and per projection
+    (1000, 5, 2, 192, 448, 2),           # several row tiles per expert, ragged, an expert with no rows; N = 448 and 192 end inside a column tile
+    (21, 5, 2, 200, 128, None),          # H % 64 != 0: the k range of fc_in ends inside a K-tile
+])
+def test_staged_bf16_bank_stage_by_stage(cf, dev, rows, E, k, H, Ie, zero):
+    case(f"staged bf16 gelu bank rows={rows} E={E} k={k} H={H} Ie={Ie} zero_expert={zero}")
+    b = Bank16(dev, rows, E, k, H, Ie, seed=rows + Ie + 1, zero_expert=zero)
+    mixed, ws, off, nbytes = run16(cf, b)
+    assert nbytes > 0
+    T = b.total
+    raw = host(ws)
+    take = lambda name, dtype, count: raw[off[name]: off[name] + count * np.dtype(dtype).itemsize].view(dtype)
+    index = take("INDEX", np.int32, T)
+    assert np.array_equal(index, np.concatenate([b.idx[e, : b.counts[e]] for e in range(E)]))
+    expert = np.repeat(np.arange(E), b.counts)
+    assert np.array_equal(take("X", np.uint16, T * H).reshape(T, H), b.hidden[index]), "gathered token rows"
+
+    hx = orc.bf16_to_f32(b.hidden).astype(np.float64)
+    win = orc.bf16_to_f32(b.win).astype(np.float64)
+    wout = orc.bf16_to_f32(b.wout).astype(np.float64)
+    pre = take("PRE", np.float32, T * Ie).reshape(T, Ie).astype(np.float64)
+    for e in range(E):
+        sel = expert == e
+        if not sel.any():
+            continue
+        want = hx[index[sel]] @ win[e].T
+        ad = np.abs(hx[index[sel]]) @ np.abs(win[e]).T
+        assert np.all(np.abs(pre[sel] - want) <= 2.0 ** -22 * np.abs(want) + ACC_BF16 * ad), f"fc_in expert {e}"
+
+    split = orc.bf16_to_f32(take("SPLIT", np.uint16, T * 2 * Ie).reshape(T, 2, Ie)).astype(np.float64)
+    act = split[:, 0] + split[:, 1]
+    g = gelu64(pre)
+    tol = 2.0 ** -16 * np.abs(g) + 4e-7 * (np.abs(pre) + 1e-3)
+    assert (np.abs(act - g) / tol).max() <= 1.0, "two bf16 terms carry the GELU to 16 bits"
+    assert np.all(np.abs(split[:, 1]) <= 2.0 ** -8 * np.abs(split[:, 0]) + 1e-30), "the second term is the first one's rounding error"
+
+    y = orc.bf16_to_f32(take("Y", np.uint16, T * H).reshape(T, H)).astype(np.float64)
+    for e in range(E):
+        sel = expert == e
+        if not sel.any():
+            continue
+        want = act[sel] @ wout[e].T
+        ad = (np.abs(split[sel, 0]) + np.abs(split[sel, 1])) @ np.abs(wout[e]).T
+        tol = 0.505 * orc.bf16_ulp(np.maximum(np.abs(want), np.abs(y[sel]))) + ACC_BF16 * ad
+        worst = np.abs(y[sel] - want) / tol
+        assert worst.max() <= 1.0, f"fc_out expert {e}: worst {worst.max():.3f}"
+    check_result16(b, mixed)
+
+
+def test_staged_bf16_bank_other_shapes_pass_through(cf, dev):
+    case("staged bf16 gelu bank entry on a shape of the one-kernel forms")
+    b = Bank16(dev, 50, 3, 2, 64, 40, seed=2)
+    mixed, _, _, nbytes = run16(cf, b)
+    assert nbytes == 0
+    check_result16(b, mixed)

@@ -9,6 +9,7 @@
 #include "common.hpp"
 
 #include <mutex>
+#include <type_traits>
 
 namespace cf {
 namespace {
@@ -127,29 +128,53 @@ __global__ __launch_bounds__(kThreads) void k_topk_wave(float* __restrict__ scor
     if (live) s[lane] = kept ? v * inv_sum : 0.0f;
 }
 
-// ---- top-k, any E up to 2048: one lane per row ----------------------------------
+// ---- top-k, 64 < E <= 2048: one wavefront per row, lane l holds experts l, l + 64, ... ----------
+// A pick is the largest remaining score, the lowest expert among equals; scores must beat -1 strictly (NaN never
+// does).  Each lane scans its own experts in ascending order, the wavefront agrees on the largest value and then on
+// the lowest expert that holds it.  The kept sum runs in ascending expert order, one fp32 add per kept expert.
 constexpr int kMaxExpertsGeneric = 2048;
-__global__ __launch_bounds__(128) void k_topk_generic(float* __restrict__ scores, float* __restrict__ row_sum_save,
-                                                      int rows, int E, int top_k, int normalize) {
-    const int row = blockIdx.x * blockDim.x + threadIdx.x;
+__global__ __launch_bounds__(kThreads) void k_topk_wide(float* __restrict__ scores, float* __restrict__ row_sum_save,
+                                                        int rows, int E, int top_k, int normalize) {
+    constexpr int J = kMaxExpertsGeneric / 64;
+    const int row = blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
     if (row >= rows) return;
+    const int lane = threadIdx.x & 63;
     float* s = scores + static_cast<size_t>(row) * E;
-    uint32_t kept[kMaxExpertsGeneric / 32];
-    for (int w = 0; w < (E + 31) / 32; ++w) kept[w] = 0u;
+    float v[J];
+#pragma unroll
+    for (int j = 0; j < J; ++j) v[j] = j * 64 + lane < E ? s[j * 64 + lane] : -2.0f;
+    uint32_t kept = 0u;            // bit j: expert j * 64 + lane is kept
     const int k = min(top_k, E);
     for (int pick = 0; pick < k; ++pick) {
-        int best = -1;
-        float best_v = -1.0f;
-        for (int e = 0; e < E; ++e)
-            if (!((kept[e >> 5] >> (e & 31)) & 1u) && s[e] > best_v) { best_v = s[e]; best = e; }
-        if (best < 0) break;
-        kept[best >> 5] |= 1u << (best & 31);
+        float best = -1.0f;
+        int bj = -1;
+#pragma unroll
+        for (int j = 0; j < J; ++j)
+            if (!((kept >> j) & 1u) && v[j] > best) { best = v[j]; bj = j; }
+        float top = best;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) top = fmaxf(top, __shfl_xor(top, off, kWave));
+        int who = (bj >= 0 && best == top) ? bj * 64 + lane : 0x7fffffff;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) who = min(who, __shfl_xor(who, off, kWave));
+        if (who == 0x7fffffff) break;                      // nothing left that beats -1
+        if ((who & 63) == lane) kept |= 1u << (who >> 6);
     }
     float sum = 0.0f;
-    for (int e = 0; e < E; ++e) if ((kept[e >> 5] >> (e & 31)) & 1u) sum += s[e];
-    if (row_sum_save) row_sum_save[row] = sum;
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+        unsigned long long mask = j * 64 < E ? __ballot((kept >> j) & 1u) : 0ull;
+        while (mask) {
+            const int l = __builtin_ctzll(mask);
+            mask &= mask - 1;
+            sum += __shfl(v[j], l, kWave);
+        }
+    }
+    if (row_sum_save && lane == 0) row_sum_save[row] = sum;
     const float inv_sum = (normalize && sum > 0.0f) ? (1.0f / sum) : 1.0f;
-    for (int e = 0; e < E; ++e) s[e] = ((kept[e >> 5] >> (e & 31)) & 1u) ? s[e] * inv_sum : 0.0f;
+#pragma unroll
+    for (int j = 0; j < J; ++j)
+        if (j * 64 + lane < E) s[j * 64 + lane] = ((kept >> j) & 1u) ? v[j] * inv_sum : 0.0f;
 }
 
 // ---- per-expert row lists ----------------------------------------------------------
@@ -442,16 +467,6 @@ __global__ __launch_bounds__(kThreads) void k_unpermute(uint16_t* __restrict__ m
     }
 }
 
-// ---- grouped GELU expert bank, reference semantics ------------------------------------------
-// mixed[row] += w * fc_out(gelu(fc_in(hidden[row]))) for every selected (expert,row): operands are
-// dequantised with per-tensor descales, the exact-erf GELU output stays in fp32 (it is not
-// re-quantised), products are accumulated in fp32, and the result is added to the bf16 output with a
-// 32-bit compare-and-swap on the word holding it.  One workgroup per (expert, tile of 16 rows);
-// workgroups past an expert's row count leave at once.  This fp32-FMA form follows the reference
-// kernel's loop and takes any shape; shapes made of whole MFMA steps go to k_grouped_gelu_fp8_mfma below.
-constexpr int kGeluRows = 16;
-constexpr int kGeluChunk = 128;
-
 __device__ __forceinline__ void atomic_add_bf16(uint16_t* addr, float v) {
     const uintptr_t a = reinterpret_cast<uintptr_t>(addr);
     auto* word = reinterpret_cast<unsigned int*>(a & ~static_cast<uintptr_t>(3));
@@ -466,88 +481,138 @@ __device__ __forceinline__ void atomic_add_bf16(uint16_t* addr, float v) {
     }
 }
 
-// BF16: the reference's bf16 sibling (moe_grouped_expert_forward_bf16, same scheduling): hidden and weights are bf16
-// (the byte pointers then address 2-byte elements), no descales.
-template <bool BF16>
-__global__ __launch_bounds__(kThreads) void k_grouped_gelu_fp8(const uint8_t* __restrict__ hidden, const float* __restrict__ fcin_descale,
-                                                               int fcin_is_e5m2, const float* __restrict__ route_weights,
-                                                               const int* __restrict__ counts, const int* __restrict__ row_indices,
-                                                               const uint8_t* __restrict__ fc_in_w, const float* __restrict__ fc_in_descale,
-                                                               const uint8_t* __restrict__ fc_out_w, const float* __restrict__ fc_out_descale,
-                                                               uint16_t* __restrict__ mixed, int rows, int H, int Ie, int E,
-                                                               int tiles_per_expert) {
+// ---- grouped GELU expert bank, reference semantics, any shape --------------------------------
+// mixed[row] += w * fc_out(gelu(fc_in(hidden[row]))) for every selected (expert,row): per-tensor descales, the
+// exact-erf GELU output stays in fp32 (it is not re-quantised), products are accumulated in fp32, and the result is
+// added to the bf16 output with a 32-bit compare-and-swap on the word holding it.  Shapes made of whole MFMA steps
+// go to the matrix-core kernels below; this one takes everything else, with no alignment demands.
+//
+// One workgroup per (expert, R token rows); workgroups past an expert's row count leave at once.  The R hidden rows
+// sit in LDS as fp32.  A projection is wave-parallel dot products: a wavefront takes C = 32 / R output columns at a
+// time, lane l walks k = l, l + 64, ... (a weight row is contiguous in k, so the 64 lanes read 64 neighbouring
+// elements of each of the C rows; the activations of the R rows come from LDS, one bank per lane), which leaves
+// every lane with 32 partial sums; fold_values adds them over the 64 lanes in 32 exchanges instead of 32 x 6.
+// The descales multiply the finished sums.  BF16: the bf16 sibling (moe_grouped_expert_forward_bf16): hidden and
+// weights are bf16 (the byte pointers then address 2-byte elements), no descales.
+
+// The sums of 32 per-lane values over the 64 lanes: each of five halving steps hands the half of the values this
+// lane gives up to the lane across (xor 32, 16, 8, 4, 2) and adds what comes back to the half it keeps; one plain
+// step (xor 1) finishes.  Value i ends in v[0] of lanes 2 i and 2 i + 1.
+template <int N>
+__device__ __forceinline__ void fold_values(float (&v)[32], int lane) {
+    if constexpr (N > 1) {
+        constexpr int half = N / 2;
+        const bool upper = (lane & N) != 0;
+#pragma unroll
+        for (int i = 0; i < half; ++i) {
+            const float send = upper ? v[i] : v[i + half];
+            const float keep = upper ? v[i + half] : v[i];
+            v[i] = keep + __shfl_xor(send, N, kWave);
+        }
+        fold_values<half>(v, lane);
+    } else {
+        v[0] += __shfl_xor(v[0], 1, kWave);
+    }
+}
+
+// out(r, n, sum_k x[r][k] w[n][k]) for r < R and every n < N, called by one lane per (r, n); x in LDS [R][K]
+template <int R, class Elem, class Out>
+__device__ __forceinline__ void project_rows(const float* x, int K, int N, Elem&& weight, Out&& out) {
+    constexpr int C = 32 / R;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int n0 = wave * C; n0 < N; n0 += (kThreads / 64) * C) {
+        float v[32];
+#pragma unroll
+        for (int i = 0; i < 32; ++i) v[i] = 0.0f;
+        size_t wrow[C];
+#pragma unroll
+        for (int c = 0; c < C; ++c) wrow[c] = static_cast<size_t>(min(n0 + c, N - 1)) * K;
+        for (int k = lane; k < K; k += 64) {
+            float xv[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r) xv[r] = x[r * K + k];
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                const float wv = weight(wrow[c] + k);
+#pragma unroll
+                for (int r = 0; r < R; ++r) v[r * C + c] = __builtin_fmaf(xv[r], wv, v[r * C + c]);
+            }
+        }
+        fold_values<32>(v, lane);
+        const int idx = lane >> 1, r = idx / C, c = idx % C;
+        if ((lane & 1) == 0 && n0 + c < N) out(r, n0 + c, v[0]);
+    }
+}
+
+template <bool BF16, int R>
+__global__ __launch_bounds__(kThreads) void k_grouped_gelu_wave(const uint8_t* __restrict__ hidden, const float* __restrict__ fcin_descale,
+                                                                int fcin_is_e5m2, const float* __restrict__ route_weights,
+                                                                const int* __restrict__ counts, const int* __restrict__ row_indices,
+                                                                const uint8_t* __restrict__ fc_in_w, const float* __restrict__ fc_in_descale,
+                                                                const uint8_t* __restrict__ fc_out_w, const float* __restrict__ fc_out_descale,
+                                                                uint16_t* __restrict__ mixed, int rows, int H, int Ie, int E,
+                                                                int tiles_per_expert) {
     extern __shared__ float sh[];
-    float* sh_chunk = sh;                                  // [kGeluRows][kGeluChunk]
-    float* sh_act = sh + kGeluRows * kGeluChunk;           // [kGeluRows][Ie]
+    float* xs = sh;                        // [R][H]: the tile's hidden rows, decoded, not yet descaled
+    float* act = sh + R * H;               // [R][Ie]: GELU output
     const int e = blockIdx.x / tiles_per_expert, tile = blockIdx.x % tiles_per_expert;
-    const int first = tile * kGeluRows, n_active = counts[e];
+    const int first = tile * R, n_active = counts[e];
     if (first >= n_active) return;
-    const int n_rows = min(kGeluRows, n_active - first);
+    const int n_rows = min(R, n_active - first);
     const int* my_rows = row_indices + static_cast<size_t>(e) * rows + first;
-    const float d_in = BF16 ? 1.0f : *fcin_descale, d_win = BF16 ? 1.0f : *fc_in_descale, d_wout = BF16 ? 1.0f : *fc_out_descale;
     constexpr int kElem = BF16 ? 2 : 1;
     const uint8_t* w_in = fc_in_w + static_cast<size_t>(e) * H * Ie * kElem;
     const uint8_t* w_out = fc_out_w + static_cast<size_t>(e) * Ie * H * kElem;
-    auto hidden_at = [&](size_t i) {
-        if constexpr (BF16) return bf16_to_f32(reinterpret_cast<const uint16_t*>(hidden)[i]);
-        else return (fcin_is_e5m2 ? e5m2_to_f32(hidden[i]) : e4m3_to_f32(hidden[i])) * d_in;
+    const float s_in = BF16 ? 1.0f : *fcin_descale * *fc_in_descale, s_out = BF16 ? 1.0f : *fc_out_descale;
+    auto element = [](const uint8_t* p, size_t i, bool e5m2) {
+        if constexpr (BF16) return bf16_to_f32(reinterpret_cast<const uint16_t*>(p)[i]);
+        else return e5m2 ? e5m2_to_f32(p[i]) : e4m3_to_f32(p[i]);
     };
-    auto weight_at = [&](const uint8_t* w, size_t i, float d) {
-        if constexpr (BF16) return bf16_to_f32(reinterpret_cast<const uint16_t*>(w)[i]);
-        else return e4m3_to_f32(w[i]) * d;
-    };
-
-    // fc_in: 256 output columns per pass, K in chunks of 128 staged (dequantised) through LDS
-    for (int j0 = 0; j0 < Ie; j0 += kThreads) {
-        const int j = j0 + threadIdx.x;
-        float accum[kGeluRows];
-#pragma unroll
-        for (int r = 0; r < kGeluRows; ++r) accum[r] = 0.0f;
-        for (int k0 = 0; k0 < H; k0 += kGeluChunk) {
-            const int kt = min(kGeluChunk, H - k0);
-            __syncthreads();
-            for (int i = threadIdx.x; i < n_rows * kt; i += kThreads) {
-                const int r = i / kt, k = i % kt;
-                sh_chunk[r * kGeluChunk + k] = hidden_at(static_cast<size_t>(my_rows[r]) * H + k0 + k);
-            }
-            __syncthreads();
-            if (j < Ie) {
-                const size_t wr = static_cast<size_t>(j) * H + k0;
-                for (int k = 0; k < kt; ++k) {
-                    const float wv = weight_at(w_in, wr + k, d_win);
-#pragma unroll
-                    for (int r = 0; r < kGeluRows; ++r) accum[r] = __builtin_fmaf(sh_chunk[r * kGeluChunk + k], wv, accum[r]);
-                }
-            }
-        }
-        if (j < Ie) {
-#pragma unroll
-            for (int r = 0; r < kGeluRows; ++r) {
-                const float v = accum[r];
-                sh_act[r * Ie + j] = 0.5f * v * (1.0f + erff(v * 0.7071067811865476f));
-            }
-        }
+    for (int i = threadIdx.x; i < R * H; i += kThreads) {
+        const int r = i / H, k = i - r * H;
+        xs[i] = r < n_rows ? element(hidden, static_cast<size_t>(my_rows[r]) * H + k, fcin_is_e5m2 != 0) : 0.0f;
     }
     __syncthreads();
-    // fc_out: activations are resident in LDS
-    for (int h0 = 0; h0 < H; h0 += kThreads) {
-        const int h = h0 + threadIdx.x;
-        if (h >= H) continue;
-        float accum[kGeluRows];
-#pragma unroll
-        for (int r = 0; r < kGeluRows; ++r) accum[r] = 0.0f;
-        const size_t wr = static_cast<size_t>(h) * Ie;
-        for (int k = 0; k < Ie; ++k) {
-            const float wv = weight_at(w_out, wr + k, d_wout);
-#pragma unroll
-            for (int r = 0; r < kGeluRows; ++r) accum[r] = __builtin_fmaf(sh_act[r * Ie + k], wv, accum[r]);
-        }
-        for (int r = 0; r < n_rows; ++r) {
-            const int row = my_rows[r];
-            const float rw = route_weights[static_cast<size_t>(row) * E + e];
-            atomic_add_bf16(mixed + static_cast<size_t>(row) * H + h, rw * accum[r]);
-        }
-    }
+    project_rows<R>(xs, H, Ie, [&](size_t i) { return element(w_in, i, false); },
+                    [&](int r, int j, float sum) { act[r * Ie + j] = gelu_fwd(sum * s_in); });
+    __syncthreads();
+    project_rows<R>(act, Ie, H, [&](size_t i) { return element(w_out, i, false); },
+                    [&](int r, int h, float sum) {
+                        if (r >= n_rows) return;
+                        const int row = my_rows[r];
+                        atomic_add_bf16(mixed + static_cast<size_t>(row) * H + h, route_weights[static_cast<size_t>(row) * E + e] * (sum * s_out));
+                    });
+}
+
+// R token rows per workgroup: the most (of 8, 4, 2, 1) whose fp32 hidden rows and GELU rows fit the LDS
+template <bool BF16>
+int launch_grouped_gelu_wave(const uint8_t* hidden, const float* fcin_descale, int fcin_is_e5m2, const float* route_weights,
+                             const int* counts, const int* row_indices, const uint8_t* fc_in_w, const float* fc_in_descale,
+                             const uint8_t* fc_out_w, const float* fc_out_descale, uint16_t* mixed, int rows, int H, int Ie, int E,
+                             hipStream_t st) {
+    const size_t per_row = sizeof(float) * (static_cast<size_t>(H) + Ie);
+    auto go = [&](auto rc) {
+        constexpr int R = decltype(rc)::value;
+        static std::once_flag once;
+        static hipError_t attr_err = hipSuccess;
+        std::call_once(once, [] {
+            attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_grouped_gelu_wave<BF16, R>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        });
+        if (attr_err != hipSuccess) return static_cast<int>(attr_err);
+        const int tiles_per_expert = (rows + R - 1) / R;
+        if (static_cast<long long>(E) * tiles_per_expert >= (1LL << 31)) return static_cast<int>(CF_ERR_UNSUPPORTED);
+        k_grouped_gelu_wave<BF16, R><<<E * tiles_per_expert, kThreads, R * per_row, st>>>(
+            hidden, fcin_descale, fcin_is_e5m2, route_weights, counts, row_indices, fc_in_w, fc_in_descale, fc_out_w, fc_out_descale,
+            mixed, rows, H, Ie, E, tiles_per_expert);
+        return launch_status();
+    };
+    constexpr size_t kLdsBytes = 160 * 1024;
+    if (8 * per_row <= kLdsBytes) return go(std::integral_constant<int, 8>{});
+    if (4 * per_row <= kLdsBytes) return go(std::integral_constant<int, 4>{});
+    if (2 * per_row <= kLdsBytes) return go(std::integral_constant<int, 2>{});
+    if (per_row <= kLdsBytes) return go(std::integral_constant<int, 1>{});
+    return static_cast<int>(CF_ERR_UNSUPPORTED);
 }
 
 // ---- the same bank on the matrix cores -----------------------------------------------------------
@@ -1137,7 +1202,7 @@ int cf_moe_topk_route_f32(float* d_scores, int rows, int num_experts, int top_k,
                                             hipMemcpyDeviceToDevice, st);
         if (e != hipSuccess) return static_cast<int>(e);
     }
-    k_topk_generic<<<ceil_div(rows, 128), 128, 0, st>>>(d_scores, d_row_sum_save, rows, num_experts, top_k, normalize_topk);
+    k_topk_wide<<<ceil_div(rows, kThreads / 64), kThreads, 0, st>>>(d_scores, d_row_sum_save, rows, num_experts, top_k, normalize_topk);
     return launch_status();
 }
 
@@ -1531,21 +1596,10 @@ int cf_moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_fcin_
         else launch(k_grouped_gelu_fp8_mfma<false>);
         return launch_status();
     }
-    const size_t smem = sizeof(float) * static_cast<size_t>(kGeluRows) * (kGeluChunk + Ie);
-    if (smem > 160 * 1024) return CF_ERR_UNSUPPORTED;
-    static std::once_flag once;
-    static hipError_t attr_err = hipSuccess;
-    std::call_once(once, [] {
-        attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_grouped_gelu_fp8<false>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    });
-    if (attr_err != hipSuccess) return static_cast<int>(attr_err);
-    const int tiles_per_expert = (rows + kGeluRows - 1) / kGeluRows;
-    k_grouped_gelu_fp8<false><<<num_experts * tiles_per_expert, kThreads, smem, as_stream(stream)>>>(
-        static_cast<const uint8_t*>(d_hidden), d_fcin_descale, fcin_is_e5m2, d_route_weights, d_counts, d_row_indices,
-        static_cast<const uint8_t*>(d_fc_in_w), d_fc_in_descale, static_cast<const uint8_t*>(d_fc_out_w), d_fc_out_descale,
-        d_mixed, rows, H, Ie, num_experts, tiles_per_expert);
-    return launch_status();
+    return launch_grouped_gelu_wave<false>(static_cast<const uint8_t*>(d_hidden), d_fcin_descale, fcin_is_e5m2, d_route_weights, d_counts,
+                                           d_row_indices, static_cast<const uint8_t*>(d_fc_in_w), d_fc_in_descale,
+                                           static_cast<const uint8_t*>(d_fc_out_w), d_fc_out_descale, d_mixed, rows, H, Ie, num_experts,
+                                           as_stream(stream));
 }
 
 int cf_moe_grouped_expert_forward_bf16(const uint16_t* d_hidden, const float* d_route_weights, const int* d_counts,
@@ -1573,21 +1627,9 @@ int cf_moe_grouped_expert_forward_bf16(const uint16_t* d_hidden, const float* d_
             d_hidden, d_route_weights, d_counts, d_row_indices, d_fc_in_w, d_fc_out_w, d_mixed, rows, H, Ie, num_experts, tiles);
         return launch_status();
     }
-    const size_t smem = sizeof(float) * static_cast<size_t>(kGeluRows) * (kGeluChunk + Ie);
-    if (smem > 160 * 1024) return CF_ERR_UNSUPPORTED;
-    static std::once_flag once;
-    static hipError_t attr_err = hipSuccess;
-    std::call_once(once, [] {
-        attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_grouped_gelu_fp8<true>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    });
-    if (attr_err != hipSuccess) return static_cast<int>(attr_err);
-    const int tiles_per_expert = (rows + kGeluRows - 1) / kGeluRows;
-    k_grouped_gelu_fp8<true><<<num_experts * tiles_per_expert, kThreads, smem, as_stream(stream)>>>(
-        reinterpret_cast<const uint8_t*>(d_hidden), nullptr, 0, d_route_weights, d_counts, d_row_indices,
-        reinterpret_cast<const uint8_t*>(d_fc_in_w), nullptr, reinterpret_cast<const uint8_t*>(d_fc_out_w), nullptr,
-        d_mixed, rows, H, Ie, num_experts, tiles_per_expert);
-    return launch_status();
+    return launch_grouped_gelu_wave<true>(reinterpret_cast<const uint8_t*>(d_hidden), nullptr, 0, d_route_weights, d_counts, d_row_indices,
+                                          reinterpret_cast<const uint8_t*>(d_fc_in_w), nullptr, reinterpret_cast<const uint8_t*>(d_fc_out_w),
+                                          nullptr, d_mixed, rows, H, Ie, num_experts, as_stream(stream));
 }
 
 }  // extern "C"

@@ -544,7 +544,7 @@ int cf_moe_grouped_swiglu_forward_fp8(const void* d_hidden_e4m3, const float* d_
  * Ie % 64 == 0, 16-byte aligned operands and 8-byte aligned d_mixed the two projections run on
  * the matrix cores (fp8 MFMA for fc_in; fc_out as bf16 MFMA on a two-term bf16 split of the fp32
  * GELU output, relative error 2^-17, against the weights widened exactly; 32 token rows per
- * workgroup up to H = 2048, 16 beyond); other shapes take an fp32 FMA kernel.  Same contract
+ * workgroup up to H = 2048, 16 beyond); other shapes take a wave-parallel fp32 kernel.  Same contract
  * either way. */
 int cf_moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_fcin_descale,
                                       int fcin_is_e5m2, const float* d_route_weights,
@@ -607,8 +607,8 @@ int cf_moe_grouped_expert_forward_bf16_ws(const uint16_t* d_hidden, const float*
  * bf16 hidden states and bf16 weights (fc_in_w [E,Ie,H], fc_out_w [E,H,Ie]), no descales; fp32
  * accumulation, exact-erf GELU kept in fp32, compare-and-swap accumulation into d_mixed.  The
  * non-FP8 sibling: bf16 MFMA for both projections when H % 64 == 0, Ie % 64 == 0, the operands are
- * 16-byte aligned and d_mixed 8-byte aligned (16-row tiles); an fp32 FMA kernel in the reference's
- * loop form otherwise. */
+ * 16-byte aligned and d_mixed 8-byte aligned (16-row tiles); a wave-parallel fp32 kernel
+ * otherwise. */
 int cf_moe_grouped_expert_forward_bf16(const uint16_t* d_hidden, const float* d_route_weights,
                                        const int* d_counts, const int* d_offsets,
                                        const int* d_row_indices, const uint16_t* d_fc_in_w,

@@ -55,7 +55,7 @@ def test_topk_reference_fixture(cf, dev):
     assert np.array_equal(got > 0, want > 0) and np.max(np.abs(got - want)) <= 2e-7
 
 
-@pytest.mark.parametrize("E,k", [(3, 2), (8, 2), (64, 6), (64, 64), (5, 9), (40, 1), (65, 4), (128, 8), (300, 3)])
+@pytest.mark.parametrize("E,k", [(3, 2), (8, 2), (64, 6), (64, 64), (5, 9), (40, 1), (65, 4), (128, 8), (300, 3), (1000, 100), (2048, 7)])
 @pytest.mark.parametrize("normalize", [True, False])
 def test_topk_route_bit_exact(cf, dev, E, k, normalize):
     case(f"top-k E={E} k={k} normalize={normalize}")

@@ -311,3 +311,53 @@ def test_staged_bf16_bank_other_shapes_pass_through(cf, dev):
     mixed, _, _, nbytes = run16(cf, b)
     assert nbytes == 0
     check_result16(b, mixed)
+
+
+# ---- config 5 size: a sample of token rows against the double reference of exactly those rows -------------------
+
+def sample_rows(rows):
+    sel = np.sort(np.random.default_rng(1).choice(rows, 40, replace=False))
+    sel[0], sel[-1] = 0, rows - 1
+    return sel
+
+
+def test_staged_bank_config5_size(cf, dev):
+    case("staged gelu bank, config 5 size")
+    b = Bank(dev, 16384, 64, 6, 2048, 1408, False, seed=8)
+    assert b.total == 98304
+    mixed, ws, off, nbytes = run(cf, b)
+    sel = sample_rows(b.rows)
+    rw = np.ascontiguousarray(b.rw[sel])
+    counts, idx = orc.moe_build_expert_row_lists(rw)
+    start = orc.bf16_to_f32(b.mixed0[sel]).astype(np.float64)
+    ref = orc.moe_grouped_expert_forward_fp8_ref(b.hq[sel], b.d_h, False, rw, counts, idx, b.winq, b.d_in, b.woutq, b.d_out, start)
+    got = orc.bf16_to_f32(bf16_bits(mixed)[sel]).astype(np.float64)
+    assert np.sqrt(((got - ref) ** 2).sum() / (ref ** 2).sum()) <= 4e-3
+    typical = np.sqrt(((ref - start) ** 2).mean())
+    assert np.all(np.abs(got - ref) <= (2 * b.k + 1) * 2.0 ** -8 * (np.abs(start) + np.abs(ref) + 2.0 * typical))
+    # rows nobody samples: every row moved, and by a plausible amount (a tile that was skipped or written twice shows)
+    all_got = orc.bf16_to_f32(bf16_bits(mixed)).astype(np.float64)
+    delta = np.abs(all_got - orc.bf16_to_f32(b.mixed0).astype(np.float64)).mean(axis=1)
+    assert delta.min() > 0.1 * np.median(delta) and delta.max() < 10.0 * np.median(delta)
+    # a second call on the same workspace gives the same bits
+    mixed2, _, _, _ = run(cf, b)
+    assert np.array_equal(bf16_bits(mixed2), bf16_bits(mixed))
+
+
+def test_staged_bf16_bank_config5_size(cf, dev):
+    case("staged bf16 gelu bank, config 5 size")
+    b = Bank16(dev, 16384, 64, 6, 2048, 1408, seed=9)
+    assert b.total == 98304
+    mixed, ws, off, nbytes = run16(cf, b)
+    sel = sample_rows(b.rows)
+    rw = np.ascontiguousarray(b.rw[sel])
+    counts, idx = orc.moe_build_expert_row_lists(rw)
+    start = orc.bf16_to_f32(b.mixed0[sel]).astype(np.float64)
+    ref = orc.moe_grouped_expert_forward_bf16_ref(b.hidden[sel], rw, counts, idx, b.win, b.wout, start)
+    got = orc.bf16_to_f32(bf16_bits(mixed)[sel]).astype(np.float64)
+    assert np.sqrt(((got - ref) ** 2).sum() / (ref ** 2).sum()) <= 4e-3
+    typical = np.sqrt(((ref - start) ** 2).mean())
+    assert np.all(np.abs(got - ref) <= (2 * b.k + 1) * 2.0 ** -8 * (np.abs(start) + np.abs(ref) + 2.0 * typical))
+    all_got = orc.bf16_to_f32(bf16_bits(mixed)).astype(np.float64)
+    delta = np.abs(all_got - orc.bf16_to_f32(b.mixed0).astype(np.float64)).mean(axis=1)
+    assert delta.min() > 0.1 * np.median(delta) and delta.max() < 10.0 * np.median(delta)

@@ -39,6 +39,20 @@ def test_argument_errors_do_not_need_a_gpu(cf):
     assert cf.raw_cf_fp8_quantize_e4m3(None, None, None, 0, None) == 0
     assert cf.raw_cf_fp8_quantize_e4m3(None, None, None, 8, None) == -1
     assert cf.raw_cf_fp8_quantize_rows(None, -1, 4, 0, None, None, None, None) == -1
+    # the workspace forms of the expert bank: sizes are host arithmetic, argument checks come before any launch
+    import ctypes
+    n = ctypes.c_size_t(7)
+    assert cf.raw_cf_moe_grouped_expert_forward_fp8_workspace(16384, 98304, 64, 2048, 1408, None, ctypes.byref(n)) == 0
+    assert 1_300_000_000 < n.value < 1_500_000_000 and n.value % 256 == 0
+    assert cf.raw_cf_moe_grouped_expert_forward_fp8_workspace(100, 200, 4, 96, 72, None, ctypes.byref(n)) == 0 and n.value == 0
+    assert cf.raw_cf_moe_grouped_expert_forward_fp8_workspace(-1, 0, 0, 0, 0, None, ctypes.byref(n)) == -1
+    assert cf.raw_cf_moe_grouped_expert_forward_bf16_workspace(16384, 98304, 64, 2048, 1408, None, ctypes.byref(n)) == 0
+    assert 1_800_000_000 < n.value < 2_000_000_000
+    nul = [None] * 12
+    assert cf.raw_cf_moe_grouped_expert_forward_fp8_ws(None, None, 0, *nul[:9], 4, 256, 128, 2, 8, None, 0, None) == -1
+    assert cf.raw_cf_moe_grouped_expert_forward_fp8_ws(None, None, 0, *nul[:9], 0, 256, 128, 2, 0, None, 0, None) == 0
+    assert cf.raw_cf_moe_grouped_expert_forward_bf16_ws(*nul[:8], 4, 256, 128, 2, 8, None, 0, None) == -1
+    assert cf.raw_cf_moe_grouped_expert_forward_bf16_ws(*nul[:8], -4, 256, 128, 2, 8, None, 0, None) == -1
 
 
 def test_cpp_shim_compiles_links_and_maps_errors(tmp_path):

@@ -93,8 +93,8 @@ def test_delayed_scaling_step_replays_from_a_graph(cf, dev):
 
 
 def test_moe_layer_replays_from_a_graph(cf, dev):
-    """Routing, row lists, offsets and both one-call expert banks (SwiGLU; GELU with re-quantized activations) in one
-    captured graph: every buffer the routing fills is consumed on the device, so a replay on new logits and new hidden
+    """Routing, row lists, offsets and the one-call expert banks (SwiGLU; GELU with re-quantized activations; the workspace
+    forms of moe_grouped_expert_forward_fp8 and _bf16, which take no offsets) in one captured graph: every buffer the routing fills is consumed on the device, so a replay on new logits and new hidden
     states must reproduce the eager run bit for bit."""
     import ctypes
     case("graph capture: top-k route -> row lists -> offsets -> SwiGLU bank -> GELU bank")
@@ -110,6 +110,16 @@ def test_moe_layer_replays_from_a_graph(cf, dev):
     idx = torch.zeros(E * T, dtype=torch.int32, device=dev)
     out_swiglu = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
     out_gelu = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+    out_ref8 = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+    out_ref16 = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+    h16 = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+    wi16 = (0.05 * torch.randn(E * Ie, H, device=dev, generator=g)).to(torch.bfloat16)
+    wo16 = (0.05 * torch.randn(E * H, Ie, device=dev, generator=g)).to(torch.bfloat16)
+    s3, s4 = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    assert cf.raw_cf_moe_grouped_expert_forward_fp8_workspace(T, total, E, H, Ie, None, ctypes.byref(s3)) == 0 and s3.value > 0
+    assert cf.raw_cf_moe_grouped_expert_forward_bf16_workspace(T, total, E, H, Ie, None, ctypes.byref(s4)) == 0 and s4.value > 0
+    ws3 = torch.empty(s3.value + 256, dtype=torch.uint8, device=dev); p3 = ws3.data_ptr() + (-ws3.data_ptr()) % 256
+    ws4 = torch.empty(s4.value + 256, dtype=torch.uint8, device=dev); p4 = ws4.data_ptr() + (-ws4.data_ptr()) % 256
     s1, s2 = ctypes.c_size_t(0), ctypes.c_size_t(0)
     assert cf.raw_cf_moe_grouped_swiglu_workspace_bytes(total, E, H, Ie, ctypes.byref(s1)) == 0
     assert cf.raw_cf_moe_grouped_gelu_workspace_bytes(T, total, E, H, Ie, ctypes.byref(s2)) == 0
@@ -119,7 +129,7 @@ def test_moe_layer_replays_from_a_graph(cf, dev):
     def step():
         s = stream()
         rw.copy_(logits)
-        out_swiglu.zero_(); out_gelu.zero_()
+        out_swiglu.zero_(); out_gelu.zero_(); out_ref8.zero_(); out_ref16.zero_()
         cf.cf_moe_topk_route_f32(rw, T, E, k, s, None, None, 1)
         cf.cf_moe_build_expert_row_lists(rw, counts, idx, T, E, s)
         cf.cf_moe_expert_offsets_from_counts(counts, offs, E, s)
@@ -127,12 +137,16 @@ def test_moe_layer_replays_from_a_graph(cf, dev):
                                              p1, s1.value, s)
         cf.cf_moe_grouped_gelu_forward_fp8(hq, one, 0, rw, counts, offs, idx, wg, one, wd, one, out_gelu, T, H, Ie, E, total,
                                            p2, s2.value, s)
+        cf.cf_moe_grouped_expert_forward_fp8_ws(hq, one, 0, rw, counts, None, idx, wg, one, wd, one, out_ref8, T, H, Ie, E, total,
+                                                p3, s3.value, s)
+        cf.cf_moe_grouped_expert_forward_bf16_ws(h16, rw, counts, None, idx, wi16, wo16, out_ref16, T, H, Ie, E, total, p4, s4.value, s)
 
     def new_inputs(i):
         logits.copy_(torch.randn(T, E, device=dev, generator=g))
         x = torch.randn(T, H, device=dev, generator=g) * (1.0 + i)
         amax = x.abs().amax(dim=1).clamp_min(1e-12)
         hq.copy_((x * (448.0 / amax)[:, None]).to(torch.float8_e4m3fn).view(torch.uint8)); hd.copy_(amax / 448.0)
+        h16.copy_(x.to(torch.bfloat16))
 
     new_inputs(0); step(); torch.cuda.synchronize()                 # warm-up outside the capture
     graph = torch.cuda.CUDAGraph()
@@ -142,9 +156,10 @@ def test_moe_layer_replays_from_a_graph(cf, dev):
         new_inputs(i)
         step()
         torch.cuda.synchronize()
-        want = (out_swiglu.clone(), out_gelu.clone(), counts.clone(), rw.clone())
+        want = (out_swiglu.clone(), out_gelu.clone(), counts.clone(), rw.clone(), out_ref8.clone(), out_ref16.clone())
+        assert float(out_ref8.float().abs().max()) > 0 and float(out_ref16.float().abs().max()) > 0
         assert int(counts.sum()) == total
-        out_swiglu.fill_(7.0); out_gelu.fill_(7.0); counts.fill_(-1); rw.fill_(0.5)
+        out_swiglu.fill_(7.0); out_gelu.fill_(7.0); counts.fill_(-1); rw.fill_(0.5); out_ref8.fill_(7.0); out_ref16.fill_(7.0)
         scratch = torch.randn(1 << 20, device=dev).sum()
         torch.cuda.synchronize()
         graph.replay()
@@ -152,6 +167,8 @@ def test_moe_layer_replays_from_a_graph(cf, dev):
         assert torch.equal(counts, want[2]) and torch.equal(rw, want[3]), f"replay {i}"
         assert torch.equal(out_swiglu.view(torch.int16), want[0].view(torch.int16)), f"replay {i}"
         assert torch.equal(out_gelu.view(torch.int16), want[1].view(torch.int16)), f"replay {i}"
+        assert torch.equal(out_ref8.view(torch.int16), want[4].view(torch.int16)), f"replay {i}"
+        assert torch.equal(out_ref16.view(torch.int16), want[5].view(torch.int16)), f"replay {i}"
         assert float(scratch) == float(scratch)
 
 

@@ -239,6 +239,11 @@ int grouped_gemm_bf16_nt(int total_rows, int N, int Kb, int terms, int num_exper
 // then per row tile (expert, its first row, its end row, its first row tile, its row-tile count), experts back to back.
 void build_tile_map(const int* d_counts, const int* d_offsets, int num_experts, int max_row_tiles, int* tile_map,
                     hipStream_t stream);
+// One launch for what an expert bank derives from (counts, row lists [num_experts, rows]): the offsets, the compact
+// row index, the (row, expert) -> compact row table (d_slot_index may be null) and the tile table of a grouped GEMM
+// over total_rows rows.
+void bank_setup(const int* d_counts, const int* d_row_indices, int rows, int num_experts, int total_rows, int* d_offsets,
+                int* d_compact_index, int* d_slot_index, int* tile_map, hipStream_t stream);
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline unsigned ceil_div(size_t a, size_t b) { return static_cast<unsigned>((a + b - 1) / b); }

@@ -670,10 +670,11 @@ __device__ __forceinline__ void drain_tile(v16f (&acc)[4][4], TileScales<EPI>& s
 #pragma unroll
                         for (int q = 0; q < 4; ++q) {
                             if constexpr (GATE) {
-                                // the reference rounds gate and up to bf16 before the SiLU product
-                                const float gate = round_bf16_hw(acc_read(acc[2 * unit][b][g * 4 + q]) * (sa * c4[q]));
-                                const float up = round_bf16_hw(acc_read(acc[2 * unit + 1][b][g * 4 + q]) * (sa * u4[q]));
-                                v[q] = fast_silu(gate) * up;
+                                // the reference rounds gate and up to bf16 before the SiLU product: one conversion
+                                // instruction rounds both
+                                const uint32_t gu = pack_bf16x2_hw(acc_read(acc[2 * unit][b][g * 4 + q]) * (sa * c4[q]),
+                                                                   acc_read(acc[2 * unit + 1][b][g * 4 + q]) * (sa * u4[q]));
+                                v[q] = fast_silu(bf16_lo(gu)) * bf16_hi(gu);
                             } else {
                                 v[q] = acc_read(acc[unit][b][g * 4 + q]) * (sa * c4[q]);
                             }
@@ -1538,21 +1539,21 @@ int dispatch_epi(const GemmArgs& p, int epi, int scale_mode, hipStream_t st) {
 
 // one wavefront: the row tiles of every expert in expert order (lane = expert, prefix sum of the tile counts);
 // each row tile's entry describes its expert: number, row range, first row tile, row-tile count
-__global__ __launch_bounds__(64) void k_build_tile_map(const int* __restrict__ counts, const int* __restrict__ offsets,
-                                                       int num_experts, int max_row_tiles, int* __restrict__ tile_map) {
-    const int lane = threadIdx.x;
-    int carry = 0, written = 0;
+// (offsets == nullptr: the experts' rows lie back to back, the first rows are the running sum of the counts)
+__device__ __forceinline__ void build_tile_map_wave(const int* __restrict__ counts, const int* __restrict__ offsets,
+                                                    int num_experts, int max_row_tiles, int* __restrict__ tile_map, int lane) {
+    int carry = 0, carry_rows = 0, written = 0;
     for (int e0 = 0; e0 < num_experts; e0 += 64) {
         const int e = e0 + lane;
         const int cnt = e < num_experts ? counts[e] : 0;
-        const int first = e < num_experts ? offsets[e] : 0;
         const int nt = (cnt + BM - 1) / BM;
-        int incl = nt;
+        int incl = nt, incl_rows = cnt;
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
-            const int v = __shfl_up(incl, off, 64);
-            if (lane >= off) incl += v;
+            const int v = __shfl_up(incl, off, 64), r = __shfl_up(incl_rows, off, 64);
+            if (lane >= off) { incl += v; incl_rows += r; }
         }
+        const int first = offsets ? (e < num_experts ? offsets[e] : 0) : carry_rows + incl_rows - cnt;
         const int base = carry + incl - nt;
         if (base + nt <= max_row_tiles) {        // always true for counts that sum to at most the caller's total_rows
             for (int i = 0; i < nt; ++i) {
@@ -1562,11 +1563,46 @@ __global__ __launch_bounds__(64) void k_build_tile_map(const int* __restrict__ c
             if (nt > 0) written = max(written, base + nt);
         }
         carry += __shfl(incl, 63, 64);
+        carry_rows += __shfl(incl_rows, 63, 64);
     }
     // experts are written in order, so the ones that fit form a prefix: the table ends with the last of them
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) written = max(written, __shfl_xor(written, off, 64));
     if (lane == 0) tile_map[0] = written;
+}
+__global__ __launch_bounds__(64) void k_build_tile_map(const int* __restrict__ counts, const int* __restrict__ offsets,
+                                                       int num_experts, int max_row_tiles, int* __restrict__ tile_map) {
+    build_tile_map_wave(counts, offsets, num_experts, max_row_tiles, tile_map, threadIdx.x);
+}
+
+// Everything an expert bank derives from (counts, row lists) in one launch.  Workgroup e < num_experts: the offset
+// of expert e (the sum of the counts before it), its row list copied into the compact index at that offset and,
+// when slot_index is given, the inverse entries slot_index[row, e] = position.  The last workgroup: the tile table.
+__global__ __launch_bounds__(256) void k_bank_setup(const int* __restrict__ counts, const int* __restrict__ row_indices, int rows,
+                                                    int num_experts, int max_row_tiles, int* __restrict__ offsets,
+                                                    int* __restrict__ compact, int* __restrict__ slot_index,
+                                                    int* __restrict__ tile_map) {
+    const int e = blockIdx.x, tid = threadIdx.x;
+    if (e == num_experts) {
+        if (tid < 64) build_tile_map_wave(counts, nullptr, num_experts, max_row_tiles, tile_map, tid);
+        return;
+    }
+    __shared__ int part[4];
+    int sum = 0;
+    for (int i = tid; i < e; i += 256) sum += counts[i];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    if ((tid & 63) == 0) part[tid >> 6] = sum;
+    __syncthreads();
+    const int base = part[0] + part[1] + part[2] + part[3];
+    if (tid == 0) offsets[e] = base;
+    const int n = counts[e];
+    const int* list = row_indices + static_cast<size_t>(e) * rows;
+    for (int s = tid; s < n; s += 256) {
+        const int row = list[s];
+        compact[base + s] = row;
+        if (slot_index) slot_index[static_cast<size_t>(row) * num_experts + e] = base + s;
+    }
 }
 
 int gemm_nt(GemmArgs p, int fmt, int epi, int scale_mode, int force_naive, cf_stream_t stream) {
@@ -1778,6 +1814,12 @@ int cf_fp8_grouped_gemm_nt_bf16_static(int total_rows, int N, int K, int num_exp
 void cf::build_tile_map(const int* d_counts, const int* d_offsets, int num_experts, int max_row_tiles, int* tile_map,
                         hipStream_t stream) {
     k_build_tile_map<<<1, 64, 0, stream>>>(d_counts, d_offsets, num_experts, max_row_tiles, tile_map);
+}
+
+void cf::bank_setup(const int* d_counts, const int* d_row_indices, int rows, int num_experts, int total_rows, int* d_offsets,
+                    int* d_compact_index, int* d_slot_index, int* tile_map, hipStream_t stream) {
+    k_bank_setup<<<num_experts + 1, 256, 0, stream>>>(d_counts, d_row_indices, rows, num_experts, total_rows / BM + num_experts,
+                                                      d_offsets, d_compact_index, d_slot_index, tile_map);
 }
 
 // build_map = false: d_workspace already holds the tile table of these counts and offsets (an earlier call of

@@ -210,16 +210,8 @@ int cf_moe_grouped_expert_forward_fp8_ws(const void* d_hidden, const float* d_fc
     hipStream_t st = as_stream(stream);
 
     // the reference takes the row lists without their offsets; the tile table and the compact index need them
-    int rc = cf_moe_expert_offsets_from_counts(d_counts, offsets, num_experts, stream);
-    if (rc) return rc;
-    rc = cf_moe_compact_row_index(d_counts, offsets, d_row_indices, rows, num_experts, index, stream);
-    if (rc) return rc;
-    if (slot) {
-        rc = cf_moe_build_slot_index(d_counts, offsets, d_row_indices, rows, num_experts, slot, stream);
-        if (rc) return rc;
-    }
-    build_tile_map(d_counts, offsets, num_experts, total_selected_rows / 256 + num_experts, tile_map, st);
-    rc = launch_status();
+    bank_setup(d_counts, d_row_indices, rows, num_experts, total_selected_rows, offsets, index, slot, tile_map, st);
+    int rc = launch_status();
     if (rc) return rc;
     rc = grouped_gemm_nt_store_f32(total_selected_rows, Ie, H, num_experts, d_hidden, rows, H, index, d_fcin_descale, d_fc_in_w,
                                    d_fc_in_descale, pre, Ie, tile_map, fcin_is_e5m2 ? 1 : 0, stream);
@@ -289,16 +281,8 @@ int cf_moe_grouped_expert_forward_bf16_ws(const uint16_t* d_hidden, const float*
     uint16_t* xg = reinterpret_cast<uint16_t*>(base + w.off[CF_MOE_FWD_WS_X]);
     hipStream_t st = as_stream(stream);
 
-    int rc = cf_moe_expert_offsets_from_counts(d_counts, offsets, num_experts, stream);
-    if (rc) return rc;
-    rc = cf_moe_compact_row_index(d_counts, offsets, d_row_indices, rows, num_experts, index, stream);
-    if (rc) return rc;
-    if (slot) {
-        rc = cf_moe_build_slot_index(d_counts, offsets, d_row_indices, rows, num_experts, slot, stream);
-        if (rc) return rc;
-    }
-    build_tile_map(d_counts, offsets, num_experts, total_selected_rows / 256 + num_experts, tile_map, st);
-    rc = launch_status();
+    bank_setup(d_counts, d_row_indices, rows, num_experts, total_selected_rows, offsets, index, slot, tile_map, st);
+    int rc = launch_status();
     if (rc) return rc;
     rc = cf_moe_gather_rows_bf16(d_hidden, xg, index, total_selected_rows, H, stream);
     if (rc) return rc;

@@ -228,9 +228,9 @@ int grouped_gemm_nt_bf16(int total_rows, int N, int K, int num_experts, const in
 int grouped_gemm_nt_store_f32(int total_rows, int N, int K, int num_experts, const void* A, int a_rows, int lda,
                               const int* d_a_row_index, const float* a_descale, const void* B, const float* b_descale,
                               float* C, int ldc, const int* d_tile_map, int a_is_e5m2, cf_stream_t stream);
-int grouped_gemm_nt_bf16_terms(int total_rows, int N, int Kb, int terms, int num_experts, const void* A, int lda,
-                               const float* a_descale, const void* B, const float* b_descale, uint16_t* C, int ldc,
-                               const int* d_tile_map, cf_stream_t stream);
+int grouped_gemm_nt_terms(int total_rows, int N, int Kb, int terms, int num_experts, const void* A, int lda,
+                          const float* a_descale, const void* B, const float* b_descale, void* C, int ldc, bool c_is_f32,
+                          const int* d_tile_map, cf_stream_t stream);
 // The forward-pass form of the grouped bf16 GEMM (gemm_bf16.hip): C[r, :] = sum_t A[r, t*Kb:(t+1)*Kb] . B[expert(r)]^T,
 // B [num_experts, N, Kb], C bf16 or fp32, tile table already built.
 int grouped_gemm_bf16_nt(int total_rows, int N, int Kb, int terms, int num_experts, const uint16_t* A, int lda,
@@ -239,6 +239,10 @@ int grouped_gemm_bf16_nt(int total_rows, int N, int Kb, int terms, int num_exper
 // then per row tile (expert, its first row, its end row, its first row tile, its row-tile count), experts back to back.
 void build_tile_map(const int* d_counts, const int* d_offsets, int num_experts, int max_row_tiles, int* tile_map,
                     hipStream_t stream);
+// The ordered weighted add of fp32 expert outputs into bf16 rows (moe.hip): d_slot_index null = search the row lists.
+int unpermute_f32(uint16_t* d_mixed, const float* d_y, const float* d_route_weights, const int* d_slot_index,
+                  const int* d_counts, const int* d_offsets, const int* d_row_indices, int rows, int num_experts, int H,
+                  hipStream_t st);
 // One launch for what an expert bank derives from (counts, row lists [num_experts, rows]): the offsets, the compact
 // row index, the (row, expert) -> compact row table (d_slot_index may be null) and the tile table of a grouped GEMM
 // over total_rows rows.

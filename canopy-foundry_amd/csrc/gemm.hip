@@ -725,8 +725,9 @@ __device__ __forceinline__ void drain_tile(v16f (&acc)[4][4], TileScales<EPI>& s
 // sixteen lanes), non-temporal both ways.
 // STORE: C = product (nothing is fetched).  RAGGED also covers a last column tile that N cuts short (N % 4 == 0: a
 // lane's four columns are in or out as a whole).
+// sa: the descales of this lane's four output rows (1 for the per-tensor forms), s1 the scalar factor.
 template <bool RAGGED, bool OUT_BF16, bool STORE, class Landed>
-__device__ __forceinline__ void drain_tile_accum(v16f (&acc)[4][4], float s1, const GemmArgs& p, const TilePos& t,
+__device__ __forceinline__ void drain_tile_accum(v16f (&acc)[4][4], const float (&sa)[4], float s1, const GemmArgs& p, const TilePos& t,
                                                  int wm, int wn, int lane, uint8_t* stage, Landed&& landed) {
     const int row = lane & 31, khalf = lane >> 5;
     uint8_t* wr = stage + row * 256;
@@ -765,13 +766,14 @@ __device__ __forceinline__ void drain_tile_accum(v16f (&acc)[4][4], float s1, co
 #pragma unroll
         for (int uu = 0; uu < 2; ++uu) {
             const int unit = pair * 2 + uu;
+            const float sr = sa[b] * s1;
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 float4 v;
-                v.x = acc_read(acc[unit][b][g * 4 + 0]) * s1;
-                v.y = acc_read(acc[unit][b][g * 4 + 1]) * s1;
-                v.z = acc_read(acc[unit][b][g * 4 + 2]) * s1;
-                v.w = acc_read(acc[unit][b][g * 4 + 3]) * s1;
+                v.x = acc_read(acc[unit][b][g * 4 + 0]) * sr;
+                v.y = acc_read(acc[unit][b][g * 4 + 1]) * sr;
+                v.z = acc_read(acc[unit][b][g * 4 + 2]) * sr;
+                v.w = acc_read(acc[unit][b][g * 4 + 3]) * sr;
                 *reinterpret_cast<float4*>(wr + (((uu * 8 + g * 2 + khalf) ^ wswz) << 4)) = v;
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -1015,6 +1017,7 @@ void k_gemm_nt_ring(const GemmArgs p) {
                 load_row_scales<EPI, SCALE>(sc, p, t, wm, lane);
                 load_pair_scales<EPI, SCALE>(sc.cs, sc.cs2, p, t, wn, lane, 0);
             }
+            if constexpr (END && ACCUM && SCALE == SCALE_ROW && i == 10) load_row_scales<EPI, SCALE>(sc, p, t, wm, lane);
             __builtin_amdgcn_sched_barrier(0);
         });
     };
@@ -1101,8 +1104,12 @@ void k_gemm_nt_ring(const GemmArgs p) {
             uint8_t* stage = smem + a4 + wave * (64 * BK);
             if constexpr (ACCUM) {
                 constexpr bool BF = EPI == EPI_ACCUM_BF16, ST = EPI == EPI_STORE_F32;
-                if (t.m0 + BM <= t.m_end && t.n0 + BN <= p.N) drain_tile_accum<false, BF, ST>(acc, s1, p, t, wm, wn, lane, stage, landed);
-                else                      drain_tile_accum<true, BF, ST>(acc, s1, p, t, wm, wn, lane, stage, landed);
+                if constexpr (SCALE != SCALE_ROW) {
+#pragma unroll
+                    for (int b = 0; b < 4; ++b) sc.sa[b] = 1.0f;
+                }
+                if (t.m0 + BM <= t.m_end && t.n0 + BN <= p.N) drain_tile_accum<false, BF, ST>(acc, sc.sa, s1, p, t, wm, wn, lane, stage, landed);
+                else                      drain_tile_accum<true, BF, ST>(acc, sc.sa, s1, p, t, wm, wn, lane, stage, landed);
             } else {
                 constexpr int out_bn = EPI == EPI_SILU_GATE ? BN / 2 : BN;
                 if (t.m0 + BM <= t.m_end && t.n0 + out_bn <= p.N) drain_tile<EPI, SCALE, false>(acc, sc, s1, s2, p, t, wm, wn, lane, stage, landed);
@@ -1920,12 +1927,12 @@ int grouped_gemm_nt_store_f32(int total_rows, int N, int K, int num_experts, con
                      : launch_ring_only<0, EPI_STORE_F32, SCALE_TENSOR, 0>(p, st);
 }
 
-// C[r, :] = bf16( a_descale[r] * b_descale[:] * sum_t 2^(-4 t) A[r, t*Kb : (t+1)*Kb] . B[expert(r)]^T ): the activation
+// C[r, :] = a_descale[r] * b_descale[0] * sum_t 2^(-4 t) A[r, t*Kb : (t+1)*Kb] . B[expert(r)]^T, bf16 or fp32: the activation
 // rows are `terms` E4M3 terms side by side (lda >= terms * Kb), B is [num_experts, N, Kb] E4M3, b_descale one scalar
 // for all experts.  Kb % 128 == 0; terms * Kb >= 256.
-int grouped_gemm_nt_bf16_terms(int total_rows, int N, int Kb, int terms, int num_experts, const void* A, int lda,
-                               const float* a_descale, const void* B, const float* b_descale, uint16_t* C, int ldc,
-                               const int* d_tile_map, cf_stream_t stream) {
+int grouped_gemm_nt_terms(int total_rows, int N, int Kb, int terms, int num_experts, const void* A, int lda,
+                          const float* a_descale, const void* B, const float* b_descale, void* C, int ldc, bool c_is_f32,
+                          const int* d_tile_map, cf_stream_t stream) {
     if (total_rows <= 0 || N <= 0 || num_experts <= 0) return CF_OK;
     if (!A || !B || !C || !a_descale || !b_descale || !d_tile_map || terms < 1 || terms > 8) return CF_ERR_INVALID_ARG;
     const long long K = static_cast<long long>(terms) * Kb;
@@ -1938,7 +1945,9 @@ int grouped_gemm_nt_bf16_terms(int total_rows, int N, int Kb, int terms, int num
     p.A = static_cast<const uint8_t*>(A); p.lda = lda;
     p.B = static_cast<const uint8_t*>(B); p.ldb = Kb;
     p.sa = a_descale; p.sb = b_descale;
-    p.C = C; p.ldc = ldc;
+    if (c_is_f32) p.Cf = static_cast<float*>(C);
+    else p.C = static_cast<uint16_t*>(C);
+    p.ldc = ldc;
     p.tile_map = d_tile_map;
     p.a_rows = total_rows;
     p.b_expert_stride = static_cast<long long>(N) * Kb;
@@ -1946,7 +1955,8 @@ int grouped_gemm_nt_bf16_terms(int total_rows, int N, int Kb, int terms, int num
     p.b_k_period = Kb;
     p.tiles_m = total_rows / BM + num_experts;
     p.tiles_n = (N + BN - 1) / BN;
-    return launch_ring_only<0, EPI_NONE, SCALE_ROW, 1>(p, as_stream(stream));
+    return c_is_f32 ? launch_ring_only<0, EPI_STORE_F32, SCALE_ROW, 1>(p, as_stream(stream))
+                    : launch_ring_only<0, EPI_NONE, SCALE_ROW, 1>(p, as_stream(stream));
 }
 }  // namespace cf
 

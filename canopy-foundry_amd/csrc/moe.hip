@@ -386,10 +386,52 @@ __device__ __forceinline__ void combine_rows(uint16_t* __restrict__ mrow, const 
     }
 }
 
+// The same for fp32 rows of y: mixed = bf16(mixed + w * y) per listed row, product and sum rounded in fp32 as
+// separate operations (what an add of the argument `w * y` to the stored value does), one bf16 rounding per row.
+__device__ __forceinline__ uint32_t add2_bf16(uint32_t m, float y0, float y1, float w) {
+    return pack_bf16x2(bf16_lo(m) + w * y0, bf16_hi(m) + w * y1);
+}
+__device__ __forceinline__ void combine_rows(uint16_t* __restrict__ mrow, const float* __restrict__ y, int H, int n,
+                                             const int* sl_slot, const float* sl_w, int t) {
+    if ((H & 7) == 0) {
+        for (int c = t; c < H / 8; c += blockDim.x) {
+            uint4 mv = reinterpret_cast<uint4*>(mrow)[c];
+            for (int i0 = 0; i0 < n; i0 += 4) {
+                float4 ya[4], yb[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int slot = i0 + j < n ? sl_slot[i0 + j] : -1;
+                    ya[j] = yb[j] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                    if (slot >= 0) {
+                        const float4* src = reinterpret_cast<const float4*>(y + static_cast<size_t>(slot) * H) + 2 * c;
+                        ya[j] = src[0]; yb[j] = src[1];
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if (i0 + j < n && sl_slot[i0 + j] >= 0) {
+                        const float w = sl_w[i0 + j];
+                        mv.x = add2_bf16(mv.x, ya[j].x, ya[j].y, w); mv.y = add2_bf16(mv.y, ya[j].z, ya[j].w, w);
+                        mv.z = add2_bf16(mv.z, yb[j].x, yb[j].y, w); mv.w = add2_bf16(mv.w, yb[j].z, yb[j].w, w);
+                    }
+                }
+            }
+            store_stream16(reinterpret_cast<uint4*>(mrow) + c, mv);
+        }
+    } else {
+        for (int h = t; h < H; h += blockDim.x) {
+            float m = bf16_to_f32(mrow[h]);
+            for (int i = 0; i < n; ++i)
+                if (sl_slot[i] >= 0) m = bf16_to_f32(f32_to_bf16(m + sl_w[i] * y[static_cast<size_t>(sl_slot[i]) * H + h]));
+            mrow[h] = f32_to_bf16(m);
+        }
+    }
+}
+
 // The same with the slots read from a table slot_index[row, e] (filled by k_slot_index for the selected pairs):
 // no search, so a row's critical path is one load of its weights and slots, then the gathers.
-template <bool UNIT>
-__global__ __launch_bounds__(kThreads) void k_unpermute_indexed(uint16_t* __restrict__ mixed, const uint16_t* __restrict__ y,
+template <bool UNIT, class YT = uint16_t>
+__global__ __launch_bounds__(kThreads) void k_unpermute_indexed(uint16_t* __restrict__ mixed, const YT* __restrict__ y,
                                                                 const float* __restrict__ route_weights,
                                                                 const int* __restrict__ slot_index, int E, int H) {
     __shared__ int sl_slot[64];
@@ -430,8 +472,8 @@ __global__ __launch_bounds__(kThreads) void k_slot_index(const int* __restrict__
 
 // UNIT: every selected expert's row is added with factor 1 (the backward's scatter-add); the route weights
 // then only say which experts selected the row.
-template <bool UNIT>
-__global__ __launch_bounds__(kThreads) void k_unpermute(uint16_t* __restrict__ mixed, const uint16_t* __restrict__ y,
+template <bool UNIT, class YT = uint16_t>
+__global__ __launch_bounds__(kThreads) void k_unpermute(uint16_t* __restrict__ mixed, const YT* __restrict__ y,
                                                         const float* __restrict__ route_weights,
                                                         const int* __restrict__ counts, const int* __restrict__ offsets,
                                                         const int* __restrict__ row_indices, int rows, int E, int H) {
@@ -1633,3 +1675,18 @@ int cf_moe_grouped_expert_forward_bf16(const uint16_t* d_hidden, const float* d_
 }
 
 }  // extern "C"
+
+// mixed[row] += w[row, e] * y[slot(row, e)] over the row's experts in ascending order for fp32 rows of y, one bf16
+// rounding per expert; the slot table when the caller has one, the search of the row lists otherwise
+int cf::unpermute_f32(uint16_t* d_mixed, const float* d_y, const float* d_route_weights, const int* d_slot_index,
+                      const int* d_counts, const int* d_offsets, const int* d_row_indices, int rows, int num_experts, int H,
+                      hipStream_t st) {
+    if (rows <= 0 || num_experts <= 0 || H <= 0) return CF_OK;
+    if ((H & 7) == 0 && !(aligned16(d_mixed) && aligned16(d_y))) return CF_ERR_UNSUPPORTED;
+    if (d_slot_index)
+        k_unpermute_indexed<false, float><<<rows, kThreads, 0, st>>>(d_mixed, d_y, d_route_weights, d_slot_index, num_experts, H);
+    else
+        k_unpermute<false, float><<<rows, kThreads, 0, st>>>(d_mixed, d_y, d_route_weights, d_counts, d_offsets, d_row_indices, rows,
+                                                            num_experts, H);
+    return launch_status();
+}

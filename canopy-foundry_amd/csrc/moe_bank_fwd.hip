@@ -9,12 +9,11 @@
 //           each residual is exact in fp32): 12 to 13 significand bits where bf16 has 8
 //   fc_out  one grouped FP8 GEMM over K = 3 Ie: the three terms side by side against the same weights, the
 //           matrix cores weighting term t by 2^(-4 t) through the E8M0 scale of v_mfma_scale_f32_32x32x64_f8f6f4,
-//           so the three partial products meet in one fp32 accumulator; bf16 out
-//   add     mixed[row] += w * y over the row's experts in ascending order, one bf16 rounding per expert
+//           so the three partial products meet in one fp32 accumulator; fp32 out
+//   add     mixed[row] = bf16(mixed[row] + w * y) over the row's experts in ascending order, y in fp32, one bf16
+//           rounding per expert as in the reference's compare-and-swap add
 //
-// Against the reference: y is rounded to bf16 before it is weighted and added (the reference adds w * y from fp32),
-// one more bf16 rounding per (row, expert); and the sum order over experts is fixed here where the reference's
-// compare-and-swap adds land in any order.
+// Against the reference: the sum order over experts is fixed here where the reference's adds land in any order.
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -117,12 +116,12 @@ FwdWs fwd_layout(int rows, int total_rows, int num_experts, int H, int Ie, bool 
         // two bf16 terms per value, no scales; the gathered token rows
         w.off[CF_MOE_FWD_WS_SPLIT] = off; off = up(off + 2 * 2 * T * Ie);
         w.off[CF_MOE_FWD_WS_SPLIT_DESCALE] = off;
-        w.off[CF_MOE_FWD_WS_Y] = off; off = up(off + 2 * T * H);
+        w.off[CF_MOE_FWD_WS_Y] = off; off = up(off + sizeof(float) * T * H);
         w.off[CF_MOE_FWD_WS_X] = off; off = up(off + 2 * T * H);
     } else {
         w.off[CF_MOE_FWD_WS_SPLIT] = off; off = up(off + kTerms * T * Ie);
         w.off[CF_MOE_FWD_WS_SPLIT_DESCALE] = off; off = up(off + sizeof(float) * T);
-        w.off[CF_MOE_FWD_WS_Y] = off; off = up(off + 2 * T * H);
+        w.off[CF_MOE_FWD_WS_Y] = off; off = up(off + sizeof(float) * T * H);
         w.off[CF_MOE_FWD_WS_X] = off;
     }
     w.total = off;
@@ -206,7 +205,7 @@ int cf_moe_grouped_expert_forward_fp8_ws(const void* d_hidden, const float* d_fc
     float* pre = reinterpret_cast<float*>(base + w.off[CF_MOE_FWD_WS_PRE]);
     uint8_t* split = base + w.off[CF_MOE_FWD_WS_SPLIT];
     float* split_descale = reinterpret_cast<float*>(base + w.off[CF_MOE_FWD_WS_SPLIT_DESCALE]);
-    uint16_t* y = reinterpret_cast<uint16_t*>(base + w.off[CF_MOE_FWD_WS_Y]);
+    float* y = reinterpret_cast<float*>(base + w.off[CF_MOE_FWD_WS_Y]);
     hipStream_t st = as_stream(stream);
 
     // the reference takes the row lists without their offsets; the tile table and the compact index need them
@@ -226,18 +225,16 @@ int cf_moe_grouped_expert_forward_fp8_ws(const void* d_hidden, const float* d_fc
         rc = launch_status();
         if (rc) return rc;
     }
-    rc = grouped_gemm_nt_bf16_terms(total_selected_rows, H, Ie, kTerms, num_experts, split, kTerms * Ie, split_descale, d_fc_out_w,
-                                    d_fc_out_descale, y, H, tile_map, stream);
+    rc = grouped_gemm_nt_terms(total_selected_rows, H, Ie, kTerms, num_experts, split, kTerms * Ie, split_descale, d_fc_out_w,
+                               d_fc_out_descale, y, H, true, tile_map, stream);
     if (rc) return rc;
-    if (slot) return cf_moe_unpermute_indexed_bf16(d_mixed, y, d_route_weights, slot, rows, num_experts, H, 0, stream);
-    return cf_moe_unpermute_weighted_bf16(d_mixed, y, d_route_weights, d_counts, offsets, d_row_indices, rows, num_experts, H,
-                                          stream);
+    return unpermute_f32(d_mixed, y, d_route_weights, slot, d_counts, offsets, d_row_indices, rows, num_experts, H, st);
 }
 
 // moe_grouped_expert_forward_bf16 (kernels.hpp:400-407) with a workspace: the same pipeline on bf16 operands.  The
 // token rows are gathered, fc_in is one grouped bf16 GEMM with fp32 output, the GELU output goes to fc_out as two bf16
 // terms side by side (value = head + remainder to 2^-17) against the same weight columns, K = 2 Ie, so both terms add
-// in the fp32 accumulator.
+// in the fp32 accumulator; y stays fp32 until the ordered add.
 int cf_moe_grouped_expert_forward_bf16_workspace(int rows, int total_selected_rows, int num_experts, int H, int Ie,
                                                  size_t* offsets, size_t* bytes) {
     if (rows < 0 || total_selected_rows < 0 || num_experts < 0 || H < 0 || Ie < 0 || !bytes) return CF_ERR_INVALID_ARG;
@@ -277,7 +274,7 @@ int cf_moe_grouped_expert_forward_bf16_ws(const uint16_t* d_hidden, const float*
     int* slot = w.slot_bytes ? reinterpret_cast<int*>(base + w.off[CF_MOE_FWD_WS_SLOT]) : nullptr;
     float* pre = reinterpret_cast<float*>(base + w.off[CF_MOE_FWD_WS_PRE]);
     uint16_t* split = reinterpret_cast<uint16_t*>(base + w.off[CF_MOE_FWD_WS_SPLIT]);
-    uint16_t* y = reinterpret_cast<uint16_t*>(base + w.off[CF_MOE_FWD_WS_Y]);
+    float* y = reinterpret_cast<float*>(base + w.off[CF_MOE_FWD_WS_Y]);
     uint16_t* xg = reinterpret_cast<uint16_t*>(base + w.off[CF_MOE_FWD_WS_X]);
     hipStream_t st = as_stream(stream);
 
@@ -295,11 +292,9 @@ int cf_moe_grouped_expert_forward_bf16_ws(const uint16_t* d_hidden, const float*
         rc = launch_status();
         if (rc) return rc;
     }
-    rc = grouped_gemm_bf16_nt(total_selected_rows, H, Ie, 2, num_experts, split, 2 * Ie, d_fc_out_w, y, H, false, tile_map, stream);
+    rc = grouped_gemm_bf16_nt(total_selected_rows, H, Ie, 2, num_experts, split, 2 * Ie, d_fc_out_w, y, H, true, tile_map, stream);
     if (rc) return rc;
-    if (slot) return cf_moe_unpermute_indexed_bf16(d_mixed, y, d_route_weights, slot, rows, num_experts, H, 0, stream);
-    return cf_moe_unpermute_weighted_bf16(d_mixed, y, d_route_weights, d_counts, offsets, d_row_indices, rows, num_experts, H,
-                                          stream);
+    return unpermute_f32(d_mixed, y, d_route_weights, slot, d_counts, offsets, d_row_indices, rows, num_experts, H, st);
 }
 
 }  // extern "C"

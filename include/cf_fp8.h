@@ -563,13 +563,12 @@ int cf_moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_fcin_
  * E4M3 terms under one per-row scale (value * scale = q0 + q1 / 16 + q2 / 256 to 2^-13: 12 to 13 significand
  * bits, not re-quantized to a single fp8 value); fc_out is one grouped FP8 GEMM over K = 3 Ie in which the
  * matrix cores weight term t by 2^(-4 t) (E8M0 scales of the MX form of the FP8 MFMA), so the three partial
- * products add in one fp32 accumulator; w * y is then added into d_mixed per token row over its experts in
- * ascending order, one bf16 rounding per expert.  Differences from the reference kernel: y is rounded to bf16
- * before it is weighted and added (one more bf16 rounding per (row, expert)), and the order of the adds is
- * fixed.  total_selected_rows must be the sum of d_counts; d_offsets may be null (the offsets are recomputed).
+ * products add in one fp32 accumulator and y stays fp32; w * y is then added into d_mixed per token row over its
+ * experts in ascending order, one bf16 rounding per expert as in the reference's compare-and-swap add.  The
+ * one difference from the reference kernel: the order of the adds is fixed.  total_selected_rows must be the sum of d_counts; d_offsets may be null (the offsets are recomputed).
  * d_workspace 256-byte aligned; cf_moe_grouped_expert_forward_fp8_workspace gives its size and, when
  * `offsets` is not null, the byte offsets of the intermediates (CF_MOE_FWD_WS_* order), which stay valid
- * after the call: pre [total, Ie] fp32, split [total, 3 Ie] E4M3, split_descale [total] fp32, y [total, H] bf16,
+ * after the call: pre [total, Ie] fp32, split [total, 3 Ie] E4M3, split_descale [total] fp32, y [total, H] fp32,
  * experts back to back (CF_MOE_FWD_WS_X is used by the bf16 form only). */
 enum {
     CF_MOE_FWD_WS_TILE_MAP = 0, CF_MOE_FWD_WS_OFFSETS, CF_MOE_FWD_WS_INDEX, CF_MOE_FWD_WS_SLOT, CF_MOE_FWD_WS_PRE,
@@ -591,9 +590,9 @@ int cf_moe_grouped_expert_forward_fp8_ws(const void* d_hidden, const float* d_fc
  * operands are 16-byte aligned (other shapes are passed on to that function).  The selected token rows are
  * gathered (x, CF_MOE_FWD_WS_X), fc_in is one grouped bf16 GEMM with fp32 output (pre), the GELU (fp32, erf to
  * 1.5e-7 absolute) is written as two bf16 terms side by side (split [total, 2 Ie]: bf16(g) and bf16(g - bf16(g)),
- * 16 significand bits), fc_out is one grouped bf16 GEMM over K = 2 Ie against the same weight columns, bf16
- * out (y), then the ordered add into d_mixed as in cf_moe_grouped_expert_forward_fp8_ws, with the same two
- * differences from the reference kernel.  Workspace rules as there; CF_MOE_FWD_WS_SPLIT_DESCALE is unused. */
+ * 16 significand bits), fc_out is one grouped bf16 GEMM over K = 2 Ie against the same weight columns, fp32
+ * out (y), then the ordered add into d_mixed as in cf_moe_grouped_expert_forward_fp8_ws, with the same one
+ * difference from the reference kernel.  Workspace rules as there; CF_MOE_FWD_WS_SPLIT_DESCALE is unused. */
 int cf_moe_grouped_expert_forward_bf16_workspace(int rows, int total_selected_rows, int num_experts, int H,
                                                  int Ie, size_t* offsets, size_t* bytes);
 int cf_moe_grouped_expert_forward_bf16_ws(const uint16_t* d_hidden, const float* d_route_weights,

@@ -4,8 +4,8 @@ a workspace (cf_moe_grouped_expert_forward_fp8_ws), and its bf16 sibling (cf_moe
 Every stage is checked on the intermediates the call leaves in its workspace, given that stage's own (GPU) inputs:
 the fp32 projections against the double product of the dequantized operands; the three-term E4M3 split of the GELU
 against the exact-erf GELU of those projections (12 bits and better, and the row maximum lands on 448); the fc_out
-GEMM, whose matrix-core scales weight term t by 16^-t, against the double product of the recombined terms to one bf16
-rounding; the result against the oracle of the reference kernel at the bars of the one-kernel form's test."""
+GEMM, whose matrix-core scales weight term t by 16^-t, against the double product of the recombined terms at fp32
+accumulation error; the result against the oracle of the reference kernel at the bars of the one-kernel form's test."""
 import ctypes
 import math
 
@@ -19,6 +19,9 @@ from gpu_util import bf16_bits, case, dev_arr, dev_bf16, host, stream
 pytestmark = pytest.mark.gpu
 
 NAMES = ["TILE_MAP", "OFFSETS", "INDEX", "SLOT", "PRE", "SPLIT", "SPLIT_DESCALE", "Y", "X"]
+# the block-scaled FP8 MFMA aligns the products of a K-block to the largest one before adding them, so the terms it
+# scales by 2^-4 and 2^-8 lose low bits: measured up to 2 x the unscaled FP8 MFMA's accumulation error
+ACC_MX = 4.0 * orc.ACC_MFMA
 ACC_BF16 = 16.0 * 2.0 ** -24          # fp32 accumulation of bf16 products on the matrix cores, per sum |a_k b_k|
 erf = np.vectorize(math.erf, otypes=[np.float64])
 
@@ -85,10 +88,9 @@ def check_result(b, mixed):
     got = orc.bf16_to_f32(bf16_bits(mixed)).astype(np.float64)
     rel = np.sqrt(((got - ref) ** 2).sum() / (ref ** 2).sum())
     assert rel <= 4e-3, rel
-    # every one of the k accumulations rounds the running value to bf16, y is rounded once before it: bound as in the
-    # test of the one-kernel form, with one more rounding per expert
+    # every one of the k accumulations rounds the running value to bf16: the bound of the one-kernel form's test
     typical = np.sqrt(((ref - start) ** 2).mean())
-    bound = (2 * b.k + 1) * 2.0 ** -8 * (np.abs(start) + np.abs(ref) + 2.0 * typical)
+    bound = (b.k + 1) * 2.0 ** -8 * (np.abs(start) + np.abs(ref) + 2.0 * typical)
     assert np.all(np.abs(got - ref) <= bound)
     untouched = ~(b.rw > 0).any(axis=1)
     assert np.array_equal(bf16_bits(mixed)[untouched], b.mixed0[untouched])
@@ -147,8 +149,8 @@ def test_staged_bank_stage_by_stage(cf, dev, rows, E, k, H, Ie, e5m2, zero):
     assert np.abs(recon - g)[big].max() / np.abs(g)[big].max() < 2.0 ** -12
     assert np.sqrt(((recon - g)[big] ** 2).mean()) < 0.125 * np.sqrt(((bf - g)[big] ** 2).mean())
 
-    # fc_out: the matrix cores weight the terms; one bf16 rounding of the fp32 sum
-    y = orc.bf16_to_f32(take("Y", np.uint16, T * H).reshape(T, H)).astype(np.float64)
+    # fc_out: the matrix cores weight the terms; the fp32 sum is stored as it is
+    y = take("Y", np.float32, T * H).reshape(T, H).astype(np.float64)
     act = terms[:, 0] + terms[:, 1] / 16.0 + terms[:, 2] / 256.0
     act_abs = np.abs(terms[:, 0]) + np.abs(terms[:, 1]) / 16.0 + np.abs(terms[:, 2]) / 256.0
     for e in range(E):
@@ -158,8 +160,9 @@ def test_staged_bank_stage_by_stage(cf, dev, rows, E, k, H, Ie, e5m2, zero):
         rowscale = d[sel][:, None] * float(b.d_out)
         want = (act[sel] @ wout[e].T) * rowscale
         ad = (act_abs[sel] @ np.abs(wout[e]).T) * rowscale
-        tol = 0.505 * orc.bf16_ulp(np.maximum(np.abs(want), np.abs(y[sel]))) + orc.ACC_MFMA * ad
+        tol = 2.0 ** -22 * np.abs(want) + ACC_MX * ad
         worst = np.abs(y[sel] - want) / tol
+        print(f"fc_out expert {e}: worst error / tolerance {worst.max():.3f}")
         assert worst.max() <= 1.0, f"fc_out expert {e}: worst {worst.max():.3f}"
 
     check_result(b, mixed)
@@ -248,7 +251,7 @@ def check_result16(b, mixed):
     got = orc.bf16_to_f32(bf16_bits(mixed)).astype(np.float64)
     assert np.sqrt(((got - ref) ** 2).sum() / (ref ** 2).sum()) <= 4e-3
     typical = np.sqrt(((ref - start) ** 2).mean())
-    assert np.all(np.abs(got - ref) <= (2 * b.k + 1) * 2.0 ** -8 * (np.abs(start) + np.abs(ref) + 2.0 * typical))
+    assert np.all(np.abs(got - ref) <= (b.k + 1) * 2.0 ** -8 * (np.abs(start) + np.abs(ref) + 2.0 * typical))
     untouched = ~(b.rw > 0).any(axis=1)
     assert np.array_equal(bf16_bits(mixed)[untouched], b.mixed0[untouched])
 
@@ -292,14 +295,14 @@ def test_staged_bf16_bank_stage_by_stage(cf, dev, rows, E, k, H, Ie, zero):
     assert (np.abs(act - g) / tol).max() <= 1.0, "two bf16 terms carry the GELU to 16 bits"
     assert np.all(np.abs(split[:, 1]) <= 2.0 ** -8 * np.abs(split[:, 0]) + 1e-30), "the second term is the first one's rounding error"
 
-    y = orc.bf16_to_f32(take("Y", np.uint16, T * H).reshape(T, H)).astype(np.float64)
+    y = take("Y", np.float32, T * H).reshape(T, H).astype(np.float64)
     for e in range(E):
         sel = expert == e
         if not sel.any():
             continue
         want = act[sel] @ wout[e].T
         ad = (np.abs(split[sel, 0]) + np.abs(split[sel, 1])) @ np.abs(wout[e]).T
-        tol = 0.505 * orc.bf16_ulp(np.maximum(np.abs(want), np.abs(y[sel]))) + ACC_BF16 * ad
+        tol = 2.0 ** -22 * np.abs(want) + ACC_BF16 * ad
         worst = np.abs(y[sel] - want) / tol
         assert worst.max() <= 1.0, f"fc_out expert {e}: worst {worst.max():.3f}"
     check_result16(b, mixed)
@@ -334,7 +337,7 @@ def test_staged_bank_config5_size(cf, dev):
     got = orc.bf16_to_f32(bf16_bits(mixed)[sel]).astype(np.float64)
     assert np.sqrt(((got - ref) ** 2).sum() / (ref ** 2).sum()) <= 4e-3
     typical = np.sqrt(((ref - start) ** 2).mean())
-    assert np.all(np.abs(got - ref) <= (2 * b.k + 1) * 2.0 ** -8 * (np.abs(start) + np.abs(ref) + 2.0 * typical))
+    assert np.all(np.abs(got - ref) <= (b.k + 1) * 2.0 ** -8 * (np.abs(start) + np.abs(ref) + 2.0 * typical))
     # rows nobody samples: every row moved, and by a plausible amount (a tile that was skipped or written twice shows)
     all_got = orc.bf16_to_f32(bf16_bits(mixed)).astype(np.float64)
     delta = np.abs(all_got - orc.bf16_to_f32(b.mixed0).astype(np.float64)).mean(axis=1)
@@ -357,7 +360,7 @@ def test_staged_bf16_bank_config5_size(cf, dev):
     got = orc.bf16_to_f32(bf16_bits(mixed)[sel]).astype(np.float64)
     assert np.sqrt(((got - ref) ** 2).sum() / (ref ** 2).sum()) <= 4e-3
     typical = np.sqrt(((ref - start) ** 2).mean())
-    assert np.all(np.abs(got - ref) <= (2 * b.k + 1) * 2.0 ** -8 * (np.abs(start) + np.abs(ref) + 2.0 * typical))
+    assert np.all(np.abs(got - ref) <= (b.k + 1) * 2.0 ** -8 * (np.abs(start) + np.abs(ref) + 2.0 * typical))
     all_got = orc.bf16_to_f32(bf16_bits(mixed)).astype(np.float64)
     delta = np.abs(all_got - orc.bf16_to_f32(b.mixed0).astype(np.float64)).mean(axis=1)
     assert delta.min() > 0.1 * np.median(delta) and delta.max() < 10.0 * np.median(delta)

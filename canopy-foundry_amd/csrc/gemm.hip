@@ -24,6 +24,7 @@
 // Workgroup -> tile mapping is XCD aware: consecutive workgroup ids go round-robin to the 8 XCDs, so each XCD is
 // given a contiguous range of tiles, walked in 8 (M) x 4 (N) patches whose operands share its own L2.
 #include "common.hpp"
+#include "internal.hpp"
 
 #include <mutex>
 #include <type_traits>
@@ -1583,7 +1584,7 @@ __global__ __launch_bounds__(64) void k_build_tile_map(const int* __restrict__ c
 }
 
 // Everything an expert bank derives from (counts, row lists) in one launch.  Workgroup e < num_experts: the offset
-// of expert e (the sum of the counts before it), its row list copied into the compact index at that offset and,
+// of expert e (the sum of the counts before it; stored when the caller wants the array), its row list copied into the compact index at that offset and,
 // when slot_index is given, the inverse entries slot_index[row, e] = position.  The last workgroup: the tile table.
 __global__ __launch_bounds__(256) void k_bank_setup(const int* __restrict__ counts, const int* __restrict__ row_indices, int rows,
                                                     int num_experts, int max_row_tiles, int* __restrict__ offsets,
@@ -1602,7 +1603,7 @@ __global__ __launch_bounds__(256) void k_bank_setup(const int* __restrict__ coun
     if ((tid & 63) == 0) part[tid >> 6] = sum;
     __syncthreads();
     const int base = part[0] + part[1] + part[2] + part[3];
-    if (tid == 0) offsets[e] = base;
+    if (tid == 0 && offsets) offsets[e] = base;
     const int n = counts[e];
     const int* list = row_indices + static_cast<size_t>(e) * rows;
     for (int s = tid; s < n; s += 256) {

@@ -19,6 +19,7 @@
 // Rows, columns and k beyond the operands' bounds are read as zeros (buffer loads with the operand's size in their
 // descriptor), so any n_e works.
 #include "common.hpp"
+#include "internal.hpp"
 
 #include <mutex>
 #include <type_traits>
@@ -55,6 +56,8 @@ struct BfArgs {
     const int* tile_map;            // NN: [0] = row tiles, then (expert, first row, end row, first row tile, row tiles) each
     long long b_expert_stride;      // NN: elements between the experts' B matrices
     long long c_expert_stride;      // TN: elements between the experts' C matrices
+    const int* a_row_index;         // NT, GATHER: row r of the M side is row a_row_index[r] of A (a_rows rows in all)
+    int a_rows;
     int b_k_period;                 // NT: B has this many columns and k runs over them again and again (K a multiple:
                                     // A's rows are several terms side by side against the same B); 0 = B has K columns
 };
@@ -94,7 +97,9 @@ __device__ __forceinline__ v8bf read_ks(const uint8_t* lane_ptr, int krow0, int 
 
 // A_KS: the M-side operand is stored [K][M] (the weight-gradient form); otherwise [M][K].
 // B_KC: the N-side operand is stored [N][K] (a weight matrix as the forward pass holds it); otherwise [K][N].
-template <bool A_KS, int OUT, bool GROUPED, bool B_KC = false>
+// GATHER (with the [M][K] form of A): the tile's rows of A are fetched through a row index, so a token permute
+// needs no pass of its own.
+template <bool A_KS, int OUT, bool GROUPED, bool B_KC = false, bool GATHER = false>
 __global__ __launch_bounds__(kThr) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void k_gemm_bf16(const BfArgs p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -177,6 +182,19 @@ void k_gemm_bf16(const BfArgs p) {
     // [m][k] operand: this lane's row within a group of 32 rows and its 16-byte k chunk
     const uint32_t a_lane_kc = (tid >> 3) * static_cast<uint32_t>(p.lda) * 2u + (tid & 7) * 16u;
     const uint32_t b_lane_kc = (tid >> 3) * static_cast<uint32_t>(p.ldb) * 2u + (tid & 7) * 16u;
+    // GATHER: one descriptor over all of A; a lane's offset per chunk is its gathered row (beyond every size for rows
+    // past the tile's end), the position along k travels in the scalar offset
+    uint32_t a_gather[GATHER ? 8 : 1];
+    static_assert(!(GATHER && A_KS), "the row gather belongs to the [M][K] form");
+    const __amdgpu_buffer_rsrc_t a_all = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t*>(p.A), 0, static_cast<int>(static_cast<uint32_t>(GATHER ? p.a_rows : 0) * static_cast<uint32_t>(p.lda) * 2u), 0x00020000);
+    if constexpr (GATHER) {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const int r = m0 + 32 * c + (tid >> 3);
+            a_gather[c] = r < m_end ? static_cast<uint32_t>(p.a_row_index[r]) * static_cast<uint32_t>(p.lda) * 2u + (tid & 7) * 16u : kOutside;
+        }
+    }
     // NT with a period: where tile ks of the k range starts in B's columns
     const int b_period = B_KC && p.b_k_period ? p.b_k_period : 0x7fffffff;
     int kb_load = 0;              // ... for the tile the next load_one calls fetch (set by the callers)
@@ -187,6 +205,10 @@ void k_gemm_bf16(const BfArgs p) {
         if constexpr (c < NA) {
             if constexpr (A_KS) {
                 ra[c] = load_rows(p.A, p.lda, k0 + 8 * c, k_end, m0, a_lane_ks);
+            } else if constexpr (GATHER) {
+                const uint32_t off = k0 + (tid & 7) * 8 < k_end ? a_gather[c] : kOutside;
+                const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(a_all, static_cast<int>(off), k0 * 2, 0);
+                ra[c] = make_uint4(v.x, v.y, v.z, v.w);
             } else {
                 const uint32_t off = k0 + (tid & 7) * 8 < k_end ? a_lane_kc : kOutside;
                 ra[c] = load_rows(p.A, p.lda, m0 + 32 * c, m_end, k0, off);
@@ -327,11 +349,11 @@ void k_gemm_bf16(const BfArgs p) {
     }
 }
 
-template <bool A_KS, int OUT, bool GROUPED, bool B_KC = false>
+template <bool A_KS, int OUT, bool GROUPED, bool B_KC = false, bool GATHER = false>
 int launch(const BfArgs& p, dim3 grid, hipStream_t st) {
     static std::once_flag once;
     hipError_t attr = hipSuccess;
-    auto kern = k_gemm_bf16<A_KS, OUT, GROUPED, B_KC>;
+    auto kern = k_gemm_bf16<A_KS, OUT, GROUPED, B_KC, GATHER>;
     std::call_once(once, [&] {
         attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
     });
@@ -411,15 +433,17 @@ int gemm_tn(int M, int N, int K, int E, const int* counts, const int* offsets, c
 }  // namespace
 
 // C[r, :] = sum over terms t of A[r, t*Kb : (t+1)*Kb] . B[expert(r)]^T: the forward-pass form, A [total_rows, terms*Kb]
-// with its rows grouped by expert, B [num_experts, N, Kb] as a weight matrix lies in memory, C bf16 or fp32 [total, N];
+// with its rows grouped by expert (or, with d_a_row_index, gathered from the a_rows rows of A: compact row r is row
+// d_a_row_index[r]), B [num_experts, N, Kb] as a weight matrix lies in memory, C bf16 or fp32 [total, N];
 // d_tile_map is the table build_tile_map made for these counts.  Kb % 8 == 0 (% 64 with several terms), N % 8 == 0.
-int grouped_gemm_bf16_nt(int total_rows, int N, int Kb, int terms, int num_experts, const uint16_t* A, int lda,
-                         const uint16_t* B, void* C, int ldc, bool c_is_f32, const int* d_tile_map, cf_stream_t stream) {
+int grouped_gemm_bf16_nt(int total_rows, int N, int Kb, int terms, int num_experts, const uint16_t* A, int a_rows, int lda,
+                         const int* d_a_row_index, const uint16_t* B, void* C, int ldc, bool c_is_f32, const int* d_tile_map,
+                         cf_stream_t stream) {
     if (total_rows <= 0 || N <= 0 || num_experts <= 0) return CF_OK;
-    if (!A || !B || !C || !d_tile_map || terms < 1) return CF_ERR_INVALID_ARG;
+    if (!A || !B || !C || !d_tile_map || terms < 1 || a_rows < 0) return CF_ERR_INVALID_ARG;
     const long long K = static_cast<long long>(terms) * Kb;
     if ((terms > 1 ? Kb % kMaxTK : Kb % 8) != 0 || Kb <= 0 || lda < K || ldc < N || N % 8 != 0 || !operands_ok(A, lda, B, Kb, C, ldc, c_is_f32 ? 4 : 2) ||
-        static_cast<size_t>(total_rows) * lda >= (1ull << 30) || static_cast<size_t>(N) * Kb >= (1ull << 30))
+        static_cast<size_t>(d_a_row_index ? a_rows : total_rows) * lda >= (1ull << 30) || static_cast<size_t>(N) * Kb >= (1ull << 30))
         return CF_ERR_UNSUPPORTED;
     BfArgs p{};
     p.A = A; p.lda = lda; p.B = B; p.ldb = Kb; p.C = C; p.ldc = ldc;
@@ -429,9 +453,15 @@ int grouped_gemm_bf16_nt(int total_rows, int N, int Kb, int terms, int num_exper
     p.tile_map = d_tile_map;
     p.b_expert_stride = static_cast<long long>(N) * Kb;
     p.b_k_period = terms > 1 ? Kb : 0;
+    p.a_row_index = d_a_row_index;
+    p.a_rows = a_rows;
     const long long total = static_cast<long long>(p.tiles_m) * p.tiles_n;
     const dim3 grid(static_cast<unsigned>(8 * ((total + 7) / 8)));
     hipStream_t st = as_stream(stream);
+    if (d_a_row_index) {
+        if (!c_is_f32) return CF_ERR_UNSUPPORTED;      // the one caller stores fp32
+        return launch<false, OUT_STORE_F32, true, true, true>(p, grid, st);
+    }
     return c_is_f32 ? launch<false, OUT_STORE_F32, true, true>(p, grid, st) : launch<false, OUT_STORE_BF16, true, true>(p, grid, st);
 }
 }  // namespace cf

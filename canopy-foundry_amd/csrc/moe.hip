@@ -7,6 +7,7 @@
 // by (value descending, index ascending), and row lists are filled in ascending row
 // order by a scan instead of atomics.
 #include "common.hpp"
+#include "internal.hpp"
 
 #include <mutex>
 #include <type_traits>
@@ -1450,16 +1451,15 @@ int cf_moe_grouped_swiglu_forward_fp8(const void* d_hidden_e4m3, const float* d_
     // the compact index for the gather and, when the workspace holds it, its inverse for the unpermute: one launch
     const bool indexed = sizeof(int) * static_cast<size_t>(rows) * num_experts <= w.slot_bytes;
     int* slot = indexed ? reinterpret_cast<int*>(base + w.slot) : nullptr;
-    {
-        const dim3 grid(ceil_div(rows, kThreads) < 16 ? ceil_div(rows, kThreads) : 16, num_experts);
-        k_compact_index<<<grid, kThreads, 0, as_stream(stream)>>>(d_counts, d_offsets, d_row_indices, rows, index, slot, num_experts);
-    }
+    // with the tile table of both projections in the same launch
+    bank_setup(d_counts, d_row_indices, rows, num_experts, total_selected_rows, nullptr, index, slot,
+               reinterpret_cast<int*>(base + w.tile_map), as_stream(stream));
     int rc = launch_status();
     if (rc) return rc;
     // gate/up: rows gathered through the compact index (the token permute is fused into the operand fetch)
-    rc = cf_fp8_grouped_gemm_nt_bf16_ex(total_selected_rows, Ie, H, num_experts, d_counts, d_offsets, d_hidden_e4m3, rows, H, index,
-                                        d_hidden_descale, d_w_gate, d_w_gate_descale, CF_SCALE_ROW_COL, CF_EPI_SILU_GATE,
-                                        d_w_up, d_w_up_descale, act, Ie, base + w.tile_map, map_bytes, stream);
+    rc = grouped_gemm_nt_bf16(total_selected_rows, Ie, H, num_experts, d_counts, d_offsets, d_hidden_e4m3, rows, H, index,
+                              d_hidden_descale, d_w_gate, d_w_gate_descale, CF_SCALE_ROW_COL, CF_EPI_SILU_GATE, d_w_up, d_w_up_descale,
+                              act, Ie, base + w.tile_map, map_bytes, false, 0, stream);
     if (rc) return rc;
     rc = cf_fp8_quantize_rows(act, total_selected_rows, Ie, 0, actq, act_scale, act_descale, stream);
     if (rc) return rc;
@@ -1538,10 +1538,8 @@ int cf_moe_grouped_gelu_forward_fp8(const void* d_hidden, const float* d_fcin_de
     hipStream_t st = as_stream(stream);
     const bool indexed = sizeof(int) * static_cast<size_t>(rows) * num_experts <= w.s.slot_bytes;
     int* slot = indexed ? reinterpret_cast<int*>(base + w.s.slot) : nullptr;
-    {
-        const dim3 grid(ceil_div(rows, kThreads) < 16 ? ceil_div(rows, kThreads) : 16, num_experts);
-        k_compact_index<<<grid, kThreads, 0, st>>>(d_counts, d_offsets, d_row_indices, rows, index, slot, num_experts);
-    }
+    bank_setup(d_counts, d_row_indices, rows, num_experts, total_selected_rows, nullptr, index, slot,
+               reinterpret_cast<int*>(base + w.s.tile_map), st);
     int rc = launch_status();
     if (rc) return rc;
     {
@@ -1554,7 +1552,7 @@ int cf_moe_grouped_gelu_forward_fp8(const void* d_hidden, const float* d_fcin_de
     // fc_in: token rows gathered through the compact index in the operand fetch
     rc = grouped_gemm_nt_bf16(total_selected_rows, Ie, H, num_experts, d_counts, d_offsets, d_hidden, rows, H, index, hidden_descale,
                               d_fc_in_w, in_descale, CF_SCALE_ROW_COL, CF_EPI_NONE, nullptr, nullptr, act, Ie, base + w.s.tile_map,
-                              map_bytes, true, fcin_is_e5m2 ? 1 : 0, stream);
+                              map_bytes, false, fcin_is_e5m2 ? 1 : 0, stream);
     if (rc) return rc;
     // gelu_forward and the per-token quantize in one pass over the bf16 projections
     rc = cf_gelu_quantize_rows_e4m3(act, total_selected_rows, Ie, actq, act_scale, act_descale, stream);

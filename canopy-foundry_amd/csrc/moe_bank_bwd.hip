@@ -24,6 +24,7 @@
 // Nothing here is a kernel of its own except the clearing of the route-weight gradient: the stages are the library's
 // entry points, enqueued on one stream with no host synchronisation.
 #include "common.hpp"
+#include "internal.hpp"
 
 namespace cf {
 namespace {

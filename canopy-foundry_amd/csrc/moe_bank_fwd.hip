@@ -20,6 +20,7 @@
 
 #include "cf_fp8.h"
 #include "common.hpp"
+#include "internal.hpp"
 
 namespace cf {
 namespace {
@@ -113,11 +114,11 @@ FwdWs fwd_layout(int rows, int total_rows, int num_experts, int H, int Ie, bool 
     w.off[CF_MOE_FWD_WS_SLOT] = off; off = up(off + w.slot_bytes);
     w.off[CF_MOE_FWD_WS_PRE] = off; off = up(off + sizeof(float) * T * Ie);
     if (bf16_form) {
-        // two bf16 terms per value, no scales; the gathered token rows
+        // two bf16 terms per value, no scales
         w.off[CF_MOE_FWD_WS_SPLIT] = off; off = up(off + 2 * 2 * T * Ie);
         w.off[CF_MOE_FWD_WS_SPLIT_DESCALE] = off;
         w.off[CF_MOE_FWD_WS_Y] = off; off = up(off + sizeof(float) * T * H);
-        w.off[CF_MOE_FWD_WS_X] = off; off = up(off + 2 * T * H);
+        w.off[CF_MOE_FWD_WS_X] = off;
     } else {
         w.off[CF_MOE_FWD_WS_SPLIT] = off; off = up(off + kTerms * T * Ie);
         w.off[CF_MOE_FWD_WS_SPLIT_DESCALE] = off; off = up(off + sizeof(float) * T);
@@ -231,8 +232,8 @@ int cf_moe_grouped_expert_forward_fp8_ws(const void* d_hidden, const float* d_fc
     return unpermute_f32(d_mixed, y, d_route_weights, slot, d_counts, offsets, d_row_indices, rows, num_experts, H, st);
 }
 
-// moe_grouped_expert_forward_bf16 (kernels.hpp:400-407) with a workspace: the same pipeline on bf16 operands.  The
-// token rows are gathered, fc_in is one grouped bf16 GEMM with fp32 output, the GELU output goes to fc_out as two bf16
+// moe_grouped_expert_forward_bf16 (kernels.hpp:400-407) with a workspace: the same pipeline on bf16 operands.
+// fc_in is one grouped bf16 GEMM that gathers the token rows in its operand fetch, fp32 output, the GELU output goes to fc_out as two bf16
 // terms side by side (value = head + remainder to 2^-17) against the same weight columns, K = 2 Ie, so both terms add
 // in the fp32 accumulator; y stays fp32 until the ordered add.
 int cf_moe_grouped_expert_forward_bf16_workspace(int rows, int total_selected_rows, int num_experts, int H, int Ie,
@@ -260,7 +261,7 @@ int cf_moe_grouped_expert_forward_bf16_ws(const uint16_t* d_hidden, const float*
     if (rows == 0 || num_experts == 0 || H == 0 || Ie == 0 || total_selected_rows == 0) return CF_OK;
     if (!d_hidden || !d_route_weights || !d_counts || !d_row_indices || !d_fc_in_w || !d_fc_out_w || !d_mixed) return CF_ERR_INVALID_ARG;
     const bool staged = staged_shape_bf16(H, Ie) && aligned16(d_hidden) && aligned16(d_fc_in_w) && aligned16(d_fc_out_w) &&
-                        aligned16(d_mixed) && static_cast<size_t>(total_selected_rows) * H < (1ull << 30) &&
+                        aligned16(d_mixed) && static_cast<size_t>(rows) * H < (1ull << 30) &&
                         static_cast<size_t>(total_selected_rows) * 2 * Ie < (1ull << 30) && static_cast<size_t>(H) * Ie < (1ull << 30);
     if (!staged)
         return cf_moe_grouped_expert_forward_bf16(d_hidden, d_route_weights, d_counts, d_offsets, d_row_indices, d_fc_in_w, d_fc_out_w,
@@ -275,15 +276,14 @@ int cf_moe_grouped_expert_forward_bf16_ws(const uint16_t* d_hidden, const float*
     float* pre = reinterpret_cast<float*>(base + w.off[CF_MOE_FWD_WS_PRE]);
     uint16_t* split = reinterpret_cast<uint16_t*>(base + w.off[CF_MOE_FWD_WS_SPLIT]);
     float* y = reinterpret_cast<float*>(base + w.off[CF_MOE_FWD_WS_Y]);
-    uint16_t* xg = reinterpret_cast<uint16_t*>(base + w.off[CF_MOE_FWD_WS_X]);
     hipStream_t st = as_stream(stream);
 
     bank_setup(d_counts, d_row_indices, rows, num_experts, total_selected_rows, offsets, index, slot, tile_map, st);
     int rc = launch_status();
     if (rc) return rc;
-    rc = cf_moe_gather_rows_bf16(d_hidden, xg, index, total_selected_rows, H, stream);
-    if (rc) return rc;
-    rc = grouped_gemm_bf16_nt(total_selected_rows, Ie, H, 1, num_experts, xg, H, d_fc_in_w, pre, Ie, true, tile_map, stream);
+    // the token permute rides in fc_in's operand fetch
+    rc = grouped_gemm_bf16_nt(total_selected_rows, Ie, H, 1, num_experts, d_hidden, rows, H, index, d_fc_in_w, pre, Ie, true, tile_map,
+                              stream);
     if (rc) return rc;
     {
         const size_t n = static_cast<size_t>(total_selected_rows) * (Ie / 4);
@@ -292,7 +292,8 @@ int cf_moe_grouped_expert_forward_bf16_ws(const uint16_t* d_hidden, const float*
         rc = launch_status();
         if (rc) return rc;
     }
-    rc = grouped_gemm_bf16_nt(total_selected_rows, H, Ie, 2, num_experts, split, 2 * Ie, d_fc_out_w, y, H, true, tile_map, stream);
+    rc = grouped_gemm_bf16_nt(total_selected_rows, H, Ie, 2, num_experts, split, total_selected_rows, 2 * Ie, nullptr, d_fc_out_w, y, H,
+                              true, tile_map, stream);
     if (rc) return rc;
     return unpermute_f32(d_mixed, y, d_route_weights, slot, d_counts, offsets, d_row_indices, rows, num_experts, H, st);
 }

@@ -569,7 +569,7 @@ int cf_moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_fcin_
  * d_workspace 256-byte aligned; cf_moe_grouped_expert_forward_fp8_workspace gives its size and, when
  * `offsets` is not null, the byte offsets of the intermediates (CF_MOE_FWD_WS_* order), which stay valid
  * after the call: pre [total, Ie] fp32, split [total, 3 Ie] E4M3, split_descale [total] fp32, y [total, H] fp32,
- * experts back to back (CF_MOE_FWD_WS_X is used by the bf16 form only). */
+ * experts back to back (CF_MOE_FWD_WS_X is reserved and has no bytes). */
 enum {
     CF_MOE_FWD_WS_TILE_MAP = 0, CF_MOE_FWD_WS_OFFSETS, CF_MOE_FWD_WS_INDEX, CF_MOE_FWD_WS_SLOT, CF_MOE_FWD_WS_PRE,
     CF_MOE_FWD_WS_SPLIT, CF_MOE_FWD_WS_SPLIT_DESCALE, CF_MOE_FWD_WS_Y, CF_MOE_FWD_WS_X, CF_MOE_FWD_WS_COUNT
@@ -587,8 +587,8 @@ int cf_moe_grouped_expert_forward_fp8_ws(const void* d_hidden, const float* d_fc
 
 /* moe_grouped_expert_forward_bf16 (kernels.hpp:400-407) with a workspace: the same arguments and contract as
  * cf_moe_grouped_expert_forward_bf16, run as whole-matrix launches when H % 8 == 0, Ie % 64 == 0 and the
- * operands are 16-byte aligned (other shapes are passed on to that function).  The selected token rows are
- * gathered (x, CF_MOE_FWD_WS_X), fc_in is one grouped bf16 GEMM with fp32 output (pre), the GELU (fp32, erf to
+ * operands are 16-byte aligned (other shapes are passed on to that function).  fc_in is one grouped bf16 GEMM
+ * that gathers the selected token rows in its operand fetch, fp32 output (pre), the GELU (fp32, erf to
  * 1.5e-7 absolute) is written as two bf16 terms side by side (split [total, 2 Ie]: bf16(g) and bf16(g - bf16(g)),
  * 16 significand bits), fc_out is one grouped bf16 GEMM over K = 2 Ie against the same weight columns, fp32
  * out (y), then the ordered add into d_mixed as in cf_moe_grouped_expert_forward_fp8_ws, with the same one

@@ -274,7 +274,6 @@ def test_staged_bf16_bank_stage_by_stage(cf, dev, rows, E, k, H, Ie, zero):
     index = take("INDEX", np.int32, T)
     assert np.array_equal(index, np.concatenate([b.idx[e, : b.counts[e]] for e in range(E)]))
     expert = np.repeat(np.arange(E), b.counts)
-    assert np.array_equal(take("X", np.uint16, T * H).reshape(T, H), b.hidden[index]), "gathered token rows"
 
     hx = orc.bf16_to_f32(b.hidden).astype(np.float64)
     win = orc.bf16_to_f32(b.win).astype(np.float64)

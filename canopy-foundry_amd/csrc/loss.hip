@@ -3,7 +3,8 @@
 //
 // The reference (kernels/cross_entropy.cu:201-305) runs one 128-thread block per row that reads the row three
 // times (max, sum of exp, gradient); the FP8 path then reads the bf16 gradient once more to quantize it
-// (src/trainer.cu:8053-8058).  Here a 256-lane workgroup keeps a row of up to 32768 logits in registers: HBM
+// (src/trainer.cu:8053-8058).  Here a 256-lane workgroup keeps a row of up to 32768 logits in registers (a 1024-lane
+// one a row of up to 131072): HBM
 // sees 2 B read + 2 B (bf16 gradient, which the weight-gradient GEMM needs) + 1 B (E5M2) written per element.
 //
 // exp and log run on the hardware exp2 / log2 units (about 1 ulp; CUDA's expf / logf bits cannot be reproduced
@@ -15,6 +16,7 @@ namespace cf {
 namespace {
 
 constexpr int kCeThreads = 256;
+constexpr int kCeWide = 1024;                          // lanes per row for rows beyond 32768 logits
 constexpr int kCeMaxChunks = 16;                       // 8-element chunks per lane: rows up to 32768 logits
 constexpr float kLog2e = 1.44269504088896340736f, kLn2 = 0.69314718055994530942f;
 
@@ -55,17 +57,19 @@ __device__ __forceinline__ void opaque_words(const uint4& v, uint32_t (&w)[4]) {
     asm volatile("" : "+v"(w[0]), "+v"(w[1]), "+v"(w[2]), "+v"(w[3]));
 }
 
-// Row in registers: V % 8 == 0, V <= 32768, 16-byte aligned rows (8-byte for the fp8 gradient).
-template <bool QUANT>
-__global__ __launch_bounds__(kCeThreads) void k_ce_rows(const CeArgs p) {
-    __shared__ float sh[kCeThreads / 64];
+// Row in registers: V % 8 == 0, V <= 128 T, 16-byte aligned rows (8-byte for the fp8 gradient).  T lanes per row: 256
+// for rows up to 32768 logits, 1024 (a CU's sixteen wavefronts, 128 registers each) for rows up to 131072, so that a
+// 128k vocabulary is still read from memory once.
+template <bool QUANT, int T>
+__global__ __launch_bounds__(T) void k_ce_rows(const CeArgs p) {
+    __shared__ float sh[T / 64];
     const int tid = threadIdx.x, V = p.V, nchunks = V / 8;
     const size_t row = blockIdx.x;
     const int label = p.labels[row];
     uint16_t* grow = p.grad + row * V;
     uint8_t* qrow = QUANT ? p.grad8 + row * V : nullptr;
     if (label < 0) {                                     // ignored token: zero gradient, no loss (:237-241)
-        for (int c = tid; c < nchunks; c += kCeThreads) {
+        for (int c = tid; c < nchunks; c += T) {
             reinterpret_cast<uint4*>(grow)[c] = make_uint4(0, 0, 0, 0);
             if constexpr (QUANT) reinterpret_cast<uint2*>(qrow)[c] = make_uint2(0, 0);
         }
@@ -76,7 +80,7 @@ __global__ __launch_bounds__(kCeThreads) void k_ce_rows(const CeArgs p) {
     float m = -3.402823466e38f;
 #pragma unroll
     for (int j = 0; j < kCeMaxChunks; ++j) {
-        const int c = tid + j * kCeThreads;
+        const int c = tid + j * T;
         if (c < nchunks) {
             v[j] = reinterpret_cast<const uint4*>(lrow)[c];
             const uint32_t w[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
@@ -90,7 +94,7 @@ __global__ __launch_bounds__(kCeThreads) void k_ce_rows(const CeArgs p) {
     float s = 0.0f;
 #pragma unroll
     for (int j = 0; j < kCeMaxChunks; ++j) {
-        if (tid + j * kCeThreads < nchunks) {
+        if (tid + j * T < nchunks) {
             uint32_t w[4];
             opaque_words(v[j], w);
 #pragma unroll
@@ -110,7 +114,7 @@ __global__ __launch_bounds__(kCeThreads) void k_ce_rows(const CeArgs p) {
     uint32_t absacc = 0;
 #pragma unroll
     for (int j = 0; j < kCeMaxChunks; ++j) {
-        const int c = tid + j * kCeThreads;
+        const int c = tid + j * T;
         if (c < nchunks) {
             uint32_t w[4];
             opaque_words(v[j], w);
@@ -294,8 +298,9 @@ template <bool QUANT>
 int launch_ce(const CeArgs& p, int rows, hipStream_t st) {
     const bool vec = p.V % 8 == 0 && aligned16(p.logits) && aligned16(p.grad) &&
                      (!QUANT || (reinterpret_cast<uintptr_t>(p.grad8) & 7u) == 0);
-    if (vec && p.V <= kCeMaxChunks * kCeThreads * 8) k_ce_rows<QUANT><<<rows, kCeThreads, 0, st>>>(p);
-    else if (vec)                                    k_ce_rows_stream<QUANT><<<rows, kCeThreads, 0, st>>>(p);
+    if (vec && p.V <= kCeMaxChunks * kCeThreads * 8)      k_ce_rows<QUANT, kCeThreads><<<rows, kCeThreads, 0, st>>>(p);
+    else if (vec && p.V <= kCeMaxChunks * kCeWide * 8)    k_ce_rows<QUANT, kCeWide><<<rows, kCeWide, 0, st>>>(p);
+    else if (vec)                                         k_ce_rows_stream<QUANT><<<rows, kCeThreads, 0, st>>>(p);
     else                                             k_ce_rows_generic<QUANT><<<rows, kCeThreads, 0, st>>>(p);
     return launch_status();
 }

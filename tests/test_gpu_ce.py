@@ -33,7 +33,7 @@ def check_grad(got_bits, logits, labels, n_valid):
     return ref_loss
 
 
-@pytest.mark.parametrize("rows,V", [(1, 8), (9, 1000), (33, 4096), (7, 4099), (5, 32000), (3, 32768), (2, 50264), (2, 50257), (2, 128256)])
+@pytest.mark.parametrize("rows,V", [(1, 8), (9, 1000), (33, 4096), (7, 4099), (5, 32000), (3, 32768), (2, 50264), (2, 50257), (2, 128256), (2, 131072), (2, 131080)])
 def test_cross_entropy_chunk(cf, dev, rows, V):
     case(f"cross entropy rows={rows} V={V}")
     logits, labels = make(rows, V, rows * 13 + V)
@@ -57,7 +57,7 @@ def test_cross_entropy_chunk(cf, dev, rows, V):
     assert torch.equal(x.view(torch.int16), grad.view(torch.int16))
 
 
-@pytest.mark.parametrize("rows,V", [(12, 4096), (6, 32000), (5, 1001), (2, 40000), (3, 128256)])
+@pytest.mark.parametrize("rows,V", [(12, 4096), (6, 32000), (5, 1001), (2, 40000), (3, 128256), (2, 131080)])
 def test_cross_entropy_chunk_fused_with_e5m2_quantize(cf, dev, rows, V):
     case(f"cross entropy + e5m2 quantize rows={rows} V={V}")
     logits, labels = make(rows, V, rows * 17 + V)

@@ -164,6 +164,13 @@ def test_staged_bank_stage_by_stage(cf, dev, rows, E, k, H, Ie, e5m2, zero):
         worst = np.abs(y[sel] - want) / tol
         print(f"fc_out expert {e}: worst error / tolerance {worst.max():.3f}")
         assert worst.max() <= 1.0, f"fc_out expert {e}: worst {worst.max():.3f}"
+        # end to end from the exact-erf GELU in double: what the split and the matrix cores lose together, against what
+        # rounding the activations to bf16 would lose
+        exact = (g[sel] @ wout[e].T) * float(b.d_out)
+        lost = np.sqrt(((y[sel] - exact) ** 2).sum() / (exact ** 2).sum())
+        lost_bf16 = np.sqrt((((bf[sel] @ wout[e].T) * float(b.d_out) - exact) ** 2).sum() / (exact ** 2).sum())
+        print(f"fc_out expert {e}: rel L2 from exact GELU {lost:.2e}, with bf16 activations {lost_bf16:.2e}")
+        assert lost < 0.1 * lost_bf16
 
     check_result(b, mixed)
 

@@ -233,9 +233,9 @@ int cf_moe_grouped_expert_forward_fp8_ws(const void* d_hidden, const float* d_fc
 }
 
 // moe_grouped_expert_forward_bf16 (kernels.hpp:400-407) with a workspace: the same pipeline on bf16 operands.
-// fc_in is one grouped bf16 GEMM that gathers the token rows in its operand fetch, fp32 output, the GELU output goes to fc_out as two bf16
-// terms side by side (value = head + remainder to 2^-17) against the same weight columns, K = 2 Ie, so both terms add
-// in the fp32 accumulator; y stays fp32 until the ordered add.
+// fc_in is one grouped bf16 GEMM that gathers the token rows in its operand fetch, fp32 output; the GELU output goes
+// to fc_out as two bf16 terms side by side (value = head + remainder to 2^-17) against the same weight columns,
+// K = 2 Ie, so both terms add in the fp32 accumulator; y stays fp32 until the ordered add.
 int cf_moe_grouped_expert_forward_bf16_workspace(int rows, int total_selected_rows, int num_experts, int H, int Ie,
                                                  size_t* offsets, size_t* bytes) {
     if (rows < 0 || total_selected_rows < 0 || num_experts < 0 || H < 0 || Ie < 0 || !bytes) return CF_ERR_INVALID_ARG;

@@ -41,4 +41,16 @@ int unpermute_f32(uint16_t* d_mixed, const float* d_y, const float* d_route_weig
 void bank_setup(const int* d_counts, const int* d_row_indices, int rows, int num_experts, int total_rows, int* d_offsets,
                 int* d_compact_index, int* d_slot_index, int* tile_map, hipStream_t stream);
 
+// The one-kernel forms of the GELU expert bank (moe.hip): what cf_moe_grouped_expert_forward_fp8 / _bf16 run when no
+// workspace is at hand.  Arguments checked by the callers.
+int expert_forward_fp8_one_kernel(const void* d_hidden, const float* d_fcin_descale, int fcin_is_e5m2, const float* d_route_weights,
+                                  const int* d_counts, const int* d_row_indices, const void* d_fc_in_w, const float* d_fc_in_descale,
+                                  const void* d_fc_out_w, const float* d_fc_out_descale, uint16_t* d_mixed, int rows, int H, int Ie,
+                                  int num_experts, cf_stream_t stream);
+int expert_forward_bf16_one_kernel(const uint16_t* d_hidden, const float* d_route_weights, const int* d_counts,
+                                   const int* d_row_indices, const uint16_t* d_fc_in_w, const uint16_t* d_fc_out_w, uint16_t* d_mixed,
+                                   int rows, int H, int Ie, int num_experts, cf_stream_t stream);
+// The buffer lent through cf_set_workspace, (null, 0) when there is none (moe_bank_fwd.hip).
+void lent_workspace(void** d_workspace, size_t* bytes);
+
 }  // namespace cf

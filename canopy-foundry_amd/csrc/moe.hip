@@ -1571,13 +1571,32 @@ int cf_moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_fcin_
                                       const int* d_row_indices, const void* d_fc_in_w, const float* d_fc_in_descale,
                                       const void* d_fc_out_w, const float* d_fc_out_descale, uint16_t* d_mixed, int rows,
                                       int H, int Ie, int num_experts, int total_selected_rows, cf_stream_t stream) {
-    (void)d_offsets;               // as in the reference, the tiled form needs neither
-    (void)total_selected_rows;
     if (rows < 0 || H < 0 || Ie < 0 || num_experts < 0) return CF_ERR_INVALID_ARG;
     if (rows == 0 || num_experts == 0 || H == 0 || Ie == 0) return CF_OK;
     if (!d_hidden || !d_fcin_descale || !d_route_weights || !d_counts || !d_row_indices || !d_fc_in_w || !d_fc_in_descale ||
         !d_fc_out_w || !d_fc_out_descale || !d_mixed)
         return CF_ERR_INVALID_ARG;
+    // a lent workspace that is large enough sends the call to the whole-matrix form (which needs the true row total)
+    void* lent = nullptr;
+    size_t lent_bytes = 0, need = 0;
+    lent_workspace(&lent, &lent_bytes);
+    if (lent && total_selected_rows > 0 &&
+        cf_moe_grouped_expert_forward_fp8_workspace(rows, total_selected_rows, num_experts, H, Ie, nullptr, &need) == CF_OK && need > 0 &&
+        need <= lent_bytes)
+        return cf_moe_grouped_expert_forward_fp8_ws(d_hidden, d_fcin_descale, fcin_is_e5m2, d_route_weights, d_counts, d_offsets,
+                                                    d_row_indices, d_fc_in_w, d_fc_in_descale, d_fc_out_w, d_fc_out_descale, d_mixed,
+                                                    rows, H, Ie, num_experts, total_selected_rows, lent, lent_bytes, stream);
+    return expert_forward_fp8_one_kernel(d_hidden, d_fcin_descale, fcin_is_e5m2, d_route_weights, d_counts, d_row_indices, d_fc_in_w,
+                                         d_fc_in_descale, d_fc_out_w, d_fc_out_descale, d_mixed, rows, H, Ie, num_experts, stream);
+}
+
+}  // extern "C"
+
+int cf::expert_forward_fp8_one_kernel(const void* d_hidden, const float* d_fcin_descale, int fcin_is_e5m2,
+                                      const float* d_route_weights, const int* d_counts, const int* d_row_indices,
+                                      const void* d_fc_in_w, const float* d_fc_in_descale, const void* d_fc_out_w,
+                                      const float* d_fc_out_descale, uint16_t* d_mixed, int rows, int H, int Ie, int num_experts,
+                                      cf_stream_t stream) {
     const bool mfma_ok = H % 128 == 0 && Ie % 64 == 0 && aligned16(d_hidden) && aligned16(d_fc_in_w) && aligned16(d_fc_out_w) &&
                          (reinterpret_cast<uintptr_t>(d_mixed) & 7u) == 0;
     // 32 rows per workgroup where the output blocks fit a wavefront's registers and LDS holds the hidden rows plus
@@ -1642,15 +1661,32 @@ int cf_moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_fcin_
                                            as_stream(stream));
 }
 
+extern "C" {
+
 int cf_moe_grouped_expert_forward_bf16(const uint16_t* d_hidden, const float* d_route_weights, const int* d_counts,
                                        const int* d_offsets, const int* d_row_indices, const uint16_t* d_fc_in_w,
                                        const uint16_t* d_fc_out_w, uint16_t* d_mixed, int rows, int H, int Ie,
                                        int num_experts, int total_selected_rows, cf_stream_t stream) {
-    (void)d_offsets;               // as in the reference, the tiled form needs neither
-    (void)total_selected_rows;
     if (rows < 0 || H < 0 || Ie < 0 || num_experts < 0) return CF_ERR_INVALID_ARG;
     if (rows == 0 || num_experts == 0 || H == 0 || Ie == 0) return CF_OK;
     if (!d_hidden || !d_route_weights || !d_counts || !d_row_indices || !d_fc_in_w || !d_fc_out_w || !d_mixed) return CF_ERR_INVALID_ARG;
+    void* lent = nullptr;
+    size_t lent_bytes = 0, need = 0;
+    lent_workspace(&lent, &lent_bytes);
+    if (lent && total_selected_rows > 0 &&
+        cf_moe_grouped_expert_forward_bf16_workspace(rows, total_selected_rows, num_experts, H, Ie, nullptr, &need) == CF_OK && need > 0 &&
+        need <= lent_bytes)
+        return cf_moe_grouped_expert_forward_bf16_ws(d_hidden, d_route_weights, d_counts, d_offsets, d_row_indices, d_fc_in_w, d_fc_out_w,
+                                                     d_mixed, rows, H, Ie, num_experts, total_selected_rows, lent, lent_bytes, stream);
+    return expert_forward_bf16_one_kernel(d_hidden, d_route_weights, d_counts, d_row_indices, d_fc_in_w, d_fc_out_w, d_mixed, rows, H, Ie,
+                                          num_experts, stream);
+}
+
+}  // extern "C"
+
+int cf::expert_forward_bf16_one_kernel(const uint16_t* d_hidden, const float* d_route_weights, const int* d_counts,
+                                       const int* d_row_indices, const uint16_t* d_fc_in_w, const uint16_t* d_fc_out_w,
+                                       uint16_t* d_mixed, int rows, int H, int Ie, int num_experts, cf_stream_t stream) {
     // the matrix-core form where the shapes are whole MFMA steps and its tile fits the LDS
     const size_t smem_mfma = 2u * kMfmaRows * (static_cast<size_t>(H) + 8) + 4u * kMfmaRows * (static_cast<size_t>(Ie) + 8);
     if (H % 64 == 0 && Ie % 64 == 0 && smem_mfma <= 160 * 1024 && aligned16(d_hidden) && aligned16(d_fc_in_w) && aligned16(d_fc_out_w) &&
@@ -1671,8 +1707,6 @@ int cf_moe_grouped_expert_forward_bf16(const uint16_t* d_hidden, const float* d_
                                           reinterpret_cast<const uint8_t*>(d_fc_in_w), nullptr, reinterpret_cast<const uint8_t*>(d_fc_out_w),
                                           nullptr, d_mixed, rows, H, Ie, num_experts, as_stream(stream));
 }
-
-}  // extern "C"
 
 // mixed[row] += w[row, e] * y[slot(row, e)] over the row's experts in ascending order for fp32 rows of y, one bf16
 // rounding per expert; the slot table when the caller has one, the search of the row lists otherwise

@@ -18,6 +18,8 @@
 
 #include <cstdint>
 
+#include <mutex>
+
 #include "cf_fp8.h"
 #include "common.hpp"
 #include "internal.hpp"
@@ -27,6 +29,11 @@ namespace {
 
 constexpr int kSplitThreads = 256;
 constexpr int kTerms = 3;
+
+// the buffer a caller has lent through cf_set_workspace (one per process: the library is used on one GPU)
+std::mutex g_lent_mutex;
+void* g_lent = nullptr;
+size_t g_lent_bytes = 0;
 
 // Phi(v) = (1 + erf(v / sqrt 2)) / 2 from the rational-exponential form of erfc (Abramowitz & Stegun 7.1.26,
 // absolute error 1.5e-7 on erf: fp32 round-off level): for v < 0 the small tail is computed directly, not as
@@ -157,9 +164,24 @@ __global__ __launch_bounds__(kSplitThreads) void k_gelu_split2_bf16(const float*
 }  // namespace
 }  // namespace cf
 
+// (null, 0) when nothing is lent
+void cf::lent_workspace(void** d_workspace, size_t* bytes) {
+    std::lock_guard<std::mutex> lock(g_lent_mutex);
+    *d_workspace = g_lent;
+    *bytes = g_lent_bytes;
+}
+
 using namespace cf;
 
 extern "C" {
+
+int cf_set_workspace(void* d_workspace, size_t bytes) {
+    if ((d_workspace == nullptr) != (bytes == 0) || (reinterpret_cast<uintptr_t>(d_workspace) & 255u)) return CF_ERR_INVALID_ARG;
+    std::lock_guard<std::mutex> lock(g_lent_mutex);
+    g_lent = d_workspace;
+    g_lent_bytes = bytes;
+    return CF_OK;
+}
 
 int cf_moe_grouped_expert_forward_fp8_workspace(int rows, int total_selected_rows, int num_experts, int H, int Ie,
                                                 size_t* offsets, size_t* bytes) {
@@ -193,9 +215,8 @@ int cf_moe_grouped_expert_forward_fp8_ws(const void* d_hidden, const float* d_fc
                         static_cast<size_t>(total_selected_rows) * kTerms * Ie < (1ull << 32) &&
                         static_cast<size_t>(H) * Ie < (1ull << 32);
     if (!staged)
-        return cf_moe_grouped_expert_forward_fp8(d_hidden, d_fcin_descale, fcin_is_e5m2, d_route_weights, d_counts, d_offsets,
-                                                 d_row_indices, d_fc_in_w, d_fc_in_descale, d_fc_out_w, d_fc_out_descale, d_mixed,
-                                                 rows, H, Ie, num_experts, total_selected_rows, stream);
+        return expert_forward_fp8_one_kernel(d_hidden, d_fcin_descale, fcin_is_e5m2, d_route_weights, d_counts, d_row_indices, d_fc_in_w,
+                                             d_fc_in_descale, d_fc_out_w, d_fc_out_descale, d_mixed, rows, H, Ie, num_experts, stream);
     const FwdWs w = fwd_layout(rows, total_selected_rows, num_experts, H, Ie);
     if (!d_workspace || workspace_bytes < w.total || (reinterpret_cast<uintptr_t>(d_workspace) & 255u)) return CF_ERR_INVALID_ARG;
     auto* base = static_cast<uint8_t*>(d_workspace);
@@ -264,8 +285,8 @@ int cf_moe_grouped_expert_forward_bf16_ws(const uint16_t* d_hidden, const float*
                         aligned16(d_mixed) && static_cast<size_t>(rows) * H < (1ull << 30) &&
                         static_cast<size_t>(total_selected_rows) * 2 * Ie < (1ull << 30) && static_cast<size_t>(H) * Ie < (1ull << 30);
     if (!staged)
-        return cf_moe_grouped_expert_forward_bf16(d_hidden, d_route_weights, d_counts, d_offsets, d_row_indices, d_fc_in_w, d_fc_out_w,
-                                                  d_mixed, rows, H, Ie, num_experts, total_selected_rows, stream);
+        return expert_forward_bf16_one_kernel(d_hidden, d_route_weights, d_counts, d_row_indices, d_fc_in_w, d_fc_out_w, d_mixed, rows,
+                                              H, Ie, num_experts, stream);
     const FwdWs w = fwd_layout(rows, total_selected_rows, num_experts, H, Ie, true);
     if (!d_workspace || workspace_bytes < w.total || (reinterpret_cast<uintptr_t>(d_workspace) & 255u)) return CF_ERR_INVALID_ARG;
     auto* base = static_cast<uint8_t*>(d_workspace);

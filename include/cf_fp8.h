@@ -540,7 +540,7 @@ int cf_moe_grouped_swiglu_forward_fp8(const void* d_hidden_e4m3, const float* d_
  * per-tensor device descales, exact-erf GELU kept in fp32 (not re-quantised), bf16 accumulation
  * by compare-and-swap, so the last bit of d_mixed depends on arrival order as in the reference.
  * fc_in_w [E,Ie,H], fc_out_w [E,H,Ie] E4M3; hidden E4M3 or E5M2.  d_offsets and
- * total_selected_rows are accepted and unused, as in the reference.  With H % 128 == 0,
+ * total_selected_rows are accepted and unused, as in the reference (unless a workspace is lent: cf_set_workspace).  With H % 128 == 0,
  * Ie % 64 == 0, 16-byte aligned operands and 8-byte aligned d_mixed the two projections run on
  * the matrix cores (fp8 MFMA for fc_in; fc_out as bf16 MFMA on a two-term bf16 split of the fp32
  * GELU output, relative error 2^-17, against the weights widened exactly; 32 token rows per
@@ -554,6 +554,15 @@ int cf_moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_fcin_
                                       const float* d_fc_out_descale, uint16_t* d_mixed, int rows,
                                       int H, int Ie, int num_experts, int total_selected_rows,
                                       cf_stream_t stream);
+
+/* Lends the library a device buffer (256-byte aligned) that entry points with the reference's argument lists, which
+ * carry no workspace, may use: cf_moe_grouped_expert_forward_fp8 and cf_moe_grouped_expert_forward_bf16 then take
+ * their whole-matrix forms (the *_ws entry points below) whenever the buffer holds what the *_workspace query
+ * asks for; total_selected_rows must then be the true sum of the counts.  It has no counterpart in the reference
+ * (whose trainer owns one arena for such purposes, Fp8Ctx).  (null, 0) takes the buffer back.  The buffer is shared
+ * by every such call: calls that may overlap in time must be serialised by the caller; calls on one stream are
+ * ordered.  The library never frees or allocates it. */
+int cf_set_workspace(void* d_workspace, size_t bytes);
 
 /* moe_grouped_expert_forward_fp8 (kernels.hpp:400-423, kernels/moe.cu:950-1127) with a workspace: the same
  * arguments and contract as cf_moe_grouped_expert_forward_fp8, run as whole-matrix launches when H % 128 == 0,

@@ -370,3 +370,53 @@ def test_staged_bf16_bank_config5_size(cf, dev):
     all_got = orc.bf16_to_f32(bf16_bits(mixed)).astype(np.float64)
     delta = np.abs(all_got - orc.bf16_to_f32(b.mixed0).astype(np.float64)).mean(axis=1)
     assert delta.min() > 0.1 * np.median(delta) and delta.max() < 10.0 * np.median(delta)
+
+
+# ---- a lent workspace sends the reference's own argument lists to the whole-matrix forms --------------------------
+
+def test_lent_workspace_routes_the_reference_signatures(cf, dev):
+    case("cf_set_workspace: moe_grouped_expert_forward_fp8 / _bf16 under the reference's argument lists")
+    b8 = Bank(dev, 500, 8, 2, 512, 256, False, seed=21)
+    b16 = Bank16(dev, 500, 8, 2, 512, 256, seed=22)
+    want8 = bf16_bits(run(cf, b8)[0])
+    want16 = bf16_bits(run16(cf, b16)[0])
+    _, n8 = workspace(cf, b8)
+    n16 = ctypes.c_size_t()
+    cf.cf_moe_grouped_expert_forward_bf16_workspace(b16.rows, b16.total, b16.E, b16.H, b16.Ie, None, ctypes.byref(n16))
+    nbytes = max(n8, int(n16.value))
+    buf = torch.empty(nbytes + 256, dtype=torch.uint8, device=dev)
+    ptr = buf.data_ptr() + (-buf.data_ptr()) % 256
+    sc = lambda v: torch.tensor([v], dtype=torch.float32, device=dev)
+
+    def plain8(total):
+        mixed = dev_bf16(b8.mixed0, dev)
+        cf.cf_moe_grouped_expert_forward_fp8(dev_arr(b8.hq, dev), sc(b8.d_h), 0, dev_arr(b8.rw, dev), dev_arr(b8.counts, dev), None,
+                                             dev_arr(b8.idx, dev), dev_arr(b8.winq, dev), sc(b8.d_in), dev_arr(b8.woutq, dev), sc(b8.d_out),
+                                             mixed, b8.rows, b8.H, b8.Ie, b8.E, total, stream())
+        torch.cuda.synchronize()
+        return mixed
+
+    def plain16(total):
+        mixed = dev_bf16(b16.mixed0, dev)
+        cf.cf_moe_grouped_expert_forward_bf16(dev_bf16(b16.hidden, dev), dev_arr(b16.rw, dev), dev_arr(b16.counts, dev), None,
+                                              dev_arr(b16.idx, dev), dev_bf16(b16.win, dev), dev_bf16(b16.wout, dev), mixed, b16.rows, b16.H,
+                                              b16.Ie, b16.E, total, stream())
+        torch.cuda.synchronize()
+        return mixed
+
+    assert cf.raw_cf_set_workspace(ptr + 8, nbytes) == -1                    # not 256-byte aligned
+    assert cf.raw_cf_set_workspace(None, nbytes) == -1 and cf.raw_cf_set_workspace(ptr, 0) == -1
+    try:
+        cf.cf_set_workspace(ptr, nbytes)
+        # the whole-matrix forms are deterministic: the same bits as the explicit-workspace calls
+        assert np.array_equal(bf16_bits(plain8(b8.total)), want8)
+        assert np.array_equal(bf16_bits(plain16(b16.total)), want16)
+        # too small for these shapes: the one-kernel forms run, same contract
+        cf.cf_set_workspace(ptr, 4096)
+        check_result(b8, plain8(b8.total))
+        check_result16(b16, plain16(b16.total))
+    finally:
+        cf.cf_set_workspace(None, 0)
+    # taken back: the reference's unused total may be anything again
+    check_result(b8, plain8(b8.rows * b8.k + 5))
+    check_result16(b16, plain16(0))

@@ -1545,28 +1545,39 @@ int dispatch_epi(const GemmArgs& p, int epi, int scale_mode, hipStream_t st) {
     }
 }
 
-// one wavefront: the row tiles of every expert in expert order (lane = expert, prefix sum of the tile counts);
-// each row tile's entry describes its expert: number, row range, first row tile, row-tile count
-// (offsets == nullptr: the experts' rows lie back to back, the first rows are the running sum of the counts)
+// one wavefront: the row tiles of every expert in expert order (lane = expert, prefix sums of the row and tile
+// counts); each row tile's entry describes its expert: number, row range, first row tile, row-tile count
+// (offsets == nullptr: the experts' rows lie back to back, the first rows are the running sum of the counts).
+// total_rows is the caller's bound on the rows the compact buffers hold (the reference's callers pass
+// rows * top_k, src/trainer.cu:6863): an expert's range is cut at it, so that counts which sum to more than the
+// bound cannot send a tile past the end of those buffers.
 __device__ __forceinline__ void build_tile_map_wave(const int* __restrict__ counts, const int* __restrict__ offsets,
-                                                    int num_experts, int max_row_tiles, int* __restrict__ tile_map, int lane) {
+                                                    int num_experts, int max_row_tiles, int total_rows,
+                                                    int* __restrict__ tile_map, int lane) {
     int carry = 0, carry_rows = 0, written = 0;
     for (int e0 = 0; e0 < num_experts; e0 += 64) {
         const int e = e0 + lane;
-        const int cnt = e < num_experts ? counts[e] : 0;
-        const int nt = (cnt + BM - 1) / BM;
-        int incl = nt, incl_rows = cnt;
+        const int cnt = e < num_experts ? max(counts[e], 0) : 0;
+        int incl_rows = cnt;
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
-            const int v = __shfl_up(incl, off, 64), r = __shfl_up(incl_rows, off, 64);
-            if (lane >= off) { incl += v; incl_rows += r; }
+            const int r = __shfl_up(incl_rows, off, 64);
+            if (lane >= off) incl_rows += r;
         }
         const int first = offsets ? (e < num_experts ? offsets[e] : 0) : carry_rows + incl_rows - cnt;
+        const int kept = first >= 0 && first < total_rows ? min(cnt, total_rows - first) : 0;
+        const int nt = (kept + BM - 1) / BM;
+        int incl = nt;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int v = __shfl_up(incl, off, 64);
+            if (lane >= off) incl += v;
+        }
         const int base = carry + incl - nt;
-        if (base + nt <= max_row_tiles) {        // always true for counts that sum to at most the caller's total_rows
+        if (base + nt <= max_row_tiles) {        // always true when the experts' ranges do not overlap
             for (int i = 0; i < nt; ++i) {
                 int* w = tile_map + 1 + kMapWords * (base + i);
-                w[0] = e; w[1] = first; w[2] = first + cnt; w[3] = base; w[4] = nt;
+                w[0] = e; w[1] = first; w[2] = first + kept; w[3] = base; w[4] = nt;
             }
             if (nt > 0) written = max(written, base + nt);
         }
@@ -1579,32 +1590,34 @@ __device__ __forceinline__ void build_tile_map_wave(const int* __restrict__ coun
     if (lane == 0) tile_map[0] = written;
 }
 __global__ __launch_bounds__(64) void k_build_tile_map(const int* __restrict__ counts, const int* __restrict__ offsets,
-                                                       int num_experts, int max_row_tiles, int* __restrict__ tile_map) {
-    build_tile_map_wave(counts, offsets, num_experts, max_row_tiles, tile_map, threadIdx.x);
+                                                       int num_experts, int max_row_tiles, int total_rows,
+                                                       int* __restrict__ tile_map) {
+    build_tile_map_wave(counts, offsets, num_experts, max_row_tiles, total_rows, tile_map, threadIdx.x);
 }
 
 // Everything an expert bank derives from (counts, row lists) in one launch.  Workgroup e < num_experts: the offset
 // of expert e (the sum of the counts before it; stored when the caller wants the array), its row list copied into the compact index at that offset and,
 // when slot_index is given, the inverse entries slot_index[row, e] = position.  The last workgroup: the tile table.
+// Entries at or beyond total_rows (the size of the compact buffers) are left out.
 __global__ __launch_bounds__(256) void k_bank_setup(const int* __restrict__ counts, const int* __restrict__ row_indices, int rows,
-                                                    int num_experts, int max_row_tiles, int* __restrict__ offsets,
+                                                    int num_experts, int max_row_tiles, int total_rows, int* __restrict__ offsets,
                                                     int* __restrict__ compact, int* __restrict__ slot_index,
                                                     int* __restrict__ tile_map) {
     const int e = blockIdx.x, tid = threadIdx.x;
     if (e == num_experts) {
-        if (tid < 64) build_tile_map_wave(counts, nullptr, num_experts, max_row_tiles, tile_map, tid);
+        if (tid < 64) build_tile_map_wave(counts, nullptr, num_experts, max_row_tiles, total_rows, tile_map, tid);
         return;
     }
     __shared__ int part[4];
     int sum = 0;
-    for (int i = tid; i < e; i += 256) sum += counts[i];
+    for (int i = tid; i < e; i += 256) sum += max(counts[i], 0);
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
     if ((tid & 63) == 0) part[tid >> 6] = sum;
     __syncthreads();
     const int base = part[0] + part[1] + part[2] + part[3];
     if (tid == 0 && offsets) offsets[e] = base;
-    const int n = counts[e];
+    const int n = min(counts[e], total_rows - base);      // may be negative: nothing is copied then
     const int* list = row_indices + static_cast<size_t>(e) * rows;
     for (int s = tid; s < n; s += 256) {
         const int row = list[s];
@@ -1819,15 +1832,15 @@ int cf_fp8_grouped_gemm_nt_bf16_static(int total_rows, int N, int K, int num_exp
 
 }  // extern "C"
 
-void cf::build_tile_map(const int* d_counts, const int* d_offsets, int num_experts, int max_row_tiles, int* tile_map,
-                        hipStream_t stream) {
-    k_build_tile_map<<<1, 64, 0, stream>>>(d_counts, d_offsets, num_experts, max_row_tiles, tile_map);
+void cf::build_tile_map(const int* d_counts, const int* d_offsets, int num_experts, int max_row_tiles, int total_rows,
+                        int* tile_map, hipStream_t stream) {
+    k_build_tile_map<<<1, 64, 0, stream>>>(d_counts, d_offsets, num_experts, max_row_tiles, total_rows, tile_map);
 }
 
 void cf::bank_setup(const int* d_counts, const int* d_row_indices, int rows, int num_experts, int total_rows, int* d_offsets,
                     int* d_compact_index, int* d_slot_index, int* tile_map, hipStream_t stream) {
     k_bank_setup<<<num_experts + 1, 256, 0, stream>>>(d_counts, d_row_indices, rows, num_experts, total_rows / BM + num_experts,
-                                                      d_offsets, d_compact_index, d_slot_index, tile_map);
+                                                      total_rows, d_offsets, d_compact_index, d_slot_index, tile_map);
 }
 
 // build_map = false: d_workspace already holds the tile table of these counts and offsets (an earlier call of
@@ -1860,7 +1873,7 @@ int cf::grouped_gemm_nt_bf16(int total_rows, int N, int K, int num_experts, cons
     hipStream_t st = as_stream(stream);
     const int max_row_tiles = total_rows / BM + num_experts;
     int* tile_map = static_cast<int*>(d_workspace);
-    if (build_map) k_build_tile_map<<<1, 64, 0, st>>>(d_counts, d_offsets, num_experts, max_row_tiles, tile_map);
+    if (build_map) k_build_tile_map<<<1, 64, 0, st>>>(d_counts, d_offsets, num_experts, max_row_tiles, total_rows, tile_map);
     GemmArgs p{};
     p.M = total_rows; p.N = N; p.K = K;
     p.A = static_cast<const uint8_t*>(A); p.lda = lda;

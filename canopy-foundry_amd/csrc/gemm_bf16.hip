@@ -352,7 +352,7 @@ void k_gemm_bf16(const BfArgs p) {
 template <bool A_KS, int OUT, bool GROUPED, bool B_KC = false, bool GATHER = false>
 int launch(const BfArgs& p, dim3 grid, hipStream_t st) {
     static std::once_flag once;
-    hipError_t attr = hipSuccess;
+    static hipError_t attr = hipSuccess;      // kept: a failed set-up is reported by every call, not only the first
     auto kern = k_gemm_bf16<A_KS, OUT, GROUPED, B_KC, GATHER>;
     std::call_once(once, [&] {
         attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
@@ -391,7 +391,7 @@ int gemm_nn(int M, int N, int K, int E, const int* counts, const int* offsets, c
         cf_fp8_grouped_gemm_workspace_bytes(M, E, &need);
         if (ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 3u)) return CF_ERR_INVALID_ARG;
         tiles_m = M / TM + E;
-        build_tile_map(counts, offsets, E, tiles_m, static_cast<int*>(ws), st);
+        build_tile_map(counts, offsets, E, tiles_m, M, static_cast<int*>(ws), st);
         p.counts = counts; p.offsets = offsets;
         p.tile_map = static_cast<const int*>(ws);
         p.b_expert_stride = static_cast<long long>(K) * ldb;

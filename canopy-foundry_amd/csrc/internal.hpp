@@ -4,6 +4,13 @@
 
 namespace cf {
 
+// Word layout (4-byte words) of the device block behind a delayed-scaling activation slot (cf_act_slot): the ActSlot
+// scalars of src/trainer.cu:3248-3278 plus two scratch words of the one-launch steady-state step, zero between calls.
+namespace slotw {
+enum { AMAX = 0, SCALE, DESCALE, SCALE_SNAP, DESCALE_SNAP, CALIB_MIN, CALIB_MAX, CURSOR = 8, COUNT = 9, RUNNING = 10, ARRIVED = 11,
+       HISTORY = 16 };
+}
+
 // The grouped GEMM behind cf_fp8_grouped_gemm_nt_bf16_ex, for callers inside the library that run several
 // projections over one routing: build_map = false reuses the tile table an earlier call left in d_workspace;
 // a_is_e5m2 takes E5M2 activations (plain epilogue only).
@@ -29,12 +36,14 @@ int grouped_gemm_bf16_nt(int total_rows, int N, int Kb, int terms, int num_exper
                          cf_stream_t stream);
 // The tile table of a grouped GEMM (k_build_tile_map in gemm.hip): tile_map[0] = number of row tiles of 256 rows,
 // then per row tile (expert, its first row, its end row, its first row tile, its row-tile count), experts back to back.
-void build_tile_map(const int* d_counts, const int* d_offsets, int num_experts, int max_row_tiles, int* tile_map,
-                    hipStream_t stream);
-// The ordered weighted add of fp32 expert outputs into bf16 rows (moe.hip): d_slot_index null = search the row lists.
+// An expert's row range is cut at total_rows, the number of rows the compact buffers hold.
+void build_tile_map(const int* d_counts, const int* d_offsets, int num_experts, int max_row_tiles, int total_rows,
+                    int* tile_map, hipStream_t stream);
+// The ordered weighted add of fp32 expert outputs into bf16 rows (moe.hip): d_slot_index null = search the row lists;
+// slot_limit = the rows d_y holds, pairs whose slot lies at or beyond it are skipped.
 int unpermute_f32(uint16_t* d_mixed, const float* d_y, const float* d_route_weights, const int* d_slot_index,
                   const int* d_counts, const int* d_offsets, const int* d_row_indices, int rows, int num_experts, int H,
-                  hipStream_t st);
+                  int slot_limit, hipStream_t st);
 // One launch for what an expert bank derives from (counts, row lists [num_experts, rows]): the offsets, the compact
 // row index, the (row, expert) -> compact row table (d_offsets and d_slot_index may be null) and the tile table of a grouped GEMM
 // over total_rows rows.
@@ -50,7 +59,5 @@ int expert_forward_fp8_one_kernel(const void* d_hidden, const float* d_fcin_desc
 int expert_forward_bf16_one_kernel(const uint16_t* d_hidden, const float* d_route_weights, const int* d_counts,
                                    const int* d_row_indices, const uint16_t* d_fc_in_w, const uint16_t* d_fc_out_w, uint16_t* d_mixed,
                                    int rows, int H, int Ie, int num_experts, cf_stream_t stream);
-// The buffer lent through cf_set_workspace, (null, 0) when there is none (moe_bank_fwd.hip).
-void lent_workspace(void** d_workspace, size_t* bytes);
 
 }  // namespace cf

@@ -434,7 +434,7 @@ __device__ __forceinline__ void combine_rows(uint16_t* __restrict__ mrow, const 
 template <bool UNIT, class YT = uint16_t>
 __global__ __launch_bounds__(kThreads) void k_unpermute_indexed(uint16_t* __restrict__ mixed, const YT* __restrict__ y,
                                                                 const float* __restrict__ route_weights,
-                                                                const int* __restrict__ slot_index, int E, int H) {
+                                                                const int* __restrict__ slot_index, int E, int H, int slot_limit) {
     __shared__ int sl_slot[64];
     __shared__ float sl_w[64];
     __shared__ int sl_n;
@@ -445,7 +445,10 @@ __global__ __launch_bounds__(kThreads) void k_unpermute_indexed(uint16_t* __rest
             const int e = e0 + t;
             const float w = e < E ? route_weights[static_cast<size_t>(row) * E + e] : 0.0f;
             const bool sel = w > 0.0f;
-            const int slot = sel ? slot_index[static_cast<size_t>(row) * E + e] : -1;
+            // the table is filled for the pairs of the row lists only: a cell that does not name a row of y (a pair the
+            // lists do not hold, or one cut off by the caller's row bound) is skipped
+            int slot = sel ? slot_index[static_cast<size_t>(row) * E + e] : -1;
+            if (slot >= slot_limit) slot = -1;
             const unsigned long long m = __ballot(sel);
             if (sel) {
                 const int pos = __builtin_popcountll(m & ((1ull << t) - 1ull));
@@ -477,7 +480,7 @@ template <bool UNIT, class YT = uint16_t>
 __global__ __launch_bounds__(kThreads) void k_unpermute(uint16_t* __restrict__ mixed, const YT* __restrict__ y,
                                                         const float* __restrict__ route_weights,
                                                         const int* __restrict__ counts, const int* __restrict__ offsets,
-                                                        const int* __restrict__ row_indices, int rows, int E, int H) {
+                                                        const int* __restrict__ row_indices, int rows, int E, int H, int slot_limit) {
     __shared__ int sl_e[64];
     __shared__ int sl_slot[64];
     __shared__ float sl_w[64];
@@ -502,7 +505,8 @@ __global__ __launch_bounds__(kThreads) void k_unpermute(uint16_t* __restrict__ m
         for (int i = wave; i < n; i += kThreads / 64) {
             const int e = sl_e[i];
             const int pos = wave_find_sorted(row_indices + static_cast<size_t>(e) * rows, counts[e], row, lane);
-            if (lane == 0) sl_slot[i] = pos < 0 ? -1 : offsets[e] + pos;     // -1: not in the expert's list, skipped
+            // -1: not in the expert's list, or past the rows y holds: skipped
+            if (lane == 0) sl_slot[i] = pos < 0 || offsets[e] + pos >= slot_limit ? -1 : offsets[e] + pos;
         }
         __syncthreads();
         if (n > 0) combine_rows(mrow, y, H, n, sl_slot, sl_w, t);
@@ -617,7 +621,11 @@ __global__ __launch_bounds__(kThreads) void k_grouped_gelu_wave(const uint8_t* _
     }
     __syncthreads();
     project_rows<R>(xs, H, Ie, [&](size_t i) { return element(w_in, i, false); },
-                    [&](int r, int j, float sum) { act[r * Ie + j] = gelu_fwd(sum * s_in); });
+                    [&](int r, int j, float sum) {
+                        // the bf16 sibling parks the activation as bf16 (kernels/moe.cu:845); the FP8 kernel keeps fp32 (:1031)
+                        const float g = gelu_fwd(sum * s_in);
+                        act[r * Ie + j] = BF16 ? bf16_to_f32(f32_to_bf16(g)) : g;
+                    });
     __syncthreads();
     project_rows<R>(act, Ie, H, [&](size_t i) { return element(w_out, i, false); },
                     [&](int r, int h, float sum) {
@@ -1089,7 +1097,8 @@ __global__ __launch_bounds__(kMfmaThreads) void k_grouped_gelu_fp8_mfma32(const 
 
 // ---- the bf16 sibling on the matrix cores -------------------------------------------------------------
 // moe_grouped_expert_forward_bf16 in the 16-row form above: both projections are v_mfma_f32_16x16x32_bf16 (products
-// of two bf16 values are exact in the fp32 accumulator), fc_out again on the two-term split of the fp32 GELU output.
+// of two bf16 values are exact in the fp32 accumulator); the GELU output is rounded to bf16 before fc_out, as the
+// reference kernel parks it (sh_fcin[j] = __float2bfloat16(g), kernels/moe.cu:845).
 // A 128-byte run of a weight row is 64 elements: a lane fetches 32 bytes = two k-blocks of 8.  H % 64 == 0,
 // Ie % 64 == 0.
 __global__ __launch_bounds__(kMfmaThreads) void k_grouped_gelu_bf16_mfma(const uint16_t* __restrict__ hidden, const float* __restrict__ route_weights,
@@ -1102,8 +1111,7 @@ __global__ __launch_bounds__(kMfmaThreads) void k_grouped_gelu_bf16_mfma(const u
     const int hs = H + 8;                           // row strides in elements: neighbouring rows 16 bytes apart in the banks
     const int as = Ie + 8;
     uint16_t* sh_hidden = reinterpret_cast<uint16_t*>(smem);                          // [16][hs]
-    uint16_t* sh_hi = sh_hidden + kMfmaRows * hs;                                     // [16][as] bf16 head of gelu
-    uint16_t* sh_lo = sh_hi + kMfmaRows * as;                                         // [16][as] bf16 remainder
+    uint16_t* sh_hi = sh_hidden + kMfmaRows * hs;                                     // [16][as] bf16(gelu)
     const int xcd = blockIdx.x % kXcdCount, slot = blockIdx.x / kXcdCount;
     const int e = (slot / tiles_per_expert) * kXcdCount + xcd, tile = slot % tiles_per_expert;
     if (e >= E) return;
@@ -1152,16 +1160,11 @@ __global__ __launch_bounds__(kMfmaThreads) void k_grouped_gelu_bf16_mfma(const u
                 }
             }
         }
-        uint32_t hb[4], lb[4];
+        uint32_t hb[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const float act = gelu_fwd(acc0[r] + acc1[r]);
-            hb[r] = __float_as_uint(act) & 0xffff0000u;
-            lb[r] = f32_to_bf16(act - __uint_as_float(hb[r]));
-        }
+        for (int r = 0; r < 4; ++r) hb[r] = f32_to_bf16(gelu_fwd(acc0[r] + acc1[r]));
         const int at = t * as + n0 + 4 * g;
-        *reinterpret_cast<uint2*>(sh_hi + at) = make_uint2((hb[0] >> 16) | hb[1], (hb[2] >> 16) | hb[3]);
-        *reinterpret_cast<uint2*>(sh_lo + at) = make_uint2(lb[0] | (lb[1] << 16), lb[2] | (lb[3] << 16));
+        *reinterpret_cast<uint2*>(sh_hi + at) = make_uint2(hb[0] | (hb[1] << 16), hb[2] | (hb[3] << 16));
     }
     __syncthreads();
 
@@ -1170,7 +1173,6 @@ __global__ __launch_bounds__(kMfmaThreads) void k_grouped_gelu_bf16_mfma(const u
     const int row = live ? my_rows[t] : 0;
     const float rw = live ? route_weights[static_cast<size_t>(row) * E + e] : 0.0f;
     const uint16_t* ah = sh_hi + t * as + 16 * g;
-    const uint16_t* al = sh_lo + t * as + 16 * g;
     for (int h0 = wave * 16; h0 < H; h0 += kWaves * 16) {
         v4f acc_hi = {0.0f, 0.0f, 0.0f, 0.0f}, acc_lo = {0.0f, 0.0f, 0.0f, 0.0f};
         auto* quad = reinterpret_cast<unsigned long long*>(mixed + static_cast<size_t>(row) * H + h0 + 4 * g);
@@ -1187,13 +1189,10 @@ __global__ __launch_bounds__(kMfmaThreads) void k_grouped_gelu_bf16_mfma(const u
                 if (st < out_steps) {
                     const v8bf ca = wa[j], cb = wb[j];
                     if (st + kMfmaDepth < out_steps) load2(wr + (st + kMfmaDepth) * 64, wa[j], wb[j]);
-                    v8bf ha, hbv, la, lbv;
+                    v8bf ha, hbv;
                     load2(ah + st * 64, ha, hbv);
-                    load2(al + st * 64, la, lbv);
                     acc_hi = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ca, ha, acc_hi, 0, 0, 0);
-                    acc_lo = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ca, la, acc_lo, 0, 0, 0);
-                    acc_hi = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cb, hbv, acc_hi, 0, 0, 0);
-                    acc_lo = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cb, lbv, acc_lo, 0, 0, 0);
+                    acc_lo = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cb, hbv, acc_lo, 0, 0, 0);
                 }
             }
         }
@@ -1330,16 +1329,23 @@ int cf_moe_compact_row_index(const int* d_counts, const int* d_offsets, const in
     return launch_status();
 }
 
-int cf_moe_unpermute_weighted_bf16(uint16_t* d_mixed, const uint16_t* d_compact_out, const float* d_route_weights,
-                                   const int* d_counts, const int* d_offsets, const int* d_row_indices, int rows,
-                                   int num_experts, int H, cf_stream_t stream) {
+// slot_limit: the rows d_compact_out holds; (row, expert) pairs whose slot lies at or beyond it are skipped
+static int unpermute_weighted(uint16_t* d_mixed, const uint16_t* d_compact_out, const float* d_route_weights,
+                              const int* d_counts, const int* d_offsets, const int* d_row_indices, int rows,
+                              int num_experts, int H, int slot_limit, cf_stream_t stream) {
     if (rows < 0 || num_experts < 0 || H < 0) return CF_ERR_INVALID_ARG;
     if (rows == 0 || num_experts == 0 || H == 0) return CF_OK;
     if (!d_mixed || !d_compact_out || !d_route_weights || !d_counts || !d_offsets || !d_row_indices) return CF_ERR_INVALID_ARG;
     if ((H & 7) == 0 && !(aligned16(d_mixed) && aligned16(d_compact_out))) return CF_ERR_UNSUPPORTED;
     k_unpermute<false><<<rows, kThreads, 0, as_stream(stream)>>>(d_mixed, d_compact_out, d_route_weights, d_counts, d_offsets,
-                                                                 d_row_indices, rows, num_experts, H);
+                                                                 d_row_indices, rows, num_experts, H, slot_limit);
     return launch_status();
+}
+int cf_moe_unpermute_weighted_bf16(uint16_t* d_mixed, const uint16_t* d_compact_out, const float* d_route_weights,
+                                   const int* d_counts, const int* d_offsets, const int* d_row_indices, int rows,
+                                   int num_experts, int H, cf_stream_t stream) {
+    return unpermute_weighted(d_mixed, d_compact_out, d_route_weights, d_counts, d_offsets, d_row_indices, rows, num_experts, H,
+                              0x7fffffff, stream);
 }
 
 int cf_moe_scatter_add_rows_bf16(uint16_t* d_dst_full, const uint16_t* d_src_compact, const int* d_row_indices, int n_rows,
@@ -1362,7 +1368,7 @@ int cf_moe_unpermute_add_bf16(uint16_t* d_dst_full, const uint16_t* d_src_compac
     if (!d_dst_full || !d_src_compact || !d_route_weights || !d_counts || !d_offsets || !d_row_indices) return CF_ERR_INVALID_ARG;
     if ((H & 7) == 0 && !(aligned16(d_dst_full) && aligned16(d_src_compact))) return CF_ERR_UNSUPPORTED;
     k_unpermute<true><<<rows, kThreads, 0, as_stream(stream)>>>(d_dst_full, d_src_compact, d_route_weights, d_counts, d_offsets,
-                                                                d_row_indices, rows, num_experts, H);
+                                                                d_row_indices, rows, num_experts, H, 0x7fffffff);
     return launch_status();
 }
 
@@ -1376,20 +1382,26 @@ int cf_moe_build_slot_index(const int* d_counts, const int* d_offsets, const int
     return launch_status();
 }
 
-int cf_moe_unpermute_indexed_bf16(uint16_t* d_mixed, const uint16_t* d_compact_out, const float* d_route_weights,
-                                  const int* d_slot_index, int rows, int num_experts, int H, int unit_weights,
-                                  cf_stream_t stream) {
+static int unpermute_indexed(uint16_t* d_mixed, const uint16_t* d_compact_out, const float* d_route_weights,
+                             const int* d_slot_index, int rows, int num_experts, int H, int unit_weights, int slot_limit,
+                             cf_stream_t stream) {
     if (rows < 0 || num_experts < 0 || H < 0) return CF_ERR_INVALID_ARG;
     if (rows == 0 || num_experts == 0 || H == 0) return CF_OK;
     if (!d_mixed || !d_compact_out || !d_route_weights || !d_slot_index) return CF_ERR_INVALID_ARG;
     if ((H & 7) == 0 && !(aligned16(d_mixed) && aligned16(d_compact_out))) return CF_ERR_UNSUPPORTED;
     if (unit_weights)
         k_unpermute_indexed<true><<<rows, kThreads, 0, as_stream(stream)>>>(d_mixed, d_compact_out, d_route_weights, d_slot_index,
-                                                                            num_experts, H);
+                                                                            num_experts, H, slot_limit);
     else
         k_unpermute_indexed<false><<<rows, kThreads, 0, as_stream(stream)>>>(d_mixed, d_compact_out, d_route_weights, d_slot_index,
-                                                                             num_experts, H);
+                                                                             num_experts, H, slot_limit);
     return launch_status();
+}
+int cf_moe_unpermute_indexed_bf16(uint16_t* d_mixed, const uint16_t* d_compact_out, const float* d_route_weights,
+                                  const int* d_slot_index, int rows, int num_experts, int H, int unit_weights,
+                                  cf_stream_t stream) {
+    return unpermute_indexed(d_mixed, d_compact_out, d_route_weights, d_slot_index, rows, num_experts, H, unit_weights, 0x7fffffff,
+                             stream);
 }
 
 // ---- grouped SwiGLU expert bank -----------------------------------------------------------------
@@ -1468,9 +1480,9 @@ int cf_moe_grouped_swiglu_forward_fp8(const void* d_hidden_e4m3, const float* d_
                               act_descale, d_w_down, d_w_down_descale, CF_SCALE_ROW_COL, CF_EPI_NONE, nullptr, nullptr, y, H,
                               base + w.tile_map, map_bytes, false, 0, stream);
     if (rc) return rc;
-    if (indexed) return cf_moe_unpermute_indexed_bf16(d_mixed, y, d_route_weights, slot, rows, num_experts, H, 0, stream);
-    return cf_moe_unpermute_weighted_bf16(d_mixed, y, d_route_weights, d_counts, d_offsets, d_row_indices, rows,
-                                          num_experts, H, stream);
+    if (indexed) return unpermute_indexed(d_mixed, y, d_route_weights, slot, rows, num_experts, H, 0, total_selected_rows, stream);
+    return unpermute_weighted(d_mixed, y, d_route_weights, d_counts, d_offsets, d_row_indices, rows, num_experts, H,
+                              total_selected_rows, stream);
 }
 
 // ---- grouped GELU expert bank on the matrix cores -----------------------------------------------
@@ -1510,12 +1522,17 @@ int cf_moe_grouped_gelu_workspace_bytes(int rows, int total_selected_rows, int n
     return CF_OK;
 }
 
-int cf_moe_grouped_gelu_forward_fp8(const void* d_hidden, const float* d_fcin_descale, int fcin_is_e5m2,
-                                    const float* d_route_weights, const int* d_counts, const int* d_offsets,
-                                    const int* d_row_indices, const void* d_fc_in_w, const float* d_fc_in_descale,
-                                    const void* d_fc_out_w, const float* d_fc_out_descale, uint16_t* d_mixed, int rows,
-                                    int H, int Ie, int num_experts, int total_selected_rows, void* d_workspace,
-                                    size_t workspace_bytes, cf_stream_t stream) {
+namespace {
+// The per-expert activation slots of the loop's fc_out input (moe_fcout_act_slot, src/trainer.cu:6916): null states =
+// one scale per token row instead.
+struct FcoutSlots { float* states; int stride, history_len, is_e5m2, is_recompute; };
+
+int gelu_bank_forward(const void* d_hidden, const float* d_fcin_descale, int fcin_is_e5m2,
+                      const float* d_route_weights, const int* d_counts, const int* d_offsets,
+                      const int* d_row_indices, const void* d_fc_in_w, const float* d_fc_in_descale,
+                      const void* d_fc_out_w, const float* d_fc_out_descale, uint16_t* d_mixed, int rows,
+                      int H, int Ie, int num_experts, int total_selected_rows, const FcoutSlots& slots, void* d_workspace,
+                      size_t workspace_bytes, cf_stream_t stream) {
     if (rows < 0 || H < 0 || Ie < 0 || num_experts < 0 || total_selected_rows < 0) return CF_ERR_INVALID_ARG;
     if (rows == 0 || num_experts == 0 || total_selected_rows == 0) return CF_OK;
     if (!d_hidden || !d_fcin_descale || !d_route_weights || !d_counts || !d_offsets || !d_row_indices || !d_fc_in_w ||
@@ -1554,16 +1571,48 @@ int cf_moe_grouped_gelu_forward_fp8(const void* d_hidden, const float* d_fcin_de
                               d_fc_in_w, in_descale, CF_SCALE_ROW_COL, CF_EPI_NONE, nullptr, nullptr, act, Ie, base + w.s.tile_map,
                               map_bytes, false, fcin_is_e5m2 ? 1 : 0, stream);
     if (rc) return rc;
-    // gelu_forward and the per-token quantize in one pass over the bf16 projections
-    rc = cf_gelu_quantize_rows_e4m3(act, total_selected_rows, Ie, actq, act_scale, act_descale, stream);
+    // gelu_forward and the quantize in one pass over the bf16 projections: one scale per token row, or the loop's own
+    // per-expert delayed scale (fp8_quant_act on the expert's slot, src/trainer.cu:6916-6918), whose snapshot descale
+    // is spread over the expert's rows for the GEMM
+    if (slots.states)
+        rc = cf_moe_grouped_quantize_delayed(act, actq, Ie, num_experts, d_counts, d_offsets, total_selected_rows, slots.states,
+                                             slots.stride, slots.history_len, slots.is_e5m2, 1, slots.is_recompute, act_descale, stream);
+    else
+        rc = cf_gelu_quantize_rows_e4m3(act, total_selected_rows, Ie, actq, act_scale, act_descale, stream);
     if (rc) return rc;
     rc = grouped_gemm_nt_bf16(total_selected_rows, H, Ie, num_experts, d_counts, d_offsets, actq, total_selected_rows, Ie, nullptr,
                               act_descale, d_fc_out_w, out_descale, CF_SCALE_ROW_COL, CF_EPI_NONE, nullptr, nullptr, y, H,
-                              base + w.s.tile_map, map_bytes, false, 0, stream);
+                              base + w.s.tile_map, map_bytes, false, slots.states && slots.is_e5m2 ? 1 : 0, stream);
     if (rc) return rc;
-    if (indexed) return cf_moe_unpermute_indexed_bf16(d_mixed, y, d_route_weights, slot, rows, num_experts, H, 0, stream);
-    return cf_moe_unpermute_weighted_bf16(d_mixed, y, d_route_weights, d_counts, d_offsets, d_row_indices, rows,
-                                          num_experts, H, stream);
+    if (indexed) return unpermute_indexed(d_mixed, y, d_route_weights, slot, rows, num_experts, H, 0, total_selected_rows, stream);
+    return unpermute_weighted(d_mixed, y, d_route_weights, d_counts, d_offsets, d_row_indices, rows, num_experts, H,
+                              total_selected_rows, stream);
+}
+}  // namespace
+
+int cf_moe_grouped_gelu_forward_fp8(const void* d_hidden, const float* d_fcin_descale, int fcin_is_e5m2,
+                                    const float* d_route_weights, const int* d_counts, const int* d_offsets,
+                                    const int* d_row_indices, const void* d_fc_in_w, const float* d_fc_in_descale,
+                                    const void* d_fc_out_w, const float* d_fc_out_descale, uint16_t* d_mixed, int rows,
+                                    int H, int Ie, int num_experts, int total_selected_rows, void* d_workspace,
+                                    size_t workspace_bytes, cf_stream_t stream) {
+    return gelu_bank_forward(d_hidden, d_fcin_descale, fcin_is_e5m2, d_route_weights, d_counts, d_offsets, d_row_indices, d_fc_in_w,
+                             d_fc_in_descale, d_fc_out_w, d_fc_out_descale, d_mixed, rows, H, Ie, num_experts, total_selected_rows,
+                             FcoutSlots{nullptr, 0, 0, 0, 0}, d_workspace, workspace_bytes, stream);
+}
+
+int cf_moe_grouped_gelu_forward_fp8_slots(const void* d_hidden, const float* d_fcin_descale, int fcin_is_e5m2,
+                                          const float* d_route_weights, const int* d_counts, const int* d_offsets,
+                                          const int* d_row_indices, const void* d_fc_in_w, const float* d_fc_in_descale,
+                                          const void* d_fc_out_w, const float* d_fc_out_descale, uint16_t* d_mixed, int rows,
+                                          int H, int Ie, int num_experts, int total_selected_rows, float* d_fcout_slot_states,
+                                          int state_stride_words, int history_len, int fcout_is_e5m2, int is_recompute,
+                                          void* d_workspace, size_t workspace_bytes, cf_stream_t stream) {
+    if (!d_fcout_slot_states || history_len < 0 || state_stride_words < cf_act_slot_state_words(history_len)) return CF_ERR_INVALID_ARG;
+    return gelu_bank_forward(d_hidden, d_fcin_descale, fcin_is_e5m2, d_route_weights, d_counts, d_offsets, d_row_indices, d_fc_in_w,
+                             d_fc_in_descale, d_fc_out_w, d_fc_out_descale, d_mixed, rows, H, Ie, num_experts, total_selected_rows,
+                             FcoutSlots{d_fcout_slot_states, state_stride_words, history_len, fcout_is_e5m2 ? 1 : 0, is_recompute ? 1 : 0},
+                             d_workspace, workspace_bytes, stream);
 }
 
 int cf_moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_fcin_descale, int fcin_is_e5m2,
@@ -1576,16 +1625,8 @@ int cf_moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_fcin_
     if (!d_hidden || !d_fcin_descale || !d_route_weights || !d_counts || !d_row_indices || !d_fc_in_w || !d_fc_in_descale ||
         !d_fc_out_w || !d_fc_out_descale || !d_mixed)
         return CF_ERR_INVALID_ARG;
-    // a lent workspace that is large enough sends the call to the whole-matrix form (which needs the true row total)
-    void* lent = nullptr;
-    size_t lent_bytes = 0, need = 0;
-    lent_workspace(&lent, &lent_bytes);
-    if (lent && total_selected_rows > 0 &&
-        cf_moe_grouped_expert_forward_fp8_workspace(rows, total_selected_rows, num_experts, H, Ie, nullptr, &need) == CF_OK && need > 0 &&
-        need <= lent_bytes)
-        return cf_moe_grouped_expert_forward_fp8_ws(d_hidden, d_fcin_descale, fcin_is_e5m2, d_route_weights, d_counts, d_offsets,
-                                                    d_row_indices, d_fc_in_w, d_fc_in_descale, d_fc_out_w, d_fc_out_descale, d_mixed,
-                                                    rows, H, Ie, num_experts, total_selected_rows, lent, lent_bytes, stream);
+    (void)d_offsets;               // accepted and unused, as in the reference (kernels/moe.cu:1063-1071)
+    (void)total_selected_rows;
     return expert_forward_fp8_one_kernel(d_hidden, d_fcin_descale, fcin_is_e5m2, d_route_weights, d_counts, d_row_indices, d_fc_in_w,
                                          d_fc_in_descale, d_fc_out_w, d_fc_out_descale, d_mixed, rows, H, Ie, num_experts, stream);
 }
@@ -1670,14 +1711,8 @@ int cf_moe_grouped_expert_forward_bf16(const uint16_t* d_hidden, const float* d_
     if (rows < 0 || H < 0 || Ie < 0 || num_experts < 0) return CF_ERR_INVALID_ARG;
     if (rows == 0 || num_experts == 0 || H == 0 || Ie == 0) return CF_OK;
     if (!d_hidden || !d_route_weights || !d_counts || !d_row_indices || !d_fc_in_w || !d_fc_out_w || !d_mixed) return CF_ERR_INVALID_ARG;
-    void* lent = nullptr;
-    size_t lent_bytes = 0, need = 0;
-    lent_workspace(&lent, &lent_bytes);
-    if (lent && total_selected_rows > 0 &&
-        cf_moe_grouped_expert_forward_bf16_workspace(rows, total_selected_rows, num_experts, H, Ie, nullptr, &need) == CF_OK && need > 0 &&
-        need <= lent_bytes)
-        return cf_moe_grouped_expert_forward_bf16_ws(d_hidden, d_route_weights, d_counts, d_offsets, d_row_indices, d_fc_in_w, d_fc_out_w,
-                                                     d_mixed, rows, H, Ie, num_experts, total_selected_rows, lent, lent_bytes, stream);
+    (void)d_offsets;               // the row lists carry everything the kernels need
+    (void)total_selected_rows;     // the reference's launch bound (kernels/moe.cu:875); the grid here follows the row lists
     return expert_forward_bf16_one_kernel(d_hidden, d_route_weights, d_counts, d_row_indices, d_fc_in_w, d_fc_out_w, d_mixed, rows, H, Ie,
                                           num_experts, stream);
 }
@@ -1688,7 +1723,7 @@ int cf::expert_forward_bf16_one_kernel(const uint16_t* d_hidden, const float* d_
                                        const int* d_row_indices, const uint16_t* d_fc_in_w, const uint16_t* d_fc_out_w,
                                        uint16_t* d_mixed, int rows, int H, int Ie, int num_experts, cf_stream_t stream) {
     // the matrix-core form where the shapes are whole MFMA steps and its tile fits the LDS
-    const size_t smem_mfma = 2u * kMfmaRows * (static_cast<size_t>(H) + 8) + 4u * kMfmaRows * (static_cast<size_t>(Ie) + 8);
+    const size_t smem_mfma = 2u * kMfmaRows * (static_cast<size_t>(H) + 8) + 2u * kMfmaRows * (static_cast<size_t>(Ie) + 8);
     if (H % 64 == 0 && Ie % 64 == 0 && smem_mfma <= 160 * 1024 && aligned16(d_hidden) && aligned16(d_fc_in_w) && aligned16(d_fc_out_w) &&
         (reinterpret_cast<uintptr_t>(d_mixed) & 7u) == 0) {
         static std::once_flag once_mfma;
@@ -1712,13 +1747,13 @@ int cf::expert_forward_bf16_one_kernel(const uint16_t* d_hidden, const float* d_
 // rounding per expert; the slot table when the caller has one, the search of the row lists otherwise
 int cf::unpermute_f32(uint16_t* d_mixed, const float* d_y, const float* d_route_weights, const int* d_slot_index,
                       const int* d_counts, const int* d_offsets, const int* d_row_indices, int rows, int num_experts, int H,
-                      hipStream_t st) {
+                      int slot_limit, hipStream_t st) {
     if (rows <= 0 || num_experts <= 0 || H <= 0) return CF_OK;
     if ((H & 7) == 0 && !(aligned16(d_mixed) && aligned16(d_y))) return CF_ERR_UNSUPPORTED;
     if (d_slot_index)
-        k_unpermute_indexed<false, float><<<rows, kThreads, 0, st>>>(d_mixed, d_y, d_route_weights, d_slot_index, num_experts, H);
+        k_unpermute_indexed<false, float><<<rows, kThreads, 0, st>>>(d_mixed, d_y, d_route_weights, d_slot_index, num_experts, H, slot_limit);
     else
         k_unpermute<false, float><<<rows, kThreads, 0, st>>>(d_mixed, d_y, d_route_weights, d_counts, d_offsets, d_row_indices, rows,
-                                                            num_experts, H);
+                                                            num_experts, H, slot_limit);
     return launch_status();
 }

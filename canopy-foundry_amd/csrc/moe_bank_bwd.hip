@@ -51,7 +51,17 @@ __global__ __launch_bounds__(kThreads) void k_spread3(const float* __restrict__ 
     }
 }
 
-struct Layout { size_t off[CF_MOE_BWD_WS_COUNT]; size_t total; };
+struct Layout { size_t off[CF_MOE_BWD_WS_COUNT]; size_t counts; size_t total; };
+
+// counts[e] cut to what the compact buffers hold: total_rows is the caller's bound on the selected rows (the
+// reference's callers pass rows * top_k), and every later stage walks (these counts, the caller's offsets)
+__global__ __launch_bounds__(kThreads) void k_clamp_counts(const int* __restrict__ counts, const int* __restrict__ offsets, int E,
+                                                           int total_rows, int* __restrict__ out) {
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= E) return;
+    const int first = offsets[e];
+    out[e] = first >= 0 && first < total_rows ? max(0, min(counts[e], total_rows - first)) : 0;
+}
 
 Layout layout(int rows, int total_rows, int E, int H, int Ie) {
     auto up = [](size_t v) { return (v + 255) & ~static_cast<size_t>(255); };
@@ -81,6 +91,8 @@ Layout layout(int rows, int total_rows, int E, int H, int Ie) {
         l.off[i] = at;
         at = up(at + bytes[i]);
     }
+    l.counts = at;
+    at = up(at + sizeof(int) * static_cast<size_t>(E));
     l.total = at;
     return l;
 }
@@ -102,14 +114,17 @@ int cf_moe_grouped_gelu_backward_workspace(int rows, int total_selected_rows, in
     return CF_OK;
 }
 
-int cf_moe_grouped_gelu_backward_fp8(const uint16_t* d_grad_mixed, const void* d_hidden_fp8, const float* d_fcin_descale,
-                                     int fcin_is_e5m2, const uint16_t* d_hidden_bf16, const float* d_route_weights,
-                                     const int* d_counts, const int* d_offsets, const int* d_row_indices,
-                                     const void* d_fc_in_w8, const float* d_fc_in_descale, const void* d_fc_out_w8,
-                                     const float* d_fc_out_descale, const uint16_t* d_fc_in_w, const uint16_t* d_fc_out_w,
-                                     float* d_grad_route_weights, uint16_t* d_grad_fc_in, uint16_t* d_grad_fc_out,
-                                     uint16_t* d_grad_hidden, int rows, int H, int Ie, int num_experts,
-                                     int total_selected_rows, void* d_workspace, size_t workspace_bytes, cf_stream_t stream) {
+namespace {
+struct FcoutSlots { float* states; int stride, history_len, is_e5m2; };
+
+int gelu_bank_backward(const uint16_t* d_grad_mixed, const void* d_hidden_fp8, const float* d_fcin_descale,
+                       int fcin_is_e5m2, const uint16_t* d_hidden_bf16, const float* d_route_weights,
+                       const int* d_counts, const int* d_offsets, const int* d_row_indices,
+                       const void* d_fc_in_w8, const float* d_fc_in_descale, const void* d_fc_out_w8,
+                       const float* d_fc_out_descale, const uint16_t* d_fc_in_w, const uint16_t* d_fc_out_w,
+                       float* d_grad_route_weights, uint16_t* d_grad_fc_in, uint16_t* d_grad_fc_out,
+                       uint16_t* d_grad_hidden, int rows, int H, int Ie, int num_experts,
+                       int total_selected_rows, const FcoutSlots& slots, void* d_workspace, size_t workspace_bytes, cf_stream_t stream) {
     if (rows < 0 || H < 0 || Ie < 0 || num_experts < 0 || total_selected_rows < 0) return CF_ERR_INVALID_ARG;
     if (rows == 0 || num_experts == 0) return CF_OK;
     if (!d_grad_mixed || !d_hidden_fp8 || !d_fcin_descale || !d_hidden_bf16 || !d_route_weights || !d_counts || !d_offsets ||
@@ -153,7 +168,15 @@ int cf_moe_grouped_gelu_backward_fp8(const uint16_t* d_grad_mixed, const void* d
                                                            d_fc_out_descale, out_descale, nc);
     }
     if ((rc = launch_status())) return rc;
-    // entries of the index past the experts' lists (a caller's total above the sum of the counts) point at row 0: the
+    // total_selected_rows bounds the selected rows from above (the reference's callers pass rows * top_k,
+    // src/trainer.cu:6863): no stage may go past it, whatever the counts say
+    {
+        int* clamped = reinterpret_cast<int*>(base + l.counts);
+        k_clamp_counts<<<(num_experts + kThreads - 1) / kThreads, kThreads, 0, st>>>(d_counts, d_offsets, num_experts, total, clamped);
+        if ((rc = launch_status())) return rc;
+        d_counts = clamped;
+    }
+    // entries of the index past the experts' lists (a total above the sum of the counts) point at row 0: the
     // elementwise stages run over all `total` rows and must not gather from a stale index
     k_zero_i32<<<grid(static_cast<size_t>(total)), kThreads, 0, st>>>(index, static_cast<size_t>(total));
     if ((rc = launch_status())) return rc;
@@ -165,10 +188,17 @@ int cf_moe_grouped_gelu_backward_fp8(const uint16_t* d_grad_mixed, const void* d
                                    true, fcin_is_e5m2 ? 1 : 0, stream)))
         return rc;
     if ((rc = cf_gelu_forward_bf16(pre, post, static_cast<size_t>(total) * Ie, stream))) return rc;
-    if ((rc = cf_fp8_quantize_rows(post, total, Ie, 0, postq, post_scale, post_descale, stream))) return rc;
+    // one scale per token row, or the recompute call of fp8_quant_act on the expert's slot (is_recompute = true: the
+    // scale the forward's call snapshotted, no side effects; src/trainer.cu:7707-7712)
+    if (slots.states)
+        rc = cf_moe_grouped_quantize_delayed(post, postq, Ie, num_experts, d_counts, d_offsets, total, slots.states, slots.stride,
+                                             slots.history_len, slots.is_e5m2, 0, 1, post_descale, stream);
+    else
+        rc = cf_fp8_quantize_rows(post, total, Ie, 0, postq, post_scale, post_descale, stream);
+    if (rc) return rc;
     if ((rc = grouped_gemm_nt_bf16(total, H, Ie, num_experts, d_counts, d_offsets, postq, total, Ie, nullptr, post_descale,
                                    d_fc_out_w8, out_descale, CF_SCALE_ROW_COL, CF_EPI_NONE, nullptr, nullptr, d_out, H, tile_map, map_bytes,
-                                   false, 0, stream)))
+                                   false, slots.states && slots.is_e5m2 ? 1 : 0, stream)))
         return rc;
 
     // ---- route-weight gradient; the expert outputs become their gradients in place ----
@@ -193,6 +223,39 @@ int cf_moe_grouped_gelu_backward_fp8(const uint16_t* d_grad_mixed, const void* d
         return rc;
     return cf_moe_unpermute_add_bf16(d_grad_hidden, d_x, d_route_weights, d_counts, d_offsets, d_row_indices, rows, num_experts, H,
                                      stream);
+}
+}  // namespace
+
+int cf_moe_grouped_gelu_backward_fp8(const uint16_t* d_grad_mixed, const void* d_hidden_fp8, const float* d_fcin_descale,
+                                     int fcin_is_e5m2, const uint16_t* d_hidden_bf16, const float* d_route_weights,
+                                     const int* d_counts, const int* d_offsets, const int* d_row_indices,
+                                     const void* d_fc_in_w8, const float* d_fc_in_descale, const void* d_fc_out_w8,
+                                     const float* d_fc_out_descale, const uint16_t* d_fc_in_w, const uint16_t* d_fc_out_w,
+                                     float* d_grad_route_weights, uint16_t* d_grad_fc_in, uint16_t* d_grad_fc_out,
+                                     uint16_t* d_grad_hidden, int rows, int H, int Ie, int num_experts,
+                                     int total_selected_rows, void* d_workspace, size_t workspace_bytes, cf_stream_t stream) {
+    return gelu_bank_backward(d_grad_mixed, d_hidden_fp8, d_fcin_descale, fcin_is_e5m2, d_hidden_bf16, d_route_weights, d_counts, d_offsets,
+                              d_row_indices, d_fc_in_w8, d_fc_in_descale, d_fc_out_w8, d_fc_out_descale, d_fc_in_w, d_fc_out_w,
+                              d_grad_route_weights, d_grad_fc_in, d_grad_fc_out, d_grad_hidden, rows, H, Ie, num_experts,
+                              total_selected_rows, FcoutSlots{nullptr, 0, 0, 0}, d_workspace, workspace_bytes, stream);
+}
+
+int cf_moe_grouped_gelu_backward_fp8_slots(const uint16_t* d_grad_mixed, const void* d_hidden_fp8, const float* d_fcin_descale,
+                                           int fcin_is_e5m2, const uint16_t* d_hidden_bf16, const float* d_route_weights,
+                                           const int* d_counts, const int* d_offsets, const int* d_row_indices,
+                                           const void* d_fc_in_w8, const float* d_fc_in_descale, const void* d_fc_out_w8,
+                                           const float* d_fc_out_descale, const uint16_t* d_fc_in_w, const uint16_t* d_fc_out_w,
+                                           float* d_grad_route_weights, uint16_t* d_grad_fc_in, uint16_t* d_grad_fc_out,
+                                           uint16_t* d_grad_hidden, int rows, int H, int Ie, int num_experts,
+                                           int total_selected_rows, float* d_fcout_slot_states, int state_stride_words,
+                                           int history_len, int fcout_is_e5m2, void* d_workspace, size_t workspace_bytes,
+                                           cf_stream_t stream) {
+    if (!d_fcout_slot_states || history_len < 0 || state_stride_words < cf_act_slot_state_words(history_len)) return CF_ERR_INVALID_ARG;
+    return gelu_bank_backward(d_grad_mixed, d_hidden_fp8, d_fcin_descale, fcin_is_e5m2, d_hidden_bf16, d_route_weights, d_counts, d_offsets,
+                              d_row_indices, d_fc_in_w8, d_fc_in_descale, d_fc_out_w8, d_fc_out_descale, d_fc_in_w, d_fc_out_w,
+                              d_grad_route_weights, d_grad_fc_in, d_grad_fc_out, d_grad_hidden, rows, H, Ie, num_experts,
+                              total_selected_rows, FcoutSlots{d_fcout_slot_states, state_stride_words, history_len, fcout_is_e5m2 ? 1 : 0},
+                              d_workspace, workspace_bytes, stream);
 }
 
 }  // extern "C"

@@ -18,8 +18,6 @@
 
 #include <cstdint>
 
-#include <mutex>
-
 #include "cf_fp8.h"
 #include "common.hpp"
 #include "internal.hpp"
@@ -29,11 +27,6 @@ namespace {
 
 constexpr int kSplitThreads = 256;
 constexpr int kTerms = 3;
-
-// the buffer a caller has lent through cf_set_workspace (one per process: the library is used on one GPU)
-std::mutex g_lent_mutex;
-void* g_lent = nullptr;
-size_t g_lent_bytes = 0;
 
 // Phi(v) = (1 + erf(v / sqrt 2)) / 2 from the rational-exponential form of erfc (Abramowitz & Stegun 7.1.26,
 // absolute error 1.5e-7 on erf: fp32 round-off level): for v < 0 the small tail is computed directly, not as
@@ -121,8 +114,8 @@ FwdWs fwd_layout(int rows, int total_rows, int num_experts, int H, int Ie, bool 
     w.off[CF_MOE_FWD_WS_SLOT] = off; off = up(off + w.slot_bytes);
     w.off[CF_MOE_FWD_WS_PRE] = off; off = up(off + sizeof(float) * T * Ie);
     if (bf16_form) {
-        // two bf16 terms per value, no scales
-        w.off[CF_MOE_FWD_WS_SPLIT] = off; off = up(off + 2 * 2 * T * Ie);
+        // the GELU output as bf16, no scales
+        w.off[CF_MOE_FWD_WS_SPLIT] = off; off = up(off + 2 * T * Ie);
         w.off[CF_MOE_FWD_WS_SPLIT_DESCALE] = off;
         w.off[CF_MOE_FWD_WS_Y] = off; off = up(off + sizeof(float) * T * H);
         w.off[CF_MOE_FWD_WS_X] = off;
@@ -140,10 +133,10 @@ FwdWs fwd_layout(int rows, int total_rows, int num_experts, int H, int Ie, bool 
 bool staged_shape(int H, int Ie) { return H % 128 == 0 && H >= 256 && Ie % 128 == 0 && Ie >= 128 && Ie <= 4096; }
 bool staged_shape_bf16(int H, int Ie) { return H % 8 == 0 && Ie % 64 == 0; }
 
-// GELU of the fp32 projections as two bf16 terms side by side: out[r, 0:K] = bf16(g), out[r, K:2K] = bf16(g - bf16(g)),
-// 16 significand bits between them.  K % 4 == 0.
-__global__ __launch_bounds__(kSplitThreads) void k_gelu_split2_bf16(const float* __restrict__ pre, size_t rows, int K,
-                                                                    uint16_t* __restrict__ out) {
+// GELU of the fp32 projections rounded to bf16, as the reference kernel parks it before fc_out
+// (sh_fcin[j] = __float2bfloat16(g), kernels/moe.cu:845).  K % 4 == 0.
+__global__ __launch_bounds__(kSplitThreads) void k_gelu_round_bf16(const float* __restrict__ pre, size_t rows, int K,
+                                                                   uint16_t* __restrict__ out) {
     typedef float f32x4 __attribute__((ext_vector_type(4)));
     const int kv = K / 4;
     const size_t n = rows * kv;
@@ -152,36 +145,16 @@ __global__ __launch_bounds__(kSplitThreads) void k_gelu_split2_bf16(const float*
         const int c = static_cast<int>(i - r * kv) * 4;
         const f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(pre + r * K + c));
         const float g[4] = {gelu_tail_form(v[0]), gelu_tail_form(v[1]), gelu_tail_form(v[2]), gelu_tail_form(v[3])};
-        const uint32_t h01 = pack_bf16x2_hw(g[0], g[1]), h23 = pack_bf16x2_hw(g[2], g[3]);
-        const uint32_t r01 = pack_bf16x2_hw(g[0] - bf16_lo(h01), g[1] - bf16_hi(h01));
-        const uint32_t r23 = pack_bf16x2_hw(g[2] - bf16_lo(h23), g[3] - bf16_hi(h23));
-        uint16_t* o = out + r * (2 * static_cast<size_t>(K)) + c;
-        store_stream8(o, make_uint2(h01, h23));
-        store_stream8(o + K, make_uint2(r01, r23));
+        store_stream8(out + r * static_cast<size_t>(K) + c, make_uint2(pack_bf16x2_hw(g[0], g[1]), pack_bf16x2_hw(g[2], g[3])));
     }
 }
 
 }  // namespace
 }  // namespace cf
 
-// (null, 0) when nothing is lent
-void cf::lent_workspace(void** d_workspace, size_t* bytes) {
-    std::lock_guard<std::mutex> lock(g_lent_mutex);
-    *d_workspace = g_lent;
-    *bytes = g_lent_bytes;
-}
-
 using namespace cf;
 
 extern "C" {
-
-int cf_set_workspace(void* d_workspace, size_t bytes) {
-    if ((d_workspace == nullptr) != (bytes == 0) || (reinterpret_cast<uintptr_t>(d_workspace) & 255u)) return CF_ERR_INVALID_ARG;
-    std::lock_guard<std::mutex> lock(g_lent_mutex);
-    g_lent = d_workspace;
-    g_lent_bytes = bytes;
-    return CF_OK;
-}
 
 int cf_moe_grouped_expert_forward_fp8_workspace(int rows, int total_selected_rows, int num_experts, int H, int Ie,
                                                 size_t* offsets, size_t* bytes) {
@@ -250,13 +223,13 @@ int cf_moe_grouped_expert_forward_fp8_ws(const void* d_hidden, const float* d_fc
     rc = grouped_gemm_nt_terms(total_selected_rows, H, Ie, kTerms, num_experts, split, kTerms * Ie, split_descale, d_fc_out_w,
                                d_fc_out_descale, y, H, true, tile_map, stream);
     if (rc) return rc;
-    return unpermute_f32(d_mixed, y, d_route_weights, slot, d_counts, offsets, d_row_indices, rows, num_experts, H, st);
+    return unpermute_f32(d_mixed, y, d_route_weights, slot, d_counts, offsets, d_row_indices, rows, num_experts, H,
+                         total_selected_rows, st);
 }
 
 // moe_grouped_expert_forward_bf16 (kernels.hpp:400-407) with a workspace: the same pipeline on bf16 operands.
-// fc_in is one grouped bf16 GEMM that gathers the token rows in its operand fetch, fp32 output; the GELU output goes
-// to fc_out as two bf16 terms side by side (value = head + remainder to 2^-17) against the same weight columns,
-// K = 2 Ie, so both terms add in the fp32 accumulator; y stays fp32 until the ordered add.
+// fc_in is one grouped bf16 GEMM that gathers the token rows in its operand fetch, fp32 output; the GELU output is
+// rounded to bf16 for fc_out, as in the reference kernel (kernels/moe.cu:845); y stays fp32 until the ordered add.
 int cf_moe_grouped_expert_forward_bf16_workspace(int rows, int total_selected_rows, int num_experts, int H, int Ie,
                                                  size_t* offsets, size_t* bytes) {
     if (rows < 0 || total_selected_rows < 0 || num_experts < 0 || H < 0 || Ie < 0 || !bytes) return CF_ERR_INVALID_ARG;
@@ -283,7 +256,7 @@ int cf_moe_grouped_expert_forward_bf16_ws(const uint16_t* d_hidden, const float*
     if (!d_hidden || !d_route_weights || !d_counts || !d_row_indices || !d_fc_in_w || !d_fc_out_w || !d_mixed) return CF_ERR_INVALID_ARG;
     const bool staged = staged_shape_bf16(H, Ie) && aligned16(d_hidden) && aligned16(d_fc_in_w) && aligned16(d_fc_out_w) &&
                         aligned16(d_mixed) && static_cast<size_t>(rows) * H < (1ull << 30) &&
-                        static_cast<size_t>(total_selected_rows) * 2 * Ie < (1ull << 30) && static_cast<size_t>(H) * Ie < (1ull << 30);
+                        static_cast<size_t>(total_selected_rows) * Ie < (1ull << 30) && static_cast<size_t>(H) * Ie < (1ull << 30);
     if (!staged)
         return expert_forward_bf16_one_kernel(d_hidden, d_route_weights, d_counts, d_row_indices, d_fc_in_w, d_fc_out_w, d_mixed, rows,
                                               H, Ie, num_experts, stream);
@@ -309,14 +282,15 @@ int cf_moe_grouped_expert_forward_bf16_ws(const uint16_t* d_hidden, const float*
     {
         const size_t n = static_cast<size_t>(total_selected_rows) * (Ie / 4);
         const unsigned want = ceil_div(n, kSplitThreads);
-        k_gelu_split2_bf16<<<want < 16384u ? want : 16384u, kSplitThreads, 0, st>>>(pre, static_cast<size_t>(total_selected_rows), Ie, split);
+        k_gelu_round_bf16<<<want < 16384u ? want : 16384u, kSplitThreads, 0, st>>>(pre, static_cast<size_t>(total_selected_rows), Ie, split);
         rc = launch_status();
         if (rc) return rc;
     }
-    rc = grouped_gemm_bf16_nt(total_selected_rows, H, Ie, 2, num_experts, split, total_selected_rows, 2 * Ie, nullptr, d_fc_out_w, y, H,
+    rc = grouped_gemm_bf16_nt(total_selected_rows, H, Ie, 1, num_experts, split, total_selected_rows, Ie, nullptr, d_fc_out_w, y, H,
                               true, tile_map, stream);
     if (rc) return rc;
-    return unpermute_f32(d_mixed, y, d_route_weights, slot, d_counts, offsets, d_row_indices, rows, num_experts, H, st);
+    return unpermute_f32(d_mixed, y, d_route_weights, slot, d_counts, offsets, d_row_indices, rows, num_experts, H,
+                         total_selected_rows, st);
 }
 
 }  // extern "C"

@@ -6,6 +6,7 @@
 // two 128-bit loads and one 128-bit store, a wavefront reduces with xor
 // shuffles, and a workgroup issues one atomic.
 #include "common.hpp"
+#include "internal.hpp"
 #include <mutex>
 
 namespace cf {
@@ -329,6 +330,81 @@ __global__ __launch_bounds__(kAmaxThreads) void k_quant_delayed_step(const uint1
             *d.descale = hist_max / d.fp8_max;
             *d.running_amax = 0.0f;
             *d.arrived = 0u;
+        }
+    }
+}
+
+// The same step for a bank of experts in one launch: the rows of expert e (counts[e] of them, from row offsets[e] of a
+// compact [total_rows, K] buffer) are one tensor with its own delayed-scaling state block (the word layout of
+// cf_act_slot's device block; block e starts e * stride words after the first).  blockIdx.y = expert, gridDim.x
+// workgroups share an expert's rows; an expert without rows is left alone, state included (the reference's loop skips
+// it before fp8_quant_act, src/trainer.cu:6887-6888).  GELU: the tensor quantized is bf16(gelu(x)) (gelu_forward in
+// place, then fp8_quant_act, :6910-6918).  RECOMPUTE: the backward's second pass, with the snapshot scale and no side
+// effects (:4736-4743).  row_descale[r] = the descale the GEMM that consumes row r dequantizes with (the expert's
+// descale_snapshot, :6921-6924).
+template <bool E5M2, bool GELU, bool RECOMPUTE>
+__global__ __launch_bounds__(kThreads) void k_grouped_quant_delayed(const uint16_t* __restrict__ x, uint8_t* __restrict__ out, int K,
+                                                                    const int* __restrict__ counts, const int* __restrict__ offsets,
+                                                                    int total_rows, float* __restrict__ states, int stride,
+                                                                    int history_len, float fp8_max, float* __restrict__ row_descale) {
+    __shared__ float sh[kThreads / 64];
+    const int e = blockIdx.y;
+    const int first = offsets[e];
+    const int rows = first >= 0 && first < total_rows ? min(counts[e], total_rows - first) : 0;
+    if (rows <= 0) return;
+    float* st = states + static_cast<size_t>(e) * stride;
+    const float s = st[RECOMPUTE ? slotw::SCALE_SNAP : slotw::SCALE];
+    const float ds = st[RECOMPUTE ? slotw::DESCALE_SNAP : slotw::DESCALE];
+    const bool s_finite = fabsf(s) < __uint_as_float(0x7f800000u);
+    float pre_max = 0.0f;
+    int pre_cursor = 0, pre_count = 0;
+    if (!RECOMPUTE && threadIdx.x == 0 && history_len > 0) {
+        pre_cursor = reinterpret_cast<const int*>(st)[slotw::CURSOR];
+        pre_count = reinterpret_cast<const int*>(st)[slotw::COUNT];
+        if (pre_cursor < 0 || pre_cursor >= history_len) pre_cursor = 0;
+        if (pre_count < history_len) ++pre_count;
+        for (int i = 0; i < pre_count; ++i)
+            if (i != pre_cursor) pre_max = fmaxf(pre_max, st[slotw::HISTORY + i]);
+    }
+    const size_t tid = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x;
+    const size_t stride_t = static_cast<size_t>(gridDim.x) * kThreads;
+    for (size_t r = tid; r < static_cast<size_t>(rows); r += stride_t) row_descale[first + r] = ds;
+    const uint16_t* xe = x + static_cast<size_t>(first) * K;
+    uint8_t* oe = out + static_cast<size_t>(first) * K;
+    const size_t nvec = static_cast<size_t>(rows) * K / kVec;       // K % 16 == 0
+    float local = 0.0f;
+    int local_bits = 0;
+    for (size_t i = tid; i < nvec; i += stride_t) {
+        Vec16 v = load16(xe + i * kVec);
+        if constexpr (GELU) v = gelu16(v);
+        store_stream16(oe + i * kVec, quant16_track<E5M2, !RECOMPUTE>(v, s, s_finite, local_bits, local));
+    }
+    if constexpr (!RECOMPUTE) {
+        local = fmaxf(local, __uint_as_float(static_cast<uint32_t>(local_bits) << 16));
+        const float m = block_max(local, sh);
+        if (threadIdx.x == 0) {
+            unsigned* arrived = reinterpret_cast<unsigned*>(st) + slotw::ARRIVED;
+            atomic_max_nonneg(st + slotw::RUNNING, m);
+            __threadfence();
+            if (atomicAdd(arrived, 1u) == gridDim.x - 1) {
+                __threadfence();
+                const float amax = __hip_atomic_load(st + slotw::RUNNING, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                st[slotw::SCALE_SNAP] = s;
+                st[slotw::DESCALE_SNAP] = ds;
+                st[slotw::AMAX] = amax;
+                const float a = fmaxf(amax, 1e-12f);
+                float hist_max = a;
+                if (history_len > 0) {
+                    st[slotw::HISTORY + pre_cursor] = a;
+                    hist_max = fmaxf(pre_cursor < pre_count ? fmaxf(pre_max, a) : pre_max, 1e-12f);
+                    reinterpret_cast<int*>(st)[slotw::CURSOR] = (pre_cursor + 1) % history_len;
+                    reinterpret_cast<int*>(st)[slotw::COUNT] = pre_count;
+                }
+                st[slotw::SCALE] = fp8_max / hist_max;
+                st[slotw::DESCALE] = hist_max / fp8_max;
+                st[slotw::RUNNING] = 0.0f;
+                *arrived = 0u;
+            }
         }
     }
 }
@@ -839,6 +915,40 @@ int cf_fp8_quantize_f32_e5m2(const float* d_x, void* d_out, const float* d_scale
     const int vec = aligned16(d_x) && (reinterpret_cast<uintptr_t>(d_out) & 3u) == 0;
     k_quant_f32<true><<<blocks_for(vec ? (n + 3) / 4 : n), kThreads, 0, as_stream(stream)>>>(
         d_x, static_cast<uint8_t*>(d_out), d_scale, n, vec);
+    return launch_status();
+}
+
+int cf_moe_grouped_quantize_delayed(const uint16_t* d_x, void* d_out, int K, int num_experts, const int* d_counts,
+                                    const int* d_offsets, int total_rows, float* d_slot_states, int state_stride_words,
+                                    int history_len, int is_e5m2, int apply_gelu, int is_recompute, float* d_row_descale,
+                                    cf_stream_t stream) {
+    if (K < 0 || num_experts < 0 || total_rows < 0 || history_len < 0) return CF_ERR_INVALID_ARG;
+    if (K == 0 || num_experts == 0 || total_rows == 0) return CF_OK;
+    if (!d_x || !d_out || !d_counts || !d_offsets || !d_slot_states || !d_row_descale) return CF_ERR_INVALID_ARG;
+    if (state_stride_words < cf_act_slot_state_words(history_len)) return CF_ERR_INVALID_ARG;
+    if (K % kVec != 0 || !aligned16(d_x) || !aligned16(d_out)) return CF_ERR_UNSUPPORTED;
+    // enough workgroups per expert to fill the part, few enough that an expert's arrivals stay a short tail
+    unsigned per = 2048u / static_cast<unsigned>(num_experts);
+    per = per < 1u ? 1u : (per > 64u ? 64u : per);
+    const dim3 grid(per, static_cast<unsigned>(num_experts));
+    const float fp8_max = is_e5m2 ? CF_E5M2_MAX : CF_E4M3_MAX;
+    hipStream_t st = as_stream(stream);
+    auto* o = static_cast<uint8_t*>(d_out);
+    auto launch = [&](auto kernel) {
+        kernel<<<grid, kThreads, 0, st>>>(d_x, o, K, d_counts, d_offsets, total_rows, d_slot_states, state_stride_words, history_len,
+                                          fp8_max, d_row_descale);
+    };
+    const int which = (is_e5m2 ? 4 : 0) | (apply_gelu ? 2 : 0) | (is_recompute ? 1 : 0);
+    switch (which) {
+        case 0: launch(k_grouped_quant_delayed<false, false, false>); break;
+        case 1: launch(k_grouped_quant_delayed<false, false, true>); break;
+        case 2: launch(k_grouped_quant_delayed<false, true, false>); break;
+        case 3: launch(k_grouped_quant_delayed<false, true, true>); break;
+        case 4: launch(k_grouped_quant_delayed<true, false, false>); break;
+        case 5: launch(k_grouped_quant_delayed<true, false, true>); break;
+        case 6: launch(k_grouped_quant_delayed<true, true, false>); break;
+        default: launch(k_grouped_quant_delayed<true, true, true>); break;
+    }
     return launch_status();
 }
 

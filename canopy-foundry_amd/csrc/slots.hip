@@ -3,6 +3,7 @@
 // over the quantize entry points of this library.  Device scalars live in one caller-owned
 // block; the host object only carries the flags the reference keeps in its slot struct.
 #include "common.hpp"
+#include "internal.hpp"
 
 #include <new>
 
@@ -20,9 +21,9 @@ namespace cf {
 namespace {
 
 // device block layout, in 4-byte words
-enum { W_AMAX = 0, W_SCALE, W_DESCALE, W_SCALE_SNAP, W_DESCALE_SNAP, W_CALIB_MIN, W_CALIB_MAX, W_CURSOR = 8, W_COUNT = 9,
-       W_RUNNING_AMAX = 10, W_ARRIVED = 11,      // scratch of the one-launch steady-state step, zero between calls
-       W_HISTORY = 16 };
+enum { W_AMAX = slotw::AMAX, W_SCALE = slotw::SCALE, W_DESCALE = slotw::DESCALE, W_SCALE_SNAP = slotw::SCALE_SNAP,
+       W_DESCALE_SNAP = slotw::DESCALE_SNAP, W_CALIB_MIN = slotw::CALIB_MIN, W_CALIB_MAX = slotw::CALIB_MAX, W_CURSOR = slotw::CURSOR,
+       W_COUNT = slotw::COUNT, W_RUNNING_AMAX = slotw::RUNNING, W_ARRIVED = slotw::ARRIVED, W_HISTORY = slotw::HISTORY };
 
 __global__ void k_slot_init(float* st, int history_len) {
     for (int i = threadIdx.x; i < W_HISTORY + history_len; i += blockDim.x) st[i] = 0.0f;   // zero words are int 0 as well

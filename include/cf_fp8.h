@@ -11,9 +11,21 @@
  *   - work is enqueued on `stream` (a hipStream_t passed as void*) and nothing
  *     synchronises;
  *   - bf16 tensors are passed as uint16_t*, fp8 tensors as void* / uint8_t*;
- *   - the library allocates no device memory and keeps no mutable global
- *     state; the only allocation is the small host object behind
- *     cf_act_slot_create (freed by cf_act_slot_destroy).
+ *   - the library allocates no device memory; the only allocation is the
+ *     small host object behind cf_act_slot_create (freed by
+ *     cf_act_slot_destroy).  It keeps no state between calls and every entry
+ *     point may be called from several host threads and streams at once on
+ *     buffers that do not overlap, with one exception that says so where it is
+ *     declared: cf_fp8_grouped_gemm_nt_bf16_static, whose tile table is a
+ *     fixed array in the library's device image shared by all its calls on a
+ *     GPU.  One-time kernel attribute set-up runs under std::call_once;
+ *   - total_selected_rows / total_rows of the expert-bank entry points is an
+ *     UPPER BOUND on the sum of the device-side counts, as the reference's
+ *     callers pass it (rows * top_k, src/trainer.cu:6863): it sizes the
+ *     compact buffers and the workspace; the true total is taken from the
+ *     counts on the device.  Should the counts sum to more than the bound,
+ *     the rows beyond it are left out (nothing is written or read past the
+ *     buffers the bound sized) and the result misses their terms.
  * The reference functions return void and throw; the C ABI returns 0 on
  * success, a positive hipError_t when the runtime reports one, or a negative
  * CF_ERR_* code for an argument the kernels cannot honour.
@@ -422,8 +434,9 @@ int cf_moe_grouped_gemm_bf16_tn_accum_bf16(int M, int N, int total_rows, int num
  * (gradients).  Outputs: d_grad_route_weights [rows,E] fp32 (cleared, then one entry per selected pair),
  * d_grad_fc_in [E,Ie,H] and d_grad_fc_out [E,H,Ie] bf16 (accumulated into), d_grad_hidden [rows,H] bf16
  * (accumulated into, experts in ascending order).  As in cf_moe_grouped_gelu_forward_fp8 the recomputed
- * activation is quantized with one scale per token row (the loop's per-expert delayed scale is host-side slot
- * state).  H and Ie multiples of 128 and at least 256; total_selected_rows the sum of the counts; d_workspace
+ * activation is quantized with one scale per token row (cf_moe_grouped_gelu_backward_fp8_slots keeps the loop's
+ * per-expert delayed scale).  H and Ie multiples of 128 and at least 256; total_selected_rows an upper bound on
+ * the sum of the counts; d_workspace
  * 256-byte aligned.  cf_moe_grouped_gelu_backward_workspace gives the workspace size and, when `offsets` is
  * not null, the byte offsets of the intermediates inside it (CF_MOE_BWD_WS_* order), which stay valid after
  * the call: pre / post / postq / d_out / d_post / d_pre / x / d_x, experts back to back. */
@@ -540,7 +553,7 @@ int cf_moe_grouped_swiglu_forward_fp8(const void* d_hidden_e4m3, const float* d_
  * per-tensor device descales, exact-erf GELU kept in fp32 (not re-quantised), bf16 accumulation
  * by compare-and-swap, so the last bit of d_mixed depends on arrival order as in the reference.
  * fc_in_w [E,Ie,H], fc_out_w [E,H,Ie] E4M3; hidden E4M3 or E5M2.  d_offsets and
- * total_selected_rows are accepted and unused, as in the reference (unless a workspace is lent: cf_set_workspace).  With H % 128 == 0,
+ * total_selected_rows are accepted and unused, as in the reference.  With H % 128 == 0,
  * Ie % 64 == 0, 16-byte aligned operands and 8-byte aligned d_mixed the two projections run on
  * the matrix cores (fp8 MFMA for fc_in; fc_out as bf16 MFMA on a two-term bf16 split of the fp32
  * GELU output, relative error 2^-17, against the weights widened exactly; 32 token rows per
@@ -555,15 +568,6 @@ int cf_moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_fcin_
                                       int H, int Ie, int num_experts, int total_selected_rows,
                                       cf_stream_t stream);
 
-/* Lends the library a device buffer (256-byte aligned) that entry points with the reference's argument lists, which
- * carry no workspace, may use: cf_moe_grouped_expert_forward_fp8 and cf_moe_grouped_expert_forward_bf16 then take
- * their whole-matrix forms (the *_ws entry points below) whenever the buffer holds what the *_workspace query
- * asks for; total_selected_rows must then be the true sum of the counts.  It has no counterpart in the reference
- * (whose trainer owns one arena for such purposes, Fp8Ctx).  (null, 0) takes the buffer back.  The buffer is shared
- * by every such call: calls that may overlap in time must be serialised by the caller; calls on one stream are
- * ordered.  The library never frees or allocates it. */
-int cf_set_workspace(void* d_workspace, size_t bytes);
-
 /* moe_grouped_expert_forward_fp8 (kernels.hpp:400-423, kernels/moe.cu:950-1127) with a workspace: the same
  * arguments and contract as cf_moe_grouped_expert_forward_fp8, run as whole-matrix launches when H % 128 == 0,
  * H >= 256, Ie % 128 == 0, Ie <= 4096 and hidden, weights and d_mixed are 16-byte aligned (other shapes are
@@ -574,7 +578,9 @@ int cf_set_workspace(void* d_workspace, size_t bytes);
  * matrix cores weight term t by 2^(-4 t) (E8M0 scales of the MX form of the FP8 MFMA), so the three partial
  * products add in one fp32 accumulator and y stays fp32; w * y is then added into d_mixed per token row over its
  * experts in ascending order, one bf16 rounding per expert as in the reference's compare-and-swap add.  The
- * one difference from the reference kernel: the order of the adds is fixed.  total_selected_rows must be the sum of d_counts; d_offsets may be null (the offsets are recomputed).
+ * one difference from the reference kernel: the order of the adds is fixed.  total_selected_rows is an upper bound on
+ * the sum of d_counts (rows * top_k, as the reference's caller passes it); d_offsets may be null (the offsets are recomputed).
+ * The workspace belongs to the call: two calls that may overlap in time (two streams, two host threads) need two workspaces.
  * d_workspace 256-byte aligned; cf_moe_grouped_expert_forward_fp8_workspace gives its size and, when
  * `offsets` is not null, the byte offsets of the intermediates (CF_MOE_FWD_WS_* order), which stay valid
  * after the call: pre [total, Ie] fp32, split [total, 3 Ie] E4M3, split_descale [total] fp32, y [total, H] fp32,
@@ -594,14 +600,14 @@ int cf_moe_grouped_expert_forward_fp8_ws(const void* d_hidden, const float* d_fc
                                          int H, int Ie, int num_experts, int total_selected_rows,
                                          void* d_workspace, size_t workspace_bytes, cf_stream_t stream);
 
-/* moe_grouped_expert_forward_bf16 (kernels.hpp:400-407) with a workspace: the same arguments and contract as
- * cf_moe_grouped_expert_forward_bf16, run as whole-matrix launches when H % 8 == 0, Ie % 64 == 0 and the
- * operands are 16-byte aligned (other shapes are passed on to that function).  fc_in is one grouped bf16 GEMM
- * that gathers the selected token rows in its operand fetch, fp32 output (pre), the GELU (fp32, erf to
- * 1.5e-7 absolute) is written as two bf16 terms side by side (split [total, 2 Ie]: bf16(g) and bf16(g - bf16(g)),
- * 16 significand bits), fc_out is one grouped bf16 GEMM over K = 2 Ie against the same weight columns, fp32
- * out (y), then the ordered add into d_mixed as in cf_moe_grouped_expert_forward_fp8_ws, with the same one
- * difference from the reference kernel.  Workspace rules as there; CF_MOE_FWD_WS_SPLIT_DESCALE is unused. */
+/* moe_grouped_expert_forward_bf16 (kernels.hpp:400-407, kernels/moe.cu:800-851) with a workspace: the same
+ * arguments and contract as cf_moe_grouped_expert_forward_bf16, run as whole-matrix launches when H % 8 == 0,
+ * Ie % 64 == 0 and the operands are 16-byte aligned (other shapes are passed on to that function).  fc_in is one
+ * grouped bf16 GEMM that gathers the selected token rows in its operand fetch, fp32 output (pre); the GELU (fp32,
+ * erf to 1.5e-7 absolute) is rounded to bf16 as the reference kernel rounds it before fc_out (split [total, Ie]
+ * bf16); fc_out is one grouped bf16 GEMM, fp32 out (y); then the ordered add into d_mixed as in
+ * cf_moe_grouped_expert_forward_fp8_ws, with the same one difference from the reference kernel.  Workspace rules
+ * as there; CF_MOE_FWD_WS_SPLIT_DESCALE is unused. */
 int cf_moe_grouped_expert_forward_bf16_workspace(int rows, int total_selected_rows, int num_experts, int H,
                                                  int Ie, size_t* offsets, size_t* bytes);
 int cf_moe_grouped_expert_forward_bf16_ws(const uint16_t* d_hidden, const float* d_route_weights,
@@ -611,9 +617,10 @@ int cf_moe_grouped_expert_forward_bf16_ws(const uint16_t* d_hidden, const float*
                                           int Ie, int num_experts, int total_selected_rows,
                                           void* d_workspace, size_t workspace_bytes, cf_stream_t stream);
 
-/* moe_grouped_expert_forward_bf16, kernels.hpp:400-407: the same device-scheduled expert bank on
- * bf16 hidden states and bf16 weights (fc_in_w [E,Ie,H], fc_out_w [E,H,Ie]), no descales; fp32
- * accumulation, exact-erf GELU kept in fp32, compare-and-swap accumulation into d_mixed.  The
+/* moe_grouped_expert_forward_bf16, kernels.hpp:400-407 (kernel kernels/moe.cu:800-851): the same
+ * device-scheduled expert bank on bf16 hidden states and bf16 weights (fc_in_w [E,Ie,H], fc_out_w
+ * [E,H,Ie]), no descales; fp32 accumulation, exact-erf GELU rounded to bf16 before fc_out (as the
+ * kernel's shared-memory row holds it, :845), compare-and-swap accumulation into d_mixed.  The
  * non-FP8 sibling: bf16 MFMA for both projections when H % 64 == 0, Ie % 64 == 0, the operands are
  * 16-byte aligned and d_mixed 8-byte aligned (16-row tiles); a wave-parallel fp32 kernel
  * otherwise. */
@@ -637,9 +644,10 @@ int cf_gelu_quantize_rows_e4m3(const uint16_t* d_x, int rows, int K, void* d_out
  * in one call with no host round trip, on the FP8 matrix cores: same arguments as
  * cf_moe_grouped_expert_forward_fp8 plus a workspace.  Unlike that function (and like the loop)
  * the GELU output is rounded to bf16 and re-quantized to E4M3 before fc_out; its scale is per
- * token row (the loop's per-expert delayed scale needs host-side slot state).  d_offsets must be
- * the exclusive prefix sum of d_counts and total_selected_rows their sum.  H and Ie multiples of
- * 128 and at least 256; d_workspace 256-byte aligned, cf_moe_grouped_gelu_workspace_bytes() bytes. */
+ * token row; cf_moe_grouped_gelu_forward_fp8_slots below keeps the loop's per-expert delayed scale
+ * instead.  d_offsets must be the exclusive prefix sum of d_counts, total_selected_rows an upper
+ * bound on their sum.  H and Ie multiples of 128 and at least 256; d_workspace 256-byte aligned,
+ * cf_moe_grouped_gelu_workspace_bytes() bytes. */
 int cf_moe_grouped_gelu_workspace_bytes(int rows, int total_selected_rows, int num_experts, int H,
                                         int Ie, size_t* bytes);
 int cf_moe_grouped_gelu_forward_fp8(const void* d_hidden, const float* d_fcin_descale,
@@ -650,6 +658,58 @@ int cf_moe_grouped_gelu_forward_fp8(const void* d_hidden, const float* d_fcin_de
                                     const float* d_fc_out_descale, uint16_t* d_mixed, int rows,
                                     int H, int Ie, int num_experts, int total_selected_rows,
                                     void* d_workspace, size_t workspace_bytes, cf_stream_t stream);
+
+/* The steady-state branch of fp8_quant_act (src/trainer.cu:4823-4850) for a bank of per-expert activation slots in ONE
+ * launch: what the FP8 expert loop does once per expert on moe_fcout_act_slot(f8, layer, base + e) between its two
+ * GEMMs (src/trainer.cu:6910-6918).  d_x [total_rows, K] bf16 holds the experts' rows back to back (expert e:
+ * d_counts[e] rows from row d_offsets[e]); block e of d_slot_states (state_stride_words 4-byte words apart, each laid
+ * out as the device block of a cf_act_slot with this history_len) is expert e's slot.  Per expert with at least one
+ * row: the scale pair the previous call left is snapshotted, the rows are quantized with it (E4M3 or E5M2) while their
+ * amax is recorded, and history, cursor, count, scale and descale advance as fp8_update_delayed_scale does; an
+ * expert without rows keeps its state untouched, as the loop's `continue` leaves it (:6887-6888).  apply_gelu: the
+ * tensor quantized is bf16(gelu(x)) (gelu_forward in place, kernels/moe.cu:510-521, then the quantize).
+ * is_recompute: quantize with the snapshot scale and change nothing (:4736-4743).  d_row_descale [total_rows]
+ * receives, for every row, its expert's descale_snapshot: what the GEMM consuming the bytes dequantizes with
+ * (:6921-6924).  The slots must be in steady state (calibration and first use go through cf_fp8_quant_act per
+ * expert) and share one format.  K % 16 == 0, 16-byte aligned d_x and d_out.  Calls on one bank must not overlap. */
+int cf_moe_grouped_quantize_delayed(const uint16_t* d_x, void* d_out, int K, int num_experts,
+                                    const int* d_counts, const int* d_offsets, int total_rows,
+                                    float* d_slot_states, int state_stride_words, int history_len,
+                                    int is_e5m2, int apply_gelu, int is_recompute, float* d_row_descale,
+                                    cf_stream_t stream);
+
+/* cf_moe_grouped_gelu_forward_fp8 with the reference loop's activation scale: the GELU output of expert e is
+ * quantized by cf_moe_grouped_quantize_delayed on slot e of d_fcout_slot_states (fp8_quant_act on
+ * moe_fcout_act_slot(..., e), src/trainer.cu:6916-6918) and fc_out dequantizes with that slot's descale_snapshot
+ * (:6921-6924); fcout_is_e5m2 is act_fp8_type of those slots.  is_recompute replays a forward for the backward
+ * (snapshot scale, no side effects).  Same workspace as cf_moe_grouped_gelu_forward_fp8. */
+int cf_moe_grouped_gelu_forward_fp8_slots(const void* d_hidden, const float* d_fcin_descale,
+                                          int fcin_is_e5m2, const float* d_route_weights,
+                                          const int* d_counts, const int* d_offsets,
+                                          const int* d_row_indices, const void* d_fc_in_w,
+                                          const float* d_fc_in_descale, const void* d_fc_out_w,
+                                          const float* d_fc_out_descale, uint16_t* d_mixed, int rows,
+                                          int H, int Ie, int num_experts, int total_selected_rows,
+                                          float* d_fcout_slot_states, int state_stride_words,
+                                          int history_len, int fcout_is_e5m2, int is_recompute,
+                                          void* d_workspace, size_t workspace_bytes, cf_stream_t stream);
+
+/* cf_moe_grouped_gelu_backward_fp8 whose recompute quantizes the GELU output as the reference's backward loop does:
+ * fp8_quant_act with is_recompute = true on the expert's slot (src/trainer.cu:7707-7712), i.e. with the scale the
+ * forward call snapshotted and no side effects.  Same workspace as cf_moe_grouped_gelu_backward_fp8. */
+int cf_moe_grouped_gelu_backward_fp8_slots(const uint16_t* d_grad_mixed, const void* d_hidden_fp8,
+                                           const float* d_fcin_descale, int fcin_is_e5m2,
+                                           const uint16_t* d_hidden_bf16, const float* d_route_weights,
+                                           const int* d_counts, const int* d_offsets, const int* d_row_indices,
+                                           const void* d_fc_in_w8, const float* d_fc_in_descale,
+                                           const void* d_fc_out_w8, const float* d_fc_out_descale,
+                                           const uint16_t* d_fc_in_w, const uint16_t* d_fc_out_w,
+                                           float* d_grad_route_weights, uint16_t* d_grad_fc_in,
+                                           uint16_t* d_grad_fc_out, uint16_t* d_grad_hidden, int rows, int H, int Ie,
+                                           int num_experts, int total_selected_rows,
+                                           float* d_fcout_slot_states, int state_stride_words, int history_len,
+                                           int fcout_is_e5m2, void* d_workspace, size_t workspace_bytes,
+                                           cf_stream_t stream);
 
 /* ---- slot state machines (host logic of src/trainer.cu over the entry points above) ------- */
 

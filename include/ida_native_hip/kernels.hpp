@@ -201,11 +201,6 @@ inline void moe_grouped_expert_forward_fp8(const void* d_hidden, const float* d_
                                              d_row_indices, d_fc_in_w, d_fc_in_descale, d_fc_out_w, d_fc_out_descale,
                                              hip_detail::u(d_mixed), rows, H, Ie, num_experts, total_selected_rows, stream));
 }
-// Lends the library a device buffer for the calls whose reference argument lists carry no workspace (the two expert
-// banks above then run as whole-matrix GEMMs); (nullptr, 0) takes it back.  The trainer would pass a slice of its arena
-// once at start-up.
-inline void set_workspace(void* d_workspace, size_t bytes) { CF_FWD(cf_set_workspace(d_workspace, bytes)); }
-
 // The bf16 bank with a workspace slice: both projections as whole-matrix grouped bf16 GEMMs where the shape allows.
 inline size_t moe_grouped_expert_forward_bf16_workspace_bytes(int rows, int H, int Ie, int num_experts, int total_selected_rows) {
     size_t bytes = 0;

@@ -591,8 +591,9 @@ def moe_grouped_expert_forward_fp8_ref(hidden, fcin_descale, fcin_e5m2, route_we
 
 def moe_grouped_expert_forward_bf16_ref(hidden, route_weights, counts, row_indices, fc_in_w, fc_out_w, mixed0):
     """moe_grouped_expert_forward_bf16 (kernels/moe.cu, the bf16 sibling of the grouped FP8 expert forward) in
-    float64 numpy: per expert, its listed rows through fc_in [Ie,H], exact-erf GELU, fc_out [H,Ie], times the route
-    weight, summed into mixed.  hidden / weights are bf16 bit patterns; returns float64 [rows,H]."""
+    float64 numpy: per expert, its listed rows through fc_in [Ie,H], exact-erf GELU rounded to bf16 as the kernel parks
+    it in shared memory before fc_out (kernels/moe.cu:845), fc_out [H,Ie], times the route weight, summed into mixed.
+    hidden / weights are bf16 bit patterns; returns float64 [rows,H]."""
     import math
     erf = np.vectorize(math.erf, otypes=[np.float64])
     x = bf16_to_f32(hidden).astype(np.float64)
@@ -606,5 +607,6 @@ def moe_grouped_expert_forward_bf16_ref(hidden, route_weights, counts, row_indic
             continue
         pre = x[rows] @ w_in[e].T
         act = 0.5 * pre * (1.0 + erf(pre * 0.70710678118654752440))
+        act = bf16_to_f32(bf16_from_f32(act.astype(np.float32))).astype(np.float64)
         out[rows] += rw[rows, e][:, None] * (act @ w_out[e].T)
     return out

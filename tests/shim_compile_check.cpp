@@ -31,8 +31,7 @@ int main() {
     void (*f20)(const bf16*, const float*, const int*, const int*, const int*, const bf16*, const bf16*, bf16*, int, int, int, int, int,
                 void*, std::size_t, hipStream_t) = &moe_grouped_expert_forward_bf16;
     std::size_t (*f21)(int, int, int, int, int) = &moe_grouped_expert_forward_bf16_workspace_bytes;
-    void (*f22)(void*, std::size_t) = &set_workspace;
-    if (!f12 || !f13 || !f14 || !f15 || !f16 || !f17 || !f18 || !f19 || !f20 || !f21 || !f22) return 1;
+    if (!f12 || !f13 || !f14 || !f15 || !f16 || !f17 || !f18 || !f19 || !f20 || !f21) return 1;
     if (!f1 || !f2 || !f3 || !f4 || !f5 || !f6 || !f7 || !f8 || !f9 || !f10 || !f11) return 1;
     int ok = 0;
     try { swiglu_forward(nullptr, nullptr, nullptr, -1, nullptr); } catch (const std::invalid_argument&) { ++ok; }   // kernels/activations.cu:61-72

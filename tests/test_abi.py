@@ -47,8 +47,11 @@ def test_argument_errors_do_not_need_a_gpu(cf):
     assert cf.raw_cf_moe_grouped_expert_forward_fp8_workspace(100, 200, 4, 96, 72, None, ctypes.byref(n)) == 0 and n.value == 0
     assert cf.raw_cf_moe_grouped_expert_forward_fp8_workspace(-1, 0, 0, 0, 0, None, ctypes.byref(n)) == -1
     assert cf.raw_cf_moe_grouped_expert_forward_bf16_workspace(16384, 98304, 64, 2048, 1408, None, ctypes.byref(n)) == 0
-    assert 1_800_000_000 < n.value < 2_000_000_000
-    assert cf.raw_cf_set_workspace(None, 5) == -1 and cf.raw_cf_set_workspace(None, 0) == 0
+    assert 1_500_000_000 < n.value < 1_700_000_000      # bf16 form: the GELU output travels as one bf16 term
+    # the bank of per-expert delayed-scaling slots: argument checks before any launch
+    assert cf.raw_cf_moe_grouped_quantize_delayed(None, None, 256, 4, None, None, 100, None, 32, 8, 0, 1, 0, None, None) == -1
+    assert cf.raw_cf_moe_grouped_quantize_delayed(None, None, 256, 4, None, None, 0, None, 32, 8, 0, 1, 0, None, None) == 0
+    assert cf.raw_cf_moe_grouped_quantize_delayed(None, None, -1, 4, None, None, 0, None, 32, 8, 0, 1, 0, None, None) == -1
     nul = [None] * 12
     assert cf.raw_cf_moe_grouped_expert_forward_fp8_ws(None, None, 0, *nul[:9], 4, 256, 128, 2, 8, None, 0, None) == -1
     assert cf.raw_cf_moe_grouped_expert_forward_fp8_ws(None, None, 0, *nul[:9], 0, 256, 128, 2, 0, None, 0, None) == 0

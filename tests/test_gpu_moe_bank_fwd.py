@@ -372,51 +372,103 @@ def test_staged_bf16_bank_config5_size(cf, dev):
     assert delta.min() > 0.1 * np.median(delta) and delta.max() < 10.0 * np.median(delta)
 
 
-# ---- a lent workspace sends the reference's own argument lists to the whole-matrix forms --------------------------
+# ---- total_selected_rows is the caller's upper bound (rows * top_k, /root/reference/src/trainer.cu:6863) ------------
 
-def test_lent_workspace_routes_the_reference_signatures(cf, dev):
-    case("cf_set_workspace: moe_grouped_expert_forward_fp8 / _bf16 under the reference's argument lists")
-    b8 = Bank(dev, 500, 8, 2, 512, 256, False, seed=21)
+def run_total(cf, b, total, guard=4096, st=None, form="fp8"):
+    """The workspace form with `total` as the bound: workspace sized for it, guard bytes behind it that must survive."""
+    dev = b.dev
+    nbytes = ctypes.c_size_t()
+    if form == "fp8":
+        cf.cf_moe_grouped_expert_forward_fp8_workspace(b.rows, total, b.E, b.H, b.Ie, None, ctypes.byref(nbytes))
+    else:
+        cf.cf_moe_grouped_expert_forward_bf16_workspace(b.rows, total, b.E, b.H, b.Ie, None, ctypes.byref(nbytes))
+    nbytes = int(nbytes.value)
+    buf = torch.empty(nbytes + 256 + guard, dtype=torch.uint8, device=dev)
+    buf.fill_(0xA7)
+    shift = (-buf.data_ptr()) % 256
+    ws = buf[shift:shift + nbytes]
+    mixed = dev_bf16(b.mixed0, dev)
+    sc = lambda v: torch.tensor([v], dtype=torch.float32, device=dev)
+    s = stream() if st is None else st.cuda_stream
+    if form == "fp8":
+        cf.cf_moe_grouped_expert_forward_fp8_ws(dev_arr(b.hq, dev), sc(b.d_h), int(b.e5m2), dev_arr(b.rw, dev), dev_arr(b.counts, dev), None,
+                                                dev_arr(b.idx, dev), dev_arr(b.winq, dev), sc(b.d_in), dev_arr(b.woutq, dev), sc(b.d_out),
+                                                mixed, b.rows, b.H, b.Ie, b.E, total, ws, nbytes, s)
+    else:
+        cf.cf_moe_grouped_expert_forward_bf16_ws(dev_bf16(b.hidden, dev), dev_arr(b.rw, dev), dev_arr(b.counts, dev), None,
+                                                 dev_arr(b.idx, dev), dev_bf16(b.win, dev), dev_bf16(b.wout, dev), mixed, b.rows, b.H,
+                                                 b.Ie, b.E, total, ws, nbytes, s)
+    return mixed, buf, shift + nbytes
+
+
+def test_total_is_an_upper_bound(cf, dev):
+    case("workspace forms with total_selected_rows = rows * top_k above the sum of the counts (an expert nobody selects)")
+    b8 = Bank(dev, 500, 8, 2, 512, 256, False, seed=21, zero_expert=5)
     b16 = Bank16(dev, 500, 8, 2, 512, 256, seed=22)
+    # some rows select fewer than k experts once a weight underflows to zero: make that certain
+    b8.rw[::7, :] = 0.0
+    b8.rw[::7, 1] = 1.0
+    b8.counts, b8.idx = orc.moe_build_expert_row_lists(b8.rw)
+    b8.total = int(b8.counts.sum())
+    assert b8.total < b8.rows * b8.k and b8.counts[5] == 0
     want8 = bf16_bits(run(cf, b8)[0])
     want16 = bf16_bits(run16(cf, b16)[0])
-    _, n8 = workspace(cf, b8)
-    n16 = ctypes.c_size_t()
-    cf.cf_moe_grouped_expert_forward_bf16_workspace(b16.rows, b16.total, b16.E, b16.H, b16.Ie, None, ctypes.byref(n16))
-    nbytes = max(n8, int(n16.value))
-    buf = torch.empty(nbytes + 256, dtype=torch.uint8, device=dev)
-    ptr = buf.data_ptr() + (-buf.data_ptr()) % 256
+    for total in (b8.rows * b8.k, b8.rows * b8.k + 777):
+        mixed, buf, end = run_total(cf, b8, total)
+        torch.cuda.synchronize()
+        # the whole-matrix form is deterministic: the bound changes the layout, not a bit of the result
+        assert np.array_equal(bf16_bits(mixed), want8), total
+        assert bool((buf[end:] == 0xA7).all())
+    mixed, buf, end = run_total(cf, b16, b16.rows * b16.k + 300, form="bf16")
+    torch.cuda.synchronize()
+    assert np.array_equal(bf16_bits(mixed), want16)
+    assert bool((buf[end:] == 0xA7).all())
+    # the calls under the reference's own argument lists do not use the bound at all (kernels/moe.cu:1070)
     sc = lambda v: torch.tensor([v], dtype=torch.float32, device=dev)
-
-    def plain8(total):
+    for total in (b8.rows * b8.k + 5, 0):
         mixed = dev_bf16(b8.mixed0, dev)
         cf.cf_moe_grouped_expert_forward_fp8(dev_arr(b8.hq, dev), sc(b8.d_h), 0, dev_arr(b8.rw, dev), dev_arr(b8.counts, dev), None,
                                              dev_arr(b8.idx, dev), dev_arr(b8.winq, dev), sc(b8.d_in), dev_arr(b8.woutq, dev), sc(b8.d_out),
                                              mixed, b8.rows, b8.H, b8.Ie, b8.E, total, stream())
         torch.cuda.synchronize()
-        return mixed
+        check_result(b8, mixed)
 
-    def plain16(total):
-        mixed = dev_bf16(b16.mixed0, dev)
-        cf.cf_moe_grouped_expert_forward_bf16(dev_bf16(b16.hidden, dev), dev_arr(b16.rw, dev), dev_arr(b16.counts, dev), None,
-                                              dev_arr(b16.idx, dev), dev_bf16(b16.win, dev), dev_bf16(b16.wout, dev), mixed, b16.rows, b16.H,
-                                              b16.Ie, b16.E, total, stream())
-        torch.cuda.synchronize()
-        return mixed
 
-    assert cf.raw_cf_set_workspace(ptr + 8, nbytes) == -1                    # not 256-byte aligned
-    assert cf.raw_cf_set_workspace(None, nbytes) == -1 and cf.raw_cf_set_workspace(ptr, 0) == -1
-    try:
-        cf.cf_set_workspace(ptr, nbytes)
-        # the whole-matrix forms are deterministic: the same bits as the explicit-workspace calls
-        assert np.array_equal(bf16_bits(plain8(b8.total)), want8)
-        assert np.array_equal(bf16_bits(plain16(b16.total)), want16)
-        # too small for these shapes: the one-kernel forms run, same contract
-        cf.cf_set_workspace(ptr, 4096)
-        check_result(b8, plain8(b8.total))
-        check_result16(b16, plain16(b16.total))
-    finally:
-        cf.cf_set_workspace(None, 0)
-    # taken back: the reference's unused total may be anything again
-    check_result(b8, plain8(b8.rows * b8.k + 5))
-    check_result16(b16, plain16(0))
+def test_counts_beyond_the_bound_are_cut_not_written(cf, dev):
+    case("workspace forms with total_selected_rows BELOW the sum of the counts: rows beyond the bound are left out")
+    b = Bank(dev, 600, 6, 2, 512, 256, False, seed=31)
+    offs = orc.moe_expert_offsets(b.counts)
+    total = int(offs[4]) + 37                      # expert 4 keeps 37 rows, expert 5 none
+    assert total < b.total
+    mixed, buf, end = run_total(cf, b, total, guard=1 << 20)
+    torch.cuda.synchronize()
+    assert bool((buf[end:] == 0xA7).all()), "a write went past the workspace the bound sized"
+    # what is inside the bound is computed as ever: compare with a bank that holds exactly those pairs
+    kept = Bank(dev, 600, 6, 2, 512, 256, False, seed=31)
+    for e in range(b.E):
+        n_keep = max(0, min(int(b.counts[e]), total - int(offs[e])))
+        for s_ in range(n_keep, int(b.counts[e])):
+            kept.rw[b.idx[e, s_], e] = 0.0
+    kept.counts, kept.idx = orc.moe_build_expert_row_lists(kept.rw)
+    kept.total = int(kept.counts.sum())
+    assert kept.total == total
+    check_result(kept, mixed)
+
+
+def test_two_streams_two_workspaces(cf, dev):
+    case("two banks in flight at once on two streams, each with its own workspace")
+    a = Bank(dev, 700, 8, 2, 512, 384, False, seed=41)
+    b = Bank(dev, 650, 6, 3, 768, 256, False, seed=42)
+    want_a = bf16_bits(run(cf, a)[0])
+    want_b = bf16_bits(run(cf, b)[0])
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    outs = []
+    for rep in range(3):
+        ma, bufa, enda = run_total(cf, a, a.rows * a.k, st=s1)
+        mb, bufb, endb = run_total(cf, b, b.rows * b.k, st=s2)
+        outs.append((ma, mb, bufa, bufb))
+    torch.cuda.synchronize()
+    for ma, mb, _, _ in outs:
+        assert np.array_equal(bf16_bits(ma), want_a)
+        assert np.array_equal(bf16_bits(mb), want_b)

@@ -13,8 +13,14 @@ Prints ONE JSON line.  `value` is the step's GEMM work (2*M*N*K for gate, up and
 whole step time, quantize passes included.  `roofline` describes the dominant kernel (the fused
 gate/up GEMM) from HIP events recorded around that launch inside the timed region; `cpu_baseline`
 is the reference's CPU linear-forward idiom on config 1, timed on this host.  Extra keys: the step replayed
-from a HIP graph, a plain-copy HBM ceiling for the quantize kernels, socket power and shader clock sampled
-during the timed region.
+from a HIP graph, two HBM ceilings for the quantize kernels (a plain device copy, and a streaming kernel of the
+library with the quantize's own 2-read : 1-write traffic), socket power and shader clock sampled during the timed
+region.
+
+Before the W warm-up steps the same eager step runs for `--settle` seconds (default 0.5): right after the idle
+set-up phase the part is still ramping its clocks and the first tens of steps run several percent slower than the
+same step a second later.  The W warm-up steps and the K timed steps follow unchanged; the literal procedure without
+the settling phase is timed first and reported as `unsettled_ms_per_step`.
 """
 from __future__ import annotations
 
@@ -193,6 +199,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--settle", type=float, default=0.5,
+                    help="seconds of the same eager step run before the warm-up steps, so that the timed region is not the "
+                         "part's ramp after the idle set-up phase (0 = none)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--traffic-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy, so a rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this "
@@ -270,6 +279,25 @@ def main():
             dst.copy_(src)          # reads 1 GiB, writes 1 GiB
         torch.cuda.synchronize()
         del src, dst
+
+    # the literal procedure straight after set-up (W warm-up steps, K timed steps): on file beside the settled figure
+    for _ in range(args.warmup):
+        step(0)
+    torch.cuda.synchronize()
+    u0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(0)
+    torch.cuda.synchronize()
+    unsettled_ms = (time.perf_counter() - u0) * 1e3 / args.steps
+    # settling phase: the same eager step until the clocks have come up
+    settle_steps = 0
+    s0 = time.perf_counter()
+    while time.perf_counter() - s0 < args.settle:
+        for _ in range(25):
+            step(0)
+        torch.cuda.synchronize()
+        settle_steps += 25
+    settle_s = time.perf_counter() - s0
 
     for _ in range(args.warmup):
         step(0)
@@ -351,21 +379,38 @@ def main():
     # quantize (2 B read + 1 B written per element), from sources that are in no cache (five source buffers of 176 MB
     # used in turn, more than the 256 MB memory-side cache holds), bracketed like the kernels in the step.
     copy_bytes = int(1.5 * M * N)
-    srcs = [torch.full((copy_bytes,), i, dtype=torch.uint8, device=dev) for i in range(5)]
+    srcs = [torch.full((2 * M * N,), i, dtype=torch.uint8, device=dev) for i in range(5)]      # each as large as H
     dsts = [torch.empty(copy_bytes, dtype=torch.uint8, device=dev) for _ in range(2)]
     torch.cuda.synchronize()
     cts = []
     for i in range(15):
         a, b = ev(), ev()
         a.record()
-        dsts[i % 2].copy_(srcs[i % 5])
+        dsts[i % 2].copy_(srcs[i % 5][:copy_bytes])
         b.record()
         torch.cuda.synchronize()
         if i >= 5:
             cts.append(a.elapsed_time(b))
     copy_ms = sorted(cts)[len(cts) // 2]
     hbm_copy_gbps = 2.0 * copy_bytes / (copy_ms * 1e-3) / 1e9
-    del srcs, dsts
+    del dsts
+    # The like-for-like ceiling: the library's streaming kernel with the traffic shape of the H quantize (one wavefront
+    # per row, 2 x 14336 bytes read and 14336 written per row with streaming stores, no arithmetic to speak of), from
+    # the same rotation of cold sources and bracketed the same way; then back to back on one source.
+    probe_dst = torch.empty(M * N, dtype=torch.uint8, device=dev)
+    pts = []
+    for i in range(15):
+        a, b = ev(), ev()
+        a.record()
+        cf.cf_hbm_stream_probe_2r1w(srcs[i % 5], probe_dst, M, N, st)
+        b.record()
+        torch.cuda.synchronize()
+        if i >= 5:
+            pts.append(a.elapsed_time(b))
+    probe_ms = sorted(pts)[len(pts) // 2]
+    probe_b2b_ms = back_to_back(lambda: cf.cf_hbm_stream_probe_2r1w(srcs[0], probe_dst, M, N, st))
+    probe_bytes = 3.0 * M * N
+    del srcs, probe_dst
 
     # outside the timed steps: the two quantize kernels on their own (the brackets inside a step include a launch gap
     # that is a quarter of a 20 us kernel)
@@ -394,6 +439,9 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4),
+        "settle_s": round(settle_s, 3),
+        "settle_steps": settle_steps,
+        "unsettled_ms_per_step": round(unsettled_ms, 4),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -431,6 +479,17 @@ def main():
         "hbm_achievable_gbps": round(hbm_copy_gbps, 1),
         "hbm_achievable_note": f"plain device copy of {copy_bytes} bytes (as many bytes moved as the H quantize) from sources in "
                                f"no cache, one event bracket per copy like the kernels in the step: {copy_ms * 1e3:.1f} us",
+        "hbm_stream_2r1w": {
+            "note": "the library's streaming kernel with the H quantize's traffic (2 B read + 1 B written per element, one "
+                    "wavefront per row, streaming stores, no arithmetic): `cold` from sources in no cache with one event "
+                    "bracket per launch like the kernels in the step, `back_to_back` 20 launches on one source",
+            "bytes": int(probe_bytes),
+            "cold_us": round(probe_ms * 1e3, 2), "cold_gbps": round(probe_bytes / (probe_ms * 1e-3) / 1e9, 1),
+            "cold_pct_hbm_peak": round(100.0 * probe_bytes / (probe_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),
+            "back_to_back_us": round(probe_b2b_ms * 1e3, 2),
+            "back_to_back_gbps": round(probe_bytes / (probe_b2b_ms * 1e-3) / 1e9, 1),
+            "back_to_back_pct_hbm_peak": round(100.0 * probe_bytes / (probe_b2b_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),
+        },
         "graph_replay": {"ms_per_step": None if graph_ms is None else round(graph_ms, 4),
                          "tflops": None if graph_ms is None else round(total_flop / (graph_ms * 1e-3) / 1e12, 2),
                          "note": graph_note},

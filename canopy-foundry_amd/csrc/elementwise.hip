@@ -287,6 +287,21 @@ __global__ __launch_bounds__(kThreads) void k_bias_add(uint16_t* __restrict__ in
         row[c] = f32_to_bf16(bf16_to_f32(row[c]) + bf16_to_f32(bias[c]));
 }
 
+// A measuring stick, not part of the hot path: the memory traffic of a per-token quantize (32 bytes read, 16 written
+// per lane and step, one wavefront per row, the same streaming stores) with next to no arithmetic, so that what such
+// a kernel could reach on this part can be read beside what the quantize kernels do reach.
+__global__ __launch_bounds__(kThreads) void k_stream_2r1w(const uint4* __restrict__ src, uint4* __restrict__ dst, int rows, int steps) {
+    const int row = blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int lane = threadIdx.x & 63;
+    const uint4* s = src + static_cast<size_t>(row) * steps * 128;
+    uint4* d = dst + static_cast<size_t>(row) * steps * 64;
+    for (int i = 0; i < steps; ++i) {
+        const uint4 a = s[(i * 64 + lane) * 2], b = s[(i * 64 + lane) * 2 + 1];
+        store_stream16(d + i * 64 + lane, make_uint4(a.x ^ b.x, a.y ^ b.y, a.z ^ b.z, a.w ^ b.w));
+    }
+}
+
 }  // namespace
 }  // namespace cf
 
@@ -365,5 +380,15 @@ int cf_bias_add_strided_bf16(uint16_t* d_inout, const uint16_t* d_bias, int rows
 }
 
 const char* cf_version(void) { return "canopy-foundry_amd fp8 hot path, gfx950"; }
+
+int cf_hbm_stream_probe_2r1w(const void* d_src, void* d_dst, int rows, int row_bytes_out, cf_stream_t stream) {
+    if (rows < 0 || row_bytes_out < 0) return CF_ERR_INVALID_ARG;
+    if (rows == 0 || row_bytes_out == 0) return CF_OK;
+    if (!d_src || !d_dst) return CF_ERR_INVALID_ARG;
+    if (row_bytes_out % 1024 != 0 || !aligned16(d_src) || !aligned16(d_dst)) return CF_ERR_UNSUPPORTED;
+    k_stream_2r1w<<<ceil_div(rows, kThreads / 64), kThreads, 0, as_stream(stream)>>>(static_cast<const uint4*>(d_src),
+                                                                                     static_cast<uint4*>(d_dst), rows, row_bytes_out / 1024);
+    return launch_status();
+}
 
 }  // extern "C"

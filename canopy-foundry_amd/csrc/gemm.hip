@@ -55,6 +55,7 @@ struct GemmArgs {
     float* Cf;                   // fp32 [M,N] for EPI_ACCUM_F32 (C += product)
     int tiles_m, tiles_n;
     int force_staged;            // take the register-staged kernel even when the ring kernel applies
+    int duo;                     // 1: the two-workgroups-per-CU kernel where it applies, 2: the same without the stagger
     // grouped (per-expert) form, ring kernel only; all null / 0 for a dense GEMM
     const int* tile_map;         // [0] = number of row tiles, then (expert, first row, end row) per row tile
     const int* a_row_index;      // compact row r reads A row (and its descale) a_row_index[r]; null = r
@@ -1134,6 +1135,307 @@ void k_gemm_nt_ring(const GemmArgs p) {
     __builtin_amdgcn_s_waitcnt(kWaitVm0);
 }
 
+// ---- duo kernel: the ring kernel at half the tile edge, two workgroups per CU ------------------------------
+// Workgroup tile 128 x 128 x 128, four wavefronts 2 x 2, each 64 x 64 = 2 x 2 MFMA tiles (64 accumulator
+// registers), the same ring of five slots at 16 KiB each: 80 KiB, so a CU holds TWO workgroups and every SIMD two
+// wavefronts.  A tile's drain is vector-ALU work (scales, SiLU, bf16 rounding) during which the matrix cores of a
+// one-wavefront-per-SIMD kernel idle; here the other workgroup's MFMAs run under it, provided the two are out of
+// step.  The workgroup that got the upper half of the CU's LDS (readable from the hardware's LDS allocation
+// register) therefore starts half a tile late.  The price is twice the LDS and L2 bytes per FLOP of the 256 x 256
+// tile.  Dense and grouped per expert (128-row tiles over the 256-row tile table: an entry's second half may be
+// empty), E4M3 activations and weights, per-row x per-channel scales, plain or SiLU-gate epilogue; N a multiple of
+// the tile's output width.
+constexpr int DM = 128;
+constexpr int kDuoSlot = DM * BK;                  // 16 KiB
+constexpr int kDuoLds = kSlots * kDuoSlot;         // 80 KiB
+constexpr int kWaitVm4 = 0x0f74;
+
+template <int EPI, bool STAGGER>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void k_gemm_nt_duo(const GemmArgs p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    constexpr bool GATE = EPI == EPI_SILU_GATE;
+    constexpr int OUT_BN = GATE ? DM / 2 : DM;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int total_tiles = p.tiles_m * p.tiles_n;
+    int my_tiles, lin0, lstep;
+    if (gridDim.x % kXcds == 0) {
+        const int per = (total_tiles + kXcds - 1) / kXcds;
+        const int x = blockIdx.x % kXcds, i = blockIdx.x / kXcds;
+        lstep = gridDim.x / kXcds;
+        const int cnt = max(0, min(per, total_tiles - x * per));
+        my_tiles = (cnt - i + lstep - 1) / lstep;
+        lin0 = x * per + i;
+    } else {
+        lstep = gridDim.x;
+        my_tiles = (total_tiles - static_cast<int>(blockIdx.x) + lstep - 1) / lstep;
+        lin0 = blockIdx.x;
+    }
+    if (my_tiles <= 0) return;
+    const int ktiles = p.K / BK;      // >= 2, checked by the launcher
+
+    if constexpr (STAGGER) {
+        // the second workgroup of a CU (its LDS starts above the first one's) waits about half a tile's MFMA time
+        unsigned alloc;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_LDS_ALLOC, 0, 12)" : "=s"(alloc));
+        if (alloc != 0) {
+            for (int i = 0; i < (ktiles + 15) / 16; ++i) __builtin_amdgcn_s_sleep(127);
+        }
+    }
+
+    auto tile_at = [&](int seq, int& m0, int& n0) {
+        int tm, tn;
+        tile_coords(lin0 + seq * lstep, p.tiles_m, p.tiles_n, tm, tn);
+        m0 = tm * DM;
+        n0 = tn * OUT_BN;
+    };
+
+    // ---- global -> LDS: wave w copies rows [32w, 32w+32) of an operand tile, 8 rows per instruction ----
+    const int lrow = lane >> 3, lslot = lane & 7;
+    uint32_t xoff[4], woff[4];
+    // SiLU-gate: the W tile's rows are [gate 32 | up 32] for the columns of wavefront column 0, then the same for
+    // column 1, so wave w copies from one matrix only: gate for even w, up for odd w
+    const uint8_t* wsrc = (GATE && (wave & 1)) ? p.B2 : p.B;
+    auto aim = [&](int seq) {
+        int m0, n0;
+        tile_at(seq, m0, n0);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int row = wave * 32 + j * 8 + lrow;
+            const uint32_t gchunk = (lslot ^ swz(row)) * 16;
+            xoff[j] = static_cast<uint32_t>(min(m0 + row, p.M - 1)) * static_cast<uint32_t>(p.lda) + gchunk;
+            const int n = GATE ? n0 + (row >> 6) * 32 + (row & 31) : n0 + row;
+            woff[j] = static_cast<uint32_t>(min(n, p.N - 1)) * static_cast<uint32_t>(p.ldb) + gchunk;
+        }
+    };
+    uint32_t lds_wave = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(smem)) + wave * (32 * BK);
+    auto dma = [&](int slot, uint32_t voff, const uint8_t* base, auto jc) {
+        constexpr int J = decltype(jc)::value;
+        const uint32_t dst = lds_wave + slot;
+        asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3"
+                     :: "s"(dst), "n"(J * 8 * BK), "v"(voff), "s"(base) : "memory", "scc");
+    };
+    auto dma_x = [&](int slot, int k0, auto jc) { dma(slot, xoff[decltype(jc)::value], p.A + k0, jc); };
+    auto dma_w = [&](int slot, int k0, auto jc) { dma(slot, woff[decltype(jc)::value], wsrc + k0, jc); };
+
+    // ---- LDS -> MFMA operands ----
+    const int frow = lane & 31, khalf = lane >> 5, fs = swz(frow);
+    int rd[2][2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) rd[h][j] = frow * BK + (((h * 4 + khalf * 2 + j) ^ fs) << 4);
+    const uint8_t* xrd = smem + wm * 64 * BK;
+    const uint8_t* wrd = smem + wn * 64 * BK;
+
+    v16f acc[2][2];       // [weight tile][activation tile]
+    v8i wq[2][2], xq[2][2];
+    auto put = [](v8i& dst, int half, const uint4 v) {
+        dst[4 * half + 0] = (int)v.x; dst[4 * half + 1] = (int)v.y; dst[4 * half + 2] = (int)v.z; dst[4 * half + 3] = (int)v.w;
+    };
+    // read I (0..7) of k-half H: w0 x0 x1 w1, two reads each
+    auto read_one = [&](int sx, int sw, auto hc, auto ic) {
+        constexpr int H = decltype(hc)::value, I = decltype(ic)::value;
+        constexpr int t = I >> 1, half = I & 1;
+        const int r = rd[H][half];
+        if constexpr (t == 0)      put(wq[H][0], half, *reinterpret_cast<const uint4*>(wrd + sw + r));
+        else if constexpr (t <= 2) put(xq[H][t - 1], half, *reinterpret_cast<const uint4*>(xrd + sx + (t - 1) * 32 * BK + r));
+        else                       put(wq[H][1], half, *reinterpret_cast<const uint4*>(wrd + sw + 32 * BK + r));
+    };
+    auto mfma_one = [&](auto hc, auto ic, auto first_c) {
+        constexpr int H = decltype(hc)::value, I = decltype(ic)::value;
+        constexpr int a = I >> 1, b = I & 1;
+        v16f c = acc[a][b];
+        if constexpr (decltype(first_c)::value != 0) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) c[r] = 0.0f;
+        }
+        acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wq[H][a], xq[H][b], c, 0, 0, 0, 0, 0, 0);
+    };
+    using C0 = std::integral_constant<int, 0>;
+    using C1 = std::integral_constant<int, 1>;
+
+    int a0 = 0, a1 = kDuoSlot, a2 = 2 * kDuoSlot, a3 = 3 * kDuoSlot, a4 = 4 * kDuoSlot;
+
+    // what the drain needs in registers: row descales of this lane's two output rows and the channel descales of its
+    // columns (plain: cs[a][g] = four columns of quad g of weight tile a; SiLU-gate: cs[0][g] gate, cs[1][g] up)
+    float sa[2];
+    float4 cs[2][4];
+    auto load_scales = [&](int m0, int n0) {
+#pragma unroll
+        for (int b = 0; b < 2; ++b) sa[b] = p.sa[min(m0 + wm * 64 + b * 32 + (lane & 31), p.M - 1)];
+        if constexpr (GATE) {
+            const int col = n0 + wn * 32 + khalf * 4;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                cs[0][g] = *reinterpret_cast<const float4*>(p.sb + col + g * 8);
+                cs[1][g] = *reinterpret_cast<const float4*>(p.sb2 + col + g * 8);
+            }
+        } else {
+            const int col = n0 + wn * 64 + khalf * 4;
+#pragma unroll
+            for (int a = 0; a < 2; ++a)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) cs[a][g] = *reinterpret_cast<const float4*>(p.sb + col + a * 32 + g * 8);
+        }
+    };
+
+    auto ktile = [&](auto first_c, auto end_c, int dk0, int m0, int n0, bool wait) {
+        constexpr bool END = decltype(end_c)::value != 0;
+        // step (g,0): 4 MFMAs, the operand reads of (g,1), the copies of X(g+2)
+        static_for<0, 4>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            mfma_one(C0{}, ic, first_c);
+            read_one(a0, a1, C1{}, std::integral_constant<int, 2 * i>{});
+            read_one(a0, a1, C1{}, std::integral_constant<int, 2 * i + 1>{});
+            dma_x(a4, dk0, ic);
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        // step (g,1)
+        mfma_one(C1{}, C0{}, C0{});
+        __builtin_amdgcn_sched_barrier(0);
+        if (wait) __builtin_amdgcn_s_waitcnt(kWaitVm4);
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<1, 4>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            mfma_one(C1{}, ic, C0{});
+            if constexpr (!END) {
+                static_for<0, 3>([&](auto jc) {
+                    constexpr int j = (i - 1) * 3 + decltype(jc)::value;
+                    if constexpr (j < 8) read_one(a2, a3, C0{}, std::integral_constant<int, j < 8 ? j : 0>{});
+                });
+            }
+            if constexpr (i == 1) { dma_w(a0, dk0, C0{}); dma_w(a0, dk0, C1{}); }
+            if constexpr (i == 2) dma_w(a0, dk0, std::integral_constant<int, 2>{});
+            if constexpr (i == 3) dma_w(a0, dk0, std::integral_constant<int, 3>{});
+            if constexpr (END && i == 1) load_scales(m0, n0);
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+    auto rotate = [&]() {
+        const int b0 = a0, b1 = a1;
+        a0 = a2; a1 = a3; a2 = a4; a3 = b0; a4 = b1;
+    };
+
+    // copy position: two K-tiles ahead of the compute position; past the last tile the stream re-reads that tile
+    int dkt = 2 % ktiles, dseq = 2 / ktiles;
+    aim(0);
+    static_for<0, 4>([&](auto jc) { dma_x(a0, 0, jc); });
+    static_for<0, 4>([&](auto jc) { dma_w(a1, 0, jc); });
+    static_for<0, 4>([&](auto jc) { dma_x(a2, BK, jc); });
+    static_for<0, 4>([&](auto jc) { dma_w(a3, BK, jc); });
+    if (dseq == 1 && my_tiles > 1) aim(1);
+    __builtin_amdgcn_s_waitcnt(kWaitVm8);
+    __syncthreads();
+    static_for<0, 8>([&](auto ic) { read_one(a0, a1, C0{}, ic); });
+
+    auto advance_copy = [&]() {
+        if (++dkt == ktiles) {
+            dkt = 0;
+            if (++dseq < my_tiles) aim(dseq);
+        }
+    };
+
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    for (int seq = 0; seq < my_tiles; ++seq) {
+        int m0, n0;
+        tile_at(seq, m0, n0);
+        ktile(C1{}, C0{}, dkt * BK, m0, n0, seq == 0);
+        rotate(); advance_copy();
+        for (int kt = 1; kt + 1 < ktiles; ++kt) {
+            ktile(C0{}, C0{}, dkt * BK, m0, n0, true);
+            rotate(); advance_copy();
+        }
+        ktile(C0{}, C1{}, dkt * BK, m0, n0, true);
+        rotate(); advance_copy();
+
+        // ---- drain: a4 is free until this workgroup's own copies of the stream's next K-tile but one ----
+        const int row = lane & 31;
+        const int wswz = (row >> 1) & 7;
+        const int rr = lane >> 3, rc = lane & 7;
+        if constexpr (GATE) {
+            // the two wavefronts of a row half share 64 rows x 128 bytes: each writes the 64 bytes per row of its 32
+            // output columns, then (barrier) each streams out 32 whole rows
+            uint8_t* stage = smem + a4 + wm * (64 * 128);
+            uint8_t* wr = stage + row * 128 + khalf * 8;
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const float c4[4] = {cs[0][g].x, cs[0][g].y, cs[0][g].z, cs[0][g].w};
+                    const float u4[4] = {cs[1][g].x, cs[1][g].y, cs[1][g].z, cs[1][g].w};
+                    float v[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        // the reference rounds gate and up to bf16 before the SiLU product
+                        const uint32_t gu = pack_bf16x2_hw(acc[0][b][g * 4 + q] * (sa[b] * c4[q]), acc[1][b][g * 4 + q] * (sa[b] * u4[q]));
+                        v[q] = fast_silu(bf16_lo(gu)) * bf16_hi(gu);
+                    }
+                    *reinterpret_cast<uint2*>(wr + b * 32 * 128 + (((wn * 4 + g) ^ wswz) << 4)) =
+                        make_uint2(pack_bf16x2_hw(v[0], v[1]), pack_bf16x2_hw(v[2], v[3]));
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // every copy in flight is waited for before the first store (stores and copies share one counter); the tile
+            // that follows skips the wait of its first K-tile
+            __builtin_amdgcn_s_waitcnt(kWaitVm0);
+            __syncthreads();
+            const uint8_t* rdp0 = stage + (wn * 32 + rr) * 128 + ((rc ^ (rr >> 1)) << 4);
+            const uint8_t* rdp1 = stage + (wn * 32 + rr) * 128 + ((rc ^ (rr >> 1) ^ 4) << 4);
+            uint8_t* cu = reinterpret_cast<uint8_t*>(p.C + static_cast<size_t>(m0 + wm * 64 + wn * 32) * p.ldc + n0);
+            const uint32_t coff = (static_cast<uint32_t>(rr) * static_cast<uint32_t>(p.ldc) + rc * 8u) * 2u;
+            const size_t cstep = static_cast<size_t>(p.ldc) * 16;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint4 v = *reinterpret_cast<const uint4*>(((i & 1) ? rdp1 : rdp0) + i * 8 * 128);
+                if (m0 + wm * 64 + wn * 32 + rr + i * 8 < p.M) {
+                    const u32x4 vv = {v.x, v.y, v.z, v.w};
+                    __builtin_nontemporal_store(vv, reinterpret_cast<u32x4*>(cu + i * cstep + coff));
+                }
+            }
+        } else {
+            // per 32 output rows: 32 rows x 128 bytes in this wavefront's own 4 KiB, then out as whole lines
+            uint8_t* stage = smem + a4 + wave * (32 * BK);
+            uint8_t* wr = stage + row * 128 + khalf * 8;
+            const uint8_t* rdp0 = stage + rr * 128 + ((rc ^ (rr >> 1)) << 4);
+            const uint8_t* rdp1 = stage + rr * 128 + ((rc ^ (rr >> 1) ^ 4) << 4);
+            uint8_t* cu = reinterpret_cast<uint8_t*>(p.C + static_cast<size_t>(m0 + wm * 64) * p.ldc + n0 + wn * 64);
+            const uint32_t coff = (static_cast<uint32_t>(rr) * static_cast<uint32_t>(p.ldc) + rc * 8u) * 2u;
+            const size_t cstep = static_cast<size_t>(p.ldc) * 16;
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+#pragma unroll
+                for (int a = 0; a < 2; ++a)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const float c4[4] = {cs[a][g].x, cs[a][g].y, cs[a][g].z, cs[a][g].w};
+                        float v[4];
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) v[q] = acc[a][b][g * 4 + q] * (sa[b] * c4[q]);
+                        *reinterpret_cast<uint2*>(wr + (((a * 4 + g) ^ wswz) << 4)) =
+                            make_uint2(pack_bf16x2_hw(v[0], v[1]), pack_bf16x2_hw(v[2], v[3]));
+                    }
+                __builtin_amdgcn_sched_barrier(0);
+                if (b == 0) __builtin_amdgcn_s_waitcnt(kWaitVm0);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const uint4 v = *reinterpret_cast<const uint4*>(((i & 1) ? rdp1 : rdp0) + i * 8 * 128);
+                    if (m0 + wm * 64 + b * 32 + rr + i * 8 < p.M) {
+                        const u32x4 vv = {v.x, v.y, v.z, v.w};
+                        __builtin_nontemporal_store(vv, reinterpret_cast<u32x4*>(cu + (b * 4 + i) * cstep + coff));
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        static_for<0, 8>([&](auto ic) { read_one(a0, a1, C0{}, ic); });
+    }
+    __builtin_amdgcn_s_waitcnt(kWaitVm0);
+}
+
 // ---- block-scaled ring kernel ---------------------------------------------------------------
 // The block-scaled GEMM on the persistent direct-to-LDS structure.  Needs K % 128 == 0, K >= 384,
 // N % 256 == 0, operands smaller than 4 GiB, K / 128 <= 256.
@@ -1530,6 +1832,35 @@ int launch_tiled(const GemmArgs& p, hipStream_t st) {
     return launch_status();
 }
 
+// the duo kernel: E4M3 operands, per-row x per-channel scales, plain or SiLU-gate epilogue, whole column tiles
+template <int EPI>
+int launch_duo(GemmArgs p, hipStream_t st) {
+    static std::once_flag once;
+    static hipError_t err = hipSuccess;
+    std::call_once(once, [] {
+        err = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_nt_duo<EPI, true>), hipFuncAttributeMaxDynamicSharedMemorySize, kDuoLds);
+        if (err == hipSuccess)
+            err = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_nt_duo<EPI, false>), hipFuncAttributeMaxDynamicSharedMemorySize, kDuoLds);
+    });
+    if (err != hipSuccess) return static_cast<int>(err);
+    constexpr int out_bn = EPI == EPI_SILU_GATE ? DM / 2 : DM;
+    p.tiles_m = (p.M + DM - 1) / DM;
+    p.tiles_n = p.N / out_bn;
+    const int total = p.tiles_m * p.tiles_n;
+    int grid = total < 2 * num_cus() ? total : 2 * num_cus();
+    if (grid >= kXcds) grid -= grid % kXcds;
+    if (p.duo == 2) k_gemm_nt_duo<EPI, false><<<grid, kThreads, kDuoLds, st>>>(p);
+    else            k_gemm_nt_duo<EPI, true><<<grid, kThreads, kDuoLds, st>>>(p);
+    return launch_status();
+}
+inline bool duo_ok(const GemmArgs& p, int fmt, int epi, int scale_mode) {
+    const int out_bn = epi == EPI_SILU_GATE ? DM / 2 : DM;
+    return fmt == 0 && scale_mode == SCALE_ROWCOL && (epi == EPI_NONE || epi == EPI_SILU_GATE) && !p.tile_map && p.K % BK == 0 &&
+           p.K >= 2 * BK && p.N % out_bn == 0 && p.ldc % 8 == 0 && aligned16(p.C) && aligned16(p.sb) &&
+           (epi != EPI_SILU_GATE || aligned16(p.sb2)) && static_cast<size_t>(p.M) * p.lda < (1ull << 32) &&
+           static_cast<size_t>(p.N) * p.ldb < (1ull << 32);
+}
+
 template <int FMT, int EPI>
 int dispatch_scale(const GemmArgs& p, int scale_mode, hipStream_t st) {
     return scale_mode == SCALE_TENSOR ? launch_tiled<FMT, EPI, SCALE_TENSOR>(p, st)
@@ -1691,6 +2022,8 @@ int gemm_nt(GemmArgs p, int fmt, int epi, int scale_mode, int force_naive, cf_st
         }
     }
     if (fmt & 2) return CF_ERR_UNSUPPORTED;     // forward weights are always E4M3
+    if (p.duo && duo_ok(p, fmt, epi, scale_mode))
+        return epi == EPI_SILU_GATE ? launch_duo<EPI_SILU_GATE>(p, st) : launch_duo<EPI_NONE>(p, st);
     return (fmt & 1) ? dispatch_epi<1>(p, epi, scale_mode, st) : dispatch_epi<0>(p, epi, scale_mode, st);
 }
 
@@ -1726,6 +2059,7 @@ int cf_fp8_gemm_nt_bf16_ex(int M, int N, int K, const void* A, int lda, int a_is
     p.C = C; p.ldc = ldc;
     if (epilogue > EPI_SILU_GATE) return CF_ERR_INVALID_ARG;
     p.force_staged = (flags & CF_GEMM_FLAG_STAGED) != 0;
+    p.duo = (flags & CF_GEMM_FLAG_DUO) ? ((flags & CF_GEMM_FLAG_DUO_IN_STEP) ? 2 : 1) : 0;
     return gemm_nt(p, a_is_e5m2 ? 1 : 0, epilogue, scale_mode, flags & CF_GEMM_FLAG_NAIVE, stream);
 }
 

@@ -251,6 +251,10 @@ int cf_cross_entropy_fwd_bwd_chunk_quant_e5m2(const uint16_t* d_logits, const in
 
 #define CF_GEMM_FLAG_NAIVE 1   /* run the one-lane-per-output cross-check kernel  */
 #define CF_GEMM_FLAG_STAGED 2  /* take the register-staged tile kernel (the K % 64 != 0 path) */
+#define CF_GEMM_FLAG_DUO 4     /* take the 128 x 128-tile kernel that runs two workgroups per CU (a tile's epilogue under
+                                  the other workgroup's MFMAs) where it applies: E4M3, CF_SCALE_ROW_COL, plain or SiLU-gate
+                                  epilogue, N a multiple of 128 (64 with the SiLU gate) */
+#define CF_GEMM_FLAG_DUO_IN_STEP 8 /* with CF_GEMM_FLAG_DUO: do not start the CU's second workgroup half a tile late */
 
 /* lt_gemm_fp8_nt, static at src/trainer.cu:4498-4534 (plan lookup :4402-4496).
  * C[M,N] bf16 (row stride ldc) = (A[M,K] fp8, row stride lda, E4M3 or E5M2) .
@@ -710,6 +714,11 @@ int cf_moe_grouped_gelu_backward_fp8_slots(const uint16_t* d_grad_mixed, const v
                                            float* d_fcout_slot_states, int state_stride_words, int history_len,
                                            int fcout_is_e5m2, void* d_workspace, size_t workspace_bytes,
                                            cf_stream_t stream);
+
+/* A measuring stick for the benchmark, with no counterpart in the reference and no part in the hot path: a kernel
+ * with the memory traffic of the per-token quantize (per row 2 x row_bytes_out bytes read, row_bytes_out written with
+ * the same streaming stores, one wavefront per row) and next to no arithmetic.  row_bytes_out % 1024 == 0. */
+int cf_hbm_stream_probe_2r1w(const void* d_src, void* d_dst, int rows, int row_bytes_out, cf_stream_t stream);
 
 /* ---- slot state machines (host logic of src/trainer.cu over the entry points above) ------- */
 

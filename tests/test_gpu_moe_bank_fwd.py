@@ -265,8 +265,8 @@ def check_result16(b, mixed):
 
 @pytest.mark.parametrize("rows,E,k,H,Ie,zero", [
     (70, 3, 3, 2048, 1408, None),        # config 5's widths
-    (300, 6, 3, 256, 320, None),         # Ie = 5 K-tiles: the second term starts at an odd K-tile
-    (200, 4, 2, 64, 64, None),           # one K-tile per term and per projection
+    (300, 6, 3, 256, 320, None),         # Ie = 5 K-tiles
+    (200, 4, 2, 64, 64, None),           # one K-tile per projection
     (1000, 5, 2, 192, 448, 2),           # several row tiles per expert, ragged, an expert with no rows; N = 448 and 192 end inside a column tile
     (21, 5, 2, 200, 128, None),          # H % 64 != 0: the k range of fc_in ends inside a K-tile
 ])
@@ -294,12 +294,16 @@ def test_staged_bf16_bank_stage_by_stage(cf, dev, rows, E, k, H, Ie, zero):
         ad = np.abs(hx[index[sel]]) @ np.abs(win[e]).T
         assert np.all(np.abs(pre[sel] - want) <= 2.0 ** -22 * np.abs(want) + ACC_BF16 * ad), f"fc_in expert {e}"
 
-    split = orc.bf16_to_f32(take("SPLIT", np.uint16, T * 2 * Ie).reshape(T, 2, Ie)).astype(np.float64)
-    act = split[:, 0] + split[:, 1]
+    # the GELU output rounded to bf16, as the reference kernel parks it before fc_out (kernels/moe.cu:845)
+    act_bits = take("SPLIT", np.uint16, T * Ie).reshape(T, Ie)
+    act = orc.bf16_to_f32(act_bits).astype(np.float64)
     g = gelu64(pre)
-    tol = 2.0 ** -16 * np.abs(g) + 4e-7 * (np.abs(pre) + 1e-3)
-    assert (np.abs(act - g) / tol).max() <= 1.0, "two bf16 terms carry the GELU to 16 bits"
-    assert np.all(np.abs(split[:, 1]) <= 2.0 ** -8 * np.abs(split[:, 0]) + 1e-30), "the second term is the first one's rounding error"
+    gb = orc.bf16_from_f32(g.astype(np.float32))
+    # the erf form is good to 4e-7 (|pre| + 1e-3) absolute: away from zero that can only flip a rounding now and then
+    big = np.abs(g) >= 2.0 ** -6
+    off_by = np.abs(act_bits.astype(np.int64) - gb.astype(np.int64))[big]
+    assert off_by.max() <= 1 and (off_by != 0).mean() < 2e-2, (off_by.max(), (off_by != 0).mean())
+    assert (np.abs(act - g) <= 2.0 ** -8 * np.abs(g) + 4e-7 * (np.abs(pre) + 1e-3)).all()
 
     y = take("Y", np.float32, T * H).reshape(T, H).astype(np.float64)
     for e in range(E):
@@ -307,7 +311,7 @@ def test_staged_bf16_bank_stage_by_stage(cf, dev, rows, E, k, H, Ie, zero):
         if not sel.any():
             continue
         want = act[sel] @ wout[e].T
-        ad = (np.abs(split[sel, 0]) + np.abs(split[sel, 1])) @ np.abs(wout[e]).T
+        ad = np.abs(act[sel]) @ np.abs(wout[e]).T
         tol = 2.0 ** -22 * np.abs(want) + ACC_BF16 * ad
         worst = np.abs(y[sel] - want) / tol
         assert worst.max() <= 1.0, f"fc_out expert {e}: worst {worst.max():.3f}"
@@ -389,16 +393,23 @@ def run_total(cf, b, total, guard=4096, st=None, form="fp8"):
     ws = buf[shift:shift + nbytes]
     mixed = dev_bf16(b.mixed0, dev)
     sc = lambda v: torch.tensor([v], dtype=torch.float32, device=dev)
+    # the operands are returned with the result: a call on a side stream may still be reading them when this returns
+    if form == "fp8":
+        ops = [dev_arr(b.hq, dev), sc(b.d_h), dev_arr(b.rw, dev), dev_arr(b.counts, dev), dev_arr(b.idx, dev), dev_arr(b.winq, dev),
+               sc(b.d_in), dev_arr(b.woutq, dev), sc(b.d_out)]
+    else:
+        ops = [dev_bf16(b.hidden, dev), dev_arr(b.rw, dev), dev_arr(b.counts, dev), dev_arr(b.idx, dev), dev_bf16(b.win, dev),
+               dev_bf16(b.wout, dev)]
+    if st is not None:
+        st.wait_stream(torch.cuda.current_stream())      # the uploads above ran on the current stream
     s = stream() if st is None else st.cuda_stream
     if form == "fp8":
-        cf.cf_moe_grouped_expert_forward_fp8_ws(dev_arr(b.hq, dev), sc(b.d_h), int(b.e5m2), dev_arr(b.rw, dev), dev_arr(b.counts, dev), None,
-                                                dev_arr(b.idx, dev), dev_arr(b.winq, dev), sc(b.d_in), dev_arr(b.woutq, dev), sc(b.d_out),
+        cf.cf_moe_grouped_expert_forward_fp8_ws(ops[0], ops[1], int(b.e5m2), ops[2], ops[3], None, ops[4], ops[5], ops[6], ops[7], ops[8],
                                                 mixed, b.rows, b.H, b.Ie, b.E, total, ws, nbytes, s)
     else:
-        cf.cf_moe_grouped_expert_forward_bf16_ws(dev_bf16(b.hidden, dev), dev_arr(b.rw, dev), dev_arr(b.counts, dev), None,
-                                                 dev_arr(b.idx, dev), dev_bf16(b.win, dev), dev_bf16(b.wout, dev), mixed, b.rows, b.H,
+        cf.cf_moe_grouped_expert_forward_bf16_ws(ops[0], ops[1], ops[2], None, ops[3], ops[4], ops[5], mixed, b.rows, b.H,
                                                  b.Ie, b.E, total, ws, nbytes, s)
-    return mixed, buf, shift + nbytes
+    return mixed, (buf, ops), shift + nbytes
 
 
 def test_total_is_an_upper_bound(cf, dev):
@@ -414,15 +425,15 @@ def test_total_is_an_upper_bound(cf, dev):
     want8 = bf16_bits(run(cf, b8)[0])
     want16 = bf16_bits(run16(cf, b16)[0])
     for total in (b8.rows * b8.k, b8.rows * b8.k + 777):
-        mixed, buf, end = run_total(cf, b8, total)
+        mixed, keep, end = run_total(cf, b8, total)
         torch.cuda.synchronize()
         # the whole-matrix form is deterministic: the bound changes the layout, not a bit of the result
         assert np.array_equal(bf16_bits(mixed), want8), total
-        assert bool((buf[end:] == 0xA7).all())
-    mixed, buf, end = run_total(cf, b16, b16.rows * b16.k + 300, form="bf16")
+        assert bool((keep[0][end:] == 0xA7).all())
+    mixed, keep, end = run_total(cf, b16, b16.rows * b16.k + 300, form="bf16")
     torch.cuda.synchronize()
     assert np.array_equal(bf16_bits(mixed), want16)
-    assert bool((buf[end:] == 0xA7).all())
+    assert bool((keep[0][end:] == 0xA7).all())
     # the calls under the reference's own argument lists do not use the bound at all (kernels/moe.cu:1070)
     sc = lambda v: torch.tensor([v], dtype=torch.float32, device=dev)
     for total in (b8.rows * b8.k + 5, 0):
@@ -440,9 +451,9 @@ def test_counts_beyond_the_bound_are_cut_not_written(cf, dev):
     offs = orc.moe_expert_offsets(b.counts)
     total = int(offs[4]) + 37                      # expert 4 keeps 37 rows, expert 5 none
     assert total < b.total
-    mixed, buf, end = run_total(cf, b, total, guard=1 << 20)
+    mixed, keep, end = run_total(cf, b, total, guard=1 << 20)
     torch.cuda.synchronize()
-    assert bool((buf[end:] == 0xA7).all()), "a write went past the workspace the bound sized"
+    assert bool((keep[0][end:] == 0xA7).all()), "a write went past the workspace the bound sized"
     # what is inside the bound is computed as ever: compare with a bank that holds exactly those pairs
     kept = Bank(dev, 600, 6, 2, 512, 256, False, seed=31)
     for e in range(b.E):
@@ -465,9 +476,9 @@ def test_two_streams_two_workspaces(cf, dev):
     torch.cuda.synchronize()
     outs = []
     for rep in range(3):
-        ma, bufa, enda = run_total(cf, a, a.rows * a.k, st=s1)
-        mb, bufb, endb = run_total(cf, b, b.rows * b.k, st=s2)
-        outs.append((ma, mb, bufa, bufb))
+        ma, keepa, _ = run_total(cf, a, a.rows * a.k, st=s1)
+        mb, keepb, _ = run_total(cf, b, b.rows * b.k, st=s2)
+        outs.append((ma, mb, keepa, keepb))
     torch.cuda.synchronize()
     for ma, mb, _, _ in outs:
         assert np.array_equal(bf16_bits(ma), want_a)

@@ -844,7 +844,14 @@ int launch_quant_rows(const uint16_t* d_x, int rows, int K, void* d_out, float* 
             return launch_status();
         }
     }
-    if (vec && K <= 4 * 1024) k_quant_rows<E5M2, 4, GELU><<<grid, kThreads, 0, st>>>(d_x, rows, K, o, d_scale, d_descale);
+    // Rows of 2049 to 4096 elements: a workgroup of four wavefronts per row (one 32-byte load per lane) rather than a
+    // wavefront per row.  With a wavefront per row every wavefront of an 8192-row tensor is resident at once and all of
+    // them read, then all of them write; four times as many, smaller, workgroups come and go in waves, so reads and
+    // writes overlap.  Measured inside the benchmark step (input in no cache): 22.5 -> 20.9 us at 8192 x 4096, the same
+    // back to back; capping the occupancy of the wavefront-per-row form or giving each wavefront several rows with the
+    // next row's loads in flight measured the same or worse.
+    if (vec && K > 2 * 1024 && K <= 4 * 1024) k_quant_rows_block<E5M2, 1, GELU><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);
+    else if (vec && K <= 4 * 1024) k_quant_rows<E5M2, 4, GELU><<<grid, kThreads, 0, st>>>(d_x, rows, K, o, d_scale, d_descale);
     else if (vec && K <= 16 * 1024) k_quant_rows_block<E5M2, 4, GELU><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);
     else if (vec && K <= 32 * 1024) k_quant_rows_block<E5M2, 8, GELU><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);
     else k_quant_rows_generic<E5M2, GELU><<<rows, kThreads, 0, st>>>(d_x, K, o, d_scale, d_descale);

@@ -25,6 +25,9 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--only", default="", help="time only the rows whose name contains this text (for profiler runs)")
+    ap.add_argument("--sustain", type=float, default=0.0,
+                    help="after timing a GEMM row, hold it back to back for this many seconds and print the rate, the socket "
+                         "power and the shader clock over the second half of that time (sysfs, as bench.py samples them)")
     args = ap.parse_args()
     import torch
     sys.path.insert(0, str(ROOT))
@@ -78,12 +81,30 @@ def main():
 
     BF16_PEAK = 2500.0          # dense bf16 matrix peak, TFLOP/s
 
+    def sustained(fn, flop):
+        import time
+        from bench import PowerSampler
+        with PowerSampler(period_s=0.01) as ps:
+            t0 = time.perf_counter()
+            n = 0
+            while time.perf_counter() - t0 < args.sustain:
+                for _ in range(50):
+                    fn()
+                torch.cuda.synchronize()
+                n += 50
+            dt = time.perf_counter() - t0
+        r = ps.report(skip_fraction=0.5)
+        print(f"    held {dt:.1f} s: {dt / n * 1e6:9.1f} us per launch = {flop * n / dt / 1e12:6.0f} TFLOP/s, "
+              f"{r.get('socket_power_w_avg')} W of {ps.cap_watts()} W, shader clock {r.get('sclk_mhz_avg')} MHz", flush=True)
+
     def mfma16(name, shape, flop, fn):
         if args.only not in name:
             return
         t = timed(fn)
         tf = flop / t / 1e12
         print(f"{name:<64} {shape:<26} {t * 1e6:9.1f} {tf:7.0f} TFLOP/s {100 * tf / BF16_PEAK:7.1f}% (of bf16 peak)", flush=True)
+        if args.sustain > 0:
+            sustained(fn, flop)
 
     def mfma(name, shape, flop, fn):
         if args.only not in name:
@@ -92,6 +113,8 @@ def main():
         t = timed(fn)
         tf = flop / t / 1e12
         print(f"{name:<64} {shape:<26} {t * 1e6:9.1f} {tf:7.0f} TFLOP/s {100 * tf / FP8_PEAK:7.1f}%", flush=True)
+        if args.sustain > 0:
+            sustained(fn, flop)
 
     # ---- config 2 activations / weights: quantize family -------------------------------------------
     M, K, N = 8192, 4096, 14336
@@ -197,6 +220,14 @@ def main():
          lambda: cf.cf_fp8_gemm_nt_bf16_ex(M, N, K, xq, K, 0, xd, wg, K, wgd, 1, 2, None, wu, wud, c, N, 0, st))
     mfma("gemm down projection (config 2)", f"{M}x{K}x{N}", 2.0 * M * N * K,
          lambda: cf.cf_fp8_gemm_nt_bf16_ex(M, K, N, hq, N, 0, xd, wd, N, wdd, 1, 0, None, None, None, y, K, 0, st))
+    # the same two launches on the 128 x 128-tile kernel that runs two workgroups per CU (CF_GEMM_FLAG_DUO = 4;
+    # 12 = without starting the second workgroup of a CU half a tile late)
+    mfma("duo: gemm gate+up fused SiLU-gate (config 2), 2 workgroups per CU", f"{M}x2x{N}x{K}", 4.0 * M * N * K,
+         lambda: cf.cf_fp8_gemm_nt_bf16_ex(M, N, K, xq, K, 0, xd, wg, K, wgd, 1, 2, None, wu, wud, c, N, 4, st))
+    mfma("duo in step: gemm gate+up fused SiLU-gate (config 2)", f"{M}x2x{N}x{K}", 4.0 * M * N * K,
+         lambda: cf.cf_fp8_gemm_nt_bf16_ex(M, N, K, xq, K, 0, xd, wg, K, wgd, 1, 2, None, wu, wud, c, N, 12, st))
+    mfma("duo: gemm down projection (config 2), 2 workgroups per CU", f"{M}x{K}x{N}", 2.0 * M * N * K,
+         lambda: cf.cf_fp8_gemm_nt_bf16_ex(M, K, N, hq, N, 0, xd, wd, N, wdd, 1, 0, None, None, None, y, K, 4, st))
     dy = fp8(M, N, e5m2=True)
     mfma("gemm dgrad, E5M2 dY (config 4)", f"{M}x{K}x{N}", 2.0 * M * N * K,
          lambda: cf.cf_fp8_gemm_nt_bf16(M, K, N, dy, N, 1, sc, wd, de, y, K, st))
@@ -262,10 +293,21 @@ def main():
          lambda: cf.cf_fp8_grouped_gemm_nt_bf16_ex(total, Ie, H, E, counts, offs, hq, T, H, cidx, hd, wg, wgd, 1, 2, wu, wud,
                                                    act, Ie, ws, sz.value, st))
     actq = fp8(total, Ie); ad = f32(total)
+    actq_x = fp8(total, H)
     yy = torch.empty((total, H), dtype=torch.bfloat16, device=dev)
     mfma("grouped down projection (config 5)", f"{total}x{H}x{Ie}", 2.0 * total * Ie * H,
          lambda: cf.cf_fp8_grouped_gemm_nt_bf16_ex(total, H, Ie, E, counts, offs, actq, total, Ie, None, ad, wd, wdd, 1, 0, None, None,
                                                    yy, H, ws, sz.value, st))
+    # the config 5 shapes as dense GEMMs (one expert's weights for all rows): what the short K costs without the
+    # grouping, on the 256 x 256-tile kernel and on the two-workgroups-per-CU kernel
+    mfma("dense at the config 5 shape: gate+up SiLU-gate", f"{total}x2x{Ie}x{H}", 4.0 * total * Ie * H,
+         lambda: cf.cf_fp8_gemm_nt_bf16_ex(total, Ie, H, actq_x, H, 0, ad, wg, H, wgd, 1, 2, None, wu, wud, act, Ie, 0, st))
+    mfma("duo: dense at the config 5 shape: gate+up SiLU-gate", f"{total}x2x{Ie}x{H}", 4.0 * total * Ie * H,
+         lambda: cf.cf_fp8_gemm_nt_bf16_ex(total, Ie, H, actq_x, H, 0, ad, wg, H, wgd, 1, 2, None, wu, wud, act, Ie, 4, st))
+    mfma("dense at the config 5 shape: down projection", f"{total}x{H}x{Ie}", 2.0 * total * Ie * H,
+         lambda: cf.cf_fp8_gemm_nt_bf16_ex(total, H, Ie, actq, Ie, 0, ad, wd, Ie, wdd, 1, 0, None, None, None, yy, H, 0, st))
+    mfma("duo: dense at the config 5 shape: down projection", f"{total}x{H}x{Ie}", 2.0 * total * Ie * H,
+         lambda: cf.cf_fp8_gemm_nt_bf16_ex(total, H, Ie, actq, Ie, 0, ad, wd, Ie, wdd, 1, 0, None, None, None, yy, H, 4, st))
     mixed = torch.zeros((T, H), dtype=torch.bfloat16, device=dev)
     hbm("unpermute_weighted_bf16", f"{total}x{H}", 2.0 * total * H + 4.0 * T * H,
         lambda: cf.cf_moe_unpermute_weighted_bf16(mixed, yy, rw, counts, offs, idx, T, E, H, st))

@@ -179,6 +179,46 @@ def test_gemm_fused_silu_gate(cf, dev, M, N, K, mode):
         assert rel <= 4e-3, rel      # three bf16 roundings (gate, up, product): ~2^-9 * sqrt(3) relative
 
 
+DUO, DUO_IN_STEP = 4, 12
+
+
+# (300, 256, 384): ragged last row tile, three K-tiles; (1100, 384, 256): two K-tiles (the copy stream a whole tile ahead);
+# (3000, 768, 512): more tiles than workgroups; (128, 128, 1024): a single tile
+@pytest.mark.parametrize("M,N,K", [(300, 256, 384), (1100, 384, 256), (3000, 768, 512), (128, 128, 1024), (520, 512, 640)])
+@pytest.mark.parametrize("epi", [EPI_NONE, EPI_SILU])
+def test_gemm_two_workgroups_per_cu_kernel_matches_the_ring_kernel(cf, dev, M, N, K, epi):
+    """CF_GEMM_FLAG_DUO: the 128 x 128-tile kernel accumulates every output over the same sequence of MFMA steps as the
+    256 x 256-tile kernel and runs the same epilogue arithmetic, so the bits are the same; started in step or half a tile apart."""
+    case(f"gemm duo {M}x{N}x{K} epi={epi}")
+    rng = np.random.default_rng(M + N + K + epi)
+    A, sa = rand_fp8(rng, (M, K))
+    Bg, sg = rand_fp8(rng, (N, K), sigma=0.02)
+    Bu, su = rand_fp8(rng, (N, K), sigma=0.02)
+    sa = (sa * rng.uniform(0.5, 2, M)).astype(np.float32)
+    sg = (sg * rng.uniform(0.5, 2, N)).astype(np.float32)
+    su = (su * rng.uniform(0.5, 2, N)).astype(np.float32)
+    kw = dict(mode=ROW_COL, epi=epi, B2=Bu if epi == EPI_SILU else None, sb2=su if epi == EPI_SILU else None)
+    ring = run_gemm(cf, dev, A, Bg, sa, sg, **kw)
+    assert np.array_equal(run_gemm(cf, dev, A, Bg, sa, sg, flags=DUO, **kw), ring)
+    assert np.array_equal(run_gemm(cf, dev, A, Bg, sa, sg, flags=DUO_IN_STEP, **kw), ring)
+    if epi == EPI_NONE:
+        ref, absdot = orc.gemm_nt_ref(A, Bg, sa, sg, scale_mode=ROW_COL)
+        orc.assert_gemm_close(ring, ref, absdot, what=f"duo {M}x{N}x{K}")
+    # a row stride wider than N: the padding stays untouched
+    wide = run_gemm(cf, dev, A, Bg, sa, sg, flags=DUO, ldc=N + 40, **kw)
+    assert np.array_equal(wide[:, :N], ring) and np.isnan(wide[:, N:]).all()
+
+
+def test_gemm_duo_flag_on_other_shapes_takes_the_usual_kernels(cf, dev):
+    case("gemm duo flag on shapes the kernel does not take")
+    rng = np.random.default_rng(9)
+    A, sa = rand_fp8(rng, (300, 384))
+    B, sb = rand_fp8(rng, (200, 384), sigma=0.02)                # N not a multiple of 128
+    assert np.array_equal(run_gemm(cf, dev, A, B, sa, sb, flags=DUO), run_gemm(cf, dev, A, B, sa, sb))
+    B, sb = rand_fp8(rng, (256, 384), sigma=0.02)                # per-tensor scales
+    assert np.array_equal(run_gemm(cf, dev, A, B, sa, sb, flags=DUO), run_gemm(cf, dev, A, B, sa, sb))
+
+
 def test_gemm_config2_shape_sampled_rows_and_naive_crosscheck(cf, dev):
     """M=8192, K=4096, N=14336 (the benchmark shape): per-token / per-channel scales, outliers at +-40."""
     case("gemm config 2 full size")

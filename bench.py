@@ -410,6 +410,18 @@ def main():
     probe_ms = sorted(pts)[len(pts) // 2]
     probe_b2b_ms = back_to_back(lambda: cf.cf_hbm_stream_probe_2r1w(srcs[0], probe_dst, M, N, st))
     probe_bytes = 3.0 * M * N
+    # the same probe at the X quantize's shape (8192 rows of 4096 output bytes), cold sources in turn
+    pxs = []
+    for i in range(15):
+        a, b = ev(), ev()
+        a.record()
+        cf.cf_hbm_stream_probe_2r1w(srcs[i % 5], probe_dst, M, K, st)
+        b.record()
+        torch.cuda.synchronize()
+        if i >= 5:
+            pxs.append(a.elapsed_time(b))
+    probe_x_ms = sorted(pxs)[len(pxs) // 2]
+    probe_x_bytes = 3.0 * M * K
     del srcs, probe_dst
 
     # outside the timed steps: the two quantize kernels on their own (the brackets inside a step include a launch gap
@@ -489,6 +501,9 @@ def main():
             "back_to_back_us": round(probe_b2b_ms * 1e3, 2),
             "back_to_back_gbps": round(probe_bytes / (probe_b2b_ms * 1e-3) / 1e9, 1),
             "back_to_back_pct_hbm_peak": round(100.0 * probe_bytes / (probe_b2b_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),
+            "x_shape_cold_us": round(probe_x_ms * 1e3, 2),
+            "x_shape_cold_gbps": round(probe_x_bytes / (probe_x_ms * 1e-3) / 1e9, 1),
+            "x_shape_cold_pct_hbm_peak": round(100.0 * probe_x_bytes / (probe_x_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),
         },
         "graph_replay": {"ms_per_step": None if graph_ms is None else round(graph_ms, 4),
                          "tflops": None if graph_ms is None else round(total_flop / (graph_ms * 1e-3) / 1e12, 2),

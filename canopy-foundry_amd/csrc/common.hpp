@@ -171,6 +171,31 @@ __device__ __forceinline__ void atomic_max_nonneg(float* addr, float v) {
     if (__float_as_int(v) > __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(p, __float_as_int(v));
 }
 
+// "Last workgroup in" without an agent-scope fence.  A release fence at agent scope writes the XCD's whole L2 back
+// (the eight L2s are not coherent with each other) and waits for every store the wavefront has in flight: measured at
+// 15 us per workgroup under a streaming kernel.  What the pattern needs is less: that a workgroup's maximum is in place
+// before its arrival counts.  Agent-scope atomics are performed at the memory side, past the L2s; the maximum is issued
+// with its return value taken, and the arrival's operand depends on that value, so the arrival cannot be issued before
+// the maximum has been performed.  A workgroup that would not raise the maximum has nothing to publish: the value it
+// read came from an atomic that has been performed.  The caller that gets `true` arrived last of `expected`; every
+// other arrival, and with it every maximum, has been performed by then, and it reads the result with
+// atomic_load_agent().  Values are non-negative floats, which order like their bit patterns.
+__device__ __forceinline__ bool arrive_with_max(float* running, unsigned* arrived, float v, unsigned expected) {
+    int* p = reinterpret_cast<int*>(running);
+    unsigned one = 1u;
+    if (__float_as_int(v) > __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) {
+        int old = __hip_atomic_fetch_max(p, __float_as_int(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("" : "+v"(old) : : "memory");
+        one += static_cast<unsigned>(old) >> 31;             // old is a non-negative float's bits: adds nothing
+    }
+    const unsigned before = __hip_atomic_fetch_add(arrived, one, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("" : : : "memory");
+    return before == expected - 1u;
+}
+__device__ __forceinline__ float atomic_load_agent(const float* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // ---- deterministic expf ------------------------------------------------------
 // Cody-Waite reduction + degree-6 polynomial with explicit FMAs and exact
 // power-of-two scaling.  Uses only IEEE-exact operations so that a host

@@ -309,11 +309,8 @@ __global__ __launch_bounds__(kAmaxThreads) void k_quant_delayed_step(const uint1
     local = fmaxf(local, __uint_as_float(static_cast<uint32_t>(local_bits) << 16));
     const float m = block_max(local, sh);
     if (threadIdx.x == 0) {
-        atomic_max_nonneg(d.running_amax, m);
-        __threadfence();                                     // the maximum is visible before the arrival is
-        if (atomicAdd(d.arrived, 1u) == gridDim.x - 1) {
-            __threadfence();
-            const float amax = __hip_atomic_load(d.running_amax, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (arrive_with_max(d.running_amax, d.arrived, m, gridDim.x)) {
+            const float amax = atomic_load_agent(d.running_amax);
             *d.scale_snapshot = s;                           // every workgroup read the same pair at its start
             *d.descale_snapshot = pre_descale;
             *d.amax = amax;
@@ -384,11 +381,8 @@ __global__ __launch_bounds__(kThreads) void k_grouped_quant_delayed(const uint16
         const float m = block_max(local, sh);
         if (threadIdx.x == 0) {
             unsigned* arrived = reinterpret_cast<unsigned*>(st) + slotw::ARRIVED;
-            atomic_max_nonneg(st + slotw::RUNNING, m);
-            __threadfence();
-            if (atomicAdd(arrived, 1u) == gridDim.x - 1) {
-                __threadfence();
-                const float amax = __hip_atomic_load(st + slotw::RUNNING, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (arrive_with_max(st + slotw::RUNNING, arrived, m, gridDim.x)) {
+                const float amax = atomic_load_agent(st + slotw::RUNNING);
                 st[slotw::SCALE_SNAP] = s;
                 st[slotw::DESCALE_SNAP] = ds;
                 st[slotw::AMAX] = amax;
@@ -542,6 +536,109 @@ __global__ __launch_bounds__(kLutThreads) void k_gelu_quant_rows_lut(const uint1
         for (int s = 0; s < MAXS; ++s) {
             const int k = (s * 64 + lane) * kVec;
             if (k < K) store_stream16(outr + k, finite ? quant16_finite<false>(v[s], sc) : quant16<false>(v[s], sc));
+        }
+    }
+}
+
+// k_grouped_quant_delayed with GELU for large banks, on the same table: one workgroup per CU stays resident, builds
+// the 65536-entry table once and then takes the (expert, part) items w = blockIdx.x, blockIdx.x + gridDim.x, ...
+// (part p of `per` covers the expert's 16-element vectors p * 1024 + lane, stepping per * 1024).  An item ends as a
+// workgroup of the plain form does: maximum into the slot's running amax, one arrival; the item that arrives last of an
+// expert's `per` updates the slot.  The slot's state changes only in that last step, and only after every item of the
+// expert has arrived, so what a workgroup reads of it at the start of the kernel (row range and scale pair of every
+// expert, into LDS, under the table build) is the state the call started with; the history is read by the last
+// arrival alone.  Same bits as the plain form: the table holds bf16(gelu_fwd(x)) for every x.
+constexpr int kLutMaxExperts = 1024;
+template <bool E5M2, bool RECOMPUTE>
+__global__ __launch_bounds__(kLutThreads) void k_grouped_gelu_quant_delayed_lut(const uint16_t* __restrict__ x, uint8_t* __restrict__ out,
+                                                                               int K, const int* __restrict__ counts,
+                                                                               const int* __restrict__ offsets, int total_rows,
+                                                                               int num_experts, int per, float* __restrict__ states,
+                                                                               int stride, int history_len, float fp8_max,
+                                                                               float* __restrict__ row_descale) {
+    extern __shared__ uint16_t lut[];
+    __shared__ float sh[2][kLutThreads / 64];
+    __shared__ int sh_first[kLutMaxExperts], sh_rows[kLutMaxExperts];
+    __shared__ float sh_scale[kLutMaxExperts], sh_descale[kLutMaxExperts];
+    for (int e = threadIdx.x; e < num_experts; e += kLutThreads) {
+        const int first = offsets[e];
+        sh_first[e] = first;
+        sh_rows[e] = first >= 0 && first < total_rows ? min(counts[e], total_rows - first) : 0;
+        const float* st = states + static_cast<size_t>(e) * stride;
+        sh_scale[e] = st[RECOMPUTE ? slotw::SCALE_SNAP : slotw::SCALE];
+        sh_descale[e] = st[RECOMPUTE ? slotw::DESCALE_SNAP : slotw::DESCALE];
+    }
+    for (int i = threadIdx.x; i < 65536; i += kLutThreads) lut[i] = f32_to_bf16(gelu_fwd(bf16_to_f32(static_cast<uint16_t>(i))));
+    __syncthreads();
+    auto look2 = [&](uint32_t pair) { return static_cast<uint32_t>(lut[pair & 0xffffu]) | (static_cast<uint32_t>(lut[pair >> 16]) << 16); };
+    const int items = num_experts * per;
+    int parity = 0;
+    for (int w = blockIdx.x; w < items; w += gridDim.x) {
+        const int e = w / per, part = w - e * per;
+        const int rows = sh_rows[e];
+        if (rows <= 0) continue;                                     // uniform over the workgroup
+        const int first = sh_first[e];
+        const float s = sh_scale[e], ds = sh_descale[e];
+        const bool s_finite = fabsf(s) < __uint_as_float(0x7f800000u);
+        const size_t tid = static_cast<size_t>(part) * kLutThreads + threadIdx.x;
+        const size_t stride_t = static_cast<size_t>(per) * kLutThreads;
+        for (size_t r = tid; r < static_cast<size_t>(rows); r += stride_t) row_descale[first + r] = ds;
+        const uint16_t* xe = x + static_cast<size_t>(first) * K;
+        uint8_t* oe = out + static_cast<size_t>(first) * K;
+        const size_t nvec = static_cast<size_t>(rows) * K / kVec;       // K % 16 == 0
+        float local = 0.0f;
+        int local_bits = 0;
+        constexpr int kBatch = 4;                                    // loads in flight per lane
+        for (size_t i0 = tid; i0 < nvec; i0 += kBatch * stride_t) {
+            Vec16 v[kBatch];
+#pragma unroll
+            for (int b = 0; b < kBatch; ++b)
+                if (i0 + b * stride_t < nvec) v[b] = load16(xe + (i0 + b * stride_t) * kVec);
+#pragma unroll
+            for (int b = 0; b < kBatch; ++b) {
+                const size_t i = i0 + b * stride_t;
+                if (i < nvec) {
+                    v[b].lo = make_uint4(look2(v[b].lo.x), look2(v[b].lo.y), look2(v[b].lo.z), look2(v[b].lo.w));
+                    v[b].hi = make_uint4(look2(v[b].hi.x), look2(v[b].hi.y), look2(v[b].hi.z), look2(v[b].hi.w));
+                    store_stream16(oe + i * kVec, quant16_track<E5M2, !RECOMPUTE>(v[b], s, s_finite, local_bits, local));
+                }
+            }
+        }
+        if constexpr (!RECOMPUTE) {
+            local = fmaxf(local, __uint_as_float(static_cast<uint32_t>(local_bits) << 16));
+            // the two halves of sh alternate between items: the other wavefronts go on to the next item while the
+            // first lane is busy with the arrival
+            const float m = block_max(local, sh[parity]);
+            parity ^= 1;
+            if (threadIdx.x == 0) {
+                float* st = states + static_cast<size_t>(e) * stride;
+                unsigned* arrived = reinterpret_cast<unsigned*>(st) + slotw::ARRIVED;
+                if (arrive_with_max(st + slotw::RUNNING, arrived, m, static_cast<unsigned>(per))) {
+                    const float amax = atomic_load_agent(st + slotw::RUNNING);
+                    st[slotw::SCALE_SNAP] = s;
+                    st[slotw::DESCALE_SNAP] = ds;
+                    st[slotw::AMAX] = amax;
+                    const float a = fmaxf(amax, 1e-12f);
+                    float hist_max = a;
+                    if (history_len > 0) {
+                        int cursor = reinterpret_cast<const int*>(st)[slotw::CURSOR];
+                        int count = reinterpret_cast<const int*>(st)[slotw::COUNT];
+                        if (cursor < 0 || cursor >= history_len) cursor = 0;
+                        if (count < history_len) ++count;
+                        float pre_max = 0.0f;
+                        for (int i = 0; i < count; ++i)
+                            if (i != cursor) pre_max = fmaxf(pre_max, st[slotw::HISTORY + i]);
+                        st[slotw::HISTORY + cursor] = a;
+                        hist_max = fmaxf(cursor < count ? fmaxf(pre_max, a) : pre_max, 1e-12f);
+                        reinterpret_cast<int*>(st)[slotw::CURSOR] = (cursor + 1) % history_len;
+                        reinterpret_cast<int*>(st)[slotw::COUNT] = count;
+                    }
+                    st[slotw::SCALE] = fp8_max / hist_max;
+                    st[slotw::DESCALE] = hist_max / fp8_max;
+                    st[slotw::RUNNING] = 0.0f;
+                    *arrived = 0u;
+                }
+            }
         }
     }
 }
@@ -946,6 +1043,41 @@ int cf_moe_grouped_quantize_delayed(const uint16_t* d_x, void* d_out, int K, int
                                           fp8_max, d_row_descale);
     };
     const int which = (is_e5m2 ? 4 : 0) | (apply_gelu ? 2 : 0) | (is_recompute ? 1 : 0);
+    // GELU over a large bank: the table form (the direct form waits for erff, about 40 vector instructions per element)
+    if (apply_gelu && num_experts <= kLutMaxExperts && static_cast<size_t>(total_rows) * K >= (64u << 20)) {
+        static std::once_flag once;
+        static hipError_t err = hipSuccess;
+        static int cus = 256;
+        std::call_once(once, [] {
+            const void* ks[4] = {reinterpret_cast<const void*>(&k_grouped_gelu_quant_delayed_lut<false, false>),
+                                 reinterpret_cast<const void*>(&k_grouped_gelu_quant_delayed_lut<false, true>),
+                                 reinterpret_cast<const void*>(&k_grouped_gelu_quant_delayed_lut<true, false>),
+                                 reinterpret_cast<const void*>(&k_grouped_gelu_quant_delayed_lut<true, true>)};
+            for (const void* k : ks) {
+                const hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+                if (e != hipSuccess) err = e;
+            }
+            int dev = 0, n = 0;
+            if (hipGetDevice(&dev) == hipSuccess &&
+                hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+                cus = n;
+        });
+        if (err != hipSuccess) return static_cast<int>(err);
+        // parts per expert: about four items per resident workgroup, so ragged experts even out
+        int parts = (4 * cus + num_experts - 1) / num_experts;
+        parts = parts < 1 ? 1 : (parts > 64 ? 64 : parts);
+        auto launch_lut = [&](auto kernel) {
+            kernel<<<cus, kLutThreads, 128 * 1024, st>>>(d_x, o, K, d_counts, d_offsets, total_rows, num_experts, parts, d_slot_states,
+                                                         state_stride_words, history_len, fp8_max, d_row_descale);
+        };
+        switch (which & 5) {
+            case 0: launch_lut(k_grouped_gelu_quant_delayed_lut<false, false>); break;
+            case 1: launch_lut(k_grouped_gelu_quant_delayed_lut<false, true>); break;
+            case 4: launch_lut(k_grouped_gelu_quant_delayed_lut<true, false>); break;
+            default: launch_lut(k_grouped_gelu_quant_delayed_lut<true, true>); break;
+        }
+        return launch_status();
+    }
     switch (which) {
         case 0: launch(k_grouped_quant_delayed<false, false, false>); break;
         case 1: launch(k_grouped_quant_delayed<false, false, true>); break;

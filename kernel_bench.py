@@ -334,6 +334,18 @@ def main():
     mfma("grouped GELU expert bank, whole pipeline (re-quantizing)", f"T={T} E={E} k={k}", 4.0 * total * Ie * H,
          lambda: cf.cf_moe_grouped_gelu_forward_fp8(hq, one, 0, rw, counts, offs, idx, wg, one, wd, one, mixed, T, H, Ie, E, total,
                                                     ws3, sz3.value, st))
+    # the same loop with the reference's activation scale: one delayed-scaling slot per expert (state blocks of
+    # cf_act_slot_state_words(8) words, scale 1 after the first call's history update)
+    words = cf.raw_cf_act_slot_state_words(8)
+    bank = torch.zeros((E, words), dtype=torch.float32, device=dev)
+    bank[:, 1] = 64.0; bank[:, 2] = 1.0 / 64.0; bank[:, 3] = 64.0; bank[:, 4] = 1.0 / 64.0
+    bank_i = bank.view(torch.int32); bank_i[:, 8:12] = 0
+    rowd = f32(total)
+    hbm("grouped per-expert delayed-scale quantize with GELU (1 launch, 64 slots)", f"{total}x{Ie}", 3.0 * total * Ie,
+        lambda: cf.cf_moe_grouped_quantize_delayed(act, gq, Ie, E, counts, offs, total, bank, words, 8, 0, 1, 0, rowd, st))
+    mfma("grouped GELU expert bank with per-expert activation slots", f"T={T} E={E} k={k}", 4.0 * total * Ie * H,
+         lambda: cf.cf_moe_grouped_gelu_forward_fp8_slots(hq, one, 0, rw, counts, offs, idx, wg, one, wd, one, mixed, T, H, Ie, E, total,
+                                                          bank, words, 8, 0, 0, ws3, sz3.value, st))
     sz4 = ctypes.c_size_t(0)
     cf.raw_cf_moe_grouped_expert_forward_fp8_workspace(T, total, E, H, Ie, None, ctypes.byref(sz4))
     ws4 = u8(sz4.value)
@@ -349,7 +361,7 @@ def main():
     sz5 = ctypes.c_size_t(0)
     cf.raw_cf_moe_grouped_expert_forward_bf16_workspace(T, total, E, H, Ie, None, ctypes.byref(sz5))
     ws5 = u8(sz5.value)
-    mfma16("moe_grouped_expert_forward_bf16 with a workspace (grouped bf16 GEMMs, two-term GELU)", f"T={T} E={E} k={k}",
+    mfma16("moe_grouped_expert_forward_bf16 with a workspace (grouped bf16 GEMMs, GELU rounded to bf16)", f"T={T} E={E} k={k}",
            4.0 * total * Ie * H,
            lambda: cf.cf_moe_grouped_expert_forward_bf16_ws(hb16, rw, counts, None, idx, wi16, wo16, mixed, T, H, Ie, E, total,
                                                             ws5, sz5.value, st))

@@ -155,6 +155,68 @@ def test_counts_beyond_the_bound(cf, dev):
         bank.close()
 
 
+@pytest.mark.parametrize("e5m2", [False, True])
+def test_large_banks_take_the_table_form_with_the_same_bits(cf, dev, e5m2):
+    """From 64 Mi elements (rows of the bound x K) the GELU form looks bf16(gelu(x)) up in a table held in LDS by
+    workgroups that stay resident; total_rows being an upper bound, the same routing runs through both forms."""
+    case(f"grouped delayed GELU quantize, table form against the direct form, e5m2={e5m2}")
+    E, K, hist = 8, 1408, 8
+    counts = np.array([9000, 0, 7001, 300, 11000, 1, 8000, 4698], np.int32)
+    offsets = np.concatenate([[0], np.cumsum(counts)[:-1]]).astype(np.int32)
+    total = int(counts.sum())                                              # 40000 rows: 56 Mi elements, the direct form
+    bound = 50000                                                          # 70 Mi elements: the table form
+    assert total * K < (64 << 20) <= bound * K
+    gen = torch.Generator(device=dev).manual_seed(11)
+    x = (torch.randn(bound, K, device=dev, generator=gen) * 1.7).to(torch.bfloat16)
+    fp8_max = 57344.0 if e5m2 else 448.0
+    stride = cf.raw_cf_act_slot_state_words(hist) + 3
+    init = np.zeros((E, stride), np.float32)
+    init[:, W["scale"]] = fp8_max / 6.0
+    init[:, W["descale"]] = 6.0 / fp8_max
+    init[:, W["history"]] = 6.0
+    init.view(np.int32)[:, W["cursor"]] = 1
+    init.view(np.int32)[:, W["count"]] = 1
+    d_counts, d_offsets = dev_arr(counts, dev), dev_arr(offsets, dev)
+    results = []
+    for rows_bound in (total, bound):
+        state = torch.from_numpy(init.reshape(-1).copy()).to(dev)
+        per_call = []
+        for call in range(2):
+            out = torch.full((bound, K), 0xEE, dtype=torch.uint8, device=dev)
+            rd = torch.full((bound,), -1.0, dtype=torch.float32, device=dev)
+            cf.cf_moe_grouped_quantize_delayed(x, out, K, E, d_counts, d_offsets, rows_bound, state, stride, hist, int(e5m2), 1, 0, rd, stream())
+            out_r = torch.full((bound, K), 0xEE, dtype=torch.uint8, device=dev)
+            rd_r = torch.full((bound,), -1.0, dtype=torch.float32, device=dev)
+            cf.cf_moe_grouped_quantize_delayed(x, out_r, K, E, d_counts, d_offsets, rows_bound, state, stride, hist, int(e5m2), 1, 1, rd_r, stream())
+            torch.cuda.synchronize()
+            assert torch.equal(out_r, out) and torch.equal(rd_r, rd), "the recompute pass gives the forward call's bytes"
+            assert bool((out[total:] == 0xEE).all()) and bool((rd[total:] == -1.0).all())
+            per_call.append((out, rd, state.clone()))
+        results.append(per_call)
+    for call in range(2):
+        (o_a, rd_a, st_a), (o_b, rd_b, st_b) = results[0][call], results[1][call]
+        assert torch.equal(o_a, o_b), f"call {call}: bytes differ between the two forms"
+        assert torch.equal(rd_a, rd_b)
+        assert torch.equal(st_a.view(torch.int32), st_b.view(torch.int32)), f"call {call}: slot states differ"
+    # and one expert against the oracle (the GPU's own GELU values as its input)
+    e = 3
+    o, n = int(offsets[e]), int(counts[e])
+    g = torch.empty((n, K), dtype=torch.bfloat16, device=dev)
+    cf.cf_gelu_forward_bf16(x[o:o + n].contiguous(), g, n * K, stream())
+    torch.cuda.synchronize()
+    quant = orc.quantize_e5m2 if e5m2 else orc.quantize_e4m3
+    g_bits = bf16_bits(g).reshape(-1)
+    assert np.array_equal(host(results[1][0][0][o:o + n]).reshape(-1), quant(g_bits, np.float32(fp8_max / 6.0)))
+    st = results[1][0][2].cpu().numpy().reshape(E, stride)
+    amax = orc.amax_bf16(g_bits)
+    assert st[e, W["amax"]] == amax and st[e, W["history"] + 1] == max(amax, np.float32(1e-12))
+    assert st[e, W["scale"]] == np.float32(fp8_max) / max(amax, np.float32(6.0))
+    assert np.array_equal(st[1], init[1]), "an expert without rows keeps its slot"
+    second = results[1][1][0]
+    want_scale = st[e, W["scale"]]
+    assert np.array_equal(host(second[o:o + n]).reshape(-1), quant(g_bits, np.float32(want_scale)))
+
+
 class LoopBank:
     """Inputs of the FP8 GELU expert loop with per-tensor descales (the reference's slots are per tensor)."""
 

@@ -448,7 +448,7 @@ __global__ __launch_bounds__(kThreads) void k_unpermute_indexed(uint16_t* __rest
             // the table is filled for the pairs of the row lists only: a cell that does not name a row of y (a pair the
             // lists do not hold, or one cut off by the caller's row bound) is skipped
             int slot = sel ? slot_index[static_cast<size_t>(row) * E + e] : -1;
-            if (slot >= slot_limit) slot = -1;
+            if (static_cast<unsigned>(slot) >= static_cast<unsigned>(slot_limit)) slot = -1;     // also a negative cell
             const unsigned long long m = __ballot(sel);
             if (sel) {
                 const int pos = __builtin_popcountll(m & ((1ull << t) - 1ull));

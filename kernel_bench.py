@@ -220,6 +220,14 @@ def main():
          lambda: cf.cf_fp8_gemm_nt_bf16_ex(M, N, K, xq, K, 0, xd, wg, K, wgd, 1, 2, None, wu, wud, c, N, 0, st))
     mfma("gemm down projection (config 2)", f"{M}x{K}x{N}", 2.0 * M * N * K,
          lambda: cf.cf_fp8_gemm_nt_bf16_ex(M, K, N, hq, N, 0, xd, wd, N, wdd, 1, 0, None, None, None, y, K, 0, st))
+    # The same launch on operands without entropy (every byte 0x38 = 1.0): the matrix cores' power follows how much
+    # their inputs toggle, and on such data the part stays below its power cap at full clock.  What separates this
+    # row from the one on quantized data is the power cap, not the kernel (use --sustain to see power and clock).
+    if args.only in "gemm gate+up fused SiLU-gate (config 2), constant operands":
+        x1 = torch.full_like(xq, 0x38); g1 = torch.full_like(wg, 0x38); u1 = torch.full_like(wu, 0x38)
+        mfma("gemm gate+up fused SiLU-gate (config 2), constant operands", f"{M}x2x{N}x{K}", 4.0 * M * N * K,
+             lambda: cf.cf_fp8_gemm_nt_bf16_ex(M, N, K, x1, K, 0, xd, g1, K, wgd, 1, 2, None, u1, wud, c, N, 0, st))
+        del x1, g1, u1
     # the same two launches on the 128 x 128-tile kernel that runs two workgroups per CU (CF_GEMM_FLAG_DUO = 4;
     # 12 = without starting the second workgroup of a CU half a tile late)
     mfma("duo: gemm gate+up fused SiLU-gate (config 2), 2 workgroups per CU", f"{M}x2x{N}x{K}", 4.0 * M * N * K,

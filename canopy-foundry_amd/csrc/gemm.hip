@@ -56,6 +56,7 @@ struct GemmArgs {
     int tiles_m, tiles_n;
     int force_staged;            // take the register-staged kernel even when the ring kernel applies
     int duo;                     // 1: the two-workgroups-per-CU kernel where it applies, 2: the same without the stagger
+    int mfma32;                  // keep k_gemm_nt_ring (the 32 x 32 x 64 MFMA shape) where k_gemm_nt_ring16 would apply
     // grouped (per-expert) form, ring kernel only; all null / 0 for a dense GEMM
     const int* tile_map;         // [0] = number of row tiles, then (expert, first row, end row) per row tile
     const int* a_row_index;      // compact row r reads A row (and its descale) a_row_index[r]; null = r
@@ -1135,6 +1136,445 @@ void k_gemm_nt_ring(const GemmArgs p) {
     __builtin_amdgcn_s_waitcnt(kWaitVm0);
 }
 
+// ---- ring kernel on the 16 x 16 x 128 MFMA -----------------------------------------------------------------
+// The same persistent structure, ring, copy stream, tile walk and drain staging as k_gemm_nt_ring, with the
+// products taken by v_mfma_f32_16x16x128_f8f6f4 instead of v_mfma_f32_32x32x64_f8f6f4.  Both shapes do 2048 FLOP
+// per cycle and SIMD; measured on this part, MFMAs alone on random E4M3 operands, the 16 x 16 x 128 shape delivers
+// 8 - 9 % more at the same socket power (and draws 10 % less on constant operands), and these GEMMs run at the power
+// cap.  A wavefront's 128 x 128 tile is 8 x 8 blocks of 16 x 16 (four accumulator registers each, 256 in all); an
+// MFMA consumes a whole 128-byte K-tile row of both operands, so every accumulator is touched once per K-tile.
+// Operand registers: four sets of four blocks (weights: N-halves A0, A1; activations: M-halves B0, B1; 32 registers
+// each).  A K-tile is four phases of sixteen MFMAs; with parity p of the K-tile they use
+//   (A0, B[p]) -> (A0, B[1-p]) -> (A1, B[1-p]) -> (A1, B[p])
+// and the set that a phase has left behind is refilled two phases before it is needed again: B[1-p] and A1 of this
+// K-tile under phases 0 and 1, A0 and B[1-p] of the NEXT K-tile under phases 2 and 3 (after the barrier that makes
+// that K-tile visible).  The next K-tile then starts with (A0, B[1-p]): its parity is the other one, and so on.
+// Forms: plain, bias and SiLU-gate epilogues (the LDS-staged bf16 drain), every scale mode of those, dense or
+// grouped; no accumulate / fp32-store forms and no term-split form (those stay on k_gemm_nt_ring).
+typedef float v4f __attribute__((ext_vector_type(4)));
+// 16-byte chunk swizzle of this kernel's operand tiles: within any 16 rows the 16-lane groups of a ds_read_b128 (rows
+// 0-7 of one k-group with rows 8-15 of the next) land in 16 different 16-byte slots of a 256-byte line, and the
+// pattern repeats every 16 rows
+__device__ __forceinline__ int swz16(int row) { return (row ^ ((row >> 3) & 1)) & 7; }
+
+template <int EPI>
+struct TileScales16 {
+    float sa[8];           // descales of this lane's eight output rows (row j * 16 + lane % 16 of the wavefront's 128)
+    float4 cs[2][2];       // channel descales of the pair being drained: [unit in pair][16-column block], this lane's 4 columns
+    float4 cs2[2][2];      // up-projection descales (SiLU-gate)
+};
+
+template <int EPI, int SCALE>
+__device__ __forceinline__ void load_row_scales16(TileScales16<EPI>& s, const GemmArgs& p, const TilePos& t, int wm, int lane) {
+    if constexpr (SCALE == SCALE_ROWCOL || SCALE == SCALE_ROW) {
+        int r[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) r[j] = min(t.m0 + wm * 128 + j * 16 + (lane & 15), t.m_end - 1);
+        if (p.a_row_index) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) r[j] = p.a_row_index[r[j]];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) s.sa[j] = p.sa[r[j]];
+            asm volatile("; row scales through the row index" ::: "memory");
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) s.sa[j] = p.sa[r[j]];
+        }
+    }
+}
+template <int EPI, int SCALE>
+__device__ __forceinline__ void load_pair_scales16(float4 (&cs)[2][2], float4 (&cs2)[2][2], const GemmArgs& p,
+                                                   const TilePos& t, int wn, int lane, int pair) {
+    constexpr int NU = EPI == EPI_SILU_GATE ? 2 : 4;
+    const size_t col0 = t.n0 + wn * (NU * 32) + pair * 64;
+    if constexpr (SCALE == SCALE_ROWCOL) {
+        const size_t ucol = static_cast<size_t>(t.expert) * p.sb_expert_stride + col0;
+        const uint8_t* b1 = reinterpret_cast<const uint8_t*>(p.sb + ucol);
+        const uint8_t* b2 = reinterpret_cast<const uint8_t*>(EPI == EPI_SILU_GATE ? p.sb2 + ucol : p.sb);
+        const uint32_t loff = static_cast<uint32_t>(lane >> 4) * 16u;      // this lane's four columns of a 16-column block
+        if constexpr (EPI != EPI_SILU_GATE) {
+            if (t.n0 + BN > p.N) {      // a last column tile that N cuts short: unused factors are read from the last four columns
+                const int lim = (p.N - 4 - static_cast<int>(col0)) * 4;
+#pragma unroll
+                for (int u = 0; u < 2; ++u)
+#pragma unroll
+                    for (int sb = 0; sb < 2; ++sb)
+                        cs[u][sb] = *reinterpret_cast<const float4*>(b1 + min(static_cast<int>(loff + u * 128u + sb * 64u), lim));
+                return;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int sb = 0; sb < 2; ++sb) {
+                cs[u][sb] = *reinterpret_cast<const float4*>(b1 + (loff + u * 128u + sb * 64u));
+                if constexpr (EPI == EPI_SILU_GATE) cs2[u][sb] = *reinterpret_cast<const float4*>(b2 + (loff + u * 128u + sb * 64u));
+            }
+    }
+}
+
+// The drain of k_gemm_nt_ring for the 16 x 16 accumulator blocks: lane l of block (i, j) holds output row
+// j * 16 + l % 16 and the four consecutive columns i * 16 + 4 (l / 16) ... + 3 of the wavefront's 128 accumulated
+// columns.  Staging layout, read-back and stores are those of drain_tile.
+template <int EPI, int SCALE, bool RAGGED, class Landed>
+__device__ __forceinline__ void drain_tile16(v4f (&acc)[8][8], TileScales16<EPI>& s, float s1, float s2, const GemmArgs& p,
+                                             const TilePos& t, int wm, int wn, int lane, uint8_t* stage, Landed&& landed) {
+    constexpr bool GATE = EPI == EPI_SILU_GATE;
+    constexpr int NU = GATE ? 2 : 4;
+    const int row16 = lane & 15, cq = lane >> 4;
+    const int rr = lane >> 3, rc = lane & 7;
+    const uint8_t* rdp0 = stage + rr * 128 + ((rc ^ (rr >> 1)) << 4);
+    const uint8_t* rdp1 = stage + rr * 128 + ((rc ^ (rr >> 1) ^ 4) << 4);
+    const int mrow0 = t.m0 + wm * 128 + rr;
+    uint8_t* cu = reinterpret_cast<uint8_t*>(p.C + static_cast<size_t>(t.m0 + wm * 128) * p.ldc + t.n0 + wn * (NU * 32));
+    const uint32_t coff = (static_cast<uint32_t>(rr) * static_cast<uint32_t>(p.ldc) + rc * 8u) * 2u;
+    const size_t cstep = static_cast<size_t>(p.ldc) * 16;
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    uint4 bias8[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
+    if constexpr (EPI == EPI_BIAS) {
+        const int bcol = t.n0 + wn * (NU * 32) + rc * 8;
+#pragma unroll
+        for (int pair = 0; pair < NU / 2; ++pair)
+            bias8[pair] = *reinterpret_cast<const uint4*>(p.bias + (RAGGED ? min(bcol + pair * 64, p.N - 8) : bcol + pair * 64));
+    }
+    const int ncol0 = t.n0 + wn * (NU * 32) + rc * 8;
+
+#pragma unroll
+    for (int pair = 0; pair < NU / 2; ++pair) {
+        const uint4 bv = bias8[pair];
+        const float bf[8] = {bf16_lo(bv.x), bf16_hi(bv.x), bf16_lo(bv.y), bf16_hi(bv.y),
+                             bf16_lo(bv.z), bf16_hi(bv.z), bf16_lo(bv.w), bf16_hi(bv.w)};
+        float4 ncs[2][2], ncs2[2][2];
+        if (pair + 1 < NU / 2) load_pair_scales16<EPI, SCALE>(ncs, ncs2, p, t, wn, lane, pair + 1);
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj) {
+                const int j = half * 4 + jj;
+                const float sa = (SCALE == SCALE_ROWCOL || SCALE == SCALE_ROW) ? s.sa[j] : 1.0f;
+                const int R = jj * 16 + row16;                       // row of the 64-row staging block
+                uint8_t* wr = stage + R * 128 + (cq & 1) * 8;
+                const int wswz = (R >> 1) & 7;
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+#pragma unroll
+                    for (int sb = 0; sb < 2; ++sb) {
+                        float4 c = make_float4(s1, s1, s1, s1), up = make_float4(s2, s2, s2, s2);
+                        if constexpr (SCALE == SCALE_ROWCOL) {
+                            c = s.cs[u][sb];
+                            if constexpr (GATE) up = s.cs2[u][sb];
+                        }
+                        const float c4[4] = {c.x, c.y, c.z, c.w}, u4[4] = {up.x, up.y, up.z, up.w};
+                        float v[4];
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            if constexpr (GATE) {
+                                // weight rows of the wavefront: [gate 32 | up 32 | gate 32 | up 32]: unit u = blocks 4u .. 4u + 3
+                                const uint32_t gu = pack_bf16x2_hw(acc_read(acc[u * 4 + sb][j][q]) * (sa * c4[q]),
+                                                                   acc_read(acc[u * 4 + 2 + sb][j][q]) * (sa * u4[q]));
+                                v[q] = fast_silu(bf16_lo(gu)) * bf16_hi(gu);
+                            } else {
+                                v[q] = acc_read(acc[pair * 4 + u * 2 + sb][j][q]) * (sa * c4[q]);
+                            }
+                        }
+                        *reinterpret_cast<uint2*>(wr + (((u * 4 + sb * 2 + (cq >> 1)) ^ wswz) << 4)) =
+                            make_uint2(pack_bf16x2_hw(v[0], v[1]), pack_bf16x2_hw(v[2], v[3]));
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            if (pair == 0 && half == 0) {
+                __builtin_amdgcn_s_waitcnt(kWaitVm0);
+                landed();
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                uint4 v = *reinterpret_cast<const uint4*>(((i & 1) ? rdp1 : rdp0) + i * 8 * 128);
+                if constexpr (EPI == EPI_BIAS) {
+                    v.x = pack_bf16x2_hw(bf16_lo(v.x) + bf[0], bf16_hi(v.x) + bf[1]);
+                    v.y = pack_bf16x2_hw(bf16_lo(v.y) + bf[2], bf16_hi(v.y) + bf[3]);
+                    v.z = pack_bf16x2_hw(bf16_lo(v.z) + bf[4], bf16_hi(v.z) + bf[5]);
+                    v.w = pack_bf16x2_hw(bf16_lo(v.w) + bf[6], bf16_hi(v.w) + bf[7]);
+                }
+                if (!RAGGED || (mrow0 + half * 64 + i * 8 < t.m_end && ncol0 + pair * 64 < p.N)) {
+                    const u32x4 vv = {v.x, v.y, v.z, v.w};
+                    __builtin_nontemporal_store(vv, reinterpret_cast<u32x4*>(cu + ((half * 8 + i) * cstep + pair * 128) + coff));
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (pair + 1 < NU / 2) {
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int sb = 0; sb < 2; ++sb) { s.cs[u][sb] = ncs[u][sb]; s.cs2[u][sb] = ncs2[u][sb]; }
+        }
+    }
+}
+
+// KODD: the number of K-tiles per tile is odd.  A K-tile's parity is its position in the tile modulo 2 (after a drain
+// the operands are read afresh, so every tile starts at parity 0), and the sequence of K-tile bodies is straight-line
+// code for either case.
+template <int FMT, int EPI, int SCALE, bool KODD>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void k_gemm_nt_ring16(const GemmArgs p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    static_assert(EPI == EPI_NONE || EPI == EPI_BIAS || EPI == EPI_SILU_GATE, "bf16 drain forms only");
+    constexpr bool GATE = EPI == EPI_SILU_GATE;
+    constexpr int OUT_BN = GATE ? BN / 2 : BN;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int total_tiles = (p.tile_map ? p.tile_map[0] : p.tiles_m) * p.tiles_n;
+    int my_tiles, lin0, lstep;
+    if (gridDim.x % kXcds == 0) {
+        const int per = (total_tiles + kXcds - 1) / kXcds;
+        const int x = blockIdx.x % kXcds, i = blockIdx.x / kXcds;
+        lstep = gridDim.x / kXcds;
+        const int cnt = max(0, min(per, total_tiles - x * per));
+        my_tiles = (cnt - i + lstep - 1) / lstep;
+        lin0 = x * per + i;
+    } else {
+        lstep = gridDim.x;
+        my_tiles = (total_tiles - static_cast<int>(blockIdx.x) + lstep - 1) / lstep;
+        lin0 = blockIdx.x;
+    }
+    if (my_tiles <= 0) return;
+    const int ktiles = p.K / BK;      // >= 2, checked by the launcher
+
+    float s1 = 0.0f, s2 = 0.0f;
+    if constexpr (SCALE == SCALE_TENSOR) {
+        s1 = p.sa[0] * p.sb[0];
+        if constexpr (GATE) s2 = p.sa[0] * p.sb2[0];
+    }
+    if constexpr (SCALE == SCALE_ROW) s1 = p.sb[0];
+
+    // ---- global -> LDS: as in k_gemm_nt_ring ----
+    const int lrow = lane >> 3, lslot = lane & 7;
+    uint32_t xoff[8], woff[8];
+    const uint8_t* wb = p.B;
+    const uint8_t* wb2 = p.B2;
+    auto fetch_pos = [&](int seq, TilePos& t) { t = locate_tile<OUT_BN>(p, lin0 + seq * lstep); };
+    auto fetch_rows = [&](const TilePos& t, int (&rows)[8]) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int arow = min(t.m0 + wave * 64 + j * 8 + lrow, t.m_end - 1);
+            rows[j] = p.a_row_index ? p.a_row_index[arow] : arow;
+        }
+    };
+    auto fetch_tile = [&](int seq, TilePos& t, int (&rows)[8]) {
+        fetch_pos(seq, t);
+        fetch_rows(t, rows);
+    };
+    auto aim = [&](const TilePos& t, const int (&rows)[8]) {
+        wb = p.B + t.expert * p.b_expert_stride;
+        if constexpr (GATE) wb2 = p.B2 + t.expert * p.b_expert_stride;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int row = wave * 64 + j * 8 + lrow;
+            const uint32_t gchunk = (lslot ^ swz16(row)) * 16;
+            xoff[j] = static_cast<uint32_t>(rows[j]) * static_cast<uint32_t>(p.lda) + gchunk;
+            int n = t.n0 + row;
+            if constexpr (GATE) n = t.n0 + (row >> 7) * 64 + ((row >> 6) & 1) * 32 + (row & 31);
+            woff[j] = static_cast<uint32_t>(min(n, p.N - 1)) * static_cast<uint32_t>(p.ldb) + gchunk;
+        }
+    };
+    uint32_t lds_wave = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(smem)) + wave * (64 * BK);
+    auto dma = [&](int slot, uint32_t voff, const uint8_t* base, auto jc) {
+        constexpr int J = decltype(jc)::value;
+        // (the slot offsets rotate through five variables; the compiler may park one in a vector register)
+        const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_wave + slot);
+        asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3"
+                     :: "s"(dst), "n"(J * 8 * BK), "v"(voff), "s"(base) : "memory", "scc");
+    };
+    auto dma_x = [&](int slot, int k0, auto jc) { dma(slot, xoff[decltype(jc)::value], p.A + k0, jc); };
+    auto dma_w = [&](int slot, int k0, auto jc) {
+        constexpr int J = decltype(jc)::value;
+        dma(slot, woff[J], ((GATE && J >= 4) ? wb2 : wb) + k0, jc);
+    };
+
+    // ---- LDS -> MFMA operands: block b of an operand half is rows b * 16 ... + 15; lane l reads row l % 16, the
+    // 32 bytes of k-group l / 16 (two swizzled 16-byte chunks).  The swizzle is the same for every block, so a set's
+    // eight reads are two addresses plus immediates. ----
+    const int r16 = lane & 15, kg = lane >> 4;
+    int rd[2];
+#pragma unroll
+    for (int c = 0; c < 2; ++c) rd[c] = r16 * BK + (((kg * 2 + c) ^ swz16(r16)) << 4);
+    const uint8_t* xrd = smem + wm * 128 * BK;
+    const uint8_t* wrd = smem + wn * 128 * BK;
+
+    v4f acc[8][8];
+    v8i WA[2][4], XB[2][4];       // operand sets: weights N-halves, activations M-halves
+    auto put = [](v8i& dst, int half, const uint4 v) {
+        dst[4 * half + 0] = (int)v.x; dst[4 * half + 1] = (int)v.y; dst[4 * half + 2] = (int)v.z; dst[4 * half + 3] = (int)v.w;
+    };
+    // read R (0..7) of a set: block R / 2, chunk R % 2.  SET: 0, 1 = weights A0, A1 from slot `slot`; 2, 3 = activations B0, B1
+    auto read_set = [&](int slot, auto setc, auto rc_) {
+        constexpr int SET = decltype(setc)::value, R = decltype(rc_)::value;
+        constexpr int blk = R >> 1, c = R & 1;
+        constexpr int gb = (SET & 1) * 4 + blk;              // block within the wavefront's 128 rows
+        const int off = slot + gb * 16 * BK + rd[c];
+        if constexpr (SET < 2) put(WA[SET][blk], c, *reinterpret_cast<const uint4*>(wrd + off));
+        else                   put(XB[SET - 2][blk], c, *reinterpret_cast<const uint4*>(xrd + off));
+    };
+    auto mfma_blk = [&](auto sac, auto sbc, auto ic, auto first_c) {
+        constexpr int SA = decltype(sac)::value, SB = decltype(sbc)::value, I = decltype(ic)::value;
+        constexpr int ii = I >> 2, jj = I & 3;
+        v4f c = acc[SA * 4 + ii][SB * 4 + jj];
+        if constexpr (decltype(first_c)::value != 0) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) c[r] = 0.0f;
+        }
+        acc[SA * 4 + ii][SB * 4 + jj] =
+            __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(WA[SA][ii], XB[SB][jj], c, (FMT >> 1) & 1, FMT & 1, 0, 0, 0, 0);
+    };
+    using C0 = std::integral_constant<int, 0>;
+    using C1 = std::integral_constant<int, 1>;
+
+    int a0 = 0, a1 = kSlotBytes, a2 = 2 * kSlotBytes, a3 = 3 * kSlotBytes, a4 = 4 * kSlotBytes;
+    TileScales16<EPI> sc;
+    TilePos t0, t1, t2;
+    int nrows[8];
+    int fetch_seq = 0;
+
+    // One K-tile g of parity P.  Phases 0 and 1 (32 MFMAs): the X copies of K-tile g+2 into a4, the reads of B[1-P]
+    // and A1 of this K-tile; wait + barrier; phases 2 and 3: the W copies of K-tile g+2 into a0, the reads of A0 and
+    // B[1-P] of K-tile g+1 (not in a tile's last K-tile: the next tile's operands are read after the drain).
+    auto ktile = [&](auto first_c, auto end_c, auto par_c, int dk0, const TilePos& t, bool wait) {
+        constexpr bool END = decltype(end_c)::value != 0;
+        constexpr int P = decltype(par_c)::value;
+        using SBP = std::integral_constant<int, P>;             // activations set of phases 0 and 3
+        using SBQ = std::integral_constant<int, 1 - P>;         // ... of phases 1 and 2
+        using RBQ = std::integral_constant<int, 2 + (1 - P)>;   // read_set index of B[1-P]
+        static_for<0, 16>([&](auto ic) {                        // phase 0: (A0, B[P]); reads B[1-P](g)
+            constexpr int i = decltype(ic)::value;
+            mfma_blk(C0{}, SBP{}, ic, first_c);
+            if constexpr ((i & 1) == 0) read_set(a0, RBQ{}, std::integral_constant<int, i / 2>{});
+            if constexpr (i >= 4 && (i & 1) == 1) dma_x(a4, dk0, std::integral_constant<int, (i >= 4) ? (i - 5) / 2 : 0>{});
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        static_for<0, 16>([&](auto ic) {                        // phase 1: (A0, B[1-P]); reads A1(g)
+            constexpr int i = decltype(ic)::value;
+            mfma_blk(C0{}, SBQ{}, ic, first_c);
+            if constexpr ((i & 1) == 0) read_set(a1, C1{}, std::integral_constant<int, i / 2>{});
+            if constexpr (i < 4 && (i & 1) == 1) dma_x(a4, dk0, std::integral_constant<int, 6 + i / 2>{});
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        // phase 2: (A1, B[1-P])
+        mfma_blk(C1{}, SBQ{}, C0{}, first_c);
+        mfma_blk(C1{}, SBQ{}, C1{}, first_c);
+        __builtin_amdgcn_sched_barrier(0);
+        if (wait) __builtin_amdgcn_s_waitcnt(kWaitVm8);
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<2, 16>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            mfma_blk(C1{}, SBQ{}, ic, first_c);
+            if constexpr (!END && (i & 1) == 0) read_set(a3, C0{}, std::integral_constant<int, (i - 2) / 2>{});      // A0(g+1): reads 0..6
+            if constexpr ((i & 1) == 1) dma_w(a0, dk0, std::integral_constant<int, (i - 3) / 2>{});                  // W copies 0..6
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        static_for<0, 16>([&](auto ic) {                        // phase 3: (A1, B[P]); reads B[1-P](g+1)
+            constexpr int i = decltype(ic)::value;
+            mfma_blk(C1{}, SBP{}, ic, first_c);
+            if constexpr (!END && i == 0) read_set(a3, C0{}, std::integral_constant<int, 7>{});
+            if constexpr (i == 1) dma_w(a0, dk0, std::integral_constant<int, 7>{});
+            if constexpr (!END && i >= 2 && (i & 1) == 0) read_set(a2, RBQ{}, std::integral_constant<int, (i >= 2) ? (i - 2) / 2 : 0>{});   // reads 0..6
+            if constexpr (!END && i == 15) read_set(a2, RBQ{}, std::integral_constant<int, 7>{});
+            if constexpr (END && i == 5) {
+                if (fetch_seq < my_tiles) fetch_pos(fetch_seq, t2);
+            }
+            if constexpr (END && i == 3) {
+                load_row_scales16<EPI, SCALE>(sc, p, t, wm, lane);
+                load_pair_scales16<EPI, SCALE>(sc.cs, sc.cs2, p, t, wn, lane, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+    auto rotate = [&]() {
+        const int b0 = a0, b1 = a1;
+        a0 = a2; a1 = a3; a2 = a4; a3 = b0; a4 = b1;
+    };
+
+    int dkt = 2 % ktiles, dseq = 2 / ktiles;
+    const bool ahead = ktiles > 2;
+    {
+        int rows0[8] = {};
+        fetch_tile(0, t0, rows0);
+        aim(t0, rows0);
+        t1 = t0; t2 = t0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) nrows[j] = rows0[j];
+        if (ahead && my_tiles > 1) fetch_tile(1, t1, nrows);
+        __builtin_amdgcn_s_waitcnt(kWaitVm0);
+        static_for<0, 8>([&](auto jc) { dma_x(a0, 0, jc); });
+        static_for<0, 8>([&](auto jc) { dma_w(a1, 0, jc); });
+        static_for<0, 8>([&](auto jc) { dma_x(a2, BK, jc); });
+        static_for<0, 8>([&](auto jc) { dma_w(a3, BK, jc); });
+        if (!ahead && my_tiles > 1) {
+            fetch_tile(1, t1, rows0);
+            aim(t1, rows0);
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(kWaitVm16);
+    __syncthreads();
+    // a tile's first K-tile has parity 0: it starts with (A0, B0)
+    static_for<0, 8>([&](auto rc_) { read_set(a1, C0{}, rc_); });
+    static_for<0, 8>([&](auto rc_) { read_set(a0, std::integral_constant<int, 2>{}, rc_); });
+
+    auto advance_copy = [&]() {
+        if (++dkt == ktiles) {
+            dkt = 0;
+            if (++dseq < my_tiles) {
+                if (ahead) {
+                    aim(t1, nrows);
+                } else {
+                    TilePos tt;
+                    int rr[8] = {};
+                    fetch_tile(dseq, tt, rr);
+                    aim(tt, rr);
+                }
+            }
+        }
+    };
+
+    for (int seq = 0; seq < my_tiles; ++seq) {
+        if (!ahead) fetch_pos(seq, t0);
+        const TilePos t = t0;
+        ktile(C1{}, C0{}, C0{}, dkt * BK, t, !(seq > 0));
+        rotate(); advance_copy();
+        for (int kt = 1; kt + 2 < ktiles; kt += 2) {
+            ktile(C0{}, C0{}, C1{}, dkt * BK, t, true);
+            rotate(); advance_copy();
+            ktile(C0{}, C0{}, C0{}, dkt * BK, t, true);
+            rotate(); advance_copy();
+        }
+        fetch_seq = ahead ? seq + 2 : my_tiles;
+        if constexpr (KODD) {
+            ktile(C0{}, C0{}, C1{}, dkt * BK, t, true);
+            rotate(); advance_copy();
+            ktile(C0{}, C1{}, C0{}, dkt * BK, t, true);
+        } else {
+            ktile(C0{}, C1{}, C1{}, dkt * BK, t, true);
+        }
+        rotate(); advance_copy();
+        const bool more = ahead && seq + 2 < my_tiles;
+        auto landed = [&]() { if (more) fetch_rows(t2, nrows); };
+        uint8_t* stage = smem + a4 + wave * (64 * BK);
+        constexpr int out_bn = EPI == EPI_SILU_GATE ? BN / 2 : BN;
+        if (t.m0 + BM <= t.m_end && t.n0 + out_bn <= p.N) drain_tile16<EPI, SCALE, false>(acc, sc, s1, s2, p, t, wm, wn, lane, stage, landed);
+        else                                              drain_tile16<EPI, SCALE, true>(acc, sc, s1, s2, p, t, wm, wn, lane, stage, landed);
+        if (more) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) asm volatile("" :: "v"(nrows[j]));
+        }
+        t0 = t1; t1 = t2;
+        static_for<0, 8>([&](auto rc_) { read_set(a1, C0{}, rc_); });
+        static_for<0, 8>([&](auto rc_) { read_set(a0, std::integral_constant<int, 2>{}, rc_); });
+    }
+    __builtin_amdgcn_s_waitcnt(kWaitVm0);
+}
+
 // ---- duo kernel: the ring kernel at half the tile edge, two workgroups per CU ------------------------------
 // Workgroup tile 128 x 128 x 128, four wavefronts 2 x 2, each 64 x 64 = 2 x 2 MFMA tiles (64 accumulator
 // registers), the same ring of five slots at 16 KiB each: 80 KiB, so a CU holds TWO workgroups and every SIMD two
@@ -1825,6 +2265,23 @@ int launch_tiled(const GemmArgs& p, hipStream_t st) {
         const int total = p.tiles_m * p.tiles_n;     // grouped: tiles_m is the host-side upper bound of row tiles
         int grid = total < num_cus() ? total : num_cus();
         if (grid >= kXcds) grid -= grid % kXcds;
+        if constexpr (EPI == EPI_NONE || EPI == EPI_BIAS || EPI == EPI_SILU_GATE) {
+            if (!p.mfma32) {
+                static std::once_flag once16;
+                static hipError_t err16 = hipSuccess;
+                std::call_once(once16, [] {
+                    err16 = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_nt_ring16<FMT, EPI, SCALE, false>),
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, kRingLds);
+                    if (err16 == hipSuccess)
+                        err16 = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_nt_ring16<FMT, EPI, SCALE, true>),
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, kRingLds);
+                });
+                if (err16 != hipSuccess) return static_cast<int>(err16);
+                if ((p.K / BK) & 1) k_gemm_nt_ring16<FMT, EPI, SCALE, true><<<grid, kThreads, kRingLds, st>>>(p);
+                else                k_gemm_nt_ring16<FMT, EPI, SCALE, false><<<grid, kThreads, kRingLds, st>>>(p);
+                return launch_status();
+            }
+        }
         k_gemm_nt_ring<FMT, EPI, SCALE><<<grid, kThreads, kRingLds, st>>>(p);
         return launch_status();
     }
@@ -2060,6 +2517,7 @@ int cf_fp8_gemm_nt_bf16_ex(int M, int N, int K, const void* A, int lda, int a_is
     if (epilogue > EPI_SILU_GATE) return CF_ERR_INVALID_ARG;
     p.force_staged = (flags & CF_GEMM_FLAG_STAGED) != 0;
     p.duo = (flags & CF_GEMM_FLAG_DUO) ? ((flags & CF_GEMM_FLAG_DUO_IN_STEP) ? 2 : 1) : 0;
+    p.mfma32 = (flags & CF_GEMM_FLAG_MFMA32) != 0;
     return gemm_nt(p, a_is_e5m2 ? 1 : 0, epilogue, scale_mode, flags & CF_GEMM_FLAG_NAIVE, stream);
 }
 

@@ -255,6 +255,9 @@ int cf_cross_entropy_fwd_bwd_chunk_quant_e5m2(const uint16_t* d_logits, const in
                                   the other workgroup's MFMAs) where it applies: E4M3, CF_SCALE_ROW_COL, plain or SiLU-gate
                                   epilogue, N a multiple of 128 (64 with the SiLU gate) */
 #define CF_GEMM_FLAG_DUO_IN_STEP 8 /* with CF_GEMM_FLAG_DUO: do not start the CU's second workgroup half a tile late */
+#define CF_GEMM_FLAG_MFMA32 16 /* plain, bias and SiLU-gate epilogues: keep the ring kernel on v_mfma_f32_32x32x64_f8f6f4
+                                  instead of the one on v_mfma_f32_16x16x128_f8f6f4 (the default; same tiles and drain,
+                                  8 - 9 % more MFMA throughput at the same socket power) */
 
 /* lt_gemm_fp8_nt, static at src/trainer.cu:4498-4534 (plan lookup :4402-4496).
  * C[M,N] bf16 (row stride ldc) = (A[M,K] fp8, row stride lda, E4M3 or E5M2) .

@@ -209,6 +209,59 @@ def test_gemm_two_workgroups_per_cu_kernel_matches_the_ring_kernel(cf, dev, M, N
     assert np.array_equal(wide[:, :N], ring) and np.isnan(wide[:, N:]).all()
 
 
+MFMA32 = 16
+
+
+# (300, 256, 384): ragged last row tile, three K-tiles (odd); (1100, 384, 256): two K-tiles; (3000, 768, 512): more tiles than
+# workgroups; (520, 904, 640): a last column tile cut short at a multiple of 8, five K-tiles; (257, 128, 4096): 32 K-tiles
+@pytest.mark.parametrize("M,N,K", [(300, 256, 384), (1100, 384, 256), (3000, 768, 512), (520, 904, 640), (257, 128, 4096)])
+@pytest.mark.parametrize("epi", [EPI_NONE, EPI_BIAS, EPI_SILU])
+@pytest.mark.parametrize("mode", [PER_TENSOR, ROW_COL])
+def test_gemm_both_mfma_shapes_of_the_ring_kernel(cf, dev, M, N, K, epi, mode):
+    """The persistent kernel exists on two MFMA shapes: v_mfma_f32_16x16x128_f8f6f4 (the default for the bf16 epilogues)
+    and v_mfma_f32_32x32x64_f8f6f4 (CF_GEMM_FLAG_MFMA32; also what the accumulate and term-split forms run on).  Same
+    tiles, same drain arithmetic; the two differ at most by the order in which a K-tile's 128 products are added."""
+    if epi == EPI_SILU and N % 128:
+        pytest.skip("the fused gate/up form keeps whole column tiles on either kernel")
+    case(f"gemm 16x16x128 / 32x32x64 {M}x{N}x{K} epi={epi} mode={mode}")
+    rng = np.random.default_rng(M + N + K + 3 * epi + mode)
+    A, sa = rand_fp8(rng, (M, K))
+    Bg, sg = rand_fp8(rng, (N, K), sigma=0.02)
+    Bu, su = rand_fp8(rng, (N, K), sigma=0.02)
+    if mode == ROW_COL:
+        sa = (sa * rng.uniform(0.5, 2, M)).astype(np.float32)
+        sg = (sg * rng.uniform(0.5, 2, N)).astype(np.float32)
+        su = (su * rng.uniform(0.5, 2, N)).astype(np.float32)
+    bias = orc.bf16_from_f32((rng.standard_normal(N) * 0.05).astype(np.float32)) if epi == EPI_BIAS else None
+    kw = dict(mode=mode, epi=epi, bias=bias, B2=Bu if epi == EPI_SILU else None, sb2=su if epi == EPI_SILU else None)
+    new = run_gemm(cf, dev, A, Bg, sa, sg, ldc=N + 24, **kw)
+    old = run_gemm(cf, dev, A, Bg, sa, sg, flags=MFMA32, ldc=N + 24, **kw)
+    assert np.isnan(new[:, N:]).all() and np.isnan(old[:, N:]).all()
+    new, old = new[:, :N], old[:, :N]
+    if epi == EPI_NONE:
+        ref, absdot = orc.gemm_nt_ref(A, Bg, np.atleast_1d(sa), np.atleast_1d(sg), scale_mode=mode)
+        orc.assert_gemm_close(new, ref, absdot, what=f"16x16x128 {M}x{N}x{K}")
+        orc.assert_gemm_close(old, ref, absdot, what=f"32x32x64 {M}x{N}x{K}")
+    # against each other: the same value, or neighbouring bf16 values where the accumulation order moves a sum across a
+    # rounding boundary (gate, up and product each round once in the fused form)
+    tol = (3 if epi == EPI_SILU else 1) * np.maximum(orc.bf16_ulp(old), orc.bf16_ulp(new))
+    assert np.all(np.abs(new - old) <= tol), float(np.abs(new - old).max())
+    assert (new != old).mean() < 0.02
+
+
+def test_gemm_exact_integers_on_both_mfma_shapes(cf, dev):
+    case("gemm exact small integers, 16x16x128 and 32x32x64")
+    rng = np.random.default_rng(21)
+    M, N, K = 520, 384, 640
+    ai = rng.integers(-3, 4, (M, K)).astype(np.float32)
+    bi = rng.integers(-2, 3, (N, K)).astype(np.float32)
+    A, B = orc.e4m3_satfinite(ai), orc.e4m3_satfinite(bi)
+    want = orc.bf16_to_f32(orc.bf16_from_f32((ai @ bi.T).astype(np.float32))).astype(np.float64)
+    one = np.float32(1.0)
+    for flags in (0, MFMA32):
+        assert np.array_equal(run_gemm(cf, dev, A, B, one, one, flags=flags), want), flags
+
+
 def test_gemm_duo_flag_on_other_shapes_takes_the_usual_kernels(cf, dev):
     case("gemm duo flag on shapes the kernel does not take")
     rng = np.random.default_rng(9)

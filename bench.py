@@ -483,7 +483,7 @@ def main():
             "quantize_h_pct_hbm_peak": round(100.0 * qh_bytes / (qh_alone_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),
         },
         "roofline": {
-            "kernel": "k_gemm_nt_ring<e4m3,silu_gate,row_col> M=8192 N=2x14336 K=4096",
+            "kernel": "k_gemm_nt_ring16<e4m3,silu_gate,row_col> M=8192 N=2x14336 K=4096 (v_mfma_f32_16x16x128_f8f6f4)",
             "bound": "mfma", "achieved": round(gateup_tflops, 1), "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": round(gateup_tflops / FP8_PEAK_TFLOPS, 4), "traffic": traffic,
         },

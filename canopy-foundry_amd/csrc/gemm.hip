@@ -1150,7 +1150,9 @@ void k_gemm_nt_ring(const GemmArgs p) {
 // K-tile under phases 0 and 1, A0 and B[1-p] of the NEXT K-tile under phases 2 and 3 (after the barrier that makes
 // that K-tile visible).  The next K-tile then starts with (A0, B[1-p]): its parity is the other one, and so on.
 // Forms: plain, bias and SiLU-gate epilogues (the LDS-staged bf16 drain), every scale mode of those, dense or
-// grouped; no accumulate / fp32-store forms and no term-split form (those stay on k_gemm_nt_ring).
+// grouped, an even number of K-tiles.  The accumulate / fp32-store forms stay on k_gemm_nt_ring (the fp32-accumulating
+// weight gradient measured the same on either shape: its drain, not the MFMAs, sets its power), and so does the
+// term-split form.
 typedef float v4f __attribute__((ext_vector_type(4)));
 // 16-byte chunk swizzle of this kernel's operand tiles: within any 16 rows the 16-lane groups of a ds_read_b128 (rows
 // 0-7 of one k-group with rows 8-15 of the next) land in 16 different 16-byte slots of a 256-byte line, and the
@@ -1312,10 +1314,12 @@ __device__ __forceinline__ void drain_tile16(v4f (&acc)[8][8], TileScales16<EPI>
     }
 }
 
-// KODD: the number of K-tiles per tile is odd.  A K-tile's parity is its position in the tile modulo 2 (after a drain
-// the operands are read afresh, so every tile starts at parity 0), and the sequence of K-tile bodies is straight-line
-// code for either case.
-template <int FMT, int EPI, int SCALE, bool KODD>
+// A K-tile's parity is its position in the tile modulo 2 (after a drain the operands are read afresh, so every tile
+// starts at parity 0).  The number of K-tiles per tile is even (the launcher sends other shapes to k_gemm_nt_ring), so a
+// tile is first(0), pairs of (1, 0), last(1): straight-line code.  (A form for odd counts was built: its extra K-tile
+// bodies cost the register allocator its balance, reloads landed inside the K-tile loop and it ran 20 % slower than
+// k_gemm_nt_ring at K = 1408.)
+template <int FMT, int EPI, int SCALE>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void k_gemm_nt_ring16(const GemmArgs p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -1550,20 +1554,18 @@ void k_gemm_nt_ring16(const GemmArgs p) {
             rotate(); advance_copy();
         }
         fetch_seq = ahead ? seq + 2 : my_tiles;
-        if constexpr (KODD) {
-            ktile(C0{}, C0{}, C1{}, dkt * BK, t, true);
-            rotate(); advance_copy();
-            ktile(C0{}, C1{}, C0{}, dkt * BK, t, true);
-        } else {
-            ktile(C0{}, C1{}, C1{}, dkt * BK, t, true);
-        }
+        ktile(C0{}, C1{}, C1{}, dkt * BK, t, true);
         rotate(); advance_copy();
         const bool more = ahead && seq + 2 < my_tiles;
         auto landed = [&]() { if (more) fetch_rows(t2, nrows); };
         uint8_t* stage = smem + a4 + wave * (64 * BK);
+        // the drain's per-lane constants are worked out afresh for every tile: hoisted out of the tile loop they would sit
+        // in registers through the K-tile loop, which has none to spare
+        int lane_d = lane;
+        asm volatile("" : "+v"(lane_d));
         constexpr int out_bn = EPI == EPI_SILU_GATE ? BN / 2 : BN;
-        if (t.m0 + BM <= t.m_end && t.n0 + out_bn <= p.N) drain_tile16<EPI, SCALE, false>(acc, sc, s1, s2, p, t, wm, wn, lane, stage, landed);
-        else                                              drain_tile16<EPI, SCALE, true>(acc, sc, s1, s2, p, t, wm, wn, lane, stage, landed);
+        if (t.m0 + BM <= t.m_end && t.n0 + out_bn <= p.N) drain_tile16<EPI, SCALE, false>(acc, sc, s1, s2, p, t, wm, wn, lane_d, stage, landed);
+        else                                              drain_tile16<EPI, SCALE, true>(acc, sc, s1, s2, p, t, wm, wn, lane_d, stage, landed);
         if (more) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) asm volatile("" :: "v"(nrows[j]));
@@ -2266,19 +2268,16 @@ int launch_tiled(const GemmArgs& p, hipStream_t st) {
         int grid = total < num_cus() ? total : num_cus();
         if (grid >= kXcds) grid -= grid % kXcds;
         if constexpr (EPI == EPI_NONE || EPI == EPI_BIAS || EPI == EPI_SILU_GATE) {
-            if (!p.mfma32) {
+            // the bf16 epilogues on an even number of K-tiles: the kernel on the 16 x 16 x 128 MFMA
+            if (!p.mfma32 && (p.K / BK) % 2 == 0) {
                 static std::once_flag once16;
                 static hipError_t err16 = hipSuccess;
                 std::call_once(once16, [] {
-                    err16 = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_nt_ring16<FMT, EPI, SCALE, false>),
+                    err16 = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_nt_ring16<FMT, EPI, SCALE>),
                                                 hipFuncAttributeMaxDynamicSharedMemorySize, kRingLds);
-                    if (err16 == hipSuccess)
-                        err16 = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_nt_ring16<FMT, EPI, SCALE, true>),
-                                                    hipFuncAttributeMaxDynamicSharedMemorySize, kRingLds);
                 });
                 if (err16 != hipSuccess) return static_cast<int>(err16);
-                if ((p.K / BK) & 1) k_gemm_nt_ring16<FMT, EPI, SCALE, true><<<grid, kThreads, kRingLds, st>>>(p);
-                else                k_gemm_nt_ring16<FMT, EPI, SCALE, false><<<grid, kThreads, kRingLds, st>>>(p);
+                k_gemm_nt_ring16<FMT, EPI, SCALE><<<grid, kThreads, kRingLds, st>>>(p);
                 return launch_status();
             }
         }

@@ -17,7 +17,7 @@ from a HIP graph, two HBM ceilings for the quantize kernels (a plain device copy
 library with the quantize's own 2-read : 1-write traffic), socket power and shader clock sampled during the timed
 region.
 
-Before the W warm-up steps the same eager step runs for `--settle` seconds (default 0.5): right after the idle
+Before the W warm-up steps the same eager step runs for `--settle` seconds (default 1.0): right after the idle
 set-up phase the part is still ramping its clocks and the first tens of steps run several percent slower than the
 same step a second later.  The W warm-up steps and the K timed steps follow unchanged; the literal procedure without
 the settling phase is timed first and reported as `unsettled_ms_per_step`.
@@ -199,7 +199,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--settle", type=float, default=0.5,
+    ap.add_argument("--settle", type=float, default=1.0,
                     help="seconds of the same eager step run before the warm-up steps, so that the timed region is not the "
                          "part's ramp after the idle set-up phase (0 = none)")
     ap.add_argument("--no-cpu-baseline", action="store_true")

@@ -220,6 +220,12 @@ def main():
          lambda: cf.cf_fp8_gemm_nt_bf16_ex(M, N, K, xq, K, 0, xd, wg, K, wgd, 1, 2, None, wu, wud, c, N, 0, st))
     mfma("gemm down projection (config 2)", f"{M}x{K}x{N}", 2.0 * M * N * K,
          lambda: cf.cf_fp8_gemm_nt_bf16_ex(M, K, N, hq, N, 0, xd, wd, N, wdd, 1, 0, None, None, None, y, K, 0, st))
+    # the same two launches on the persistent kernel's 32 x 32 x 64 MFMA form (CF_GEMM_FLAG_MFMA32 = 16; the default for
+    # these epilogues is the 16 x 16 x 128 form, which does more at the same socket power)
+    mfma("32x32x64 MFMA: gemm gate+up fused SiLU-gate (config 2)", f"{M}x2x{N}x{K}", 4.0 * M * N * K,
+         lambda: cf.cf_fp8_gemm_nt_bf16_ex(M, N, K, xq, K, 0, xd, wg, K, wgd, 1, 2, None, wu, wud, c, N, 16, st))
+    mfma("32x32x64 MFMA: gemm down projection (config 2)", f"{M}x{K}x{N}", 2.0 * M * N * K,
+         lambda: cf.cf_fp8_gemm_nt_bf16_ex(M, K, N, hq, N, 0, xd, wd, N, wdd, 1, 0, None, None, None, y, K, 16, st))
     # The same launch on operands without entropy (every byte 0x38 = 1.0): the matrix cores' power follows how much
     # their inputs toggle, and on such data the part stays below its power cap at full clock.  What separates this
     # row from the one on quantized data is the power cap, not the kernel (use --sustain to see power and clock).

@@ -1316,9 +1316,10 @@ __device__ __forceinline__ void drain_tile16(v4f (&acc)[8][8], TileScales16<EPI>
 
 // A K-tile's parity is its position in the tile modulo 2 (after a drain the operands are read afresh, so every tile
 // starts at parity 0).  The number of K-tiles per tile is even (the launcher sends other shapes to k_gemm_nt_ring), so a
-// tile is first(0), pairs of (1, 0), last(1): straight-line code.  (A form for odd counts was built: its extra K-tile
-// bodies cost the register allocator its balance, reloads landed inside the K-tile loop and it ran 20 % slower than
-// k_gemm_nt_ring at K = 1408.)
+// tile is first(0), pairs of (1, 0), last(1): straight-line code.  (Two forms for odd counts were built and measured at
+// K = 1408 against k_gemm_nt_ring: first(0), pairs of (1, 0), 1, last(0) spilled registers inside the K-tile loop and ran
+// 20 % slower; first(0), 1, pairs of (0, 1), last(0) ran 1 % slower.  Eleven K-tiles per drain leave the matrix cores too
+// little of the launch for their lower power to pay.)
 template <int FMT, int EPI, int SCALE>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void k_gemm_nt_ring16(const GemmArgs p) {

@@ -9,13 +9,20 @@
 // lane needs eight consecutive k of one row (or column).  Such a tile is parked in LDS as it lies in memory,
 // [k][columns], and read with ds_read_b64_tr_b16: per 16 lanes the instruction takes a 4 (k) x 16 (columns) block,
 // source lane r supplying the address of row r / 4, columns 4 (r % 4) .. +3, and hands lane i the four k values of
-// column i.  Two such reads give a lane its eight k of a 32x32x16 MFMA operand.  An operand that is K-contiguous
-// in memory takes the usual path (128-byte LDS rows, 16-byte chunks xor-swizzled, ds_read_b128).
+// column i.  Two such reads give a lane its eight k of a 16x16x32 MFMA operand (lanes 16 g .. 16 g + 15 hold k rows
+// 8 g .. 8 g + 7 of a 32-deep k-step).  An operand that is K-contiguous in memory takes the usual path (128-byte LDS
+// rows, 16-byte chunks xor-swizzled, ds_read_b128).
 //
-// Workgroup tile 256 (M) x 256 (N) x 64 (K), four wavefronts 2 x 2, each 128 x 128 = 4 x 4 tiles of
-// v_mfma_f32_32x32x16_bf16 with fp32 accumulators.  The N-side operand goes to the MFMA "A" side, so a lane
-// ends up with four consecutive output columns of one output row per accumulator quad.  Global loads are
-// register staged two K-tiles ahead (16 bytes per lane), LDS is double buffered, one barrier per K-tile.
+// Workgroup tile 256 (M) x 256 (N) x 64 (K), four wavefronts 2 x 2, each 128 x 128 = 8 x 8 blocks of
+// v_mfma_f32_16x16x32_bf16 with fp32 accumulators (four registers per block).  Both bf16 MFMA shapes do 1024 FLOP per
+// cycle and SIMD; at the socket power limit, where these GEMMs run, the 16 x 16 x 32 shape delivers 14 % more (MFMAs
+// alone on random operands, probes/mfma_shape_power_bf16.hip).  The N-side operand goes to the MFMA "A" side, so a lane
+// ends up with four consecutive output columns of one output row per block.  Global loads are register staged two
+// K-tiles ahead (16 bytes per lane), LDS is double buffered, one barrier per K-tile.
+// Operand registers: four sets of four blocks (N halves N0, N1; M halves M0, M1; 16 registers each).  A 32-deep k-step
+// is four phases of sixteen MFMAs, (N0, M[p]) -> (N0, M[1-p]) -> (N1, M[1-p]) -> (N1, M[p]) with p the k-step's parity,
+// and the set a phase leaves behind is refilled two phases before it is needed again: M[1-p] and N1 of this k-step
+// under phases 0 and 1, N0 and M[1-p] of the next k-step under phases 2 and 3.  A K-tile is two k-steps.
 // Rows, columns and k beyond the operands' bounds are read as zeros (buffer loads with the operand's size in their
 // descriptor), so any n_e works.
 #include "common.hpp"
@@ -40,6 +47,7 @@ constexpr int kLds = 2 * kStage;               // 147,456 bytes: one workgroup p
 
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef __bf16 v4bf __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) v4bf* lds_v4bf_ptr;
 
 enum { OUT_STORE_BF16 = 0, OUT_ACCUM_BF16 = 1, OUT_ACCUM_F32 = 2, OUT_STORE_F32 = 3 };
@@ -78,23 +86,20 @@ __device__ __forceinline__ float acc_read(float a) {
     return v;
 }
 
-__device__ __forceinline__ int swz(int row) { return (row ^ ((row >> 3) & 3)) & 7; }
+// 16-byte chunk swizzle of a K-contiguous tile: a ds_read_b128 of a 16 x 16 x 32 operand has rows 0-7 of k-group g go
+// with rows 8-15 of k-group g ^ 1 (chunks g and g ^ 1 of the k-step), and the 16 lanes must hit 16 different 16-byte
+// slots of a 256-byte line
+__device__ __forceinline__ int swz(int row) { return (row ^ (((row >> 3) & 1) << 1)) & 7; }
 
 // Eight k of one column for every lane: two transposing reads of a [k][columns] tile.  `lane_ptr` is the tile's base
 // plus this lane's share of the address (ks_lane_offset); the k-step and the column block are compile-time
 // constants, so they end up in the instructions' immediate offsets and no address register is spent on them.
+// k rows 8 .. 15 (mod 16) of a [k][columns] tile are parked 32 bytes to the right (into the row's pad), so that the
+// k-groups that one instruction serves together do not meet on the same banks.
 __device__ __forceinline__ int ks_lane_offset(int pitch, int lane) {
-    const int b = lane >> 4, r = lane & 15;
-    return (8 * (b >> 1) + (r >> 2)) * pitch + (16 * (b & 1) + 4 * (r & 3)) * 2;
+    const int g = lane >> 4, r = lane & 15;
+    return (8 * g + (r >> 2)) * pitch + (g & 1) * 32 + 4 * (r & 3) * 2;
 }
-template <int PITCH>
-__device__ __forceinline__ v8bf read_ks(const uint8_t* lane_ptr, int krow0, int col0) {
-    const uint8_t* p = lane_ptr + krow0 * PITCH + col0 * 2;
-    const v4bf lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_v4bf_ptr)(p));
-    const v4bf hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_v4bf_ptr)(p + 4 * PITCH));
-    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-}
-
 // A_KS: the M-side operand is stored [K][M] (the weight-gradient form); otherwise [M][K].
 // B_KC: the N-side operand is stored [N][K] (a weight matrix as the forward pass holds it); otherwise [K][N].
 // GATHER (with the [M][K] form of A): the tile's rows of A are fetched through a row index, so a token permute
@@ -226,7 +231,7 @@ void k_gemm_bf16(const BfArgs p) {
         uint8_t* as = smem + stage * kStage;
         if constexpr (c < NA) {
             if constexpr (A_KS) {
-                *reinterpret_cast<uint4*>(as + ((tid >> 5) + 8 * c) * kPitchM + (tid & 31) * 16) = ra[c];
+                *reinterpret_cast<uint4*>(as + ((tid >> 5) + 8 * c) * kPitchM + (c & 1) * 32 + (tid & 31) * 16) = ra[c];
             } else {
                 const int r = (tid >> 3) + 32 * c;
                 *reinterpret_cast<uint4*>(as + r * kPitchKC + (((tid & 7) ^ swz(r)) << 4)) = ra[c];
@@ -235,60 +240,83 @@ void k_gemm_bf16(const BfArgs p) {
             const int r = (tid >> 3) + 32 * (c - NA);
             *reinterpret_cast<uint4*>(as + kATile + r * kPitchKC + (((tid & 7) ^ swz(r)) << 4)) = rb[c - NA];
         } else {
-            *reinterpret_cast<uint4*>(as + kATile + ((tid >> 5) + 8 * (c - NA)) * kPitchN + (tid & 31) * 16) = rb[c - NA];
+            *reinterpret_cast<uint4*>(as + kATile + ((tid >> 5) + 8 * (c - NA)) * kPitchN + ((c - NA) & 1) * 32 + (tid & 31) * 16) = rb[c - NA];
         }
     };
 
     // ---- LDS -> MFMA ----
-    v16f acc[4][4];      // [n tile][m tile]
+    v4f acc[8][8];      // [n block][m block]
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < 8; ++j)
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < 8; ++i)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[j][i][r] = 0.0f;
+            for (int r = 0; r < 4; ++r) acc[j][i][r] = 0.0f;
 
-    const int frow = lane & 31, khalf = lane >> 5;
+    const int r16 = lane & 15, kg = lane >> 4;
     const int ks_n = ks_lane_offset(kPitchN, lane) + wn * 128 * 2, ks_m = ks_lane_offset(kPitchM, lane) + wm * 128 * 2;
-    // operand fragments, two sets: k-step s of any K-tile lives in set s % 2
-    v8bf nop[2][4], mop[2][4];
-    // fragment u (0..3: N side, 4..7: M side) of k-step s of the K-tile in LDS stage `stage`
-    auto read_unit = [&](int stage, auto sc, auto uc) {
-        constexpr int ks16 = decltype(sc)::value, u = decltype(uc)::value;
+    // K-contiguous tiles: this lane's row within a block and its chunk for either k-step (the swizzle depends on the
+    // row modulo 16 only, so the block is an immediate offset)
+    int kc[2];
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) kc[s2] = r16 * kPitchKC + (((4 * s2 + kg) ^ swz(r16)) << 4);
+    // operand sets: [half of the wavefront's 128 columns / rows][block]
+    v8bf nset[2][4], mset[2][4];
+    // block R (0..3) of set SET (0, 1: N halves; 2, 3: M halves) for k-step S of the K-tile in LDS stage `stage`: one
+    // ds_read_b128 of a K-contiguous operand, two transposing reads (k rows + 0 .. 3 and + 4 .. 7) of a [k][columns] one
+    auto read_set = [&](int stage, auto sc, auto setc, auto rc_) {
+        constexpr int S = decltype(sc)::value, SET = decltype(setc)::value, R = decltype(rc_)::value;
         const uint8_t* as = smem + stage * kStage;
-        if constexpr (u < 4 && B_KC) {
-            const int row = wn * 128 + 32 * u + frow;
-            nop[ks16 & 1][u] = *reinterpret_cast<const v8bf*>(as + kATile + row * kPitchKC + (((2 * ks16 + khalf) ^ swz(row)) << 4));
-        } else if constexpr (u < 4) {
-            nop[ks16 & 1][u] = read_ks<kPitchN>(as + kATile + ks_n, 16 * ks16, 32 * u);
-        } else if constexpr (A_KS) {
-            mop[ks16 & 1][u - 4] = read_ks<kPitchM>(as + ks_m, 16 * ks16, 32 * (u - 4));
+        constexpr bool NSIDE = SET < 2;
+        constexpr bool KC = NSIDE ? B_KC : !A_KS;
+        constexpr int half = SET & 1, blk = half * 4 + R;
+        v8bf v;
+        if constexpr (KC) {
+            const uint8_t* base = as + (NSIDE ? kATile + wn * 128 * kPitchKC : wm * 128 * kPitchKC);
+            v = *reinterpret_cast<const v8bf*>(base + blk * 16 * kPitchKC + kc[S]);
         } else {
-            const int row = wm * 128 + 32 * (u - 4) + frow;
-            mop[ks16 & 1][u - 4] = *reinterpret_cast<const v8bf*>(as + row * kPitchKC + (((2 * ks16 + khalf) ^ swz(row)) << 4));
+            constexpr int PITCH = NSIDE ? kPitchN : kPitchM;
+            const uint8_t* pl = as + (NSIDE ? kATile + ks_n : ks_m) + 32 * S * PITCH + 16 * blk * 2;
+            const v4bf lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_v4bf_ptr)(pl));
+            const v4bf hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_v4bf_ptr)(pl + 4 * PITCH));
+            v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
         }
+        if constexpr (NSIDE) nset[half][R] = v; else mset[half][R] = v;
     };
+    constexpr int RN = 4, RM = 4;       // read_set calls per set
 
-    // One K-tile (64 MFMAs per wavefront) with everything else woven between them, one item per MFMA at most (one
+    // One K-tile: two k-steps of four phases, 128 MFMAs per wavefront, with everything else woven between them (one
     // wavefront per SIMD: whatever waits, the matrix cores wait with it).  While tile ks is multiplied from `stage`:
-    //   - the fragments of k-step s + 1 are read during k-step s;
-    //   - the 16 loads of tile ks + 2 go out one every fourth MFMA, into the register set tile ks just left;
-    //   - tile ks + 1 (requested one tile ago) is parked in the other stage one chunk every third MFMA, done by MFMA 47;
-    //   - the barrier follows, and the first fragments of tile ks + 1 are read under the last 16 MFMAs.
+    //   - a phase refills the set the phase before it left behind (see the top of the file);
+    //   - the 16 loads of tile ks + 2 go out one every eighth MFMA, into the register set tile ks just left;
+    //   - tile ks + 1 (requested one tile ago) is parked in the other stage one chunk every sixth MFMA, done by MFMA 92;
+    //   - the barrier follows MFMA 95, and the first sets of tile ks + 1 are read under the last 32 MFMAs.
     // A tile past the end of the k range is fetched as zeros (it lies beyond the descriptors) and adds nothing, so the
     // loop needs no tail.
     auto ktile = [&](auto stage_c, int ks, uint4 (&ra_new)[NA], uint4 (&rb_new)[NB], const uint4 (&ra_next)[NA], const uint4 (&rb_next)[NB]) {
         constexpr int stage = decltype(stage_c)::value;
-        static_for<0, 64>([&](auto mc) {
-            constexpr int m = decltype(mc)::value, ks16 = m / 16, q = m % 16;
-            acc[q >> 2][q & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(nop[ks16 & 1][q >> 2], mop[ks16 & 1][q & 3], acc[q >> 2][q & 3], 0, 0, 0);
-            if constexpr (q < 8) {
-                if constexpr (ks16 < 3) read_unit(stage, std::integral_constant<int, (ks16 + 1) % 4>{}, std::integral_constant<int, q % 8>{});
-                else                    read_unit(stage ^ 1, std::integral_constant<int, 0>{}, std::integral_constant<int, q % 8>{});
+        static_for<0, 128>([&](auto mc) {
+            constexpr int m = decltype(mc)::value, S = m / 64, ph = (m % 64) / 16, q = m % 16;
+            // k-step S has parity S: phases (N0, M[S]), (N0, M[1-S]), (N1, M[1-S]), (N1, M[S])
+            constexpr int nh = ph >> 1, mh = (ph == 0 || ph == 3) ? S : 1 - S;
+            constexpr int jn = nh * 4 + (q >> 2), im = mh * 4 + (q & 3);
+            // issued through inline assembly with the accumulator tied to the destination: left to the compiler, the 64
+            // four-register accumulators come out of a K-tile in other registers than they went in and are moved back
+            // through the vector ALU at the loop's end (several hundred moves per K-tile pair)
+            asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[jn][im]) : "v"(nset[nh][q >> 2]), "v"(mset[mh][q & 3]));
+            // refills: ph 0: M[1-S] of this k-step; ph 1: N1 of this k-step; ph 2: N0 of the next k-step; ph 3: M[1-S] of the next
+            if constexpr (ph == 0) {
+                if constexpr (q < 2 * RM && q % 2 == 0) read_set(stage, std::integral_constant<int, S>{}, std::integral_constant<int, 2 + (1 - S)>{}, std::integral_constant<int, (q / 2) % RM>{});
+            } else if constexpr (ph == 1) {
+                if constexpr (q < 2 * RN && q % 2 == 0) read_set(stage, std::integral_constant<int, S>{}, std::integral_constant<int, 1>{}, std::integral_constant<int, (q / 2) % RN>{});
+            } else if constexpr (ph == 2) {
+                if constexpr (q < 2 * RN && q % 2 == 0) read_set(S == 0 ? stage : stage ^ 1, std::integral_constant<int, 1 - S>{}, std::integral_constant<int, 0>{}, std::integral_constant<int, (q / 2) % RN>{});
+            } else {
+                if constexpr (q < 2 * RM && q % 2 == 0) read_set(S == 0 ? stage : stage ^ 1, std::integral_constant<int, 1 - S>{}, std::integral_constant<int, 2 + (1 - S)>{}, std::integral_constant<int, (q / 2) % RM>{});
             }
-            if constexpr (m % 4 == 1) load_one(ks + 2, std::integral_constant<int, m / 4>{}, ra_new, rb_new);
-            if constexpr (m < 48 && m % 3 == 2) park_one(stage ^ 1, std::integral_constant<int, (m / 3) % 16>{}, ra_next, rb_next);
-            if constexpr (m == 47) __syncthreads();
+            if constexpr (m % 8 == 7) load_one(ks + 2, std::integral_constant<int, m / 8>{}, ra_new, rb_new);
+            if constexpr (m < 96 && m % 6 == 2) park_one(stage ^ 1, std::integral_constant<int, (m / 6) % 16>{}, ra_next, rb_next);
+            if constexpr (m == 95) __syncthreads();
             __builtin_amdgcn_sched_barrier(0);
         });
         if constexpr (B_KC) {          // the next K-tile's loads are one tile further
@@ -305,47 +333,49 @@ void k_gemm_bf16(const BfArgs p) {
     if constexpr (B_KC) kb_load = (2 * TK) % b_period;
     static_for<0, 16>([&](auto c) { park_one(0, c, ra0, rb0); });
     __syncthreads();
-    static_for<0, 8>([&](auto u) { read_unit(0, std::integral_constant<int, 0>{}, u); });
+    // the first k-step (parity 0) starts with (N0, M0)
+    static_for<0, RN>([&](auto r) { read_set(0, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, r); });
+    static_for<0, RM>([&](auto r) { read_set(0, std::integral_constant<int, 0>{}, std::integral_constant<int, 2>{}, r); });
     for (int ks = 0; ks < nk; ks += 2) {
         ktile(std::integral_constant<int, 0>{}, ks, ra0, rb0, ra1, rb1);
         ktile(std::integral_constant<int, 1>{}, ks + 1, ra1, rb1, ra0, rb0);
     }
 
-    // ---- epilogue: accumulator register r of tile (j, i) is output row m0 + wm*128 + 32 i + lane % 32,
-    //      column n0 + wn*128 + 32 j + 8 (r / 4) + 4 (lane / 32) + r % 4 ----
+    // the MFMAs above are opaque to the compiler's hazard handling: leave the wait states between the last of them and
+    // the first read of an accumulator explicitly
+    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+    // ---- epilogue: accumulator register q of block (j, i) is output row m0 + wm*128 + 16 i + lane % 16,
+    //      column n0 + wn*128 + 16 j + 4 (lane / 16) + q ----
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int m = m0 + wm * 128 + 32 * i + frow;
+    for (int i = 0; i < 8; ++i) {
+        const int m = m0 + wm * 128 + 16 * i + r16;
         if (m >= m_end) continue;
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int n = n0 + wn * 128 + 32 * j + 8 * q + 4 * khalf;
-                if (n >= p.N) continue;                      // N % 8 == 0: a quad is inside or outside as a whole
-                const size_t at = c_base + static_cast<size_t>(m) * p.ldc + n;
-                float v[4] = {acc_read(acc[j][i][4 * q]), acc_read(acc[j][i][4 * q + 1]), acc_read(acc[j][i][4 * q + 2]),
-                              acc_read(acc[j][i][4 * q + 3])};
-                if constexpr (OUT == OUT_STORE_F32) {
-                    *reinterpret_cast<float4*>(static_cast<float*>(p.C) + at) = make_float4(v[0], v[1], v[2], v[3]);
-                } else if constexpr (OUT == OUT_ACCUM_F32) {
-                    float4* dst = reinterpret_cast<float4*>(static_cast<float*>(p.C) + at);
-                    float4 c = *dst;
-                    c.x += v[0]; c.y += v[1]; c.z += v[2]; c.w += v[3];
-                    *dst = c;
-                } else {
-                    uint2* dst = reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.C) + at);
-                    if constexpr (OUT == OUT_ACCUM_BF16) {
-                        // fp32 sum of the old value and the product, one rounding (cublasGemmEx with a bf16 C, beta = 1)
-                        const uint2 c = *dst;
-                        v[0] += bf16_lo(c.x); v[1] += bf16_hi(c.x); v[2] += bf16_lo(c.y); v[3] += bf16_hi(c.y);
-                    }
-                    *dst = make_uint2(pack_bf16x2_hw(v[0], v[1]), pack_bf16x2_hw(v[2], v[3]));
+        for (int j = 0; j < 8; ++j) {
+            const int n = n0 + wn * 128 + 16 * j + 4 * kg;
+            if (n >= p.N) continue;                      // N % 8 == 0: a quad is inside or outside as a whole
+            const size_t at = c_base + static_cast<size_t>(m) * p.ldc + n;
+            float v[4] = {acc_read(acc[j][i][0]), acc_read(acc[j][i][1]), acc_read(acc[j][i][2]), acc_read(acc[j][i][3])};
+            if constexpr (OUT == OUT_STORE_F32) {
+                *reinterpret_cast<float4*>(static_cast<float*>(p.C) + at) = make_float4(v[0], v[1], v[2], v[3]);
+            } else if constexpr (OUT == OUT_ACCUM_F32) {
+                float4* dst = reinterpret_cast<float4*>(static_cast<float*>(p.C) + at);
+                float4 c = *dst;
+                c.x += v[0]; c.y += v[1]; c.z += v[2]; c.w += v[3];
+                *dst = c;
+            } else {
+                uint2* dst = reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.C) + at);
+                if constexpr (OUT == OUT_ACCUM_BF16) {
+                    // fp32 sum of the old value and the product, one rounding (cublasGemmEx with a bf16 C, beta = 1)
+                    const uint2 c = *dst;
+                    v[0] += bf16_lo(c.x); v[1] += bf16_hi(c.x); v[2] += bf16_lo(c.y); v[3] += bf16_hi(c.y);
                 }
-                // one quad's loads and stores at a time: pulling the whole tile's reads of C to the front would need
-                // more registers than the main loop leaves
-                if constexpr (OUT == OUT_ACCUM_BF16 || OUT == OUT_ACCUM_F32) __builtin_amdgcn_sched_barrier(0);
+                *dst = make_uint2(pack_bf16x2_hw(v[0], v[1]), pack_bf16x2_hw(v[2], v[3]));
             }
+            // one quad's loads and stores at a time: pulling the whole tile's reads of C to the front would need
+            // more registers than the main loop leaves
+            if constexpr (OUT == OUT_ACCUM_BF16 || OUT == OUT_ACCUM_F32) __builtin_amdgcn_sched_barrier(0);
+        }
     }
 }
 

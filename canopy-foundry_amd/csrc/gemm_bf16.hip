@@ -164,21 +164,24 @@ void k_gemm_bf16(const BfArgs p) {
     // A buffer load takes a descriptor with a base and a size in bytes and returns zeros for a lane whose offset lies
     // beyond the size, so every load is issued unconditionally (loads under branches would keep the compiler from
     // counting the loads in flight: it would wait for all of them, the prefetch included, before the first LDS store)
-    // and the zero fill of the ragged ends costs nothing.  Each load gets a descriptor of its own, built with scalar
-    // instructions: the base is the first of the eight-row (32-row) group it fetches, the size what is left of the
-    // operand from there (nothing, past the end of the k range), so the lane's offset is one constant per operand: its
-    // row within the group and its 16-byte column; a lane whose columns lie outside the operand (or, for the
-    // K-contiguous form, whose k chunk lies beyond K) uses an offset beyond every size.  The launcher keeps operands
-    // below 2 GiB.
+    // and the zero fill of the ragged ends costs nothing.  Each operand gets one descriptor per K-tile, built with scalar
+    // instructions: the base is the tile's first row (and first k), the size what is left of the operand from there
+    // (nothing, past the end of the k range).  A lane's offset is its row within the first eight-row (32-row) group and
+    // its 16-byte column, plus the group's distance from the tile's first row; a lane whose columns lie outside the
+    // operand (or, for the K-contiguous form, whose k chunk lies beyond K) starts from an offset beyond every size.
+    // The launcher keeps operands below 2 GiB, so the sum does not wrap.  (A descriptor per load costs about ten
+    // scalar instructions in front of one MFMA in every eight, more than the MFMA's 16 cycles cover.)
     constexpr uint32_t kOutside = 0x80000000u;
     typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
     // rows [row0, row_end) of a row-major operand with `ld` elements per row, seen from element `col0` of row row0
-    auto load_rows = [](const uint16_t* base, int ld, int row0, int row_end, int col0, uint32_t lane_off) {
+    auto rows_rsrc = [](const uint16_t* base, int ld, int row0, int row_end, int col0) {
         const int rows_left = max(row_end - row0, 0);
-        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+        return __builtin_amdgcn_make_buffer_rsrc(
             const_cast<uint16_t*>(base + static_cast<size_t>(row0) * ld + col0), 0,
             static_cast<int>(static_cast<uint32_t>(rows_left) * static_cast<uint32_t>(ld) * 2u), 0x00020000);
-        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rs, static_cast<int>(lane_off), 0, 0);
+    };
+    auto load_at = [](__amdgpu_buffer_rsrc_t rs, uint32_t off) {
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rs, static_cast<int>(off), 0, 0);
         return make_uint4(v.x, v.y, v.z, v.w);
     };
     // [k][columns] operands: this lane's row within a group of eight k rows and its 16-byte column
@@ -204,25 +207,43 @@ void k_gemm_bf16(const BfArgs p) {
     const int b_period = B_KC && p.b_k_period ? p.b_k_period : 0x7fffffff;
     int kb_load = 0;              // ... for the tile the next load_one calls fetch (set by the callers)
     // chunk c (0 .. NA-1: M side, NA .. NA+NB-1: N side) of K-tile ks into its staging register
+    // One descriptor per operand and K-tile, built by the tile's first load of that operand; the chunks of the tile
+    // differ in the lane offset only (one vector add each).
+    __amdgpu_buffer_rsrc_t rs_a = a_all, rs_b = a_all;
+    uint32_t off_a = kOutside, off_b = kOutside;
+    const uint32_t a_step = (A_KS ? 8u : 32u) * static_cast<uint32_t>(p.lda) * 2u;
+    const uint32_t b_step = (B_KC ? 32u : 8u) * static_cast<uint32_t>(p.ldb) * 2u;
     auto load_one = [&](int ks, auto cc, uint4 (&ra)[NA], uint4 (&rb)[NB]) {
         constexpr int c = decltype(cc)::value;
         const int k0 = k_begin + ks * TK;
-        if constexpr (c < NA) {
+        if constexpr (c == 0 && !GATHER) {
             if constexpr (A_KS) {
-                ra[c] = load_rows(p.A, p.lda, k0 + 8 * c, k_end, m0, a_lane_ks);
-            } else if constexpr (GATHER) {
+                rs_a = rows_rsrc(p.A, p.lda, k0, k_end, m0);
+                off_a = a_lane_ks;
+            } else {
+                rs_a = rows_rsrc(p.A, p.lda, m0, m_end, k0);
+                off_a = k0 + (tid & 7) * 8 < k_end ? a_lane_kc : kOutside;
+            }
+        }
+        if constexpr (c == NA) {
+            if constexpr (B_KC) {
+                rs_b = rows_rsrc(B, p.ldb, n0, p.N, kb_load);
+                off_b = k0 + (tid & 7) * 8 < k_end ? b_lane_kc : kOutside;
+            } else {
+                rs_b = rows_rsrc(B, p.ldb, k0, k_end, n0);
+                off_b = b_lane;
+            }
+        }
+        if constexpr (c < NA) {
+            if constexpr (GATHER) {
                 const uint32_t off = k0 + (tid & 7) * 8 < k_end ? a_gather[c] : kOutside;
                 const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(a_all, static_cast<int>(off), k0 * 2, 0);
                 ra[c] = make_uint4(v.x, v.y, v.z, v.w);
             } else {
-                const uint32_t off = k0 + (tid & 7) * 8 < k_end ? a_lane_kc : kOutside;
-                ra[c] = load_rows(p.A, p.lda, m0 + 32 * c, m_end, k0, off);
+                ra[c] = load_at(rs_a, off_a + c * a_step);
             }
-        } else if constexpr (B_KC) {
-            const uint32_t off = k0 + (tid & 7) * 8 < k_end ? b_lane_kc : kOutside;
-            rb[c - NA] = load_rows(B, p.ldb, n0 + 32 * (c - NA), p.N, kb_load, off);
         } else {
-            rb[c - NA] = load_rows(B, p.ldb, k0 + 8 * (c - NA), k_end, n0, b_lane);
+            rb[c - NA] = load_at(rs_b, off_b + (c - NA) * b_step);
         }
     };
     // the same chunk from its staging register into LDS stage `stage`

@@ -25,6 +25,10 @@
 // under phases 0 and 1, N0 and M[1-p] of the next k-step under phases 2 and 3.  A K-tile is two k-steps.
 // Rows, columns and k beyond the operands' bounds are read as zeros (buffer loads with the operand's size in their
 // descriptor), so any n_e works.
+// The kernel is persistent: one workgroup per CU walks a sequence of output tiles with the operand fetch running on
+// across the tile boundaries, and writes a finished tile through LDS in whole 256-byte (bf16) or 512-byte (fp32) row
+// pieces.  Per output tile that leaves about 14 thousand cycles beside the K-tiles (11 of them the stores' way to memory)
+// where one workgroup per tile with stores straight from the accumulator layout took 27 thousand.
 #include "common.hpp"
 #include "internal.hpp"
 
@@ -112,53 +116,103 @@ void k_gemm_bf16(const BfArgs p) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
 
-    // ---- which tile ----
+    // ---- which tiles ----
+    // Persistent: one workgroup per CU walks a sequence of output tiles, and the operand fetch runs on across the tile
+    // boundaries (the last two K-tiles of a tile already request the first two of the next), so only the first tile of a
+    // workgroup waits for memory with idle matrix cores.
     // Workgroups go to the 8 XCDs round-robin (launch position % 8), each XCD with its own 4 MiB L2.  Position b is
     // therefore read as (XCD x = b % 8, that XCD's i-th workgroup), and what an XCD runs at one time is made to share
     // operands: in the row-major forms XCD x walks the contiguous range [x * per, (x + 1) * per) of the tile order in
-    // patches of 8 row tiles x 4 column tiles; in the grouped weight-gradient form XCD x owns experts x, x + 8, ...
-    // whole, so that all tiles of an expert stream the same rows through one L2.
-    const int x = blockIdx.x % 8, xi = blockIdx.x / 8;
-    int m0, n0, m_end = p.M, k_begin = 0, k_end = p.K;
-    const uint16_t* B = p.B;
-    size_t c_base = 0;
-    if constexpr (GROUPED && A_KS) {
-        const int tiles = p.tiles_m * p.tiles_n;
-        const int e = x + 8 * (xi / tiles), t = xi % tiles;
-        if (e >= p.num_experts) return;
-        m0 = (t % p.tiles_m) * TM;
-        n0 = (t / p.tiles_m) * TN;
-        // uniform values, but loaded through the vector path: moved to scalar registers, where the descriptors need them
-        k_begin = __builtin_amdgcn_readfirstlane(p.offsets[e]);
-        k_end = k_begin + __builtin_amdgcn_readfirstlane(p.counts[e]);
-        c_base = static_cast<size_t>(e) * p.c_expert_stride;
-    } else {
-        const int row_tiles = GROUPED ? __builtin_amdgcn_readfirstlane(p.tile_map[0]) : p.tiles_m;
-        const int total = row_tiles * p.tiles_n;
-        const int per = (total + 7) / 8;
-        const int t = x * per + xi;
-        if (xi >= per || t >= total) return;
-        constexpr int GM = 8;
-        const int group = t / (GM * p.tiles_n), first = group * GM;
-        const int gm = min(GM, row_tiles - first), in_group = t - group * GM * p.tiles_n;
-        const int tmi = first + in_group % gm;
-        n0 = (in_group / gm) * TN;
-        m0 = tmi * TM;
-        if constexpr (GROUPED) {
-            const int* e = p.tile_map + 1 + 5 * tmi;
-            const int expert = __builtin_amdgcn_readfirstlane(e[0]), first_row = __builtin_amdgcn_readfirstlane(e[1]);
-            const int end_row = __builtin_amdgcn_readfirstlane(e[2]), first_tile = __builtin_amdgcn_readfirstlane(e[3]);
-            m0 = first_row + (tmi - first_tile) * TM;
-            m_end = min(m0 + TM, end_row);
-            B += static_cast<size_t>(expert) * p.b_expert_stride;
-        }
-    }
-    if (k_end <= k_begin) {
-        if constexpr (OUT == OUT_ACCUM_BF16 || OUT == OUT_ACCUM_F32) return;      // nothing to add
-    }
+    // patches of 8 row tiles x 4 column tiles, its workgroups taking every (grid / 8)-th tile of it; in the grouped
+    // weight-gradient form XCD x owns experts x, x + 8, ... whole, so that all tiles of an expert stream the same rows
+    // through one L2.
+    const int x = blockIdx.x % 8, xi_step = gridDim.x / 8;
     constexpr int TK = 64;
     constexpr int NA = A_KS ? TK / 8 : 8, NB = TK / 8;       // 16-byte chunks per lane and K-tile
-    const int nk = (k_end - k_begin + TK - 1) / TK;
+    constexpr uint32_t kOutside = 0x80000000u;
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    int row_tiles = p.tiles_m;
+    if constexpr (GROUPED && !A_KS) row_tiles = __builtin_amdgcn_readfirstlane(p.tile_map[0]);
+    const int total = row_tiles * p.tiles_n, per = (total + 7) / 8;     // the row-major forms
+    const int tiles_mn = p.tiles_m * p.tiles_n;                          // the grouped weight-gradient form: per expert
+
+    struct Tile {
+        int m0, n0, m_end, k_begin, k_end;
+        int nk2;                // K-tiles, rounded up to an even number (at least two): the pad tile lies beyond the k range
+        long long b_off;        // elements from p.B to the expert's matrix
+        size_t c_base;
+        bool valid;
+    };
+    // The grouped forms read what they need of a tile from memory (its row of the tile table, or the expert's offset
+    // and count).  That read is issued one tile before its values are used, through buffer loads whose offsets lie
+    // beyond the descriptor for positions past the end of the sequence: no branch, no wait.
+    [[maybe_unused]] const __amdgpu_buffer_rsrc_t rs_map = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<int*>(GROUPED && !A_KS ? p.tile_map : nullptr), 0, GROUPED && !A_KS ? (1 + 5 * p.tiles_m) * 4 : 0, 0x00020000);
+    [[maybe_unused]] const __amdgpu_buffer_rsrc_t rs_offsets = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<int*>(GROUPED && A_KS ? p.offsets : nullptr), 0, GROUPED && A_KS ? p.num_experts * 4 : 0, 0x00020000);
+    [[maybe_unused]] const __amdgpu_buffer_rsrc_t rs_counts = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<int*>(GROUPED && A_KS ? p.counts : nullptr), 0, GROUPED && A_KS ? p.num_experts * 4 : 0, 0x00020000);
+    // position xi of this XCD's sequence -> (valid, row tile, first column) for the row-major forms
+    auto place = [&](int xi, int& tmi, int& n0) {
+        const int t = x * per + xi;
+        const bool valid = xi < per && t < total;
+        constexpr int GM = 8;
+        const int tt = valid ? t : 0;
+        const int group = tt / (GM * p.tiles_n), first = group * GM;
+        const int gm = max(min(GM, row_tiles - first), 1), in_group = tt - group * GM * p.tiles_n;
+        tmi = first + in_group % gm;
+        n0 = (in_group / gm) * TN;
+        return valid;
+    };
+    auto fetch = [&](int xi) {
+        int2 rec = make_int2(0, 0);
+        if constexpr (GROUPED && A_KS) {
+            const int e = x + 8 * (xi / tiles_mn);
+            const uint32_t off = e < p.num_experts ? static_cast<uint32_t>(e) * 4u : kOutside;
+            rec.x = __builtin_amdgcn_raw_buffer_load_b32(rs_offsets, static_cast<int>(off), 0, 0);
+            rec.y = __builtin_amdgcn_raw_buffer_load_b32(rs_counts, static_cast<int>(off), 0, 0);
+        } else if constexpr (GROUPED) {
+            int tmi, n0;
+            const bool valid = place(xi, tmi, n0);
+            const uint32_t off = valid && lane < 5 ? static_cast<uint32_t>(1 + 5 * tmi + lane) * 4u : kOutside;
+            rec.x = __builtin_amdgcn_raw_buffer_load_b32(rs_map, static_cast<int>(off), 0, 0);     // lane l: word l of the row
+        }
+        return rec;
+    };
+    auto decode = [&](int xi, int2 rec) {
+        Tile t{};
+        if constexpr (GROUPED && A_KS) {
+            const int e = x + 8 * (xi / tiles_mn), ti = xi % tiles_mn;
+            t.valid = e < p.num_experts;
+            t.m0 = (ti % p.tiles_m) * TM;
+            t.n0 = (ti / p.tiles_m) * TN;
+            t.m_end = p.M;
+            t.k_begin = __builtin_amdgcn_readfirstlane(rec.x);
+            t.k_end = t.k_begin + __builtin_amdgcn_readfirstlane(rec.y);
+            t.c_base = static_cast<size_t>(t.valid ? e : 0) * p.c_expert_stride;
+        } else {
+            int tmi;
+            t.valid = place(xi, tmi, t.n0);
+            t.m0 = tmi * TM;
+            t.m_end = p.M;
+            t.k_end = p.K;
+            if constexpr (GROUPED) {
+                const int expert = __builtin_amdgcn_readlane(rec.x, 0), first_row = __builtin_amdgcn_readlane(rec.x, 1);
+                const int end_row = __builtin_amdgcn_readlane(rec.x, 2), first_tile = __builtin_amdgcn_readlane(rec.x, 3);
+                t.m0 = first_row + (tmi - first_tile) * TM;
+                t.m_end = min(t.m0 + TM, end_row);
+                t.b_off = static_cast<long long>(expert) * p.b_expert_stride;
+            }
+        }
+        if (!t.valid) {         // a position past the end: every load of it lies beyond its descriptor
+            t.m0 = t.n0 = t.m_end = t.k_begin = t.k_end = 0;
+            t.b_off = 0;
+            t.c_base = 0;
+        }
+        const int nk = (max(t.k_end - t.k_begin, 0) + TK - 1) / TK;
+        t.nk2 = max((nk + 1) & ~1, 2);
+        return t;
+    };
 
     // ---- global -> registers -> LDS: 16-byte chunks through buffer loads ----
     // A buffer load takes a descriptor with a base and a size in bytes and returns zeros for a lane whose offset lies
@@ -171,8 +225,6 @@ void k_gemm_bf16(const BfArgs p) {
     // operand (or, for the K-contiguous form, whose k chunk lies beyond K) starts from an offset beyond every size.
     // The launcher keeps operands below 2 GiB, so the sum does not wrap.  (A descriptor per load costs about ten
     // scalar instructions in front of one MFMA in every eight, more than the MFMA's 16 cycles cover.)
-    constexpr uint32_t kOutside = 0x80000000u;
-    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
     // rows [row0, row_end) of a row-major operand with `ld` elements per row, seen from element `col0` of row row0
     auto rows_rsrc = [](const uint16_t* base, int ld, int row0, int row_end, int col0) {
         const int rows_left = max(row_end - row0, 0);
@@ -185,58 +237,117 @@ void k_gemm_bf16(const BfArgs p) {
         return make_uint4(v.x, v.y, v.z, v.w);
     };
     // [k][columns] operands: this lane's row within a group of eight k rows and its 16-byte column
-    const uint32_t b_lane = n0 + (tid & 31) * 8 < p.N ? (tid >> 5) * static_cast<uint32_t>(p.ldb) * 2u + (tid & 31) * 16u : kOutside;
-    const uint32_t a_lane_ks = m0 + (tid & 31) * 8 < p.M ? (tid >> 5) * static_cast<uint32_t>(p.lda) * 2u + (tid & 31) * 16u : kOutside;
+    const uint32_t b_lane_ks = (tid >> 5) * static_cast<uint32_t>(p.ldb) * 2u + (tid & 31) * 16u;
+    const uint32_t a_lane_ks = (tid >> 5) * static_cast<uint32_t>(p.lda) * 2u + (tid & 31) * 16u;
     // [m][k] operand: this lane's row within a group of 32 rows and its 16-byte k chunk
     const uint32_t a_lane_kc = (tid >> 3) * static_cast<uint32_t>(p.lda) * 2u + (tid & 7) * 16u;
     const uint32_t b_lane_kc = (tid >> 3) * static_cast<uint32_t>(p.ldb) * 2u + (tid & 7) * 16u;
     // GATHER: one descriptor over all of A; a lane's offset per chunk is its gathered row (beyond every size for rows
-    // past the tile's end), the position along k travels in the scalar offset
-    uint32_t a_gather[GATHER ? 8 : 1];
+    // past the tile's end), the position along k travels in the scalar offset.  The row index is itself read through
+    // a descriptor, one tile before the rows are.
     static_assert(!(GATHER && A_KS), "the row gather belongs to the [M][K] form");
     const __amdgpu_buffer_rsrc_t a_all = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t*>(p.A), 0, static_cast<int>(static_cast<uint32_t>(GATHER ? p.a_rows : 0) * static_cast<uint32_t>(p.lda) * 2u), 0x00020000);
-    if constexpr (GATHER) {
+    [[maybe_unused]] const __amdgpu_buffer_rsrc_t rs_index = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<int*>(GATHER ? p.a_row_index : nullptr), 0, GATHER ? p.M * 4 : 0, 0x00020000);
+    constexpr int NG = GATHER ? 8 : 1;
+    auto gather_rows = [&](const Tile& t, int (&rows)[NG]) {       // the index values, as loaded
+        if constexpr (GATHER) {
 #pragma unroll
-        for (int c = 0; c < 8; ++c) {
-            const int r = m0 + 32 * c + (tid >> 3);
-            a_gather[c] = r < m_end ? static_cast<uint32_t>(p.a_row_index[r]) * static_cast<uint32_t>(p.lda) * 2u + (tid & 7) * 16u : kOutside;
+            for (int c = 0; c < 8; ++c) {
+                const int r = t.m0 + 32 * c + (tid >> 3);
+                rows[c] = __builtin_amdgcn_raw_buffer_load_b32(rs_index, static_cast<int>(r < t.m_end ? static_cast<uint32_t>(r) * 4u : kOutside), 0, 0);
+            }
         }
-    }
-    // NT with a period: where tile ks of the k range starts in B's columns
+    };
+    auto gather_offsets = [&](const Tile& t, const int (&rows)[NG], uint32_t (&offs)[NG]) {
+        if constexpr (GATHER) {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                const int r = t.m0 + 32 * c + (tid >> 3);
+                offs[c] = r < t.m_end ? static_cast<uint32_t>(rows[c]) * static_cast<uint32_t>(p.lda) * 2u + (tid & 7) * 16u : kOutside;
+            }
+        }
+    };
+
+    // ---- the fetch cursor: K-tile lks of tile L, two K-tiles ahead of the MFMAs ----
+    // L_after is the tile after L (decoded a tile ahead, so that its gathered row numbers can be on their way), rec_next
+    // the record of the tile after that; L_before is the tile L came from: when the MFMAs finish a tile, the fetch is in
+    // the next one or, if that has two K-tiles only, already in the one after it (tiles_ahead says which).
     const int b_period = B_KC && p.b_k_period ? p.b_k_period : 0x7fffffff;
-    int kb_load = 0;              // ... for the tile the next load_one calls fetch (set by the callers)
-    // chunk c (0 .. NA-1: M side, NA .. NA+NB-1: N side) of K-tile ks into its staging register
+    int xi_next = blockIdx.x / 8;
+    Tile L = decode(xi_next, fetch(xi_next));
+    if (!L.valid) return;
+    xi_next += xi_step;
+    Tile L_after = decode(xi_next, fetch(xi_next));
+    xi_next += xi_step;
+    int2 rec_next = fetch(xi_next);
+    Tile L_before = L;
+    int tiles_ahead = 0;
+    int lks = 0;
+    int kb_load = 0;              // NT with a period: where K-tile lks starts in B's columns
+    uint32_t a_gather[NG];
+    int rows_after[NG];
+    {
+        int rows_now[NG];
+        gather_rows(L, rows_now);
+        gather_offsets(L, rows_now, a_gather);
+        gather_rows(L_after, rows_after);
+    }
+    // to the next K-tile, after the 16 loads of one.  Tiles have an even number of K-tiles and the cursor starts on an
+    // even one, so only the step off an odd K-tile (END_OF_PAIR) can leave the tile: the other needs no branch.
+    auto advance = [&](auto end_of_pair) {
+        ++lks;
+        if constexpr (B_KC) {
+            kb_load += TK;
+            if (kb_load >= b_period) kb_load -= b_period;
+        }
+        if constexpr (!decltype(end_of_pair)::value) return;
+        if (lks == L.nk2) {
+            L_before = L;
+            L = L_after;
+            gather_offsets(L, rows_after, a_gather);
+            L_after = decode(xi_next, rec_next);
+            xi_next += xi_step;
+            rec_next = fetch(xi_next);
+            gather_rows(L_after, rows_after);
+            ++tiles_ahead;
+            lks = 0;
+            kb_load = 0;
+        }
+    };
     // One descriptor per operand and K-tile, built by the tile's first load of that operand; the chunks of the tile
     // differ in the lane offset only (one vector add each).
     __amdgpu_buffer_rsrc_t rs_a = a_all, rs_b = a_all;
     uint32_t off_a = kOutside, off_b = kOutside;
     const uint32_t a_step = (A_KS ? 8u : 32u) * static_cast<uint32_t>(p.lda) * 2u;
     const uint32_t b_step = (B_KC ? 32u : 8u) * static_cast<uint32_t>(p.ldb) * 2u;
-    auto load_one = [&](int ks, auto cc, uint4 (&ra)[NA], uint4 (&rb)[NB]) {
+    // chunk c (0 .. NA-1: M side, NA .. NA+NB-1: N side) of the cursor's K-tile into its staging register
+    auto load_one = [&](auto cc, uint4 (&ra)[NA], uint4 (&rb)[NB]) {
         constexpr int c = decltype(cc)::value;
-        const int k0 = k_begin + ks * TK;
+        const int k0 = L.k_begin + lks * TK;
         if constexpr (c == 0 && !GATHER) {
             if constexpr (A_KS) {
-                rs_a = rows_rsrc(p.A, p.lda, k0, k_end, m0);
-                off_a = a_lane_ks;
+                rs_a = rows_rsrc(p.A, p.lda, k0, L.k_end, L.m0);
+                off_a = L.m0 + (tid & 31) * 8 < p.M ? a_lane_ks : kOutside;
             } else {
-                rs_a = rows_rsrc(p.A, p.lda, m0, m_end, k0);
-                off_a = k0 + (tid & 7) * 8 < k_end ? a_lane_kc : kOutside;
+                rs_a = rows_rsrc(p.A, p.lda, L.m0, L.m_end, k0);
+                off_a = k0 + (tid & 7) * 8 < L.k_end ? a_lane_kc : kOutside;
             }
         }
         if constexpr (c == NA) {
+            const uint16_t* B = p.B + L.b_off;
             if constexpr (B_KC) {
-                rs_b = rows_rsrc(B, p.ldb, n0, p.N, kb_load);
-                off_b = k0 + (tid & 7) * 8 < k_end ? b_lane_kc : kOutside;
+                rs_b = rows_rsrc(B, p.ldb, L.n0, p.N, kb_load);
+                off_b = k0 + (tid & 7) * 8 < L.k_end ? b_lane_kc : kOutside;
             } else {
-                rs_b = rows_rsrc(B, p.ldb, k0, k_end, n0);
-                off_b = b_lane;
+                rs_b = rows_rsrc(B, p.ldb, k0, L.k_end, L.n0);
+                off_b = L.n0 + (tid & 31) * 8 < p.N ? b_lane_ks : kOutside;
             }
         }
         if constexpr (c < NA) {
             if constexpr (GATHER) {
-                const uint32_t off = k0 + (tid & 7) * 8 < k_end ? a_gather[c] : kOutside;
+                const uint32_t off = k0 + (tid & 7) * 8 < L.k_end ? a_gather[c] : kOutside;
                 const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(a_all, static_cast<int>(off), k0 * 2, 0);
                 ra[c] = make_uint4(v.x, v.y, v.z, v.w);
             } else {
@@ -267,12 +378,15 @@ void k_gemm_bf16(const BfArgs p) {
 
     // ---- LDS -> MFMA ----
     v4f acc[8][8];      // [n block][m block]
+    auto clear_acc = [&] {
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
+        for (int j = 0; j < 8; ++j)
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
+            for (int i = 0; i < 8; ++i)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) acc[j][i][r] = 0.0f;
+                for (int r = 0; r < 4; ++r) acc[j][i][r] = 0.0f;
+    };
+    clear_acc();
 
     const int r16 = lane & 15, kg = lane >> 4;
     const int ks_n = ks_lane_offset(kPitchN, lane) + wn * 128 * 2, ks_m = ks_lane_offset(kPitchM, lane) + wm * 128 * 2;
@@ -306,15 +420,40 @@ void k_gemm_bf16(const BfArgs p) {
     };
     constexpr int RN = 4, RM = 4;       // read_set calls per set
 
+    // The forms that add to C read it in the epilogue, with idle matrix cores: a round trip to HBM per pass.  Under the
+    // tile's last pair of K-tiles every 128-byte line of the wavefront's 128 x 128 block of C is therefore touched once
+    // (one dword per lane, distinct lines), so that the epilogue's reads find it in the L2 / the memory-side cache.
+    // The touches are issued in every pair, from offsets beyond the descriptor in all but the last.
+    constexpr bool ACCUM = OUT == OUT_ACCUM_BF16 || OUT == OUT_ACCUM_F32;
+    constexpr int CE = OUT == OUT_ACCUM_F32 || OUT == OUT_STORE_F32 ? 4 : 2;        // bytes per element of C
+    constexpr int NTOUCH = ACCUM ? 2 * CE : 1;              // 128 rows x CE lines / 64 lanes
+    [[maybe_unused]] int touched[NTOUCH] = {};
+    [[maybe_unused]] __amdgpu_buffer_rsrc_t rs_c = a_all;
+    [[maybe_unused]] bool touch_ok = false;
+    [[maybe_unused]] const uint32_t touch_lane = (lane / CE) * static_cast<uint32_t>(p.ldc) * CE + (lane % CE) * 128u;
+    [[maybe_unused]] const uint32_t touch_step = (64 / CE) * static_cast<uint32_t>(p.ldc) * CE;
+    [[maybe_unused]] auto touch_one = [&](auto tc) {
+        constexpr int t = decltype(tc)::value;
+        touched[t] = __builtin_amdgcn_raw_buffer_load_b32(rs_c, static_cast<int>(touch_ok ? touch_lane + t * touch_step : kOutside), 0, 0);
+    };
+    // the wavefront's block of the output tile `t`, rows beyond the tile's end cut off
+    [[maybe_unused]] auto c_block_rsrc = [&](const Tile& t) {
+        const int row_w = t.m0 + wm * 128;
+        const int rows = min(max(t.m_end - row_w, 0), 128);
+        return __builtin_amdgcn_make_buffer_rsrc(
+            static_cast<uint8_t*>(p.C) + (t.c_base + static_cast<size_t>(row_w) * p.ldc + t.n0 + wn * 128) * CE, 0,
+            static_cast<int>(static_cast<uint32_t>(rows) * static_cast<uint32_t>(p.ldc) * CE), 0x00020000);
+    };
+
     // One K-tile: two k-steps of four phases, 128 MFMAs per wavefront, with everything else woven between them (one
     // wavefront per SIMD: whatever waits, the matrix cores wait with it).  While tile ks is multiplied from `stage`:
     //   - a phase refills the set the phase before it left behind (see the top of the file);
-    //   - the 16 loads of tile ks + 2 go out one every eighth MFMA, into the register set tile ks just left;
+    //   - the 16 loads of tile ks + 2 (the fetch cursor's) go out one every eighth MFMA, into the register set tile ks just left;
     //   - tile ks + 1 (requested one tile ago) is parked in the other stage one chunk every sixth MFMA, done by MFMA 92;
     //   - the barrier follows MFMA 95, and the first sets of tile ks + 1 are read under the last 32 MFMAs.
     // A tile past the end of the k range is fetched as zeros (it lies beyond the descriptors) and adds nothing, so the
-    // loop needs no tail.
-    auto ktile = [&](auto stage_c, int ks, uint4 (&ra_new)[NA], uint4 (&rb_new)[NB], const uint4 (&ra_next)[NA], const uint4 (&rb_next)[NB]) {
+    // loop needs no tail; past the last K-tile of an output tile, "tile ks + 1" is the first of the next output tile.
+    auto ktile = [&](auto stage_c, uint4 (&ra_new)[NA], uint4 (&rb_new)[NB], const uint4 (&ra_next)[NA], const uint4 (&rb_next)[NB]) {
         constexpr int stage = decltype(stage_c)::value;
         static_for<0, 128>([&](auto mc) {
             constexpr int m = decltype(mc)::value, S = m / 64, ph = (m % 64) / 16, q = m % 16;
@@ -335,69 +474,183 @@ void k_gemm_bf16(const BfArgs p) {
             } else {
                 if constexpr (q < 2 * RM && q % 2 == 0) read_set(S == 0 ? stage : stage ^ 1, std::integral_constant<int, 1 - S>{}, std::integral_constant<int, 2 + (1 - S)>{}, std::integral_constant<int, (q / 2) % RM>{});
             }
-            if constexpr (m % 8 == 7) load_one(ks + 2, std::integral_constant<int, m / 8>{}, ra_new, rb_new);
+            if constexpr (m % 8 == 7) load_one(std::integral_constant<int, m / 8>{}, ra_new, rb_new);
+            if constexpr (ACCUM && stage == 0 && m % 8 == 1 && m / 8 < NTOUCH) touch_one(std::integral_constant<int, m / 8>{});
             if constexpr (m < 96 && m % 6 == 2) park_one(stage ^ 1, std::integral_constant<int, (m / 6) % 16>{}, ra_next, rb_next);
             if constexpr (m == 95) __syncthreads();
             __builtin_amdgcn_sched_barrier(0);
         });
-        if constexpr (B_KC) {          // the next K-tile's loads are one tile further
-            kb_load += TK;
-            if (kb_load >= b_period) kb_load -= b_period;
-        }
+        advance(std::integral_constant<bool, stage == 1>{});
     };
 
     static_assert(NA + NB == 16, "the weave above places 16 loads and 16 LDS stores per K-tile");
     uint4 ra0[NA], rb0[NB], ra1[NA], rb1[NB];
-    static_for<0, 16>([&](auto c) { load_one(0, c, ra0, rb0); });
-    if constexpr (B_KC) kb_load = TK % b_period;
-    static_for<0, 16>([&](auto c) { load_one(1, c, ra1, rb1); });
-    if constexpr (B_KC) kb_load = (2 * TK) % b_period;
+    Tile cur = L;
+    static_for<0, 16>([&](auto c) { load_one(c, ra0, rb0); });
+    advance(std::false_type{});
+    static_for<0, 16>([&](auto c) { load_one(c, ra1, rb1); });
+    advance(std::true_type{});
     static_for<0, 16>([&](auto c) { park_one(0, c, ra0, rb0); });
     __syncthreads();
     // the first k-step (parity 0) starts with (N0, M0)
     static_for<0, RN>([&](auto r) { read_set(0, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, r); });
     static_for<0, RM>([&](auto r) { read_set(0, std::integral_constant<int, 0>{}, std::integral_constant<int, 2>{}, r); });
-    for (int ks = 0; ks < nk; ks += 2) {
-        ktile(std::integral_constant<int, 0>{}, ks, ra0, rb0, ra1, rb1);
-        ktile(std::integral_constant<int, 1>{}, ks + 1, ra1, rb1, ra0, rb0);
-    }
-
-    // the MFMAs above are opaque to the compiler's hazard handling: leave the wait states between the last of them and
-    // the first read of an accumulator explicitly
-    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
-    // ---- epilogue: accumulator register q of block (j, i) is output row m0 + wm*128 + 16 i + lane % 16,
-    //      column n0 + wn*128 + 16 j + 4 (lane / 16) + q ----
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int m = m0 + wm * 128 + 16 * i + r16;
-        if (m >= m_end) continue;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const int n = n0 + wn * 128 + 16 * j + 4 * kg;
-            if (n >= p.N) continue;                      // N % 8 == 0: a quad is inside or outside as a whole
-            const size_t at = c_base + static_cast<size_t>(m) * p.ldc + n;
-            float v[4] = {acc_read(acc[j][i][0]), acc_read(acc[j][i][1]), acc_read(acc[j][i][2]), acc_read(acc[j][i][3])};
-            if constexpr (OUT == OUT_STORE_F32) {
-                *reinterpret_cast<float4*>(static_cast<float*>(p.C) + at) = make_float4(v[0], v[1], v[2], v[3]);
-            } else if constexpr (OUT == OUT_ACCUM_F32) {
-                float4* dst = reinterpret_cast<float4*>(static_cast<float*>(p.C) + at);
-                float4 c = *dst;
-                c.x += v[0]; c.y += v[1]; c.z += v[2]; c.w += v[3];
-                *dst = c;
-            } else {
-                uint2* dst = reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.C) + at);
-                if constexpr (OUT == OUT_ACCUM_BF16) {
-                    // fp32 sum of the old value and the product, one rounding (cublasGemmEx with a bf16 C, beta = 1)
-                    const uint2 c = *dst;
-                    v[0] += bf16_lo(c.x); v[1] += bf16_hi(c.x); v[2] += bf16_lo(c.y); v[3] += bf16_hi(c.y);
-                }
-                *dst = make_uint2(pack_bf16x2_hw(v[0], v[1]), pack_bf16x2_hw(v[2], v[3]));
-            }
-            // one quad's loads and stores at a time: pulling the whole tile's reads of C to the front would need
-            // more registers than the main loop leaves
-            if constexpr (OUT == OUT_ACCUM_BF16 || OUT == OUT_ACCUM_F32) __builtin_amdgcn_sched_barrier(0);
+    while (true) {
+        if constexpr (ACCUM) rs_c = c_block_rsrc(cur);
+        for (int ks = 0; ks < cur.nk2; ks += 2) {
+            if constexpr (ACCUM) touch_ok = ks + 2 >= cur.nk2 && cur.n0 + wn * 128 + (lane % CE) * (128 / CE) < p.N;
+            ktile(std::integral_constant<int, 0>{}, ra0, rb0, ra1, rb1);
+            ktile(std::integral_constant<int, 1>{}, ra1, rb1, ra0, rb0);
         }
+        // the MFMAs above are opaque to the compiler's hazard handling: leave the wait states between the last of them
+        // and the first read of an accumulator explicitly
+        asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+        // ---- epilogue: accumulator register q of block (j, i) is output row m0 + wm*128 + 16 i + lane % 16,
+        //      column n0 + wn*128 + 16 j + 4 (lane / 16) + q.  Written from there a store instruction would cover sixteen
+        //      rows with 32 bytes each; instead the wavefront turns its 128 x 128 outputs round in LDS, 64 rows (bf16) or
+        //      32 rows (fp32) at a time, and stores (or adds to) whole 256-byte / 512-byte row pieces.  The staging area
+        //      is the wavefront's quarter of LDS stage 1: every output tile ends on that stage, nobody reads it after
+        //      the last K-tile's barrier, and nobody parks into it before the barrier below.
+        //      An empty k range adds nothing (and must not turn a -0 of C into +0). ----
+        const bool nothing_to_add = (OUT == OUT_ACCUM_BF16 || OUT == OUT_ACCUM_F32) && cur.k_end <= cur.k_begin;
+        if constexpr (ACCUM) {
+#pragma unroll
+            for (int t = 0; t < NTOUCH; ++t) asm volatile("" : : "v"(touched[t]));     // the touches end here
+        }
+        if (!nothing_to_add) {
+            // C is reached through a descriptor over the wavefront's block (rows beyond the tile's end lie beyond its size;
+            // a lane whose columns lie beyond N uses an offset beyond every size): loads return zeros there and stores
+            // are dropped, so the epilogue has no branches and its loads can be issued ahead of the staging.
+            uint8_t* stg = smem + kStage + wave * (kStage / 4);
+            if constexpr (!ACCUM) rs_c = c_block_rsrc(cur);
+            const int col_w = cur.n0 + wn * 128;
+            if constexpr (OUT == OUT_STORE_BF16 || OUT == OUT_ACCUM_BF16) {
+                // a lane's piece: eight columns (16 bytes of C) of row lane / 16 of every group of four rows
+                const uint32_t c_lane = col_w + 8 * (lane & 15) < p.N ? (lane >> 4) * static_cast<uint32_t>(p.ldc) * 2u + (lane & 15) * 16u : kOutside;
+                const uint32_t c_rows4 = 4u * static_cast<uint32_t>(p.ldc) * 2u;
+                if constexpr (OUT == OUT_STORE_BF16) {
+                    constexpr int PB = 128 * 2 + 32;                    // staged row: 128 bf16 + pad
+                    static_assert(64 * PB <= kStage / 4, "two passes of 64 rows");
+#pragma unroll
+                    for (int half = 0; half < 2; ++half) {
+#pragma unroll
+                        for (int ii = 0; ii < 4; ++ii)
+#pragma unroll
+                            for (int j = 0; j < 8; ++j) {
+                                const v4f a = acc[j][4 * half + ii];
+                                *reinterpret_cast<uint2*>(stg + (16 * ii + r16) * PB + (16 * j + 4 * kg) * 2) =
+                                    make_uint2(pack_bf16x2_hw(acc_read(a[0]), acc_read(a[1])), pack_bf16x2_hw(acc_read(a[2]), acc_read(a[3])));
+                            }
+#pragma unroll
+                        for (int t = 0; t < 16; ++t) {
+                            const u32x4 v = *reinterpret_cast<const u32x4*>(stg + ((lane >> 4) + 4 * t) * PB + (lane & 15) * 16);
+                            __builtin_amdgcn_raw_buffer_store_b128(v, rs_c, static_cast<int>(c_lane + (16 * half + t) * c_rows4), 0, 0);
+                        }
+                    }
+                } else {
+                    // fp32 sum of the old value and the product, one rounding (cublasGemmEx with a bf16 C, beta = 1)
+                    constexpr int PF = 128 * 4 + 32;                    // staged row: 128 fp32 + pad
+                    static_assert(32 * PF <= kStage / 4, "four passes of 32 rows");
+                    // the next pass's rows of C are requested before this pass's are added to and stored
+                    u32x4 c[8], c_ahead[8];
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) c_ahead[t] = __builtin_amdgcn_raw_buffer_load_b128(rs_c, static_cast<int>(c_lane + t * c_rows4), 0, 0);
+#pragma unroll
+                    for (int pass = 0; pass < 4; ++pass) {
+#pragma unroll
+                        for (int t = 0; t < 8; ++t) c[t] = c_ahead[t];
+                        if (pass < 3) {
+#pragma unroll
+                            for (int t = 0; t < 8; ++t) c_ahead[t] = __builtin_amdgcn_raw_buffer_load_b128(rs_c, static_cast<int>(c_lane + (8 * (pass + 1) + t) * c_rows4), 0, 0);
+                        }
+#pragma unroll
+                        for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+                            for (int j = 0; j < 8; ++j) {
+                                const v4f a = acc[j][2 * pass + ii];
+                                *reinterpret_cast<float4*>(stg + (16 * ii + r16) * PF + (16 * j + 4 * kg) * 4) =
+                                    make_float4(acc_read(a[0]), acc_read(a[1]), acc_read(a[2]), acc_read(a[3]));
+                            }
+#pragma unroll
+                        for (int t = 0; t < 8; ++t) {
+                            const uint8_t* src = stg + ((lane >> 4) + 4 * t) * PF + (lane & 15) * 32;
+                            const float4 lo = *reinterpret_cast<const float4*>(src), hi = *reinterpret_cast<const float4*>(src + 16);
+                            u32x4 v;
+                            v.x = pack_bf16x2_hw(lo.x + bf16_lo(c[t].x), lo.y + bf16_hi(c[t].x));
+                            v.y = pack_bf16x2_hw(lo.z + bf16_lo(c[t].y), lo.w + bf16_hi(c[t].y));
+                            v.z = pack_bf16x2_hw(hi.x + bf16_lo(c[t].z), hi.y + bf16_hi(c[t].z));
+                            v.w = pack_bf16x2_hw(hi.z + bf16_lo(c[t].w), hi.w + bf16_hi(c[t].w));
+                            __builtin_amdgcn_raw_buffer_store_b128(v, rs_c, static_cast<int>(c_lane + (8 * pass + t) * c_rows4), 0, 0);
+                        }
+                    }
+                }
+            } else {
+                // fp32 C.  A lane's piece: four columns (16 bytes) of row lane / 32 of every pair of rows
+                constexpr int PF = 128 * 4 + 32;
+                static_assert(32 * PF <= kStage / 4, "four passes of 32 rows");
+                const uint32_t c_lane = col_w + 4 * (lane & 31) < p.N ? (lane >> 5) * static_cast<uint32_t>(p.ldc) * 4u + (lane & 31) * 16u : kOutside;
+                const uint32_t c_rows2 = 2u * static_cast<uint32_t>(p.ldc) * 4u;
+                // ACCUM: C is read in groups of eight row pairs, a group ahead of the adds and stores
+                [[maybe_unused]] u32x4 c[8], c_ahead[8];
+                if constexpr (OUT == OUT_ACCUM_F32) {
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) c_ahead[t] = __builtin_amdgcn_raw_buffer_load_b128(rs_c, static_cast<int>(c_lane + t * c_rows2), 0, 0);
+                }
+#pragma unroll
+                for (int pass = 0; pass < 4; ++pass) {
+#pragma unroll
+                    for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            const v4f a = acc[j][2 * pass + ii];
+                            *reinterpret_cast<float4*>(stg + (16 * ii + r16) * PF + (16 * j + 4 * kg) * 4) =
+                                make_float4(acc_read(a[0]), acc_read(a[1]), acc_read(a[2]), acc_read(a[3]));
+                        }
+#pragma unroll
+                    for (int hg = 0; hg < 2; ++hg) {
+                        if constexpr (OUT == OUT_ACCUM_F32) {
+#pragma unroll
+                            for (int t = 0; t < 8; ++t) c[t] = c_ahead[t];
+                            if (2 * pass + hg < 7) {
+#pragma unroll
+                                for (int t = 0; t < 8; ++t)
+                                    c_ahead[t] = __builtin_amdgcn_raw_buffer_load_b128(rs_c, static_cast<int>(c_lane + (8 * (2 * pass + hg + 1) + t) * c_rows2), 0, 0);
+                            }
+                        }
+#pragma unroll
+                        for (int t = 0; t < 8; ++t) {
+                            const int tt = 8 * hg + t;
+                            float4 v = *reinterpret_cast<const float4*>(stg + ((lane >> 5) + 2 * tt) * PF + (lane & 31) * 16);
+                            if constexpr (OUT == OUT_ACCUM_F32) {
+                                v.x += __uint_as_float(c[t].x); v.y += __uint_as_float(c[t].y); v.z += __uint_as_float(c[t].z); v.w += __uint_as_float(c[t].w);
+                            }
+                            u32x4 o;
+                            o.x = __float_as_uint(v.x); o.y = __float_as_uint(v.y); o.z = __float_as_uint(v.z); o.w = __float_as_uint(v.w);
+                            __builtin_amdgcn_raw_buffer_store_b128(o, rs_c, static_cast<int>(c_lane + (16 * pass + tt) * c_rows2), 0, 0);
+                        }
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        // the next tile: the one the fetch is in, or the one it has just left
+        cur = tiles_ahead == 1 ? L : L_before;
+        --tiles_ahead;
+        if (!cur.valid) break;
+        clear_acc();
     }
+}
+
+// one workgroup per CU, a multiple of 8 of them (launch position % 8 is the XCD), and no more than there are tiles
+dim3 persistent_grid(long long tiles) {
+    static const int cus = [] {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) != hipSuccess) return 256;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v < 8) return 256;
+        return v - v % 8;
+    }();
+    const long long want = 8 * ((tiles + 7) / 8);
+    return dim3(static_cast<unsigned>(want < cus ? want : cus));
 }
 
 template <bool A_KS, int OUT, bool GROUPED, bool B_KC = false, bool GATHER = false>
@@ -414,7 +667,8 @@ int launch(const BfArgs& p, dim3 grid, hipStream_t st) {
 }
 
 bool operands_ok(const void* A, int lda, const void* B, int ldb, const void* C, int ldc, int c_elem_bytes) {
-    return aligned16(A) && aligned16(B) && lda % 8 == 0 && ldb % 8 == 0 && ldc % 4 == 0 &&
+    // (the epilogue addresses a wavefront's 128 rows of C by 32-bit byte offsets from the block's first element)
+    return aligned16(A) && aligned16(B) && lda % 8 == 0 && ldb % 8 == 0 && ldc % 4 == 0 && ldc < (1 << 21) &&
            (reinterpret_cast<uintptr_t>(C) & (4u * c_elem_bytes - 1u)) == 0;
 }
 
@@ -433,10 +687,7 @@ int gemm_nn(int M, int N, int K, int E, const int* counts, const int* offsets, c
     p.M = M; p.N = N; p.K = K;
     p.tiles_n = (N + TN - 1) / TN;
     int tiles_m = (M + TM - 1) / TM;
-    auto grid_for = [&](int row_tiles) {      // 8 XCDs x the per-XCD share of the tiles, rounded up
-        const long long total = static_cast<long long>(row_tiles) * p.tiles_n;
-        return dim3(static_cast<unsigned>(8 * ((total + 7) / 8)));
-    };
+    auto grid_for = [&](int row_tiles) { return persistent_grid(static_cast<long long>(row_tiles) * p.tiles_n); };
     if (grouped) {
         size_t need = 0;
         cf_fp8_grouped_gemm_workspace_bytes(M, E, &need);
@@ -476,9 +727,9 @@ int gemm_tn(int M, int N, int K, int E, const int* counts, const int* offsets, c
         p.c_expert_stride = static_cast<long long>(M) * ldc;
         const long long blocks = 8LL * ((E + 7) / 8) * tiles;
         if (blocks >= (1LL << 31)) return CF_ERR_UNSUPPORTED;
-        return launch<true, OUT, true>(p, dim3(static_cast<unsigned>(blocks)), st);
+        return launch<true, OUT, true>(p, persistent_grid(blocks), st);
     }
-    return launch<true, OUT, false>(p, dim3(static_cast<unsigned>(8 * ((tiles + 7) / 8))), st);
+    return launch<true, OUT, false>(p, persistent_grid(tiles), st);
 }
 
 }  // namespace
@@ -507,7 +758,7 @@ int grouped_gemm_bf16_nt(int total_rows, int N, int Kb, int terms, int num_exper
     p.a_row_index = d_a_row_index;
     p.a_rows = a_rows;
     const long long total = static_cast<long long>(p.tiles_m) * p.tiles_n;
-    const dim3 grid(static_cast<unsigned>(8 * ((total + 7) / 8)));
+    const dim3 grid = persistent_grid(total);
     hipStream_t st = as_stream(stream);
     if (d_a_row_index) {
         if (!c_is_f32) return CF_ERR_UNSUPPORTED;      // the one caller stores fp32

@@ -84,6 +84,63 @@ def test_gemm_bf16_exact_integers_equal_numpy(cf, dev):
     assert not np.array_equal(want[:136, :136], want[:136, :136].T)
 
 
+@pytest.mark.parametrize("K", [64, 72, 200])
+def test_gemm_bf16_more_tiles_than_workgroups_exact(cf, dev, K):
+    """306 output tiles on at most 256 persistent workgroups: a workgroup walks from one tile into the next with its
+    operand fetch two K-tiles ahead (at K = 64 and 72 a tile has one or two real K-tiles, so the fetch is two tiles
+    ahead of the MFMAs).  Small integers, exact in fp32: all three forms must match numpy to the bit."""
+    case(f"bf16 GEMMs, 306 tiles, K={K}")
+    rng = np.random.default_rng(K)
+    M, N = 17 * 256, 17 * 256 + 8
+    a = rng.integers(-4, 5, (M, K)).astype(np.float32)
+    b = rng.integers(-3, 4, (K, N)).astype(np.float32)
+    C = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=dev)
+    cf.cf_gemm_bf16_nn(M, N, K, dev_bf16(orc.bf16_from_f32(a), dev), K, dev_bf16(orc.bf16_from_f32(b), dev), N, C, N, stream())
+    torch.cuda.synchronize()
+    assert np.array_equal(bf16_bits(C), orc.bf16_from_f32(a @ b))
+    # tn: the same product from the transposed left operand, added to C
+    at = np.ascontiguousarray(a.T)
+    c0 = rng.integers(-50, 51, (M, N)).astype(np.float32)
+    Cf = torch.from_numpy(c0).to(dev)
+    cf.cf_gemm_bf16_tn_accum_f32(M, N, K, dev_bf16(orc.bf16_from_f32(at), dev), M, dev_bf16(orc.bf16_from_f32(b), dev), N, Cf, N, stream())
+    Cb = dev_bf16(orc.bf16_from_f32(c0), dev)
+    cf.cf_gemm_bf16_tn_accum_bf16(M, N, K, dev_bf16(orc.bf16_from_f32(at), dev), M, dev_bf16(orc.bf16_from_f32(b), dev), N, Cb, N, stream())
+    torch.cuda.synchronize()
+    want = c0 + a @ b
+    assert np.array_equal(host(Cf), want)
+    assert np.array_equal(bf16_bits(Cb), orc.bf16_from_f32(want))
+
+
+def test_grouped_bf16_weight_gradient_leaves_empty_experts_alone(cf, dev):
+    """An expert without rows adds nothing: its block of C keeps its bits, negative zeros included (a sum with an
+    all-zero product would turn them into +0), also when such experts sit between experts of a few rows each."""
+    case("grouped bf16 wgrad, empty experts between short ones")
+    rng = np.random.default_rng(11)
+    E, H, Ie = 19, 520, 1032                           # 15 tiles per expert, 360 tile positions on 256 workgroups
+    counts = np.array([0, 3, 0, 0, 70, 1, 0, 130, 0, 64, 0, 0, 0, 5, 0, 65, 0, 0, 0], np.int32)
+    offsets = orc.moe_expert_offsets(counts)
+    total = int(counts.sum()) + 7                      # the compact buffers may hold more rows than the lists fill
+    d_out, act = rand_bf16(rng, (total, H), 1e-2), rand_bf16(rng, (total, Ie))
+    g0 = np.full((E, H, Ie), 0x8000, np.uint16)        # -0.0 everywhere
+    g_bf = dev_bf16(g0, dev)
+    g_f32 = torch.from_numpy(orc.bf16_to_f32(g0)).to(dev)
+    dc, do = dev_arr(counts, dev), dev_arr(offsets, dev)
+    cf.cf_moe_grouped_gemm_bf16_tn_accum_bf16(H, Ie, total, E, dc, do, dev_bf16(d_out, dev), H, dev_bf16(act, dev), Ie, g_bf, stream())
+    cf.cf_moe_grouped_gemm_bf16_tn_accum_f32(H, Ie, total, E, dc, do, dev_bf16(d_out, dev), H, dev_bf16(act, dev), Ie, g_f32, stream())
+    torch.cuda.synchronize()
+    got_g, got_gf = bf16_bits(g_bf), host(g_f32)
+    for e in range(E):
+        n, o = int(counts[e]), int(offsets[e])
+        if n == 0:
+            assert np.array_equal(got_g[e], g0[e]), f"expert {e}"
+            assert np.array_equal(got_gf[e].view(np.uint32), np.full((H, Ie), 0x80000000, np.uint32)), f"expert {e}"
+            continue
+        ref = orc.gemm_bf16_tn_ref(d_out[o:o + n], act[o:o + n])
+        ad = absdot(d_out[o:o + n], act[o:o + n], tn=True)
+        check_bf16_out(got_g[e], ref, ad, f"g_out expert {e}")
+        assert np.all(np.abs(got_gf[e] - ref) <= ACC * ad + 2.0 ** -22 * np.abs(ref))
+
+
 @pytest.mark.parametrize("M,N,K", [(256, 128, 64), (264, 200, 131), (8, 8, 1), (1408, 512, 777), (520, 136, 2000)])
 def test_gemm_bf16_tn_accumulate(cf, dev, M, N, K):
     case(f"bf16 tn {M}x{N}x{K}")

@@ -449,7 +449,7 @@ void k_gemm_bf16(const BfArgs p) {
     // wavefront per SIMD: whatever waits, the matrix cores wait with it).  While tile ks is multiplied from `stage`:
     //   - a phase refills the set the phase before it left behind (see the top of the file);
     //   - the 16 loads of tile ks + 2 (the fetch cursor's) go out one every eighth MFMA, into the register set tile ks just left;
-    //   - tile ks + 1 (requested one tile ago) is parked in the other stage one chunk every sixth MFMA, done by MFMA 92;
+    //   - tile ks + 1 (requested one tile ago) is parked in the other stage three chunks per phase, done by MFMA 83;
     //   - the barrier follows MFMA 95, and the first sets of tile ks + 1 are read under the last 32 MFMAs.
     // A tile past the end of the k range is fetched as zeros (it lies beyond the descriptors) and adds nothing, so the
     // loop needs no tail; past the last K-tile of an output tile, "tile ks + 1" is the first of the next output tile.
@@ -476,7 +476,9 @@ void k_gemm_bf16(const BfArgs p) {
             }
             if constexpr (m % 8 == 7) load_one(std::integral_constant<int, m / 8>{}, ra_new, rb_new);
             if constexpr (ACCUM && stage == 0 && m % 8 == 1 && m / 8 < NTOUCH) touch_one(std::integral_constant<int, m / 8>{});
-            if constexpr (m < 96 && m % 6 == 2) park_one(stage ^ 1, std::integral_constant<int, (m / 6) % 16>{}, ra_next, rb_next);
+            // three LDS stores per sixteen MFMAs, after MFMAs that have neither an operand read nor a load behind them
+            constexpr int park = 3 * (m / 16) + (q == 3 ? 0 : q == 10 ? 1 : 2);
+            if constexpr ((q == 3 || q == 10 || q == 13) && park < 16) park_one(stage ^ 1, std::integral_constant<int, park % 16>{}, ra_next, rb_next);
             if constexpr (m == 95) __syncthreads();
             __builtin_amdgcn_sched_barrier(0);
         });

@@ -187,8 +187,9 @@ void k_gemm_bf16(const BfArgs p) {
             t.m0 = (ti % p.tiles_m) * TM;
             t.n0 = (ti / p.tiles_m) * TN;
             t.m_end = p.M;
-            t.k_begin = __builtin_amdgcn_readfirstlane(rec.x);
-            t.k_end = t.k_begin + __builtin_amdgcn_readfirstlane(rec.y);
+            // an expert's row range is cut at the rows the compact buffers hold (p.K), as the tile table cuts it
+            t.k_begin = min(max(__builtin_amdgcn_readfirstlane(rec.x), 0), p.K);
+            t.k_end = min(t.k_begin + max(__builtin_amdgcn_readfirstlane(rec.y), 0), p.K);
             t.c_base = static_cast<size_t>(t.valid ? e : 0) * p.c_expert_stride;
         } else {
             int tmi;

@@ -423,7 +423,8 @@ int cf_moe_grouped_gemm_bf16_nn(int total_rows, int N, int K, int num_experts, c
                                 uint16_t* d_C, int ldc, void* d_workspace, size_t workspace_bytes,
                                 cf_stream_t stream);
 /* For each expert e: C[e] += A[rows of e, :M]^T . B[rows of e, :N]  with C [num_experts, M, N]
- * (the two weight-gradient calls, src/trainer.cu:7727, 7736); an expert without rows leaves its C alone. */
+ * (the two weight-gradient calls, src/trainer.cu:7727, 7736); an expert without rows leaves its C alone.
+ * total_rows is the number of rows A and B hold: an expert's row range is cut there. */
 int cf_moe_grouped_gemm_bf16_tn_accum_f32(int M, int N, int total_rows, int num_experts, const int* d_counts,
                                           const int* d_offsets, const uint16_t* d_A, int lda,
                                           const uint16_t* d_B, int ldb, float* d_C, cf_stream_t stream);

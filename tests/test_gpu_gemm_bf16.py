@@ -111,6 +111,35 @@ def test_gemm_bf16_more_tiles_than_workgroups_exact(cf, dev, K):
     assert np.array_equal(bf16_bits(Cb), orc.bf16_from_f32(want))
 
 
+def test_grouped_bf16_weight_gradient_cuts_row_ranges_at_total_rows(cf, dev):
+    """Counts that run past the rows the compact buffers hold (a caller passing an upper bound that is too small):
+    the row ranges are cut at total_rows, nothing beyond the buffers is read (NaN rows lie behind them)."""
+    case("grouped bf16 wgrad, counts beyond total_rows")
+    rng = np.random.default_rng(12)
+    E, H, Ie = 4, 136, 264
+    counts = np.array([100, 70, 90, 30], np.int32)
+    offsets = orc.moe_expert_offsets(counts)
+    total = 200                                         # cuts expert 2 after 30 rows and expert 3 entirely
+    d_out, act = rand_bf16(rng, (total, H), 1e-2), rand_bf16(rng, (total, Ie))
+    nan_rows = np.full((96, max(H, Ie)), 0x7fc0, np.uint16)
+    a_dev = dev_bf16(np.concatenate([d_out, nan_rows[:, :H]]), dev)
+    b_dev = dev_bf16(np.concatenate([act, nan_rows[:, :Ie]]), dev)
+    g0 = rand_bf16(rng, (E, H, Ie), 1e-2)
+    g_bf = dev_bf16(g0, dev)
+    dc, do = dev_arr(counts, dev), dev_arr(offsets, dev)
+    cf.cf_moe_grouped_gemm_bf16_tn_accum_bf16(H, Ie, total, E, dc, do, a_dev, H, b_dev, Ie, g_bf, stream())
+    torch.cuda.synchronize()
+    got = bf16_bits(g_bf)
+    for e in range(E):
+        o = min(int(offsets[e]), total)
+        n = min(int(counts[e]), total - o)
+        if n == 0:
+            assert np.array_equal(got[e], g0[e]), f"expert {e}"
+            continue
+        ref = orc.bf16_to_f32(g0[e]).astype(np.float64) + orc.gemm_bf16_tn_ref(d_out[o:o + n], act[o:o + n])
+        check_bf16_out(got[e], ref, absdot(d_out[o:o + n], act[o:o + n], tn=True), f"g_out expert {e}")
+
+
 def test_grouped_bf16_weight_gradient_leaves_empty_experts_alone(cf, dev):
     """An expert without rows adds nothing: its block of C keeps its bits, negative zeros included (a sum with an
     all-zero product would turn them into +0), also when such experts sit between experts of a few rows each."""

@@ -2066,8 +2066,9 @@ void k_gemm_nt_block_ring(const GemmArgs p) {
     // One K-tile g at position kt of its tile.  FOLD: the previous K-tile's partial products are folded, each tile
     // right before the MFMA that overwrites it (not for a tile's first K-tile).  After the barrier the copies of
     // K-tile g+3 (K offset dk0, position dkt of its tile) start.
-    auto ktile = [&](auto fold_c, int kt, int parity, int dk0, int dkt) {
-        constexpr bool FOLD = decltype(fold_c)::value != 0;
+    // END: a tile's last K-tile: its copies are left to the caller (the epilogue stages the output in the stage they go to).
+    auto ktile = [&](auto fold_c, auto end_c, int kt, int parity, int dk0, int dkt) {
+        constexpr bool FOLD = decltype(fold_c)::value != 0, END = decltype(end_c)::value != 0;
         // step (g,0): 4 MFMAs from a zero C, the operand reads of (g,1)
         static_for<0, 4>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
@@ -2095,7 +2096,7 @@ void k_gemm_nt_block_ring(const GemmArgs p) {
             static_for<0, 3>([&](auto jc) {
                 constexpr int j = (i - 1) * 3 + decltype(jc)::value;
                 if constexpr (j < 8) read_one(s1, C0{}, std::integral_constant<int, j < 8 ? j : 0>{});
-                if constexpr (j < 7) copy_one(s0, i0, dk0, dkt, std::integral_constant<int, j < 7 ? j : 0>{});
+                if constexpr (j < 7 && !END) copy_one(s0, i0, dk0, dkt, std::integral_constant<int, j < 7 ? j : 0>{});
             });
             __builtin_amdgcn_sched_barrier(0);
         });
@@ -2133,41 +2134,81 @@ void k_gemm_nt_block_ring(const GemmArgs p) {
 
     const int khalf4 = khalf * 4;
     const bool vec_ok = (p.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(p.C) & 7u) == 0);
+    const bool lines_ok = (p.ldc % 8 == 0) && ((reinterpret_cast<uintptr_t>(p.C) & 15u) == 0);        // whole 128-byte lines of C per row of a wavefront's tile
     for (int seq = 0; seq < my_tiles; ++seq) {
         int m0, n0;
         tile_at(seq, m0, n0);
         const int parity = seq & 1;
-        ktile(C0{}, 0, parity, dkt * BK, dkt);
+        ktile(C0{}, C0{}, 0, parity, dkt * BK, dkt);
         rotate(); advance_copy();
-        for (int kt = 1; kt < ktiles; ++kt) {
-            ktile(C1{}, kt, parity, dkt * BK, dkt);
+        for (int kt = 1; kt + 1 < ktiles; ++kt) {
+            ktile(C1{}, C0{}, kt, parity, dkt * BK, dkt);
             rotate(); advance_copy();
         }
-        // the last K-tile's partial products, then the sums leave as bf16: a lane holds four consecutive columns per quad
+        ktile(C1{}, C1{}, ktiles - 1, parity, dkt * BK, dkt);
+        // the last K-tile's partial products, then the sums leave as bf16
         static_for<0, 4>([&](auto ic) { fold_plain(f, ic); });
+        if (lines_ok) {
+            // A lane holds four consecutive columns of one row per quad: written from there a store instruction would
+            // cover 32 rows with 16 bytes each.  The wavefront turns its 64 x 64 outputs round in LDS instead, 32 rows
+            // at a time (128-byte rows, 16-byte chunks xor-swizzled by row), and stores whole lines, eight rows per
+            // instruction.  The staging area is the 4 KiB of the stage just finished that this wavefront's own weight
+            // copies of the K-tile three ahead go to: nobody reads that stage after the K-tile's barrier, and the
+            // copies are issued below, in program order after the last staging read.
+            uint8_t* stg = smem + s0 + kBsX + wave * (32 * BK);
+            const int srow = lane & 31, rrow = lane >> 3, rchunk = lane & 7;
+            typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 #pragma unroll
-        for (int b = 0; b < 2; ++b) {
-            const int m = m0 + wm * 64 + b * 32 + (lane & 31);
+            for (int b = 0; b < 2; ++b) {
 #pragma unroll
-            for (int a = 0; a < 2; ++a)
+                for (int a = 0; a < 2; ++a)
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int n = n0 + wn * 64 + a * 32 + g * 8 + khalf4;
-                    const uint32_t o01 = pack_bf16x2_hw(sum[a][b][g * 4 + 0], sum[a][b][g * 4 + 1]);
-                    const uint32_t o23 = pack_bf16x2_hw(sum[a][b][g * 4 + 2], sum[a][b][g * 4 + 3]);
-                    if (m < p.M) {
-                        uint16_t* crow = p.C + static_cast<size_t>(m) * p.ldc + n;
-                        if (vec_ok) {
-                            *reinterpret_cast<uint2*>(crow) = make_uint2(o01, o23);
-                        } else {
-                            crow[0] = static_cast<uint16_t>(o01 & 0xffffu); crow[1] = static_cast<uint16_t>(o01 >> 16);
-                            crow[2] = static_cast<uint16_t>(o23 & 0xffffu); crow[3] = static_cast<uint16_t>(o23 >> 16);
-                        }
+                    for (int g = 0; g < 4; ++g) {
+                        const uint32_t o01 = pack_bf16x2_hw(sum[a][b][g * 4 + 0], sum[a][b][g * 4 + 1]);
+                        const uint32_t o23 = pack_bf16x2_hw(sum[a][b][g * 4 + 2], sum[a][b][g * 4 + 3]);
+                        *reinterpret_cast<uint2*>(stg + srow * 128 + (((a * 4 + g) ^ (srow & 7)) << 4) + khalf * 8) = make_uint2(o01, o23);
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) sum[a][b][g * 4 + q] = 0.0f;
                     }
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) sum[a][b][g * 4 + q] = 0.0f;
+                for (int t = 0; t < 4; ++t) {
+                    const int row = rrow + 8 * t;
+                    const uint4 v = *reinterpret_cast<const uint4*>(stg + row * 128 + ((rchunk ^ (row & 7)) << 4));
+                    const int m = m0 + wm * 64 + b * 32 + row;
+                    if (m < p.M) {
+                        const u32x4 vv = {v.x, v.y, v.z, v.w};
+                        *reinterpret_cast<u32x4*>(p.C + static_cast<size_t>(m) * p.ldc + n0 + wn * 64 + rchunk * 8) = vv;
+                    }
                 }
+            }
+        } else {
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                const int m = m0 + wm * 64 + b * 32 + (lane & 31);
+#pragma unroll
+                for (int a = 0; a < 2; ++a)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const int n = n0 + wn * 64 + a * 32 + g * 8 + khalf4;
+                        const uint32_t o01 = pack_bf16x2_hw(sum[a][b][g * 4 + 0], sum[a][b][g * 4 + 1]);
+                        const uint32_t o23 = pack_bf16x2_hw(sum[a][b][g * 4 + 2], sum[a][b][g * 4 + 3]);
+                        if (m < p.M) {
+                            uint16_t* crow = p.C + static_cast<size_t>(m) * p.ldc + n;
+                            if (vec_ok) {
+                                *reinterpret_cast<uint2*>(crow) = make_uint2(o01, o23);
+                            } else {
+                                crow[0] = static_cast<uint16_t>(o01 & 0xffffu); crow[1] = static_cast<uint16_t>(o01 >> 16);
+                                crow[2] = static_cast<uint16_t>(o23 & 0xffffu); crow[3] = static_cast<uint16_t>(o23 >> 16);
+                            }
+                        }
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) sum[a][b][g * 4 + q] = 0.0f;
+                    }
+            }
         }
+        // the copies the last K-tile left out
+        static_for<0, 7>([&](auto jc) { copy_one(s0, i0, dkt * BK, dkt, jc); });
+        rotate(); advance_copy();
     }
     // the copies started past the end of the stream must have landed before the LDS is given back
     __builtin_amdgcn_s_waitcnt(kWaitVm0);

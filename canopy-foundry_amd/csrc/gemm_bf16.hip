@@ -532,7 +532,7 @@ void k_gemm_bf16(const BfArgs p) {
                 const uint32_t c_lane = col_w + 8 * (lane & 15) < p.N ? (lane >> 4) * static_cast<uint32_t>(p.ldc) * 2u + (lane & 15) * 16u : kOutside;
                 const uint32_t c_rows4 = 4u * static_cast<uint32_t>(p.ldc) * 2u;
                 if constexpr (OUT == OUT_STORE_BF16) {
-                    constexpr int PB = 128 * 2 + 32;                    // staged row: 128 bf16 + pad
+                    constexpr int PB = 128 * 2 + 16;                    // staged row: 128 bf16 + pad (sixteen rows x two quads of a write: 64 banks)
                     static_assert(64 * PB <= kStage / 4, "two passes of 64 rows");
 #pragma unroll
                     for (int half = 0; half < 2; ++half) {
@@ -552,7 +552,7 @@ void k_gemm_bf16(const BfArgs p) {
                     }
                 } else {
                     // fp32 sum of the old value and the product, one rounding (cublasGemmEx with a bf16 C, beta = 1)
-                    constexpr int PF = 128 * 4 + 32;                    // staged row: 128 fp32 + pad
+                    constexpr int PF = 128 * 4 + 16;                    // staged row: 128 fp32 + pad (the sixteen rows of a quad column: 64 banks)
                     static_assert(32 * PF <= kStage / 4, "four passes of 32 rows");
                     // the next pass's rows of C are requested before this pass's are added to and stored
                     u32x4 c[8], c_ahead[8];
@@ -589,7 +589,7 @@ void k_gemm_bf16(const BfArgs p) {
                 }
             } else {
                 // fp32 C.  A lane's piece: four columns (16 bytes) of row lane / 32 of every pair of rows
-                constexpr int PF = 128 * 4 + 32;
+                constexpr int PF = 128 * 4 + 16;
                 static_assert(32 * PF <= kStage / 4, "four passes of 32 rows");
                 const uint32_t c_lane = col_w + 4 * (lane & 31) < p.N ? (lane >> 5) * static_cast<uint32_t>(p.ldc) * 4u + (lane & 31) * 16u : kOutside;
                 const uint32_t c_rows2 = 2u * static_cast<uint32_t>(p.ldc) * 4u;

@@ -427,6 +427,17 @@ def main():
     mfma16("grouped bf16 wgrad: g_in += d_pre^T . x (tn, bf16 C)", f"{Ie}x{H}x~{total // E} x{E}", fl,
            lambda: cf.cf_moe_grouped_gemm_bf16_tn_accum_bf16(Ie, H, total, E, counts, offs, gpost, Ie, xg, H, g_in, st))
 
+    # the same kernel, dense, on constant operands (no data toggling: full clock, below the power cap) with ten output
+    # tiles per workgroup at two K: the difference is the K loop's time, the rest the per-tile cost
+    if args.only is None or "bf16 dense" in args.only or args.only in "bf16 dense":
+        Md, Nd = 16384, 10240
+        for Kd in (2048, 8192):
+            ad = torch.ones((Md, Kd), dtype=torch.bfloat16, device=dev); bd = torch.ones((Kd, Nd), dtype=torch.bfloat16, device=dev)
+            cd = torch.empty((Md, Nd), dtype=torch.bfloat16, device=dev)
+            mfma16(f"bf16 dense nn, constant operands, K = {Kd}", f"{Md}x{Nd}x{Kd}", 2.0 * Md * Nd * Kd,
+                   lambda: cf.cf_gemm_bf16_nn(Md, Nd, Kd, ad, Kd, bd, Nd, cd, Nd, st))
+            del ad, bd, cd
+
     # the whole selected-expert backward of the GELU bank in one call: FP8 recompute, route gradient, four bf16 GEMMs,
     # gelu_backward, scatter-add (16 launches per expert in the reference's host loop)
     szb = ctypes.c_size_t(0)

@@ -111,6 +111,77 @@ def test_gemm_bf16_more_tiles_than_workgroups_exact(cf, dev, K):
     assert np.array_equal(bf16_bits(Cb), orc.bf16_from_f32(want))
 
 
+def test_gemm_bf16_seeded_shapes_exact(cf, dev):
+    """Forty seeded shapes (ragged rows, columns and k, padded strides; some with several tiles per workgroup), small
+    integers: the dense forms against numpy, to the bit."""
+    rng = np.random.default_rng(2024)
+    for it in range(40):
+        M = int(rng.integers(1, 900)); N = 8 * int(rng.integers(1, 90)); K = 8 * int(rng.integers(1, 60))
+        pa, pb, pc = (8 * int(rng.integers(0, 3)) for _ in range(3))
+        case(f"bf16 nn seeded {it}: {M}x{N}x{K} pads {pa} {pb} {pc}")
+        a = rng.integers(-4, 5, (M, K)).astype(np.float32)
+        b = rng.integers(-3, 4, (K, N)).astype(np.float32)
+        C = torch.full((M, N + pc), float("nan"), dtype=torch.bfloat16, device=dev)
+        cf.cf_gemm_bf16_nn(M, N, K, dev_bf16(padded(orc.bf16_from_f32(a), K + pa), dev), K + pa,
+                           dev_bf16(padded(orc.bf16_from_f32(b), N + pb), dev), N + pb, C, N + pc, stream())
+        torch.cuda.synchronize()
+        got = bf16_bits(C)
+        assert np.array_equal(got[:, :N], orc.bf16_from_f32(a @ b)), f"nn {M}x{N}x{K}"
+        assert np.all((got[:, N:] & 0x7fff) > 0x7f80)
+        # tn with the contraction over M rows: C2[K, N2] += a^T . b2, any M
+        N2 = 8 * int(rng.integers(1, 60))
+        b2 = rng.integers(-3, 4, (M, N2)).astype(np.float32)
+        c0 = rng.integers(-50, 51, (K, N2)).astype(np.float32)
+        Cf = torch.from_numpy(c0).to(dev)
+        Cb = dev_bf16(orc.bf16_from_f32(c0), dev)
+        a_dev, b2_dev = dev_bf16(padded(orc.bf16_from_f32(a), K + pa), dev), dev_bf16(orc.bf16_from_f32(b2), dev)
+        cf.cf_gemm_bf16_tn_accum_f32(K, N2, M, a_dev, K + pa, b2_dev, N2, Cf, N2, stream())
+        cf.cf_gemm_bf16_tn_accum_bf16(K, N2, M, a_dev, K + pa, b2_dev, N2, Cb, N2, stream())
+        torch.cuda.synchronize()
+        want = c0 + a.T @ b2
+        assert np.array_equal(host(Cf), want), f"tn f32 {K}x{N2}x{M}"
+        assert np.array_equal(bf16_bits(Cb), orc.bf16_from_f32(want)), f"tn bf16 {K}x{N2}x{M}"
+
+
+def test_grouped_bf16_seeded_routings_exact(cf, dev):
+    """Twenty seeded expert banks (1 to 12 experts of 0 to 400 rows, ragged widths), small integers: both grouped forms
+    against numpy per expert, to the bit."""
+    rng = np.random.default_rng(77)
+    for it in range(20):
+        E = int(rng.integers(1, 13)); H = 8 * int(rng.integers(1, 50)); Ie = 8 * int(rng.integers(1, 70))
+        counts = rng.integers(0, 401, E).astype(np.int32)
+        counts[rng.integers(0, E)] = 0
+        offsets = orc.moe_expert_offsets(counts)
+        total = int(counts.sum()) + int(rng.integers(0, 300))
+        case(f"grouped bf16 seeded {it}: E={E} H={H} Ie={Ie} total={total}")
+        if total == 0:
+            continue
+        d_out = rng.integers(-4, 5, (total, H)).astype(np.float32)
+        act = rng.integers(-3, 4, (total, Ie)).astype(np.float32)
+        w = rng.integers(-3, 4, (E, H, Ie)).astype(np.float32)
+        g0 = rng.integers(-40, 41, (E, H, Ie)).astype(np.float32)
+        dc, do = dev_arr(counts, dev), dev_arr(offsets, dev)
+        ws, ws_bytes = workspace(cf, dev, total, E)
+        d_act = torch.full((total, Ie), float("nan"), dtype=torch.bfloat16, device=dev)
+        cf.cf_moe_grouped_gemm_bf16_nn(total, Ie, H, E, dc, do, dev_bf16(orc.bf16_from_f32(d_out), dev), H, dev_bf16(orc.bf16_from_f32(w), dev),
+                                       d_act, Ie, ws, ws_bytes, stream())
+        g_bf = dev_bf16(orc.bf16_from_f32(g0), dev)
+        g_f32 = torch.from_numpy(g0.copy()).to(dev)
+        cf.cf_moe_grouped_gemm_bf16_tn_accum_bf16(H, Ie, total, E, dc, do, dev_bf16(orc.bf16_from_f32(d_out), dev), H, dev_bf16(orc.bf16_from_f32(act), dev), Ie, g_bf, stream())
+        cf.cf_moe_grouped_gemm_bf16_tn_accum_f32(H, Ie, total, E, dc, do, dev_bf16(orc.bf16_from_f32(d_out), dev), H, dev_bf16(orc.bf16_from_f32(act), dev), Ie, g_f32, stream())
+        torch.cuda.synchronize()
+        got_act, got_g, got_gf = bf16_bits(d_act), bf16_bits(g_bf), host(g_f32)
+        filled = int(counts.sum())
+        assert np.all((got_act[filled:] & 0x7fff) > 0x7f80), "rows past the experts' lists were written"
+        for e in range(E):
+            n, o = int(counts[e]), int(offsets[e])
+            want_g = g0[e] + d_out[o:o + n].T @ act[o:o + n]
+            assert np.array_equal(got_gf[e], want_g), f"bank {it} expert {e} g (fp32)"
+            assert np.array_equal(got_g[e], orc.bf16_from_f32(want_g)), f"bank {it} expert {e} g (bf16)"
+            if n:
+                assert np.array_equal(got_act[o:o + n], orc.bf16_from_f32(d_out[o:o + n] @ w[e])), f"bank {it} expert {e} d_act"
+
+
 def test_grouped_bf16_weight_gradient_cuts_row_ranges_at_total_rows(cf, dev):
     """Counts that run past the rows the compact buffers hold (a caller passing an upper bound that is too small):
     the row ranges are cut at total_rows, nothing beyond the buffers is read (NaN rows lie behind them)."""

@@ -619,6 +619,27 @@ def test_gemm_block_scaled(cf, dev, M, N, K, flags):
     orc.assert_gemm_close(got, ref, absdot, what=f"block {M}x{N}x{K}", acc=orc.ACC_FP32 * 4 if flags else orc.ACC_MFMA)
 
 
+@pytest.mark.parametrize("pad", [4, 2, 8])
+def test_gemm_block_scaled_row_strides_of_c(cf, dev, pad):
+    """The persistent block-scaled kernel stores whole 128-byte lines when C's rows allow 16-byte accesses and falls
+    back to 8-byte or 2-byte stores otherwise: the same bits in all three, and the padding of C's rows untouched."""
+    case(f"gemm block-scaled, ldc = N + {pad}")
+    M, N, K = 300, 512, 640
+    rng = np.random.default_rng(pad)
+    xb = orc.bf16_from_f32(rng.standard_normal((M, K)).astype(np.float32))
+    wb = orc.bf16_from_f32((0.02 * rng.standard_normal((N, K))).astype(np.float32))
+    xq, xs, xd = block_quant_gpu(cf, dev, dev_bf16(xb, dev), "1x128")
+    wq, ws, wd = block_quant_gpu(cf, dev, dev_bf16(wb, dev), "128x128")
+    C0 = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=dev)
+    cf.cf_fp8_gemm_nt_bf16_ex(M, N, K, xq, K, 0, xd, wq, K, wd, BLOCK, EPI_NONE, None, None, None, C0, N, 0, stream())
+    C1 = torch.full((M, N + pad), float("nan"), dtype=torch.bfloat16, device=dev)
+    cf.cf_fp8_gemm_nt_bf16_ex(M, N, K, xq, K, 0, xd, wq, K, wd, BLOCK, EPI_NONE, None, None, None, C1, N + pad, 0, stream())
+    torch.cuda.synchronize()
+    got = bf16_bits(C1)
+    assert np.array_equal(got[:, :N], bf16_bits(C0))
+    assert np.all((got[:, N:] & 0x7fff) > 0x7f80)
+
+
 def test_config3_block_scaled_full_size_sampled(cf, dev):
     """M=4096, N=7168, K=7168; activations 1x128 groups, weights 128x128 blocks, fp32 scale tensors."""
     case("config 3 block-scaled, full size")

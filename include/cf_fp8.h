@@ -403,8 +403,9 @@ int cf_fp8_grouped_gemm_nt_bf16_static(int total_rows, int N, int K, int num_exp
  * forms run every expert in one launch over the forward's saved counts / offsets, the experts' rows
  * lying back to back in compact buffers (expert e owns rows offsets[e] .. offsets[e] + counts[e]).
  * fp32 accumulation on the matrix cores, one rounding to bf16.  Needs 16-byte aligned operands, row
- * strides that are multiples of 8 elements, N % 8 == 0, and K % 8 == 0 (nn) or M % 8 == 0 (tn); the
- * contraction length of the tn forms (an expert's row count) is arbitrary. */
+ * strides that are multiples of 8 elements (C: of 4, below 2^21), N % 8 == 0, and K % 8 == 0 (nn) or
+ * M % 8 == 0 (tn); the contraction length of the tn forms (an expert's row count) is arbitrary.
+ * Shapes outside these return CF_ERR_UNSUPPORTED. */
 
 /* C[M,N] = A[M,K] . B[K,N]   (gemm_bf16 with alpha = 1, beta = 0, src/trainer.cu:3069-3090) */
 int cf_gemm_bf16_nn(int M, int N, int K, const uint16_t* d_A, int lda, const uint16_t* d_B, int ldb,

@@ -373,6 +373,7 @@ def test_gemm_bf16_argument_errors(cf, dev):
     assert cf.raw_cf_gemm_bf16_nn(8, 12, 8, p(a), 8, p(a), 16, p(c), 16, None) == -2        # N % 8
     assert cf.raw_cf_gemm_bf16_nn(8, 8, 8, p(a) + 2, 8, p(a), 8, p(c), 8, None) == -2       # unaligned operand
     assert cf.raw_cf_gemm_bf16_nn(0, 8, 8, p(a), 8, p(a), 8, p(c), 8, None) == 0
+    assert cf.raw_cf_gemm_bf16_nn(1, 8, 8, p(a), 8, p(a), 8, p(c), 1 << 21, None) == -2     # a row stride of C the epilogue's 32-bit offsets do not cover
     assert cf.raw_cf_gemm_bf16_tn_accum_bf16(12, 8, 8, p(a), 16, p(a), 8, p(c), 8, None) == -2   # M % 8
     assert cf.raw_cf_gemm_bf16_tn_accum_bf16(8, 8, 0, p(a), 8, p(a), 8, p(c), 8, None) == 0
     torch.cuda.synchronize()
